@@ -1,0 +1,65 @@
+"""Compile the HIP sources under ``csrc/`` into ``csrc/libchr_nf4_amd.so`` for gfx950.
+
+hipcc cross-compiles without a GPU, so this runs anywhere the ROCm toolchain is
+installed.  The library is built in-tree; nothing is installed.
+"""
+
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+
+CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
+LIB = os.path.join(CSRC, "libchr_nf4_amd.so")
+SOURCES = ("nf4_gemv.hip", "nf4_attn.hip", "nf4_gemm.hip")
+HEADERS = ("nf4_common.h", os.path.join("..", "..", "include", "chr_nf4_amd.h"))
+
+#: -packed-fp32-ops is switched off on purpose: the kernels are written for
+#: scalar fp32 VALU ops only.
+HIPCC_FLAGS = (
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-shared",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+)
+
+
+def hipcc() -> str:
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found; the NF4 kernels need the ROCm toolchain to build")
+    return exe
+
+
+def stale() -> bool:
+    if not os.path.exists(LIB):
+        return True
+    t = os.path.getmtime(LIB)
+    deps = [os.path.join(CSRC, s) for s in SOURCES + HEADERS]
+    return any(os.path.getmtime(d) > t for d in deps)
+
+
+def build(force: bool = True, verbose: bool = False) -> str:
+    """Run hipcc.  ``force=False`` skips the compile when the library is newer
+    than every source."""
+    if not force and not stale():
+        return LIB
+    cmd = [hipcc(), *HIPCC_FLAGS, "-o", LIB, *[os.path.join(CSRC, s) for s in SOURCES]]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    # hipcc's host pass does not know the device-only target feature and says so
+    # once per source; that line is noise, everything else is shown.
+    noise = "is not a recognized feature for this target"
+    err = "\n".join(l for l in proc.stderr.splitlines() if noise not in l)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{err}")
+    if verbose and err.strip():
+        print(err, file=sys.stderr)
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build(force=True, verbose=True))

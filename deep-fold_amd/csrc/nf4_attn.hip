@@ -1,0 +1,489 @@
+// Decode attention for gfx950: split-KV flash-decode over the valid prefix of a
+// static bf16 KV cache with fused rotate-half RoPE and cache write, the merge of
+// the split partials, and the standalone RoPE + cache write.
+// Replaces chr_nf4_attn / chr_nf4_rope_kv (gpu/nf4/nf4_gemv.cu:497-727, 926-994).
+//
+// One 64-lane wavefront serves one (query head, split).  A cache row of hd
+// values is read by LPT = hd/8 lanes with one 16-byte load each, so a wavefront
+// walks 64/LPT time steps per iteration (four at hd = 128); each lane group
+// keeps its own online-softmax state and the groups are folded once at the end.
+// Split s owns the time steps t with t % n_split == s.
+//
+// Numerics (gpu/nf4/nf4_gemv.cu:599-727): the rotated query and the rotated
+// current key stay fp32; older keys and all values come from the bf16 cache;
+// running max starts at -1e30; exp is the fast hardware exponential.
+
+#include "nf4_common.h"
+
+namespace chr {
+namespace {
+
+constexpr float kNegBig = -1.0e30f;
+
+__device__ __forceinline__ void widen8(const uint4 v, float *f) {
+  f[0] = bf16_lo(v.x);
+  f[1] = bf16_hi(v.x);
+  f[2] = bf16_lo(v.y);
+  f[3] = bf16_hi(v.y);
+  f[4] = bf16_lo(v.z);
+  f[5] = bf16_hi(v.z);
+  f[6] = bf16_lo(v.w);
+  f[7] = bf16_hi(v.w);
+}
+
+__device__ __forceinline__ uint4 narrow8(const float *f) {
+  uint4 v;
+  v.x = f32_to_bf16(f[0]) | (static_cast<uint32_t>(f32_to_bf16(f[1])) << 16);
+  v.y = f32_to_bf16(f[2]) | (static_cast<uint32_t>(f32_to_bf16(f[3])) << 16);
+  v.z = f32_to_bf16(f[4]) | (static_cast<uint32_t>(f32_to_bf16(f[5])) << 16);
+  v.w = f32_to_bf16(f[6]) | (static_cast<uint32_t>(f32_to_bf16(f[7])) << 16);
+  return v;
+}
+
+// Rotate-half on the eight dims [d0, d0+8) of a head vector `t` (bf16 in
+// memory), fp32 result.  half = hd/2; d0 is a multiple of 8 and so never
+// straddles the half boundary.  out[d] = t[d]*cos[d] - t[d+half]*sin[d] for
+// d < half, t[d]*cos[d] + t[d-half]*sin[d] otherwise.
+__device__ __forceinline__ void rope8(const uint16_t *t, const uint16_t *cos, const uint16_t *sin,
+                                      int d0, int half, float *out) {
+  float a[8], b[8], c[8], s[8];
+  const bool low = d0 < half;
+  const int partner = low ? d0 + half : d0 - half;
+  widen8(*reinterpret_cast<const uint4 *>(t + d0), a);
+  widen8(*reinterpret_cast<const uint4 *>(t + partner), b);
+  widen8(*reinterpret_cast<const uint4 *>(cos + d0), c);
+  widen8(*reinterpret_cast<const uint4 *>(sin + d0), s);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float rot = low ? -b[i] : b[i];
+    out[i] = a[i] * c[i] + rot * s[i];
+  }
+}
+
+struct AttnArgs {
+  const uint16_t *q;
+  const uint16_t *k_cache;
+  const uint16_t *v_cache;
+  float *m_s;
+  float *l_s;
+  float *o_s;
+  const int32_t *valid_len;
+  const uint16_t *k_act;
+  const uint16_t *v_act;
+  const uint16_t *cos;
+  const uint16_t *sin;
+  const int64_t *position;
+  int n_q, n_kv, hd, n_split, max_seq;
+  float scale;
+};
+
+// LPT lanes per time step, 8 dims per lane: hd == 8*LPT.
+template <int LPT>
+__global__ __launch_bounds__(kWave) void attn_flash(const AttnArgs a) {
+  constexpr int TPW = kWave / LPT;  // time steps per wavefront iteration
+  const int head = blockIdx.x / a.n_split;
+  const int split = blockIdx.x % a.n_split;
+  const int lane = threadIdx.x;
+  const int li = lane % LPT;  // which 8 dims of the head
+  const int grp = lane / LPT; // which time step of the iteration
+  const int hd = a.hd;
+  const int d0 = li * 8;
+  const int n_rep = a.n_q / a.n_kv;
+  const int kv_head = head / n_rep;
+  const int vl = min(*a.valid_len, a.max_seq);
+
+  float qf[8];
+  float kcur[8];
+  float vcur[8];
+  int pos = -1;
+  bool fuse = false;
+  const uint16_t *qh = a.q + static_cast<size_t>(head) * hd;
+  bool rotated = false;
+  if (a.cos != nullptr && a.sin != nullptr && a.position != nullptr) {
+    const long long p = *a.position;
+    if (p >= 0 && p < a.max_seq) {
+      pos = static_cast<int>(p);
+      const uint16_t *c = a.cos + static_cast<size_t>(pos) * hd;
+      const uint16_t *s = a.sin + static_cast<size_t>(pos) * hd;
+      rope8(qh, c, s, d0, hd / 2, qf);
+      rotated = true;
+      if (a.k_act != nullptr && a.v_act != nullptr) {
+        fuse = true;
+        const uint16_t *ka = a.k_act + static_cast<size_t>(kv_head) * hd;
+        const uint16_t *va = a.v_act + static_cast<size_t>(kv_head) * hd;
+        rope8(ka, c, s, d0, hd / 2, kcur);
+        const uint4 vraw = *reinterpret_cast<const uint4 *>(va + d0);
+        widen8(vraw, vcur);
+        // Exactly one wavefront per KV head stores the new cache row.
+        if (head == kv_head * n_rep && split == pos % a.n_split && grp == 0) {
+          const size_t off = (static_cast<size_t>(pos) * a.n_kv + kv_head) * hd + d0;
+          *reinterpret_cast<uint4 *>(const_cast<uint16_t *>(a.k_cache) + off) = narrow8(kcur);
+          *reinterpret_cast<uint4 *>(const_cast<uint16_t *>(a.v_cache) + off) = vraw;
+        }
+      }
+    }
+  }
+  if (!rotated) {
+    widen8(*reinterpret_cast<const uint4 *>(qh + d0), qf);
+  }
+
+  float m = kNegBig;
+  float l = 0.f;
+  float acc[8] = {};
+  const size_t row_stride = static_cast<size_t>(a.n_kv) * hd;
+  for (int t0 = split; t0 < vl; t0 += a.n_split * TPW) {
+    const int t = t0 + grp * a.n_split;
+    const bool live = t < vl;
+    const bool cur = fuse && t == pos;
+    float kf[8], vf[8];
+    if (live && !cur) {
+      const size_t off = static_cast<size_t>(t) * row_stride + static_cast<size_t>(kv_head) * hd + d0;
+      widen8(*reinterpret_cast<const uint4 *>(a.k_cache + off), kf);
+      widen8(*reinterpret_cast<const uint4 *>(a.v_cache + off), vf);
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        kf[i] = cur ? kcur[i] : 0.f;
+        vf[i] = cur ? vcur[i] : 0.f;
+      }
+    }
+    float dot = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      dot = fmaf(qf[i], kf[i], dot);
+    }
+    dot = group_sum<LPT>(dot) * a.scale;
+    if (live) {
+      const float m2 = fmaxf(m, dot);
+      const float alpha = __expf(m - m2);
+      const float e = __expf(dot - m2);
+      l = l * alpha + e;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        acc[i] = acc[i] * alpha + e * vf[i];
+      }
+      m = m2;
+    }
+  }
+
+  // Fold the TPW lane groups: lanes with equal li hold states of different
+  // time-step subsets.
+  if constexpr (TPW > 1) {
+    float mg = m;
+#pragma unroll
+    for (int off = LPT; off < kWave; off <<= 1) {
+      mg = fmaxf(mg, __shfl_xor(mg, off, kWave));
+    }
+    const float w = __expf(m - mg);
+    l *= w;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      acc[i] *= w;
+    }
+#pragma unroll
+    for (int off = LPT; off < kWave; off <<= 1) {
+      l += __shfl_xor(l, off, kWave);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        acc[i] += __shfl_xor(acc[i], off, kWave);
+      }
+    }
+    m = mg;
+  }
+
+  const size_t slot = static_cast<size_t>(head) * a.n_split + split;
+  if (lane == 0) {
+    a.m_s[slot] = m;
+    a.l_s[slot] = l;
+  }
+  if (grp == 0) {
+    float *oh = a.o_s + slot * hd + d0;
+    *reinterpret_cast<float4 *>(oh) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+    *reinterpret_cast<float4 *>(oh + 4) = make_float4(acc[4], acc[5], acc[6], acc[7]);
+  }
+}
+
+// Any hd <= 256: lane l owns dims l, l+64, l+128, l+192; one time step per
+// iteration.  Slow path for head sizes that are not 8 * 2^n.
+__global__ __launch_bounds__(kWave) void attn_flash_generic(const AttnArgs a) {
+  const int head = blockIdx.x / a.n_split;
+  const int split = blockIdx.x % a.n_split;
+  const int lane = threadIdx.x;
+  const int hd = a.hd;
+  const int half = hd / 2;
+  const int n_rep = a.n_q / a.n_kv;
+  const int kv_head = head / n_rep;
+  const int vl = min(*a.valid_len, a.max_seq);
+  const uint16_t *qh = a.q + static_cast<size_t>(head) * hd;
+
+  float qf[4] = {}, kcur[4] = {}, vcur[4] = {};
+  int pos = -1;
+  bool fuse = false;
+  bool rotated = false;
+  if (a.cos != nullptr && a.sin != nullptr && a.position != nullptr) {
+    const long long p = *a.position;
+    if (p >= 0 && p < a.max_seq) {
+      pos = static_cast<int>(p);
+      rotated = true;
+      const uint16_t *c = a.cos + static_cast<size_t>(pos) * hd;
+      const uint16_t *s = a.sin + static_cast<size_t>(pos) * hd;
+      fuse = a.k_act != nullptr && a.v_act != nullptr;
+      const uint16_t *ka = fuse ? a.k_act + static_cast<size_t>(kv_head) * hd : nullptr;
+      const uint16_t *va = fuse ? a.v_act + static_cast<size_t>(kv_head) * hd : nullptr;
+      const bool writer = fuse && head == kv_head * n_rep && split == pos % a.n_split;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int d = lane + 64 * i;
+        if (d < hd) {
+          const bool low = d < half;
+          const int pd = low ? d + half : d - half;
+          const float cd = bf16_to_f32(c[d]), sd = bf16_to_f32(s[d]);
+          const float tq = bf16_to_f32(qh[d]), pq = bf16_to_f32(qh[pd]);
+          qf[i] = tq * cd + (low ? -pq : pq) * sd;
+          if (fuse) {
+            const float tk = bf16_to_f32(ka[d]), pk = bf16_to_f32(ka[pd]);
+            kcur[i] = tk * cd + (low ? -pk : pk) * sd;
+            vcur[i] = bf16_to_f32(va[d]);
+            if (writer) {
+              const size_t off = (static_cast<size_t>(pos) * a.n_kv + kv_head) * hd + d;
+              const_cast<uint16_t *>(a.k_cache)[off] = f32_to_bf16(kcur[i]);
+              const_cast<uint16_t *>(a.v_cache)[off] = va[d];
+            }
+          }
+        }
+      }
+    }
+  }
+  if (!rotated) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int d = lane + 64 * i;
+      if (d < hd) {
+        qf[i] = bf16_to_f32(qh[d]);
+      }
+    }
+  }
+
+  float m = kNegBig, l = 0.f;
+  float acc[4] = {};
+  const size_t row_stride = static_cast<size_t>(a.n_kv) * hd;
+  for (int t = split; t < vl; t += a.n_split) {
+    const bool cur = fuse && t == pos;
+    const size_t off = static_cast<size_t>(t) * row_stride + static_cast<size_t>(kv_head) * hd;
+    float kf[4] = {}, vf[4] = {};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int d = lane + 64 * i;
+      if (d < hd) {
+        kf[i] = cur ? kcur[i] : bf16_to_f32(a.k_cache[off + d]);
+        vf[i] = cur ? vcur[i] : bf16_to_f32(a.v_cache[off + d]);
+      }
+    }
+    float dot = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      dot = fmaf(qf[i], kf[i], dot);
+    }
+    dot = wave_sum(dot) * a.scale;
+    const float m2 = fmaxf(m, dot);
+    const float alpha = __expf(m - m2);
+    const float e = __expf(dot - m2);
+    l = l * alpha + e;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      acc[i] = acc[i] * alpha + e * vf[i];
+    }
+    m = m2;
+  }
+  const size_t slot = static_cast<size_t>(head) * a.n_split + split;
+  if (lane == 0) {
+    a.m_s[slot] = m;
+    a.l_s[slot] = l;
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int d = lane + 64 * i;
+    if (d < hd) {
+      a.o_s[slot * hd + d] = acc[i];
+    }
+  }
+}
+
+// out[head] = sum_s a_s o_s / sum_s a_s l_s with a_s = exp(m_s - max m); an
+// empty split has m = -1e30 and l = 0, so its weight underflows to zero.
+__global__ __launch_bounds__(kWave) void attn_merge(const float *__restrict__ m_s,
+                                                    const float *__restrict__ l_s,
+                                                    const float *__restrict__ o_s,
+                                                    uint16_t *__restrict__ out, int hd,
+                                                    int n_split) {
+  const int head = blockIdx.x;
+  const int lane = threadIdx.x;
+  const float *mh = m_s + static_cast<size_t>(head) * n_split;
+  const float *lh = l_s + static_cast<size_t>(head) * n_split;
+  float m = kNegBig;
+  for (int s = 0; s < n_split; ++s) {
+    m = fmaxf(m, mh[s]);
+  }
+  float l = 0.f;
+  float acc[4] = {};
+  for (int s = 0; s < n_split; ++s) {
+    const float w = __expf(mh[s] - m);
+    l += w * lh[s];
+    const float *oh = o_s + (static_cast<size_t>(head) * n_split + s) * hd;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int d = lane + 64 * i;
+      if (d < hd) {
+        acc[i] += w * oh[d];
+      }
+    }
+  }
+  uint16_t *dst = out + static_cast<size_t>(head) * hd;
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int d = lane + 64 * i;
+    if (d < hd) {
+      dst[d] = f32_to_bf16(l > 0.f ? acc[i] * inv : 0.f);
+    }
+  }
+}
+
+// Standalone RoPE + cache write: one wavefront per head (q heads first, then kv).
+__global__ __launch_bounds__(kWave) void rope_kv(uint16_t *__restrict__ q, uint16_t *__restrict__ k,
+                                                 const uint16_t *__restrict__ v,
+                                                 uint16_t *__restrict__ k_cache,
+                                                 uint16_t *__restrict__ v_cache,
+                                                 const uint16_t *__restrict__ cos,
+                                                 const uint16_t *__restrict__ sin,
+                                                 const int64_t *__restrict__ position, int n_q,
+                                                 int n_kv, int hd, int max_seq) {
+  const long long p = *position;
+  if (p < 0 || p >= max_seq) {
+    return;
+  }
+  const int pos = static_cast<int>(p);
+  const int hid = blockIdx.x;
+  const bool is_q = hid < n_q;
+  const int head = is_q ? hid : hid - n_q;
+  uint16_t *vec = (is_q ? q : k) + static_cast<size_t>(head) * hd;
+  const uint16_t *c = cos + static_cast<size_t>(pos) * hd;
+  const uint16_t *s = sin + static_cast<size_t>(pos) * hd;
+  const int half = hd / 2;
+  // Read both halves before either is overwritten.
+  float lo[2], hi[2];
+  for (int i = 0; i < 2; ++i) {
+    const int d = threadIdx.x + 64 * i;
+    if (d < half) {
+      const float t0 = bf16_to_f32(vec[d]);
+      const float t1 = bf16_to_f32(vec[d + half]);
+      lo[i] = t0 * bf16_to_f32(c[d]) + (-t1) * bf16_to_f32(s[d]);
+      hi[i] = t1 * bf16_to_f32(c[d + half]) + t0 * bf16_to_f32(s[d + half]);
+    }
+  }
+  const size_t off = (static_cast<size_t>(pos) * n_kv + head) * hd;
+  for (int i = 0; i < 2; ++i) {
+    const int d = threadIdx.x + 64 * i;
+    if (d < half) {
+      const uint16_t a = f32_to_bf16(lo[i]);
+      const uint16_t b = f32_to_bf16(hi[i]);
+      vec[d] = a;
+      vec[d + half] = b;
+      if (!is_q) {
+        k_cache[off + d] = a;
+        k_cache[off + d + half] = b;
+        v_cache[off + d] = v[static_cast<size_t>(head) * hd + d];
+        v_cache[off + d + half] = v[static_cast<size_t>(head) * hd + d + half];
+      }
+    }
+  }
+}
+
+}  // namespace
+}  // namespace chr
+
+using namespace chr;
+
+extern "C" int chr_nf4_rope_kv(void *q, void *k, const void *v, void *k_cache, void *v_cache,
+                               const void *cos, const void *sin, const void *position,
+                               int32_t n_q, int32_t n_kv, int32_t hd, int32_t max_seq,
+                               void *stream) {
+  if (q == nullptr || k == nullptr || v == nullptr || k_cache == nullptr || v_cache == nullptr ||
+      cos == nullptr || sin == nullptr || position == nullptr) {
+    return -1;
+  }
+  if (n_q < 1 || n_kv < 1 || hd < 2 || (hd & 1) != 0 || hd > 256 || max_seq < 1) {
+    return -3;
+  }
+  rope_kv<<<dim3(static_cast<unsigned>(n_q + n_kv)), dim3(kWave), 0,
+            static_cast<hipStream_t>(stream)>>>(
+      static_cast<uint16_t *>(q), static_cast<uint16_t *>(k), static_cast<const uint16_t *>(v),
+      static_cast<uint16_t *>(k_cache), static_cast<uint16_t *>(v_cache),
+      static_cast<const uint16_t *>(cos), static_cast<const uint16_t *>(sin),
+      static_cast<const int64_t *>(position), n_q, n_kv, hd, max_seq);
+  return launch_rc();
+}
+
+extern "C" int chr_nf4_attn(const void *q, const void *k, const void *v, void *out,
+                            const void *valid_len, float *ws, int32_t n_q, int32_t n_kv,
+                            int32_t hd, int32_t n_split, float scale, void *stream,
+                            const void *k_act, const void *v_act, const void *cos,
+                            const void *sin, const void *position, int32_t max_seq) {
+  if (q == nullptr || k == nullptr || v == nullptr || out == nullptr || valid_len == nullptr ||
+      ws == nullptr) {
+    return -1;
+  }
+  if (n_q < 1 || n_kv < 1 || hd < 1 || hd > 256 || (n_q % n_kv) != 0 || n_split < 1 ||
+      n_split > 64 || max_seq < 1) {
+    return -3;
+  }
+  const bool rope = cos != nullptr && sin != nullptr && position != nullptr;
+  if (rope && (hd & 1) != 0) {
+    return -3;
+  }
+  AttnArgs a{};
+  const int nml = n_q * n_split;
+  a.q = static_cast<const uint16_t *>(q);
+  a.k_cache = static_cast<const uint16_t *>(k);
+  a.v_cache = static_cast<const uint16_t *>(v);
+  a.m_s = ws;
+  a.l_s = ws + nml;
+  a.o_s = ws + 2 * static_cast<size_t>(nml);
+  a.valid_len = static_cast<const int32_t *>(valid_len);
+  a.k_act = static_cast<const uint16_t *>(k_act);
+  a.v_act = static_cast<const uint16_t *>(v_act);
+  a.cos = static_cast<const uint16_t *>(cos);
+  a.sin = static_cast<const uint16_t *>(sin);
+  a.position = static_cast<const int64_t *>(position);
+  a.n_q = n_q;
+  a.n_kv = n_kv;
+  a.hd = hd;
+  a.n_split = n_split;
+  a.max_seq = max_seq;
+  a.scale = scale;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const dim3 grid(static_cast<unsigned>(nml));
+  const dim3 block(kWave);
+  // The vector path needs 16-byte aligned rows and 16-byte aligned fp32 partials.
+  const bool vec_ok = aligned16(q) && aligned16(k) && aligned16(v) &&
+                      (k_act == nullptr || aligned16(k_act)) &&
+                      (v_act == nullptr || aligned16(v_act)) &&
+                      (cos == nullptr || aligned16(cos)) && (sin == nullptr || aligned16(sin)) &&
+                      aligned16(a.o_s);
+  if (vec_ok && hd == 128) {
+    attn_flash<16><<<grid, block, 0, st>>>(a);
+  } else if (vec_ok && hd == 64) {
+    attn_flash<8><<<grid, block, 0, st>>>(a);
+  } else if (vec_ok && hd == 256) {
+    attn_flash<32><<<grid, block, 0, st>>>(a);
+  } else if (vec_ok && hd == 32) {
+    attn_flash<4><<<grid, block, 0, st>>>(a);
+  } else if (vec_ok && hd == 16) {
+    attn_flash<2><<<grid, block, 0, st>>>(a);
+  } else {
+    attn_flash_generic<<<grid, block, 0, st>>>(a);
+  }
+  attn_merge<<<dim3(static_cast<unsigned>(n_q)), block, 0, st>>>(
+      a.m_s, a.l_s, a.o_s, static_cast<uint16_t *>(out), hd, n_split);
+  return launch_rc();
+}

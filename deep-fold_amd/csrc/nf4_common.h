@@ -1,0 +1,162 @@
+// Shared device helpers for the gfx950 NF4 kernels: the 16-level codebook,
+// bf16 / binary16 bit conversions, and 64-lane wavefront reductions.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "../../include/chr_nf4_amd.h"
+
+namespace chr {
+
+constexpr int kGroup = 64;  // weights per scale
+constexpr int kWave = 64;   // lanes per wavefront on gfx950
+
+// binary32 bit patterns of the QLoRA NF4 levels (internal/nf4/nf4.go:18-35,
+// bits as listed in internal/nf4/nf4_test.go:12-29).
+__device__ __constant__ const uint32_t kLutBits[16] = {
+    0xBF800000u, 0xBF3239B1u, 0xBF066B30u, 0xBECA32A0u, 0xBE91A24Du, 0xBE3D353Fu,
+    0xBDBA7871u, 0x00000000u, 0x3DA2FAFFu, 0x3E24CAE3u, 0x3E7C04DDu, 0x3EAD033Au,
+    0x3EE1A4B8u, 0x3F1007ABu, 0x3F3913B3u, 0x3F800000u,
+};
+
+__device__ __forceinline__ float bits_to_f32(uint32_t u) { return __uint_as_float(u); }
+__device__ __forceinline__ uint32_t f32_to_bits(float f) { return __float_as_uint(f); }
+
+// bf16 bits -> f32: the 16 bits are the top half of the binary32 word.
+__device__ __forceinline__ float bf16_lo(uint32_t pair) { return bits_to_f32(pair << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t pair) { return bits_to_f32(pair & 0xFFFF0000u); }
+__device__ __forceinline__ float bf16_to_f32(uint16_t h) {
+  return bits_to_f32(static_cast<uint32_t>(h) << 16);
+}
+
+// f32 -> bf16 bits, round to nearest even; NaN stays NaN
+// (same closed form as internal/f16/f16.go:93-106).
+__device__ __forceinline__ uint16_t f32_to_bf16(float f) {
+  uint32_t b = f32_to_bits(f);
+  if ((b & 0x7FFFFFFFu) > 0x7F800000u) {
+    uint32_t n = b >> 16;
+    if ((n & 0x7Fu) == 0) {
+      n |= 1u;
+    }
+    return static_cast<uint16_t>(n);
+  }
+  b += 0x7FFFu + ((b >> 16) & 1u);
+  return static_cast<uint16_t>(b >> 16);
+}
+
+// binary16 bits -> f32, exact (v_cvt_f32_f16 widens subnormals exactly).
+__device__ __forceinline__ float f16_to_f32(uint16_t h) {
+  return static_cast<float>(__builtin_bit_cast(_Float16, h));
+}
+
+// f32 -> binary16 bits, round to nearest even, written out in integer
+// arithmetic so it matches internal/f16/f16.go:8-57 case for case.
+__device__ __forceinline__ uint16_t f32_to_f16_rne(float f) {
+  const uint32_t b = f32_to_bits(f);
+  const uint32_t sign = (b >> 16) & 0x8000u;
+  const int exp = static_cast<int>((b >> 23) & 0xFFu);
+  uint32_t man = b & 0x7FFFFFu;
+  if (exp == 0xFF) {
+    if (man != 0) {
+      uint32_t n = man >> 13;
+      if (n == 0) {
+        n = 1;
+      }
+      return static_cast<uint16_t>(sign | 0x7C00u | n);
+    }
+    return static_cast<uint16_t>(sign | 0x7C00u);
+  }
+  const int e = exp - 127 + 15;
+  if (e >= 0x1F) {
+    return static_cast<uint16_t>(sign | 0x7C00u);
+  }
+  if (e <= 0) {
+    if (e < -10) {
+      return static_cast<uint16_t>(sign);
+    }
+    man |= 1u << 23;
+    const uint32_t shift = static_cast<uint32_t>(14 - e);
+    const uint32_t round = (man >> (shift - 1)) & 1u;
+    const uint32_t tail = man & ((1u << (shift - 1)) - 1u);
+    uint32_t m = man >> shift;
+    if (round != 0 && (tail != 0 || (m & 1u) != 0)) {
+      ++m;
+    }
+    return static_cast<uint16_t>(sign | m);
+  }
+  uint32_t half = sign | (static_cast<uint32_t>(e) << 10) | (man >> 13);
+  const uint32_t rem = man & 0x1FFFu;
+  if (rem > 0x1000u || (rem == 0x1000u && (half & 1u) != 0)) {
+    ++half;
+  }
+  return static_cast<uint16_t>(half);
+}
+
+// ---- cross-lane helpers ------------------------------------------------------
+// DPP controls (row = 16 lanes).
+constexpr int kDppQuadXor1 = 0xB1;       // quad_perm [1,0,3,2]
+constexpr int kDppQuadXor2 = 0x4E;       // quad_perm [2,3,0,1]
+constexpr int kDppRowHalfMirror = 0x141; // lane i <-> 7-i inside each 8
+constexpr int kDppRowMirror = 0x140;     // lane i <-> 15-i inside each 16
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+  const int r = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true);
+  return __int_as_float(r);
+}
+
+// Sum over aligned groups of LANES lanes (a power of two); every lane of the
+// group ends with the group's sum.  Up to 16 lanes this is pure DPP.
+template <int LANES>
+__device__ __forceinline__ float group_sum(float v) {
+  static_assert(LANES == 1 || LANES == 2 || LANES == 4 || LANES == 8 || LANES == 16 ||
+                    LANES == 32 || LANES == 64,
+                "group size must be a power of two up to 64");
+  if constexpr (LANES >= 2) v += dpp_f32<kDppQuadXor1>(v);
+  if constexpr (LANES >= 4) v += dpp_f32<kDppQuadXor2>(v);
+  if constexpr (LANES >= 8) v += dpp_f32<kDppRowHalfMirror>(v);
+  if constexpr (LANES >= 16) v += dpp_f32<kDppRowMirror>(v);
+  if constexpr (LANES >= 32) v += __shfl_xor(v, 16, kWave);
+  if constexpr (LANES >= 64) v += __shfl_xor(v, 32, kWave);
+  return v;
+}
+
+template <int LANES>
+__device__ __forceinline__ float group_max(float v) {
+  if constexpr (LANES >= 2) v = fmaxf(v, dpp_f32<kDppQuadXor1>(v));
+  if constexpr (LANES >= 4) v = fmaxf(v, dpp_f32<kDppQuadXor2>(v));
+  if constexpr (LANES >= 8) v = fmaxf(v, dpp_f32<kDppRowHalfMirror>(v));
+  if constexpr (LANES >= 16) v = fmaxf(v, dpp_f32<kDppRowMirror>(v));
+  if constexpr (LANES >= 32) v = fmaxf(v, __shfl_xor(v, 16, kWave));
+  if constexpr (LANES >= 64) v = fmaxf(v, __shfl_xor(v, 32, kWave));
+  return v;
+}
+
+// Whole-wavefront sum, result uniform in every lane: four DPP steps fold each
+// row of 16, then the four row totals are read as scalars and added in a fixed
+// order (deterministic, no atomics).
+__device__ __forceinline__ float wave_sum(float v) {
+  v = group_sum<16>(v);
+  const float r0 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+  const float r1 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+  const float r2 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+  const float r3 = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+  return (r0 + r1) + (r2 + r3);
+}
+
+// ---- host-side argument checks shared by the entry points -------------------
+inline bool k_pad_ok(int K, int K_pad) {
+  if (K < 1 || K_pad < K) {
+    return false;
+  }
+  return K_pad == kGroup * ((K + kGroup - 1) / kGroup);
+}
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline bool aligned2(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 1u) == 0; }
+
+inline int launch_rc() { return hipGetLastError() == hipSuccess ? 0 : -6; }
+
+}  // namespace chr

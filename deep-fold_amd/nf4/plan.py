@@ -1,0 +1,137 @@
+"""Host-side mirror of the ``chr_nf4_gemm`` launch planner.
+
+Pure Python, no GPU and no library: the same arithmetic as ``plan_impl`` in
+``csrc/nf4_gemm.hip``, so grid sizes and workspace needs can be asserted
+anywhere.  If the two diverge the library is the truth; ``tests/test_plan.py``
+checks they agree.  Plays the part of the reference's ``gpu/nf4/plan.py:161-236``
+for this library's gfx950 tiles.
+
+Kernel families by token count ``N`` (the reference's name for it; out features
+are ``M``, in features ``K``):
+
+* ``N == 1``  row-streaming GEMV, no split-K (path ``GEMV``).
+* ``N = 2..16`` / ``17..32``  MFMA tile, 128 rows x 32 columns per workgroup,
+  split-K over ``grid_y`` (paths ``PREFILL`` / ``PREFILL_N32``).
+* ``N = 33..64``  described by the planner, never launched (``PREFILL_N64``).
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+__all__ = [
+    "GEMV",
+    "PREFILL",
+    "PREFILL_N32",
+    "PREFILL_N64",
+    "ONE_WAVE",
+    "GROUP_SIZE",
+    "LIVE_MAX_N",
+    "PLAN_MAX_N",
+    "Plan",
+    "k_pad",
+    "gemv_rows_per_wavefront",
+    "plan",
+]
+
+GEMV = 1
+PREFILL = 2
+PREFILL_N32 = 3
+PREFILL_N64 = 4
+
+GROUP_SIZE = 64
+
+#: compute units of an MI355X; the unit the split-K target is expressed in when
+#: the caller gives no ``one_wave`` and no device is visible.
+ONE_WAVE = 256
+
+#: live ``chr_nf4_gemm`` ceiling (``gpu/nf4/plan.py:57``)
+LIVE_MAX_N = 32
+#: the planner also describes N = 33..64 (``gpu/nf4/plan.py:59``)
+PLAN_MAX_N = 64
+
+_BM = 128
+_BK = 256
+_BLOCK = 256
+_X_LDS = 32 * (_BK + 8) * 2  # staged activation tile, bf16, padded rows
+
+_PATH_NAME = {GEMV: "gemv", PREFILL: "prefill", PREFILL_N32: "prefill_n32",
+              PREFILL_N64: "prefill_n64"}
+
+
+def k_pad(k: int) -> int:
+    """``64 * ceil(K / 64)``."""
+    return GROUP_SIZE * ((int(k) + GROUP_SIZE - 1) // GROUP_SIZE)
+
+
+def _ceil_div(a: int, b: int) -> int:
+    return -(-int(a) // int(b))
+
+
+def gemv_rows_per_wavefront(m: int, forced: int = 0) -> int:
+    """Rows one wavefront of the GEMV walks together (they share x)."""
+    if forced in (1, 2, 4, 8):
+        return forced
+    if m >= 8192:
+        return 4
+    if m >= 2048:
+        return 2
+    return 1
+
+
+@dataclass(frozen=True)
+class Plan:
+    path: int
+    grid_x: int
+    grid_y: int
+    block: int
+    bm: int
+    bk: int
+    n_ktiles: int
+    tiles_per_split: int
+    ctas: int
+    smem_bytes: int
+    ws_floats: int
+
+    @property
+    def path_name(self) -> str:
+        return _PATH_NAME[self.path]
+
+    @property
+    def live(self) -> bool:
+        return self.path != PREFILL_N64
+
+
+def _pick_split(grid_x: int, n_ktiles: int, have_ws: bool, force_split: int,
+                one_wave: int) -> tuple[int, int]:
+    want = 1
+    if have_ws:
+        target = max(1, int(one_wave) * 2)
+        want = force_split if force_split > 0 else _ceil_div(target, grid_x)
+    want = max(1, min(want, n_ktiles))
+    tiles_per_split = _ceil_div(n_ktiles, want)
+    return _ceil_div(n_ktiles, tiles_per_split), tiles_per_split
+
+
+def plan(M: int, K: int, N: int = 1, *, K_pad: int | None = None, have_ws: bool = True,  # noqa: N803
+         force_split: int = 0, one_wave: int = ONE_WAVE, gemv_rows: int = 0) -> Plan:
+    M, K, N = int(M), int(K), int(N)
+    if M < 1 or K < 1:
+        raise ValueError(f"M and K must be >= 1, got M={M} K={K}")
+    if not 1 <= N <= PLAN_MAX_N:
+        raise ValueError(f"N={N} not in 1..{PLAN_MAX_N} (live launch is 1..{LIVE_MAX_N})")
+    kp = k_pad(K) if K_pad is None else int(K_pad)
+    if kp != k_pad(K):
+        raise ValueError(f"K_pad={kp} != 64*ceil(K/64) = {k_pad(K)}")
+    if N == 1:
+        bm = 4 * gemv_rows_per_wavefront(M, gemv_rows)
+        n_ktiles = _ceil_div(kp, 2048)
+        grid_x = _ceil_div(M, bm)
+        return Plan(GEMV, grid_x, 1, 256, bm, 2048, n_ktiles, n_ktiles, grid_x, 16 * 4 + 4 * 4, 0)
+    path = PREFILL if N <= 16 else (PREFILL_N32 if N <= 32 else PREFILL_N64)
+    grid_x = _ceil_div(M, _BM)
+    n_ktiles = _ceil_div(kp, _BK)
+    split, tps = _pick_split(grid_x, n_ktiles, have_ws, force_split, one_wave)
+    ws = split * M * N if split > 1 else 0
+    smem = (1 if N <= 32 else 2) * _X_LDS
+    return Plan(path, grid_x, split, _BLOCK, _BM, _BK, n_ktiles, tps, grid_x * split, smem, ws)

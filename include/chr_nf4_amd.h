@@ -1,0 +1,160 @@
+/* C ABI of the MI355X (gfx950) NF4 packed-linear library, libchr_nf4_amd.so.
+ *
+ * Every entry point below replaces the reference entry point of the same name;
+ * the citation after each one is the reference declaration (gpu/include/chr_gpu.h)
+ * and definition it stands in for.  Struct layouts are the reference's, field for
+ * field, so a binding written against chr_gpu.h binds this library unchanged.
+ *
+ * Conventions shared by all calls
+ *   - plain pointers and sizes only; every buffer is caller-owned device memory;
+ *     nothing here allocates, frees or synchronises
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream)
+ *   - activations are bfloat16 bits, scales are IEEE binary16 bits
+ *   - return 0 on success, else
+ *       -1 null pointer            -5 packed or x not 16-byte aligned
+ *       -2 N out of range             (scale not 2-byte aligned)
+ *       -3 bad dims / null blobs   -6 launch failure
+ *       -4 K_pad != 64*ceil(K/64)  -7 split-K workspace too small
+ *     (chr_gpu.h:30-33; gpu/nf4/nf4_gemm.cu:1621-1644, 1683-1698)
+ *
+ * Naming follows the reference: M = out features, K = in features,
+ * N = token columns; y[M,N] = dequant(W[M,K]) @ x[K,N].
+ */
+#pragma once
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Weight descriptor (chr_gpu.h:11-17).  packed is [M, K_pad/2] row-major, low
+ * nibble = even column; scale is [M, K_pad/64] binary16 bits. */
+typedef struct {
+  int32_t M;
+  int32_t K;
+  int32_t K_pad;
+  const uint8_t *packed;
+  const uint16_t *scale;
+} chr_nf4_dev_t;
+
+/* Launch plan (chr_gpu.h:48-60).  Same fields and meaning; the numbers describe
+ * this library's gfx950 tiles, not the reference's sm_86 ones.
+ * path: 1 = N==1 row-streaming GEMV tile, 2 = MFMA tile for N<=16,
+ *       3 = MFMA tile for N<=32, 4 = MFMA tile for N<=64 (plan only). */
+typedef struct {
+  int32_t path;
+  int32_t grid_x;          /* ceil(M / bm) */
+  int32_t grid_y;          /* split_k */
+  int32_t block;           /* threads per workgroup */
+  int32_t bm;              /* rows of M per workgroup */
+  int32_t bk;              /* K per staged tile */
+  int32_t n_ktiles;        /* ceil(K_pad / bk) */
+  int32_t tiles_per_split; /* K tiles one workgroup walks */
+  int32_t ctas;            /* grid_x * grid_y */
+  int32_t smem_bytes;      /* LDS bytes per workgroup */
+  int64_t ws_floats;       /* FP32 partials; 0 when grid_y == 1 */
+} chr_nf4_plan_t;
+
+/* y[M,N] = dequant(W) @ x[K,N]; x and y are bf16 row-major (token index
+ * fastest).  N in [1, 32].  No workspace, so split_k == 1.
+ * Replaces chr_nf4_gemm (chr_gpu.h:34-35; nf4_gemm.cu:1779-1785). */
+int chr_nf4_gemm(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N,
+                 void *stream);
+
+/* Pure launch math; only M/K/K_pad are read.  N in [1, 64].
+ * Replaces chr_nf4_gemm_plan (chr_gpu.h:64-65; nf4_gemm.cu:1656-1667). */
+int chr_nf4_gemm_plan(const chr_nf4_dev_t *w, int32_t N, int32_t have_ws,
+                      chr_nf4_plan_t *out);
+
+/* As chr_nf4_gemm with a caller-owned FP32 workspace of at least
+ * plan.ws_floats floats (ws == NULL means "no split-K").  N in [1, 32].
+ * Replaces chr_nf4_gemm_ws (chr_gpu.h:70-71; nf4_gemm.cu:1773-1777). */
+int chr_nf4_gemm_ws(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N,
+                    float *ws, int64_t ws_floats, void *stream);
+
+/* Same launch, N up to max_n (clamped to [1, 64]); N > 32 is refused with -2
+ * because no 64-column tile is built, as in the reference's live path.
+ * Replaces chr_nf4_gemm_ws_max (chr_gpu.h:75-76; nf4_gemm.cu:1669-1771). */
+int chr_nf4_gemm_ws_max(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N,
+                        float *ws, int64_t ws_floats, void *stream, int32_t max_n);
+
+/* Process-wide planner override: path 0 auto; split_k 0 auto, >0 forced;
+ * one_wave = compute units the split-K target is expressed in, 0 = this GPU's.
+ * Initial values come from CHR_NF4_PATH / CHR_NF4_SPLIT_K / CHR_NF4_ONE_WAVE.
+ * Replaces chr_nf4_set_tuning (chr_gpu.h:84; nf4_gemm.cu:1648-1654). */
+void chr_nf4_set_tuning(int32_t path, int32_t split_k, int32_t one_wave);
+
+/* N=1 GEMV.  x bf16 [K], y bf16 [M].  add: optional bf16 [M] residual, may
+ * alias y.  rms_w: optional bf16 [K]; when set, RMSNorm(x, rms_w, rms_eps),
+ * rounded to bf16, is what the dots consume.
+ * Replaces chr_nf4_gemv (chr_gpu.h:92-93; nf4_gemv.cu:790-834). */
+int chr_nf4_gemv(const chr_nf4_dev_t *w, const void *x, void *y, void *stream,
+                 const void *add, const void *rms_w, float rms_eps);
+
+/* One launch over q.M + k.M + v.M rows sharing x; optional bf16 biases are
+ * added in fp32 before the single bf16 rounding.
+ * Replaces chr_nf4_gemv_qkv (chr_gpu.h:99-103; nf4_gemv.cu:836-874). */
+int chr_nf4_gemv_qkv(const chr_nf4_dev_t *q, const chr_nf4_dev_t *k,
+                     const chr_nf4_dev_t *v, const void *x, void *yq, void *yk,
+                     void *yv, const void *bq, const void *bk, const void *bv,
+                     void *stream, const void *rms_w, float rms_eps);
+
+/* y[r] = bf16( silu(gate_r . x) * (up_r . x) ), both dots kept in fp32.
+ * Replaces chr_nf4_gemv_swiglu (chr_gpu.h:108-110; nf4_gemv.cu:876-924). */
+int chr_nf4_gemv_swiglu(const chr_nf4_dev_t *gate, const chr_nf4_dev_t *up,
+                        const void *x, void *y, void *stream, const void *rms_w,
+                        float rms_eps);
+
+/* In-place rotate-half RoPE on q [n_q,hd] and k [n_kv,hd] (rounded to bf16),
+ * then k and v are written to the caches [max_seq,n_kv,hd] at *position (int64).
+ * Replaces chr_nf4_rope_kv (chr_gpu.h:115-118; nf4_gemv.cu:926-950). */
+int chr_nf4_rope_kv(void *q, void *k, const void *v, void *k_cache, void *v_cache,
+                    const void *cos, const void *sin, const void *position,
+                    int32_t n_q, int32_t n_kv, int32_t hd, int32_t max_seq,
+                    void *stream);
+
+/* GQA decode attention over t < *valid_len (int32 on device).  With
+ * k_act/v_act/cos/sin/position it also rotates q and the current k in fp32,
+ * writes bf16(k_rot) and v into the caches at *position, and serves that slot
+ * from registers.  ws: n_q*n_split*(hd+2) floats.  hd <= 256, n_split <= 64.
+ * Replaces chr_nf4_attn (chr_gpu.h:124-128; nf4_gemv.cu:952-994). */
+int chr_nf4_attn(const void *q, const void *k, const void *v, void *out,
+                 const void *valid_len, float *ws, int32_t n_q, int32_t n_kv,
+                 int32_t hd, int32_t n_split, float scale, void *stream,
+                 const void *k_act, const void *v_act, const void *cos,
+                 const void *sin, const void *position, int32_t max_seq);
+
+/* y[i] = bf16( (w[i]*x[i]) * rsqrt(mean(x^2) + eps) ); x, w, y bf16 [n].
+ * Replaces chr_nf4_rms (chr_gpu.h:131-132; nf4_gemv.cu:996-1011). */
+int chr_nf4_rms(const void *x, const void *w, void *y, int32_t n, float eps,
+                void *stream);
+
+/* ---- entry points whose reference counterpart is not a C function ---------- */
+
+/* out[M,K] fp32 = LUT[code] * f32(scale), one binary32 multiply per weight,
+ * padding columns dropped.  Device twin of the CPU codec's Decode
+ * (internal/nf4/nf4.go:85-121), used to prove bit-exact unpacking. */
+int chr_nf4_dequant(const chr_nf4_dev_t *w, float *out, void *stream);
+
+/* Decode rows ids[0..n) of a packed table to bf16 [n, K]:
+ * bf16( LUT[code] * f32(scale) ).  ids are int64 on device.
+ * Replaces dequant_nf4_rows (gpu/host/embedding.py:74-107), the embedding
+ * gather of the decode step. */
+int chr_nf4_embed_rows(const chr_nf4_dev_t *table, const void *ids, int32_t n,
+                       void *out, void *stream);
+
+/* Quantise src[M,K] fp32 (device) into dst->packed / dst->scale (device,
+ * writable despite the const in the struct).  Device twin of the CPU codec's
+ * Encode (internal/nf4/nf4.go:46-82,129-185), bit for bit, used to make
+ * synthetic weights at model scale.  *status (int32 on device, may be NULL)
+ * is OR-ed with 1 when a non-finite weight was met (its group is skipped). */
+int chr_nf4_quantize(const float *src, const chr_nf4_dev_t *dst, int32_t *status,
+                     void *stream);
+
+/* Library version, for the loader's sanity check. */
+int chr_nf4_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
