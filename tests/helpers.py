@@ -1,0 +1,73 @@
+"""Helpers shared by the GPU parity tests: uploads, bf16 views, error bounds."""
+
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from oracle import nf4_oracle as oc
+
+DEV = "cuda"
+
+#: Floor-1 bound of the reference's kernel checks at rms(x) ~ 1
+#: (gpu/nf4/verify.py:70, gpu/nf4/numerics.py:191-202).
+MAXABS_FLOOR = 0.05
+#: max |y - y_ref| / max |y_ref| bound for bf16 outputs with fp32 accumulation.
+MAX_REL = 1e-2
+
+
+def up(a: np.ndarray) -> torch.Tensor:
+    return torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+def up_scale(scale: np.ndarray) -> torch.Tensor:
+    return torch.from_numpy(np.ascontiguousarray(scale).view(np.float16)).to(DEV)
+
+
+def bf16_tensor(a: np.ndarray) -> torch.Tensor:
+    """float32 array -> bf16 tensor on the GPU (rounded on the host, by torch)."""
+    return torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).to(torch.bfloat16).to(DEV)
+
+
+def to_f32(t: torch.Tensor) -> np.ndarray:
+    return t.detach().float().cpu().numpy()
+
+
+def bf16_bits(t: torch.Tensor) -> np.ndarray:
+    return t.detach().cpu().contiguous().view(torch.int16).numpy().view(np.uint16)
+
+
+def rand_x(k: int, n: int | None, seed: int) -> np.ndarray:
+    """N(0,1) activations already rounded to bf16 (as float32), so input rounding
+    is not charged to the kernel (gpu/tests/oracle_gate.py:113-124)."""
+    rng = np.random.default_rng(seed)
+    shape = (k,) if n is None else (k, n)
+    return oc.bf16_round(rng.standard_normal(shape).astype(np.float32))
+
+
+def ulp_bf16(v: np.ndarray) -> np.ndarray:
+    a = np.abs(np.asarray(v, dtype=np.float64))
+    e = np.floor(np.log2(np.maximum(a, 2.0 ** -126)))
+    return 2.0 ** (e - 7)
+
+
+def check_linear(y: torch.Tensor, y_ref: np.ndarray, *, what: str = "", ulps: float = 1.0) -> dict:
+    """y (bf16 on GPU) against a float32/float64 oracle result of the same shape.
+
+    Three bounds: the reference's floor-1 bound max(0.05, ULP/2); max-rel 1e-2;
+    and a tighter one of this build: within ``ulps`` bf16 ULP of the oracle value
+    (plus 1e-3 of the output's rms for cancellation-heavy rows)."""
+    got = to_f32(y).reshape(-1).astype(np.float64)
+    ref = np.asarray(y_ref, dtype=np.float64).reshape(-1)
+    assert got.shape == ref.shape, (got.shape, ref.shape)
+    assert np.isfinite(got).all(), f"{what}: non-finite output"
+    err = np.abs(got - ref)
+    u = ulp_bf16(ref)
+    rms = float(np.sqrt((ref ** 2).mean())) if ref.size else 0.0
+    assert (err <= np.maximum(MAXABS_FLOOR, 0.5 * u) + 1e-12).all(), f"{what}: maxabs {err.max():.6f}"
+    denom = np.abs(ref).max()
+    if denom > 0:
+        assert err.max() / denom <= MAX_REL, f"{what}: max-rel {err.max() / denom:.3e}"
+    assert (err <= ulps * u + 1e-3 * rms + 1e-30).all(), (
+        f"{what}: worst {np.max(err / (u + 1e-30)):.2f} bf16 ULP")
+    return {"maxabs": float(err.max()), "rms": rms}

@@ -1,0 +1,503 @@
+"""GPU parity: every NF4 kernel, through the C ABI, against the CPU oracle."""
+
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from deepfold_amd import nf4
+from oracle import nf4_oracle as oc
+
+from helpers import (DEV, bf16_bits, bf16_tensor, check_linear, rand_x, to_f32, up, up_scale)
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+def blobs(m, k, seed, **kw):
+    p, s = oc.toy_blobs(m, k, seed, **kw)
+    return p, s, up(p), up_scale(s)
+
+
+def quantized(m, k, seed, sigma=0.02):
+    rng = np.random.default_rng(seed)
+    w = (rng.standard_normal((m, k)) * sigma).astype(np.float32)
+    p, s = oc.c_encode(w)
+    return w, p, s, up(p), up_scale(s)
+
+
+# ---------------------------------------------------------------- codec twins
+@pytest.mark.parametrize("m,k", [(1, 64), (128, 256), (130, 65), (7, 1), (33, 5120), (4, 200)])
+def test_dequant_bit_exact(m, k):
+    say("dequant", m, k)
+    p, s, dp, ds = blobs(m, k, 100 + m + k)
+    got = nf4.nf4_dequant(dp, ds, m, k, oc.k_pad(k)).cpu().numpy()
+    want = oc.c_decode(p, s, m, k)
+    assert (got.view(np.uint32) == want.view(np.uint32)).all()
+
+
+def test_dequant_every_scale_pattern():
+    # all finite positive binary16 scales (incl. subnormals) x all 16 codes
+    bits = np.arange(1, 0x7C00, dtype=np.uint16)
+    m = bits.size
+    s = bits.view(np.float16).reshape(m, 1)
+    codes = np.tile(np.arange(16, dtype=np.uint8), 4)[None, :].repeat(m, 0)
+    p = oc.np_pack(codes)
+    got = nf4.nf4_dequant(up(p), up_scale(s), m, 64, 64).cpu().numpy()
+    want = oc.c_decode(p, s, m, 64)
+    assert (got.view(np.uint32) == want.view(np.uint32)).all()
+
+
+def test_dequant_golden_row():
+    w = (np.arange(64, dtype=np.float32) / np.float32(63)).reshape(1, 64)
+    p, s = oc.c_encode(w)
+    got = nf4.nf4_dequant(up(p), up_scale(s), 1, 64, 64).cpu().numpy()
+    assert (got.view(np.uint32) == oc.c_decode(p, s, 1, 64).view(np.uint32)).all()
+    # zero matrix decodes to +0 bits
+    z = nf4.nf4_dequant(up(np.full((3, 32), 0x77, np.uint8)), up_scale(np.full((3, 1), 1.0, np.float16)), 3, 64, 64)
+    assert (z.cpu().numpy().view(np.uint32) == 0).all()
+
+
+@pytest.mark.parametrize("m,k,sigma", [(1, 64, 1.0), (2, 64, 1.0), (64, 256, 0.02), (130, 65, 0.05),
+                                       (17, 5120, 0.02), (5, 1, 3.0), (9, 200, 1e-3)])
+def test_quantize_bit_exact(m, k, sigma):
+    say("quantize", m, k)
+    rng = np.random.default_rng(m * 1000 + k)
+    w = (rng.standard_normal((m, k)) * sigma).astype(np.float32)
+    if m == 2 and k == 64:
+        i = np.arange(64, dtype=np.float32)
+        w = np.stack([i / np.float32(63), (np.float32(2) * i - np.float32(63)) / np.float32(63)]).astype(np.float32)
+    dp, ds = nf4.nf4_quantize(up(w))
+    p, s = oc.c_encode(w)
+    assert (dp.cpu().numpy() == p).all()
+    assert (ds.cpu().numpy().view(np.uint16) == s.view(np.uint16)).all()
+
+
+def test_quantize_edge_groups():
+    w = np.zeros((6, 64), dtype=np.float32)
+    w[1] = 1e-12            # scale underflows binary16 -> zero group
+    w[2] = 1e6              # scale overflows -> clamp to 65504
+    w[3] = -2.25
+    w[4, :] = np.linspace(-1, 1, 64)
+    w[5, 0] = 6.1e-5        # binary16 subnormal/normal boundary
+    dp, ds = nf4.nf4_quantize(up(w))
+    p, s = oc.c_encode(w)
+    assert (dp.cpu().numpy() == p).all()
+    assert (ds.cpu().numpy().view(np.uint16) == s.view(np.uint16)).all()
+    bad = w.copy()
+    bad[2, 5] = np.nan
+    with pytest.raises(ValueError):
+        nf4.nf4_quantize(up(bad))
+    bad[2, 5] = np.inf
+    with pytest.raises(ValueError):
+        nf4.nf4_quantize(up(bad))
+
+
+def test_quantize_midpoint_neighbourhood():
+    mids = np.array([0xBF591CD8, 0xBF1C5270, 0xBEEB8480, 0xBEADEA76, 0xBE703CEC, 0xBE0D38BC,
+                     0xBD3A7871, 0x3D22FAFF, 0x3DF64862, 0x3E5067E0, 0x3E9582D4, 0x3EC753F9,
+                     0x3F006D04, 0x3F248DAF, 0x3F5C89DA], dtype=np.int64)
+    near = (mids[:, None] + np.arange(-33, 30)[None, :]).astype(np.uint32).view(np.float32)
+    w = np.concatenate([np.ones((15, 1), np.float32), near], axis=1)  # scale pinned to 1
+    dp, ds = nf4.nf4_quantize(up(w))
+    p, s = oc.c_encode(w)
+    assert (dp.cpu().numpy() == p).all() and (ds.cpu().numpy().view(np.uint16) == s.view(np.uint16)).all()
+
+
+def test_embed_rows_bit_exact():
+    m, k = 300, 200
+    p, s, dp, ds = blobs(m, k, 77)
+    ids = np.array([0, 299, 5, 5, 17, 128], dtype=np.int64)
+    got = nf4.nf4_embed_rows(dp, ds, up(ids), k)
+    want = oc.bf16_round_bits(oc.c_decode(p, s, m, k)[ids])
+    assert (bf16_bits(got) == want).all()
+
+
+# ---------------------------------------------------------------------- GEMV
+GEMV_SHAPES = [(128, 256), (130, 65), (4, 64), (1, 2048), (37, 5120), (260, 13824), (2050, 1024),
+               (8200, 128), (16, 11008), (3, 192)]
+
+
+@pytest.mark.parametrize("m,k", GEMV_SHAPES)
+def test_gemv_toy_blobs(m, k):
+    say("gemv", m, k)
+    p, s, dp, ds = blobs(m, k, 20260912 + m + k)
+    x = rand_x(k, None, m)
+    y = nf4.nf4_gemv(dp, ds, bf16_tensor(x), m, k, oc.k_pad(k))
+    assert tuple(y.shape) == (m, 1)
+    ref = oc.c_matmul_f64(oc.c_decode(p, s, m, k), x[:, None])
+    check_linear(y, ref, what=f"gemv {m}x{k}")
+    # same inputs, same bits
+    y2 = nf4.nf4_gemv(dp, ds, bf16_tensor(x), m, k, oc.k_pad(k))
+    assert (bf16_bits(y) == bf16_bits(y2)).all()
+
+
+def test_gemv_pad_codes_do_not_matter():
+    m, k = 130, 65
+    pa, sa = oc.toy_blobs(m, k, 5, pad_garbage=True)
+    pb, _ = oc.toy_blobs(m, k, 5, pad_garbage=False)
+    assert (pa != pb).any()
+    x = bf16_tensor(rand_x(k, None, 1))
+    ya = nf4.nf4_gemv(up(pa), up_scale(sa), x, m, k, 128)
+    yb = nf4.nf4_gemv(up(pb), up_scale(sa), x, m, k, 128)
+    assert (bf16_bits(ya) == bf16_bits(yb)).all()
+    xn = bf16_tensor(rand_x(k, 5, 2))
+    ga = nf4.nf4_gemm(up(pa), up_scale(sa), xn, m, k, 128)
+    gb = nf4.nf4_gemm(up(pb), up_scale(sa), xn, m, k, 128)
+    assert (bf16_bits(ga) == bf16_bits(gb)).all()
+
+
+def test_gemv_zero_level_matrix():
+    m, k = 64, 256
+    _, s = oc.toy_blobs(m, k, 9)
+    p = np.full((m, k // 2), 0x77, np.uint8)
+    y = nf4.nf4_gemv(up(p), up_scale(s), bf16_tensor(rand_x(k, None, 3)), m, k, k)
+    assert (to_f32(y) == 0).all()
+
+
+def test_gemv_config1_shape_quantized_weights():
+    m, k = 13824, 5120
+    say("gemv config 1", m, k)
+    w, p, s, dp, ds = quantized(m, k, 1)
+    x = rand_x(k, None, 2)
+    y = nf4.nf4_gemv(dp, ds, bf16_tensor(x), m, k, k)
+    ref = oc.c_matmul_f64(oc.c_decode(p, s, m, k), x[:, None])
+    check_linear(y, ref, what="config 1")
+    # the float32 two-pass CPU linear of the reference agrees to the same bound
+    check_linear(y, oc.c_linear(p, s, m, k, x[:, None]), what="config 1 vs f32 oracle", ulps=1.5)
+
+
+@pytest.mark.parametrize("rows", [1, 2, 4, 8])
+def test_gemv_rows_per_wavefront_agree(rows, monkeypatch):
+    m, k = 1030, 5120
+    p, s, dp, ds = blobs(m, k, 31)
+    x = rand_x(k, None, 4)
+    monkeypatch.setenv("CHR_NF4_GEMV_NR", str(rows))
+    y = nf4.nf4_gemv(dp, ds, bf16_tensor(x), m, k, k)
+    check_linear(y, oc.c_matmul_f64(oc.c_decode(p, s, m, k), x[:, None]), what=f"NR={rows}")
+
+
+def test_gemv_residual_add_may_alias_out():
+    m, k = 2048, 2048
+    p, s, dp, ds = blobs(m, k, 41)
+    x = rand_x(k, None, 5)
+    res = oc.bf16_round(np.random.default_rng(6).standard_normal(m).astype(np.float32))
+    dest = bf16_tensor(res)
+    out = nf4.nf4_gemv(dp, ds, bf16_tensor(x), m, k, k, dest, dest)
+    assert out.data_ptr() == dest.data_ptr()
+    ref = oc.c_matmul_f64(oc.c_decode(p, s, m, k), x[:, None]).reshape(-1) + res.astype(np.float64)
+    check_linear(dest, ref, what="residual")
+    # separate out and add give the same bits
+    out2 = torch.empty(m, dtype=torch.bfloat16, device=DEV)
+    nf4.nf4_gemv(dp, ds, bf16_tensor(x), m, k, k, out2, bf16_tensor(res))
+    assert (bf16_bits(out2) == bf16_bits(dest)).all()
+
+
+@pytest.mark.parametrize("m,k", [(256, 2048), (130, 65)])
+def test_gemv_fused_rms(m, k):
+    p, s, dp, ds = blobs(m, k, 51)
+    rng = np.random.default_rng(7)
+    x = oc.bf16_round(rng.standard_normal(k).astype(np.float32) * 3)
+    g = oc.bf16_round(1 + 0.1 * rng.standard_normal(k).astype(np.float32))
+    eps = 1e-6
+    y = nf4.nf4_gemv(dp, ds, bf16_tensor(x), m, k, oc.k_pad(k), rms_w=bf16_tensor(g), rms_eps=eps)
+    inv = 1.0 / np.sqrt((x.astype(np.float64) ** 2).mean() + eps)
+    xh = oc.bf16_round(((g.astype(np.float64) * x) * inv).astype(np.float32))
+    # normalised x is rounded to bf16 before the dots; allow one bf16 step of x
+    ref = oc.c_matmul_f64(oc.c_decode(p, s, m, k), xh[:, None])
+    check_linear(y, ref, what="fused rms", ulps=4)
+    # equals the two-launch form bit for bit when the RMS rounding agrees
+    h = torch.empty(k, dtype=torch.bfloat16, device=DEV)
+    nf4.nf4_rms(bf16_tensor(x), bf16_tensor(g), h, eps)
+    y2 = nf4.nf4_gemv(dp, ds, h, m, k, oc.k_pad(k))
+    check_linear(y, to_f32(y2), what="fused rms vs rms+gemv", ulps=1)
+
+
+def test_gemv_nan_behaviour():
+    m, k = 256, 512
+    p, s, dp, ds = blobs(m, k, 61)
+    x = rand_x(k, None, 8)
+    xn = x.copy()
+    xn[17] = np.nan
+    y = to_f32(nf4.nf4_gemv(dp, ds, bf16_tensor(xn), m, k, k))
+    assert not np.isfinite(y).any()        # a NaN in x poisons every row
+    s2 = s.copy()
+    s2[5, 3] = np.float16(np.nan)
+    y = to_f32(nf4.nf4_gemv(dp, up_scale(s2), bf16_tensor(x), m, k, k)).reshape(-1)
+    assert not np.isfinite(y[5])           # a NaN scale poisons its own row ...
+    assert np.isfinite(np.delete(y, 5)).all()  # ... and only that row
+
+
+def test_wrapper_rejects_lying_arguments():
+    m, k = 128, 256
+    p, s, dp, ds = blobs(m, k, 71)
+    x = bf16_tensor(rand_x(k, None, 9))
+    for bad in (
+        lambda: nf4.nf4_gemv(dp[: m // 2], ds, x, m, k, k),
+        lambda: nf4.nf4_gemv(dp, ds[: m // 2], x, m, k, k),
+        lambda: nf4.nf4_gemv(dp, ds, x, m, k, k + 64),
+        lambda: nf4.nf4_gemv(dp, ds, x[: k - 8], m, k, k),
+        lambda: nf4.nf4_gemv(dp, ds, x.cpu(), m, k, k),
+        lambda: nf4.nf4_gemv(dp, ds, x.to(torch.float16), m, k, k),
+        lambda: nf4.nf4_gemm(dp, ds, x.reshape(k, 1).repeat(1, 33), m, k, k),
+        lambda: nf4.nf4_gemm(dp[: m // 2], ds, x.reshape(k, 1).repeat(1, 4), m, k, k),
+    ):
+        with pytest.raises(RuntimeError):
+            bad()
+    # the context is still healthy
+    check_linear(nf4.nf4_gemv(dp, ds, x, m, k, k),
+                 oc.c_matmul_f64(oc.c_decode(p, s, m, k), to_f32(x)[:, None]), what="after refusals")
+
+
+# ----------------------------------------------------------------- QKV / SwiGLU
+@pytest.mark.parametrize("mq,mk,k,bias", [(2048, 256, 2048, True), (5120, 1024, 5120, True),
+                                          (64, 32, 64, False), (130, 33, 65, True)])
+def test_qkv_equals_three_gemvs(mq, mk, k, bias):
+    say("qkv", mq, mk, k)
+    kp = oc.k_pad(k)
+    mats = [blobs(mq, k, 81), blobs(mk, k, 82), blobs(mk, k, 83)]
+    rng = np.random.default_rng(10)
+    x = rand_x(k, None, 11)
+    biases = [oc.bf16_round(rng.standard_normal(m).astype(np.float32)) if bias else None
+              for m in (mq, mk, mk)]
+    outs = [torch.empty(m, dtype=torch.bfloat16, device=DEV) for m in (mq, mk, mk)]
+    dx = bf16_tensor(x)
+    nf4.nf4_qkv(mats[0][2], mats[0][3], mats[1][2], mats[1][3], mats[2][2], mats[2][3], dx,
+                mq, mk, mk, k, kp, outs[0], outs[1], outs[2],
+                *[None if b is None else bf16_tensor(b) for b in biases])
+    for (p, s, dp, ds), m, b, o in zip(mats, (mq, mk, mk), biases, outs):
+        ref = oc.c_matmul_f64(oc.c_decode(p, s, m, k), x[:, None]).reshape(-1)
+        if b is not None:
+            ref = ref + b
+        check_linear(o, ref, what="qkv")
+        single = torch.empty(m, dtype=torch.bfloat16, device=DEV)
+        nf4.nf4_gemv(dp, ds, dx, m, k, kp, single, None if b is None else bf16_tensor(b))
+        assert np.abs(to_f32(single) - to_f32(o)).max() <= 1e-3 + np.abs(to_f32(o)).max() * 2 ** -7
+
+
+@pytest.mark.parametrize("m,k", [(11008, 2048), (512, 5120), (130, 65), (4100, 256)])
+def test_swiglu_equals_pair(m, k):
+    say("swiglu", m, k)
+    kp = oc.k_pad(k)
+    pg, sg, dpg, dsg = blobs(m, k, 91)
+    pu, su, dpu, dsu = blobs(m, k, 92)
+    x = rand_x(k, None, 12)
+    out = torch.empty(m, dtype=torch.bfloat16, device=DEV)
+    nf4.nf4_swiglu(dpg, dsg, dpu, dsu, bf16_tensor(x), m, k, kp, out)
+    g = oc.c_matmul_f64(oc.c_decode(pg, sg, m, k), x[:, None]).reshape(-1)
+    u = oc.c_matmul_f64(oc.c_decode(pu, su, m, k), x[:, None]).reshape(-1)
+    ref = g / (1 + np.exp(-g)) * u
+    check_linear(out, ref, what="swiglu", ulps=1.5)
+
+
+# ------------------------------------------------------------------------ RMS
+@pytest.mark.parametrize("n", [64, 2048, 5120, 6144, 100])
+def test_rms(n):
+    rng = np.random.default_rng(n)
+    x = oc.bf16_round(rng.standard_normal(n).astype(np.float32) * 2)
+    w = oc.bf16_round(1 + 0.2 * rng.standard_normal(n).astype(np.float32))
+    y = torch.empty(n, dtype=torch.bfloat16, device=DEV)
+    nf4.nf4_rms(bf16_tensor(x), bf16_tensor(w), y, 1e-6)
+    ref = (w.astype(np.float64) * x) / np.sqrt((x.astype(np.float64) ** 2).mean() + 1e-6)
+    check_linear(y, ref, what="rms", ulps=1)
+    tref = F.rms_norm(torch.from_numpy(x), (n,), torch.from_numpy(w), 1e-6).numpy()
+    check_linear(y, tref, what="rms vs torch", ulps=1)
+
+
+# ----------------------------------------------------------------------- GEMM
+GEMM_SHAPES = [(128, 256), (130, 65), (64, 2048), (300, 5120), (129, 13824), (5120, 512)]
+
+
+@pytest.mark.parametrize("m,k", GEMM_SHAPES)
+@pytest.mark.parametrize("n", [2, 3, 8, 16, 17, 32])
+def test_gemm_vs_oracle(m, k, n):
+    say("gemm", m, k, n)
+    p, s, dp, ds = blobs(m, k, 200 + m + k)
+    x = rand_x(k, n, n)
+    y = nf4.nf4_gemm(dp, ds, bf16_tensor(x), m, k, oc.k_pad(k))
+    assert tuple(y.shape) == (m, n)
+    w = oc.c_decode(p, s, m, k)
+    # the MFMA path rounds each weight to bf16 before multiplying
+    ref_b = oc.c_matmul_f64(oc.bf16_round(w), x)
+    check_linear(y, ref_b, what=f"gemm {m}x{k} n{n} (bf16 weights)")
+    # and stays inside the reference's floor-1 bound against unrounded weights
+    ref = oc.c_matmul_f64(w, x)
+    err = np.abs(to_f32(y).astype(np.float64) - ref)
+    assert (err <= np.maximum(0.05, 2 ** (np.floor(np.log2(np.maximum(np.abs(ref), 1e-30))) - 8))).all()
+    assert err.max() / np.abs(ref).max() <= 1e-2
+
+
+def test_gemm_column_subset_equals_padded():
+    m, k = 256, 1024
+    p, s, dp, ds = blobs(m, k, 301)
+    x = rand_x(k, 16, 13)
+    x3 = x.copy()
+    x3[:, 3:] = 0
+    y16 = nf4.nf4_gemm(dp, ds, bf16_tensor(x3), m, k, k)
+    y3 = nf4.nf4_gemm(dp, ds, bf16_tensor(x[:, :3]), m, k, k)
+    assert (bf16_bits(y3) == bf16_bits(y16[:, :3].contiguous())).all()
+    assert (to_f32(y16[:, 3:]) == 0).all()
+
+
+@pytest.mark.parametrize("n", [8, 32])
+def test_gemm_every_split_agrees(n):
+    m, k = 512, 4096
+    p, s, dp, ds = blobs(m, k, 302)
+    x = bf16_tensor(rand_x(k, n, 14))
+    outs = []
+    try:
+        for split in (1, 2, 3, 5, 16):
+            nf4.nf4_set_tuning(split_k=split)
+            assert nf4.nf4_plan(m, k, n)["grid_y"] == min(split, 16) or split == 5
+            outs.append(to_f32(nf4.nf4_gemm(dp, ds, x, m, k, k)))
+    finally:
+        nf4.nf4_set_tuning()
+    for o in outs[1:]:
+        d = np.abs(o - outs[0])
+        assert (d <= 2.0 ** (np.floor(np.log2(np.maximum(np.abs(outs[0]), 2.0 ** -120))) - 7) + 1e-30).all()
+
+
+def test_gemm_n1_routes_to_gemv():
+    m, k = 384, 2048
+    p, s, dp, ds = blobs(m, k, 303)
+    x = bf16_tensor(rand_x(k, None, 15))
+    y = nf4.nf4_gemm(dp, ds, x, m, k, k)
+    assert tuple(y.shape) == (m, 1)
+    assert (bf16_bits(y) == bf16_bits(nf4.nf4_gemv(dp, ds, x, m, k, k))).all()
+
+
+def test_gemm_quantized_prefill_shape():
+    m, k, n = 7168, 5120, 32
+    say("gemm qkv shape", m, k, n)
+    w, p, s, dp, ds = quantized(m, k, 21)
+    x = rand_x(k, n, 16)
+    y = nf4.nf4_gemm(dp, ds, bf16_tensor(x), m, k, k)
+    check_linear(y, oc.c_matmul_f64(oc.bf16_round(oc.c_decode(p, s, m, k)), x), what="prefill qkv")
+
+
+# ------------------------------------------------------------------ attention
+def rope_tables(max_seq, hd, theta=10000.0):
+    inv = 1.0 / (np.float32(theta) ** (np.arange(0, hd, 2, dtype=np.float32) / np.float32(hd)))
+    fr = np.outer(np.arange(max_seq, dtype=np.float32), inv.astype(np.float32)).astype(np.float32)
+    emb = np.concatenate([fr, fr], axis=-1)
+    return oc.bf16_round(np.cos(emb).astype(np.float32)), oc.bf16_round(np.sin(emb).astype(np.float32))
+
+
+def rot_half(t, cos, sin):
+    d = t.shape[-1] // 2
+    rot = np.concatenate([-t[..., d:], t[..., :d]], axis=-1)
+    return t * cos + rot * sin
+
+
+def attn_ref(q, kc, vc, valid, scale, n_rep):
+    """q [n_q,hd] float64; kc/vc [T,n_kv,hd]; softmax over t < valid."""
+    n_q, hd = q.shape
+    out = np.zeros((n_q, hd))
+    for h in range(n_q):
+        kv = h // n_rep
+        sc = (kc[:valid, kv] @ q[h]) * scale
+        w = np.exp(sc - sc.max())
+        w /= w.sum()
+        out[h] = w @ vc[:valid, kv]
+    return out
+
+
+@pytest.mark.parametrize("n_q,n_kv,hd,max_seq,valid", [
+    (4, 2, 16, 16, 5), (8, 2, 64, 32, 32), (16, 2, 128, 256, 200), (40, 8, 128, 2048, 2048),
+    (4, 4, 32, 64, 1), (6, 3, 256, 40, 33), (4, 2, 48, 64, 50), (16, 2, 128, 300, 37)])
+def test_attn_plain(n_q, n_kv, hd, max_seq, valid):
+    say("attn", n_q, n_kv, hd, max_seq, valid)
+    rng = np.random.default_rng(hd + valid)
+    q = oc.bf16_round(rng.standard_normal((n_q, hd)).astype(np.float32))
+    kc = oc.bf16_round(rng.standard_normal((max_seq, n_kv, hd)).astype(np.float32))
+    vc = oc.bf16_round(rng.standard_normal((max_seq, n_kv, hd)).astype(np.float32))
+    kc[valid:] = 1e4  # a dirty tail must be ignored
+    vc[valid:] = -1e4
+    out = torch.zeros(n_q * hd, dtype=torch.bfloat16, device=DEV)
+    vl = torch.tensor(valid, dtype=torch.int32, device=DEV)
+    scale = hd ** -0.5
+    nf4.nf4_attn(bf16_tensor(q), bf16_tensor(kc), bf16_tensor(vc), out, vl, scale)
+    ref = attn_ref(q.astype(np.float64), kc.astype(np.float64), vc.astype(np.float64), valid, scale,
+                   n_q // n_kv)
+    got = to_f32(out).reshape(n_q, hd)
+    assert np.abs(got - ref).max() <= 0.02
+    # library cross-check: torch SDPA in float32
+    tq = torch.from_numpy(q).reshape(1, n_kv, n_q // n_kv, hd)
+    tk = torch.from_numpy(kc[:valid]).permute(1, 0, 2).unsqueeze(0)
+    tv = torch.from_numpy(vc[:valid]).permute(1, 0, 2).unsqueeze(0)
+    sd = F.scaled_dot_product_attention(tq, tk, tv, scale=scale).reshape(n_q, hd).numpy()
+    assert np.abs(got - sd).max() <= 0.02
+
+
+@pytest.mark.parametrize("n_q,n_kv,hd,max_seq,pos", [(4, 2, 16, 16, 0), (4, 2, 16, 16, 7),
+                                                     (16, 2, 128, 128, 100), (40, 8, 128, 2048, 1500),
+                                                     (4, 2, 48, 32, 9)])
+def test_attn_fused_rope_and_cache_write(n_q, n_kv, hd, max_seq, pos):
+    say("attn fused", n_q, n_kv, hd, max_seq, pos)
+    rng = np.random.default_rng(pos + hd)
+    cos, sin = rope_tables(max_seq, hd)
+    q = oc.bf16_round(rng.standard_normal((n_q, hd)).astype(np.float32))
+    ka = oc.bf16_round(rng.standard_normal((n_kv, hd)).astype(np.float32))
+    va = oc.bf16_round(rng.standard_normal((n_kv, hd)).astype(np.float32))
+    kc = oc.bf16_round(rng.standard_normal((max_seq, n_kv, hd)).astype(np.float32))
+    vc = oc.bf16_round(rng.standard_normal((max_seq, n_kv, hd)).astype(np.float32))
+    dk, dv = bf16_tensor(kc), bf16_tensor(vc)
+    out = torch.zeros(n_q * hd, dtype=torch.bfloat16, device=DEV)
+    vl = torch.tensor(pos + 1, dtype=torch.int32, device=DEV)
+    position = torch.tensor(pos, dtype=torch.int64, device=DEV)
+    scale = hd ** -0.5
+    nf4.nf4_attn(bf16_tensor(q), dk, dv, out, vl, scale, None, nf4.ATTN_SPLIT, bf16_tensor(ka),
+                 bf16_tensor(va), bf16_tensor(cos), bf16_tensor(sin), position)
+    qr = rot_half(q.astype(np.float64), cos[pos], sin[pos])
+    kr = rot_half(ka.astype(np.float64), cos[pos], sin[pos])
+    # cache row pos now holds bf16(k_rot) and v; every other row is untouched
+    kc2 = to_f32(dk)
+    vc2 = to_f32(dv)
+    assert (oc.bf16_round_bits(kr.astype(np.float32)) == bf16_bits(dk[pos])).mean() > 0.99
+    assert np.abs(kc2[pos] - kr).max() <= 2 ** -6
+    assert (vc2[pos] == va).all()
+    mask = np.ones(max_seq, bool)
+    mask[pos] = False
+    assert (kc2[mask] == kc[mask]).all() and (vc2[mask] == vc[mask]).all()
+    # attention uses the unrounded rotated key for the current slot
+    kfull = kc.astype(np.float64).copy()
+    vfull = vc.astype(np.float64).copy()
+    kfull[pos], vfull[pos] = kr, va
+    ref = attn_ref(qr, kfull, vfull, pos + 1, scale, n_q // n_kv)
+    assert np.abs(to_f32(out).reshape(n_q, hd) - ref).max() <= 0.02
+
+
+def test_attn_empty_prefix_gives_zero():
+    n_q, n_kv, hd, max_seq = 4, 2, 64, 16
+    out = torch.ones(n_q * hd, dtype=torch.bfloat16, device=DEV)
+    z = torch.zeros((max_seq, n_kv, hd), dtype=torch.bfloat16, device=DEV)
+    nf4.nf4_attn(torch.ones((n_q, hd), dtype=torch.bfloat16, device=DEV), z, z, out,
+                 torch.tensor(0, dtype=torch.int32, device=DEV), 0.125)
+    assert (to_f32(out) == 0).all()
+
+
+@pytest.mark.parametrize("n_q,n_kv,hd,pos", [(4, 2, 16, 3), (16, 2, 128, 60), (6, 3, 256, 0)])
+def test_rope_kv(n_q, n_kv, hd, pos):
+    max_seq = 64
+    rng = np.random.default_rng(hd)
+    cos, sin = rope_tables(max_seq, hd)
+    q = oc.bf16_round(rng.standard_normal((n_q, hd)).astype(np.float32))
+    k = oc.bf16_round(rng.standard_normal((n_kv, hd)).astype(np.float32))
+    v = oc.bf16_round(rng.standard_normal((n_kv, hd)).astype(np.float32))
+    dq, dk, dv = bf16_tensor(q), bf16_tensor(k), bf16_tensor(v)
+    kc = torch.zeros((max_seq, n_kv, hd), dtype=torch.bfloat16, device=DEV)
+    vc = torch.zeros_like(kc)
+    nf4.nf4_rope_kv(dq, dk, dv, kc, vc, bf16_tensor(cos), bf16_tensor(sin),
+                    torch.tensor(pos, dtype=torch.int64, device=DEV))
+    qr = rot_half(q.astype(np.float64), cos[pos], sin[pos])
+    kr = rot_half(k.astype(np.float64), cos[pos], sin[pos])
+    assert np.abs(to_f32(dq) - qr).max() <= 2 ** -6
+    assert np.abs(to_f32(dk) - kr).max() <= 2 ** -6
+    assert (bf16_bits(kc[pos]) == bf16_bits(dk)).all()
+    assert (to_f32(vc[pos]) == v).all()
+    assert (to_f32(kc[:pos]) == 0).all() and (to_f32(kc[pos + 1:]) == 0).all()
