@@ -35,7 +35,9 @@ namespace chr {
 
 int gemv_entry(const chr_nf4_dev_t *w, const void *x, void *y, void *stream, const void *add,
                const void *rms_w, float rms_eps);
-int gemv_rows_per_wg(int M);
+int gemv_rows_per_wg(int M, int K_pad);
+int gemv_threads_per_wg(int M, int K_pad);
+int gemv_lds_bytes(int K_pad);
 
 namespace {
 
@@ -130,14 +132,14 @@ int plan_impl(const chr_nf4_dev_t &h, int32_t N, int32_t have_ws, chr_nf4_plan_t
   if (N == 1) {
     // Row-streaming GEMV: every wavefront walks whole rows, no split-K.
     p.path = 1;
-    p.bm = gemv_rows_per_wg(h.M);
+    p.bm = gemv_rows_per_wg(h.M, h.K_pad);
     p.bk = 2048;  // codes one wavefront load step covers
-    p.block = 256;
+    p.block = gemv_threads_per_wg(h.M, h.K_pad);
     p.grid_x = ceil_div(h.M, p.bm);
     p.grid_y = 1;
     p.n_ktiles = ceil_div(h.K_pad, p.bk);
     p.tiles_per_split = p.n_ktiles;
-    p.smem_bytes = 16 * 4 + 4 * 4;
+    p.smem_bytes = gemv_lds_bytes(h.K_pad);
     p.ws_floats = 0;
   } else {
     p.path = N <= 16 ? 2 : (N <= 32 ? 3 : 4);

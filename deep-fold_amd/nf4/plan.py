@@ -2,7 +2,7 @@
 
 Pure Python, no GPU and no library: the same arithmetic as ``plan_impl`` in
 ``csrc/nf4_gemm.hip``, so grid sizes and workspace needs can be asserted
-anywhere.  If the two diverge the library is the truth; ``tests/test_plan.py``
+anywhere.  If the two diverge the library is the truth; ``tests/test_abi.py``
 checks they agree.  Plays the part of the reference's ``gpu/nf4/plan.py:161-236``
 for this library's gfx950 tiles.
 
@@ -70,13 +70,9 @@ def _ceil_div(a: int, b: int) -> int:
 
 def gemv_rows_per_wavefront(m: int, forced: int = 0) -> int:
     """Rows one wavefront of the GEMV walks together (they share x)."""
-    if forced in (1, 2, 4, 8):
+    if forced in (1, 2, 4):
         return forced
-    if m >= 8192:
-        return 4
-    if m >= 2048:
-        return 2
-    return 1
+    return 2 if m >= 4096 else 1
 
 
 @dataclass(frozen=True)
@@ -127,7 +123,8 @@ def plan(M: int, K: int, N: int = 1, *, K_pad: int | None = None, have_ws: bool 
         bm = 4 * gemv_rows_per_wavefront(M, gemv_rows)
         n_ktiles = _ceil_div(kp, 2048)
         grid_x = _ceil_div(M, bm)
-        return Plan(GEMV, grid_x, 1, 256, bm, 2048, n_ktiles, n_ktiles, grid_x, 16 * 4 + 4 * 4, 0)
+        lds = (16 + 16) * 4  # codebook + reduction partials
+        return Plan(GEMV, grid_x, 1, 256, bm, 2048, n_ktiles, n_ktiles, grid_x, lds, 0)
     path = PREFILL if N <= 16 else (PREFILL_N32 if N <= 32 else PREFILL_N64)
     grid_x = _ceil_div(M, _BM)
     n_ktiles = _ceil_div(kp, _BK)
