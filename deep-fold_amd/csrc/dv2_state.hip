@@ -1,0 +1,116 @@
+// Device-side bookkeeping of the resident decode step, so that a greedy step
+// needs no host read and only one small launch at each end:
+//   chr_dv2_mark_written   valid_len = position + 1   (gpu/decodev2/kv.py:118-120)
+//   chr_dv2_argmax_commit  next = argmax(logits), then token = next,
+//                          position += 1, finished |= (next == eos)
+//                          (gpu/decodev2/step.py:182, gpu/decodev2/state.py:98-103)
+// The argmax runs on the bf16 logits as stored and the lowest index wins a tie,
+// which is what the CPU oracle's argmax does.
+
+#include "nf4_common.h"
+
+namespace chr {
+namespace {
+
+__global__ void mark_written(const int64_t *__restrict__ position, int32_t *__restrict__ valid_len) {
+  if (threadIdx.x == 0) {
+    *valid_len = static_cast<int32_t>(*position) + 1;
+  }
+}
+
+constexpr int kArgmaxBlock = 1024;
+
+// Total order on (value, index): larger value first, then smaller index.  NaN
+// compares as larger than everything, so a NaN logit is surfaced, not hidden.
+__device__ __forceinline__ bool better(float v, int i, float bv, int bi) {
+  const bool vn = v != v, bn = bv != bv;
+  if (vn != bn) {
+    return vn;
+  }
+  if (vn && bn) {
+    return i < bi;
+  }
+  return v > bv || (v == bv && i < bi);
+}
+
+__global__ __launch_bounds__(kArgmaxBlock) void argmax_commit(
+    const uint16_t *__restrict__ logits, int n, int64_t *__restrict__ next_token,
+    int64_t *__restrict__ token, int64_t *__restrict__ position, uint8_t *__restrict__ finished,
+    const int64_t *__restrict__ eos_id, int commit) {
+  __shared__ float sv[kArgmaxBlock / kWave];
+  __shared__ int si[kArgmaxBlock / kWave];
+  float bv = -__builtin_inff();
+  int bi = 0x7FFFFFFF;
+  for (int i = threadIdx.x; i < n; i += kArgmaxBlock) {
+    const float v = bf16_to_f32(logits[i]);
+    if (better(v, i, bv, bi)) {
+      bv = v;
+      bi = i;
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(bv, off, kWave);
+    const int oi = __shfl_xor(bi, off, kWave);
+    if (better(ov, oi, bv, bi)) {
+      bv = ov;
+      bi = oi;
+    }
+  }
+  if ((threadIdx.x & (kWave - 1)) == 0) {
+    sv[threadIdx.x >> 6] = bv;
+    si[threadIdx.x >> 6] = bi;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < kArgmaxBlock / kWave; ++w) {
+      if (better(sv[w], si[w], bv, bi)) {
+        bv = sv[w];
+        bi = si[w];
+      }
+    }
+    const int64_t nt = bi;
+    *next_token = nt;
+    if (commit) {
+      *token = nt;
+      *position += 1;
+      if (nt == *eos_id) {
+        *finished |= 1;
+      }
+    }
+  }
+}
+
+}  // namespace
+}  // namespace chr
+
+using namespace chr;
+
+extern "C" int chr_dv2_mark_written(const void *position, void *valid_len, void *stream) {
+  if (position == nullptr || valid_len == nullptr) {
+    return -1;
+  }
+  mark_written<<<dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream)>>>(
+      static_cast<const int64_t *>(position), static_cast<int32_t *>(valid_len));
+  return launch_rc();
+}
+
+extern "C" int chr_dv2_argmax_commit(const void *logits, int32_t n, void *next_token, void *token,
+                                     void *position, void *finished, const void *eos_id,
+                                     int32_t commit, void *stream) {
+  if (logits == nullptr || next_token == nullptr) {
+    return -1;
+  }
+  if (commit != 0 && (token == nullptr || position == nullptr || finished == nullptr ||
+                      eos_id == nullptr)) {
+    return -1;
+  }
+  if (n < 1) {
+    return -3;
+  }
+  argmax_commit<<<dim3(1), dim3(kArgmaxBlock), 0, static_cast<hipStream_t>(stream)>>>(
+      static_cast<const uint16_t *>(logits), n, static_cast<int64_t *>(next_token),
+      static_cast<int64_t *>(token), static_cast<int64_t *>(position),
+      static_cast<uint8_t *>(finished), static_cast<const int64_t *>(eos_id), commit);
+  return launch_rc();
+}

@@ -37,6 +37,8 @@ __all__ = [
     "nf4_dequant",
     "nf4_embed_rows",
     "nf4_quantize",
+    "dv2_mark_written",
+    "dv2_argmax_commit",
     "library_path",
 ]
 
@@ -101,6 +103,8 @@ EXPORTS = (
     ("chr_nf4_dequant", ctypes.c_int, [_DP, _P, _P]),
     ("chr_nf4_embed_rows", ctypes.c_int, [_DP, _P, _I, _P, _P]),
     ("chr_nf4_quantize", ctypes.c_int, [_P, _DP, _P, _P]),
+    ("chr_dv2_mark_written", ctypes.c_int, [_P, _P, _P]),
+    ("chr_dv2_argmax_commit", ctypes.c_int, [_P, _I, _P, _P, _P, _P, _P, _I, _P]),
     ("chr_nf4_abi_version", ctypes.c_int, []),
 )
 
@@ -536,3 +540,39 @@ def nf4_quantize(w: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
     if int(status.item()) != 0:
         raise ValueError("nf4: non-finite weight")
     return packed, scale
+
+
+def dv2_mark_written(position: torch.Tensor, valid_len: torch.Tensor) -> None:
+    """``valid_len = position + 1`` on the device (``gpu/decodev2/kv.py:118-120``)."""
+    _need(position.is_cuda and position.dtype == torch.int64 and position.numel() == 1,
+          "position must be a CUDA int64 scalar")
+    _need(valid_len.is_cuda and valid_len.dtype == torch.int32 and valid_len.numel() == 1,
+          "valid_len must be a CUDA int32 scalar")
+    rc = _load_ext().chr_dv2_mark_written(position.data_ptr(), valid_len.data_ptr(), _stream())
+    _check_rc("chr_dv2_mark_written", rc)
+
+
+def dv2_argmax_commit(logits: torch.Tensor, next_token: torch.Tensor, token: torch.Tensor | None = None,
+                      position: torch.Tensor | None = None, finished: torch.Tensor | None = None,
+                      eos_id: torch.Tensor | None = None, commit: bool = False) -> None:
+    """``next_token = argmax(logits)`` (first maximum wins); with ``commit`` also
+    ``token = next``, ``position += 1``, ``finished |= next == eos``
+    (``gpu/decodev2/step.py:182``, ``gpu/decodev2/state.py:98-103``)."""
+    _need(logits.is_cuda and logits.dtype == torch.bfloat16 and logits.is_contiguous(),
+          "logits must be contiguous CUDA bf16")
+    _need(next_token.is_cuda and next_token.dtype == torch.int64 and next_token.numel() == 1,
+          "next_token must be a CUDA int64 scalar")
+    ptrs = [None, None, None, None]
+    if commit:
+        _need(token is not None and token.is_cuda and token.dtype == torch.int64, "token must be CUDA int64")
+        _need(position is not None and position.is_cuda and position.dtype == torch.int64,
+              "position must be CUDA int64")
+        _need(finished is not None and finished.is_cuda and finished.dtype == torch.uint8,
+              "finished must be CUDA uint8")
+        _need(eos_id is not None and eos_id.is_cuda and eos_id.dtype == torch.int64,
+              "eos_id must be CUDA int64")
+        ptrs = [token.data_ptr(), position.data_ptr(), finished.data_ptr(), eos_id.data_ptr()]
+    rc = _load_ext().chr_dv2_argmax_commit(logits.data_ptr(), int(logits.numel()), next_token.data_ptr(),
+                                           ptrs[0], ptrs[1], ptrs[2], ptrs[3], 1 if commit else 0,
+                                           _stream())
+    _check_rc("chr_dv2_argmax_commit", rc)

@@ -152,6 +152,21 @@ int chr_nf4_embed_rows(const chr_nf4_dev_t *table, const void *ids, int32_t n,
 int chr_nf4_quantize(const float *src, const chr_nf4_dev_t *dst, int32_t *status,
                      void *stream);
 
+/* valid_len (int32 on device) = *position (int64 on device) + 1.
+ * Replaces GraphSafeKV.mark_written (gpu/decodev2/kv.py:118-120), three tensor
+ * ops in the reference, one launch here. */
+int chr_dv2_mark_written(const void *position, void *valid_len, void *stream);
+
+/* *next_token = argmax over logits[0..n) (bf16; the lowest index wins a tie; a
+ * NaN logit wins outright).  With commit != 0 it also feeds the id back:
+ * *token = next, *position += 1, *finished |= (next == *eos_id); all scalars
+ * live on the device (int64, int64, int64, uint8, int64).
+ * Replaces the argmax of forward_decode plus DecodeState.commit_step
+ * (gpu/decodev2/step.py:182, gpu/decodev2/state.py:98-103). */
+int chr_dv2_argmax_commit(const void *logits, int32_t n, void *next_token, void *token,
+                          void *position, void *finished, const void *eos_id, int32_t commit,
+                          void *stream);
+
 /* Library version, for the loader's sanity check. */
 int chr_nf4_abi_version(void);
 

@@ -19,7 +19,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 def header_symbols():
     text = open(os.path.join(ROOT, "include", "chr_nf4_amd.h")).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(chr_nf4_\w+)\s*\(", text)))
+    return sorted(set(re.findall(r"\b(chr_(?:nf4|dv2)_\w+)\s*\(", text)))
 
 
 def test_library_exports_every_declared_symbol():

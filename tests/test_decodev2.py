@@ -1,0 +1,199 @@
+"""GPU: the resident decoder (eager step, HIP graph, chunked prefill) against the
+CPU float32 step oracle on seeded synthetic models."""
+
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+
+from deepfold_amd import decodev2 as dv2
+from deepfold_amd.decodev2.synth import build
+from oracle import nf4_oracle as oc
+from oracle import step_oracle as so
+
+pytestmark = pytest.mark.gpu
+
+PROMPT = [1, 3, 5, 7]
+SHORT = [4, 5, 6]
+LONG = [4, 5, 6, 7, 1, 2, 3, 4]
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+def session(spec, seed):
+    model = build(spec, seed)          # quantised by the library's GPU encoder
+    weights = dv2.DeviceWeights.from_synth(model, "cuda")
+    state = dv2.DecodeState.allocate(spec, device="cuda")
+    return model, state, weights
+
+
+def greedy_token_at_a_time(state, weights, prompt, n_new, step=dv2.greedy_decode):
+    state.reset()
+    for t in prompt:
+        dv2.teacher_force_token(state, weights, t)
+    out = [int(state.next_token.item())]
+    if out[0] == state.spec.eos_id:
+        return out
+    state.token.copy_(state.next_token)
+    for _ in range(n_new - 1):
+        step(state, weights)
+        out.append(int(state.token.item()))
+        if int(state.finished.item()) == 1:
+            break
+    return out
+
+
+def test_gpu_encoder_builds_the_same_model_as_the_cpu_codec():
+    a = build(dv2.TINY_LLAMA, 0)
+    b = build(dv2.TINY_LLAMA, 0, encode=oc.c_encode)
+    for la, lb in zip(a.layers, b.layers):
+        for name in ("q", "k", "v", "o", "gate", "up", "down"):
+            ma, mb = getattr(la, name), getattr(lb, name)
+            assert (ma.packed == mb.packed).all(), name
+            assert (np.asarray(ma.scale).view(np.uint16) == mb.scale.view(np.uint16)).all(), name
+    assert (a.lm_head.packed == b.lm_head.packed).all()
+
+
+@pytest.mark.parametrize("spec,seed,prompt", [
+    (dv2.TINY_LLAMA, 0, SHORT), (dv2.TINY_LLAMA, 0, PROMPT), (dv2.TINY_INTERNLM, 1, SHORT),
+    (dv2.MEDIUM_LLAMA, 0, SHORT)])
+def test_eager_greedy_matches_the_oracle(spec, seed, prompt):
+    say("greedy", spec.name, seed, prompt)
+    model, state, weights = session(spec, seed)
+    want, margins = so.greedy_ids(model, prompt, 8, return_margins=True)
+    got = greedy_token_at_a_time(state, weights, prompt, 8)
+    say("  oracle", want, "min margin", min(margins))
+    assert got == want
+    assert int(state.valid_len.item()) == len(prompt) + max(0, len(got) - 1)
+
+
+def test_teacher_forced_logits_track_the_oracle():
+    spec = dv2.MEDIUM_LLAMA
+    model, state, weights = session(spec, 0)
+    toks = [4, 5, 6, 7, 1, 2, 3, 4, 9, 100]
+    want = so.teacher_logits(model, toks)
+    state.reset()
+    for i, t in enumerate(toks):
+        dv2.teacher_force_token(state, weights, t)
+        got = state.arena.logits.float().cpu().numpy()[0]
+        # bf16 activations through 4 layers: a loose absolute bound on O(1) logits
+        assert np.abs(got - want[i]).max() <= 0.06 * max(1.0, np.abs(want[i]).max()), i
+        assert int(state.next_token.item()) == int(got.argmax())
+
+
+def test_dirty_kv_tail_is_ignored():
+    spec = dv2.TINY_LLAMA
+    _, clean, w = session(spec, 0)
+    dirty = dv2.DecodeState.allocate(spec, device="cuda")
+    for s in (clean, dirty):
+        dv2.teacher_force_token(s, w, 1)
+    dirty.kv.k[:, 2:].fill_(1.0e4)
+    dirty.kv.v[:, 2:].fill_(1.0e4)
+    for s in (clean, dirty):
+        dv2.teacher_force_token(s, w, 3)
+    assert torch.equal(clean.arena.logits, dirty.arena.logits)
+
+
+def test_reset_reproduces_a_run():
+    spec = dv2.TINY_LLAMA
+    _, state, w = session(spec, 0)
+    a = greedy_token_at_a_time(state, w, PROMPT, 8)
+    b = greedy_token_at_a_time(state, w, PROMPT, 8)   # KV is dirty now; valid_len hides it
+    assert a == b
+
+
+@pytest.mark.parametrize("spec,seed", [(dv2.TINY_LLAMA, 0), (dv2.TINY_INTERNLM, 1), (dv2.MEDIUM_LLAMA, 0)])
+def test_graph_replay_equals_eager(spec, seed):
+    say("graph", spec.name)
+    model, state, weights = session(spec, seed)
+    eager = greedy_token_at_a_time(state, weights, SHORT, 10)
+    state.reset()
+    graph = dv2.capture_greedy(state, weights, warmup=2)
+    before = torch.cuda.memory_allocated()
+    for rep in range(3):   # several replays, eager work and syncs between them
+        got = greedy_token_at_a_time(state, weights, SHORT, 10, step=graph)
+        assert got == eager, rep
+        torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated() == before       # the step allocates nothing
+    assert got == so.greedy_ids(model, SHORT, 10)
+    with pytest.raises(RuntimeError):
+        graph(dv2.DecodeState.allocate(spec, device="cuda"), weights)
+
+
+def test_graph_bookkeeping():
+    spec = dv2.TINY_LLAMA
+    _, state, weights = session(spec, 0)
+    graph = dv2.capture_greedy(state, weights, warmup=1)
+    state.reset()
+    state.load_token(5)
+    graph.replay()
+    torch.cuda.synchronize()
+    assert int(state.position.item()) == 1 and int(state.valid_len.item()) == 1
+    assert int(state.token.item()) == int(state.next_token.item())
+    graph.replay()
+    torch.cuda.synchronize()
+    assert int(state.position.item()) == 2 and int(state.valid_len.item()) == 2
+
+
+@pytest.mark.parametrize("spec,seed", [(dv2.TINY_LLAMA, 0), (dv2.TINY_INTERNLM, 1), (dv2.MEDIUM_LLAMA, 0)])
+def test_chunked_prefill_equals_token_at_a_time_and_the_oracle(spec, seed):
+    say("prefill", spec.name)
+    model, state, weights = session(spec, seed)
+    want = so.greedy_ids(model, LONG, 6)
+    one = greedy_token_at_a_time(state, weights, LONG, 6)
+    outs = {}
+    for chunk in (1, 2, 4, 8, None):
+        state.reset()
+        outs[chunk] = dv2.generate(state, weights, LONG, 6, chunk=chunk)
+        assert int(state.valid_len.item()) == len(LONG) + max(0, len(outs[chunk]) - 1)
+    assert one == want
+    for chunk, got in outs.items():
+        assert got == want, chunk
+
+
+def test_suffix_prefill_equals_full_prefill():
+    spec = dv2.TINY_LLAMA
+    _, full, w = session(spec, 0)
+    part = dv2.DecodeState.allocate(spec, device="cuda")
+    dv2.consume_prompt(full, w, LONG, chunk=2)
+    dv2.consume_prompt(part, w, LONG[:3], chunk=2)
+    dv2.consume_prompt(part, w, LONG[3:], start=3, chunk=2)
+    assert int(full.valid_len.item()) == int(part.valid_len.item()) == len(LONG)
+    assert int(full.next_token.item()) == int(part.next_token.item())
+    # the two runs cut the prompt into different chunks, so some positions went
+    # through the N=1 kernel (fp32 weights) in one and the MFMA tile (bf16 weights)
+    # in the other: equal up to bf16 rounding, not bit for bit
+    a = full.kv.k[:, : len(LONG)].float()
+    b = part.kv.k[:, : len(LONG)].float()
+    assert (a - b).abs().max().item() <= 0.02 * max(1.0, a.abs().max().item())
+
+
+def test_prompt_errors():
+    spec = dv2.TINY_LLAMA
+    _, state, w = session(spec, 0)
+    with pytest.raises(ValueError):
+        dv2.consume_prompt(state, w, [])
+    with pytest.raises(ValueError):
+        dv2.consume_prompt(state, w, list(range(spec.max_seq + 1)))
+    with pytest.raises(ValueError):
+        dv2.consume_prompt(state, w, [1, 2], start=-1)
+    with pytest.raises(RuntimeError):
+        dv2.DecodeState.allocate(spec, device="cpu")
+
+
+def test_packed_embedding_rows_and_random_weights_step():
+    spec = dv2.ArchSpec("rand", "llama_swiglu", 2, 256, 4, 2, 64, 512, 1000, 64, qkv_bias=True)
+    w = dv2.DeviceWeights.random(spec, 7)
+    assert isinstance(w.embed, dv2.PackedEmbed)
+    ids = torch.tensor([0, 999, 17], device="cuda")
+    rows = dv2.gather_embed(w.embed, ids)
+    dense = oc.c_decode(w.embed.packed.cpu().numpy(), w.embed.scale.cpu().numpy(), 1000, 256)
+    assert (rows.float().cpu().numpy() == oc.bf16_round(dense[[0, 999, 17]])).all()
+    state = dv2.DecodeState.allocate(spec, device="cuda")
+    state.load_token(17)
+    dv2.greedy_decode(state, w)
+    assert torch.isfinite(state.arena.logits.float()).all()
+    assert 0 <= int(state.token.item()) < 1000 and int(state.position.item()) == 1
