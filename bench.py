@@ -2,17 +2,21 @@
 
 ``python bench.py --gpus 1 --steps K --warmup W`` prints ONE JSON line.
 
-A step is one launch of the decode GEMV over the headline layer
-(x [1,5120] bf16 times W [13824,5120], NF4 group-64) on weights that rotate
-through > 512 MB of distinct copies, so neither L2 nor the 256 MB Infinity
-Cache can serve them.  ``value`` is the achieved algorithmic bandwidth in GB/s
-(packed codes + scales + x + y per launch), inputs resident in HBM.
+Primary workload (``metric``/``value``): a step is one launch of the decode GEMV
+over the headline layer (x [1,5120] bf16 times W [13824,5120], NF4 group-64) on
+weights that rotate through > 512 MB of distinct copies, so neither L2 nor the
+256 MB Infinity Cache can serve them.  ``value`` is the achieved algorithmic
+bandwidth in GB/s (packed codes + scales + x + y per launch), inputs resident in
+HBM.  Launches are replayed from one HIP graph and timed with events on the
+launch stream, so ``ms_per_step`` is the kernel's own average duration.
 
 Extra objects on the same line:
   roofline      algorithmic bytes / average launch duration, against 8 TB/s
   cpu_baseline  the oracle's two-pass CPU linear (decode, then fp32 matmul)
                 timed on this box's host cores on a bounded number of passes
-  decode / prefill  secondary figures (filled when those paths are enabled)
+  decode        resident greedy decode of the 14B-shaped model: tokens/s from
+                graph replays and its fraction of the bandwidth roofline
+  prefill       MFMA GEMM chunks at the 14B linear shapes, N in {8, 16, 32}
 """
 
 from __future__ import annotations
@@ -28,6 +32,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
 
 M, K = 13824, 5120  # headline layer: 14B gate/up projection
 
@@ -51,60 +56,157 @@ def make_weights(torch, nf4, m: int, k: int, copies: int, seed: int):
     return out
 
 
-def time_gemv(torch, nf4, weights, x, m, k, steps: int, warmup: int):
-    y = torch.empty(m, dtype=torch.bfloat16, device="cuda")
-    n = len(weights)
-    for i in range(warmup):
-        p, s = weights[i % n]
-        nf4.nf4_gemv(p, s, x, m, k, k, y)
-    torch.cuda.synchronize()
-    # Per-launch durations from events recorded on the launch stream.
-    evs = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
-    t0 = time.perf_counter()
-    evs[0].record()
-    for i in range(steps):
-        p, s = weights[i % n]
-        nf4.nf4_gemv(p, s, x, m, k, k, y)
-        evs[i + 1].record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    per = [evs[i].elapsed_time(evs[i + 1]) for i in range(steps)]  # ms, includes launch gaps
-    return wall, per
-
-
-def time_gemv_graph(torch, nf4, weights, x, m, k, steps: int):
-    """The same launches replayed from one HIP graph: back-to-back kernels with
-    no host launch cost between them, so total/steps is the kernel's own
-    duration (plus the in-graph dispatch gap)."""
-    y = torch.empty(m, dtype=torch.bfloat16, device="cuda")
-    n = len(weights)
+def graph_time(torch, launch, n_launches: int, reps: int = 5) -> float:
+    """Capture ``n_launches`` calls of ``launch(i)`` into one HIP graph and return
+    the best average milliseconds per launch over ``reps`` replays (events on the
+    capture stream bracket each replay)."""
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
-        for i in range(n):
-            p, s = weights[i]
-            nf4.nf4_gemv(p, s, x, m, k, k, y)
+        for i in range(min(n_launches, 32)):
+            launch(i)
         side.synchronize()
         graph = torch.cuda.CUDAGraph()
         graph.capture_begin()
-        for i in range(steps):
-            p, s = weights[i % n]
-            nf4.nf4_gemv(p, s, x, m, k, k, y)
+        for i in range(n_launches):
+            launch(i)
         graph.capture_end()
+        graph.replay()
+        side.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        best = None
+        for _ in range(reps):
+            e0.record(side)
+            graph.replay()
+            e1.record(side)
+            side.synchronize()
+            ms = e0.elapsed_time(e1)
+            best = ms if best is None else min(best, ms)
     torch.cuda.current_stream().wait_stream(side)
-    graph.replay()
+    return best / n_launches
+
+
+def bench_gemv(torch, nf4, steps: int, warmup: int, copies: int):
+    by = algorithmic_bytes(M, K)
+    copies = max(copies, -(-512 * 1024 * 1024 // by) + 1)
+    weights = make_weights(torch, nf4, M, K, copies, seed=1234)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(99)
+    x = torch.randn(K, generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+    y = torch.empty(M, dtype=torch.bfloat16, device="cuda")
+
+    def launch(i):
+        p, s = weights[i % copies]
+        nf4.nf4_gemv(p, s, x, M, K, K, y)
+
+    # eager loop: W warm-up steps, then exactly K steps between two syncs
+    for i in range(warmup):
+        launch(i)
     torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        launch(i)
+    torch.cuda.synchronize()
+    eager_ms = (time.perf_counter() - t0) * 1e3 / steps
+    ms = graph_time(torch, launch, steps)
+    del weights
+    torch.cuda.empty_cache()
+    return ms, eager_ms, copies, by
+
+
+def bench_prefill(torch, nf4):
+    """MFMA GEMM chunks at the 14B linear shapes; weights rotate through > 512 MB."""
+    shapes = {"qkv": (7168, 5120), "o": (5120, 5120), "gate_up": (13824, 5120), "down": (5120, 13824)}
+    rows = []
+    for name, (m, k) in shapes.items():
+        by1 = algorithmic_bytes(m, k, 1)
+        copies = -(-512 * 1024 * 1024 // by1) + 1
+        weights = make_weights(torch, nf4, m, k, copies, seed=4321)
+        for n in (8, 16, 32):
+            x = (torch.randn((k, n), device="cuda") ).to(torch.bfloat16)
+
+            def launch(i):
+                p, s = weights[i % copies]
+                nf4.nf4_gemm(p, s, x, m, k, k)
+
+            ms = graph_time(torch, launch, 3 * copies, reps=3)
+            by = algorithmic_bytes(m, k, n)
+            rows.append({"layer": name, "M": m, "K": k, "N": n, "us": ms * 1e3,
+                         "gbps": by / (ms * 1e-3) / 1e9,
+                         "hbm_frac": by / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                         "mfma_frac": 2.0 * m * k * n / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS})
+        del weights
+        torch.cuda.empty_cache()
+    return rows
+
+
+def bench_decode(torch, spec_name: str, prompt_len: int, new_tokens: int):
+    """Resident greedy decode on random-init weights: chunked prefill of a random
+    prompt, then ``new_tokens`` graph replays with no host read in between."""
+    from deepfold_amd import decodev2 as dv2
+
+    spec = {"3b": dv2.QWEN25_3B, "14b": dv2.QWEN25_14B, "20b": dv2.INTERNLM25_20B,
+            "32b": dv2.QWEN25_32B}[spec_name]
+    t0 = time.perf_counter()
+    weights = dv2.DeviceWeights.random(spec, seed=2026)
+    torch.cuda.synchronize()
+    load_s = time.perf_counter() - t0
+    state = dv2.DecodeState.allocate(spec, device="cuda")
+    g = torch.Generator(device="cpu")
+    g.manual_seed(7)
+    prompt = torch.randint(0, spec.vocab, (prompt_len,), generator=g).tolist()
+    # prefill (eager, 32-position chunks)
+    state.reset()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    dv2.consume_prompt(state, weights, prompt)
+    torch.cuda.synchronize()
+    prefill_ms = (time.perf_counter() - t0) * 1e3
+    state.token.copy_(state.next_token)
+    # graph capture advances the state by warmup+1 tokens; that is part of the run
+    graph = dv2.capture_greedy(state, weights, warmup=2)
+    torch.cuda.synchronize()
+    start_pos = int(state.position.item())
     e0 = torch.cuda.Event(enable_timing=True)
     e1 = torch.cuda.Event(enable_timing=True)
-    best = None
-    for _ in range(5):
-        e0.record()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(new_tokens):
         graph.replay()
-        e1.record()
-        torch.cuda.synchronize()
-        ms = e0.elapsed_time(e1)
-        best = ms if best is None else min(best, ms)
-    return best / steps  # ms per launch
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    dev_ms = e0.elapsed_time(e1)
+    end_pos = int(state.position.item())
+    assert end_pos == start_pos + new_tokens
+    # eager step for comparison (a few tokens)
+    t0 = time.perf_counter()
+    for _ in range(8):
+        dv2.greedy_decode(state, weights)
+    torch.cuda.synchronize()
+    eager_ms = (time.perf_counter() - t0) * 1e3 / 8
+    ms_tok = dev_ms / new_tokens
+    mean_ctx = (start_pos + end_pos) / 2.0
+    bytes_tok = spec.weight_bytes_per_token() + spec.kv_bytes(mean_ctx)
+    roof_ms = bytes_tok / (HBM_PEAK_GBPS * 1e9) * 1e3
+    out = {
+        "model": spec.name, "layers": spec.n_layers, "hidden": spec.hidden, "ffn": spec.intermediate,
+        "vocab": spec.vocab, "max_seq": spec.max_seq, "prompt_tokens": prompt_len,
+        "new_tokens": new_tokens, "context_start": start_pos, "context_end": end_pos,
+        "tok_s": 1e3 / ms_tok, "ms_per_token": ms_tok, "tok_s_host_clock": new_tokens / wall,
+        "eager_ms_per_token": eager_ms, "prefill_ms": prefill_ms,
+        "prefill_tok_s": prompt_len / (prefill_ms * 1e-3),
+        "weight_gb_per_token": spec.weight_bytes_per_token() / 1e9,
+        "kv_mb_per_token_mean": spec.kv_bytes(mean_ctx) / 1e6,
+        "roofline_ms_per_token": roof_ms, "roofline_tok_s": 1e3 / roof_ms,
+        "roofline_frac": roof_ms / ms_tok, "achieved_gbps": bytes_tok / (ms_tok * 1e-3) / 1e9,
+        "weights_load_s": load_s,
+    }
+    del graph, state, weights
+    torch.cuda.empty_cache()
+    return out
 
 
 def cpu_baseline(m: int, k: int, budget_s: float = 12.0) -> dict:
@@ -162,6 +264,11 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--copies", type=int, default=16, help="distinct weight copies to rotate through")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-decode", action="store_true", help="skip the model decode leg")
+    ap.add_argument("--no-prefill", action="store_true", help="skip the prefill GEMM sweep")
+    ap.add_argument("--decode-models", default="14b", help="comma list of 3b,14b,20b,32b")
+    ap.add_argument("--prompt", type=int, default=512)
+    ap.add_argument("--new-tokens", type=int, default=256)
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build drives one GPU; --gpus N with N > 1 is not supported "
@@ -176,17 +283,9 @@ def main() -> int:
         print("bench.py: no GPU visible", file=sys.stderr)
         return 2
     torch.cuda.set_device(0)
-    by = algorithmic_bytes(M, K)
-    copies = max(args.copies, -(-512 * 1024 * 1024 // by) + 1)
-    weights = make_weights(torch, nf4, M, K, copies, seed=1234)
-    g = torch.Generator(device="cuda")
-    g.manual_seed(99)
-    x = torch.randn(K, generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16)
 
-    wall, per = time_gemv(torch, nf4, weights, x, M, K, args.steps, args.warmup)
-    graph_ms = time_gemv_graph(torch, nf4, weights, x, M, K, max(args.steps, 64))
-    kernel_s = graph_ms * 1e-3
-    achieved = by / kernel_s / 1e9
+    ms, eager_ms, copies, by = bench_gemv(torch, nf4, args.steps, args.warmup, args.copies)
+    achieved = by / (ms * 1e-3) / 1e9
     out = {
         "metric": "nf4_gemv_hbm_gbps",
         "value": achieved,
@@ -194,19 +293,18 @@ def main() -> int:
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": graph_ms,
+        "ms_per_step": ms,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f32",
         "data": "synthetic",
         "config": {
-            "workload": f"decode GEMV x[1,{K}] bf16 @ W[{M},{K}] NF4 group-64, {copies} rotating weight copies "
-                        f"({copies * by / 2**20:.0f} MiB)",
+            "workload": f"decode GEMV x[1,{K}] bf16 @ W[{M},{K}] NF4 group-64, {copies} rotating weight "
+                        f"copies ({copies * by / 2**20:.0f} MiB)",
             "M": M, "K": K, "N": 1,
         },
-        "eager_ms_per_step": wall * 1e3 / args.steps,
-        "eager_event_median_ms": sorted(per)[len(per) // 2],
+        "eager_ms_per_step": eager_ms,
         "roofline": {
             "bound": "hbm",
             "achieved": achieved,
@@ -214,10 +312,15 @@ def main() -> int:
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS,
             "traffic": None,
-            "kernel": "gemv_rows",
+            "kernel": "gemv_stream",
             "algorithmic_bytes_per_launch": by,
         },
     }
+    if not args.no_decode:
+        out["decode"] = [bench_decode(torch, name.strip(), args.prompt, args.new_tokens)
+                         for name in args.decode_models.split(",") if name.strip()]
+    if not args.no_prefill:
+        out["prefill"] = bench_prefill(torch, nf4)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(M, K)
     print(json.dumps(out), flush=True)

@@ -41,7 +41,24 @@ __global__ __launch_bounds__(kArgmaxBlock) void argmax_commit(
   __shared__ int si[kArgmaxBlock / kWave];
   float bv = -__builtin_inff();
   int bi = 0x7FFFFFFF;
-  for (int i = threadIdx.x; i < n; i += kArgmaxBlock) {
+  // Eight logits per 16-byte load when the buffer allows it; indices rise within
+  // a thread, so "strictly better" keeps the lowest index of equal values.
+  const bool vec = (reinterpret_cast<uintptr_t>(logits) & 15u) == 0;
+  const int n8 = vec ? n >> 3 : 0;
+  for (int c = threadIdx.x; c < n8; c += kArgmaxBlock) {
+    const uint4 raw = reinterpret_cast<const uint4 *>(logits)[c];
+    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float v = (j & 1) ? bf16_hi(w[j >> 1]) : bf16_lo(w[j >> 1]);
+      const int i = (c << 3) + j;
+      if (better(v, i, bv, bi)) {
+        bv = v;
+        bi = i;
+      }
+    }
+  }
+  for (int i = (n8 << 3) + threadIdx.x; i < n; i += kArgmaxBlock) {
     const float v = bf16_to_f32(logits[i]);
     if (better(v, i, bv, bi)) {
       bv = v;

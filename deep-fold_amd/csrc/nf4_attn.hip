@@ -311,6 +311,10 @@ __global__ __launch_bounds__(kWave) void attn_flash_generic(const AttnArgs a) {
 
 // out[head] = sum_s a_s o_s / sum_s a_s l_s with a_s = exp(m_s - max m); an
 // empty split has m = -1e30 and l = 0, so its weight underflows to zero.
+// One wavefront per head.  Lane s first takes split s's (m, l) so the maximum
+// and the denominator are wavefront reductions; then every lane owns dims
+// l, l+64, .. and walks the splits with all loads independent (unrolled), the
+// sum over splits running in split order.
 __global__ __launch_bounds__(kWave) void attn_merge(const float *__restrict__ m_s,
                                                     const float *__restrict__ l_s,
                                                     const float *__restrict__ o_s,
@@ -320,31 +324,46 @@ __global__ __launch_bounds__(kWave) void attn_merge(const float *__restrict__ m_
   const int lane = threadIdx.x;
   const float *mh = m_s + static_cast<size_t>(head) * n_split;
   const float *lh = l_s + static_cast<size_t>(head) * n_split;
-  float m = kNegBig;
-  for (int s = 0; s < n_split; ++s) {
-    m = fmaxf(m, mh[s]);
-  }
-  float l = 0.f;
-  float acc[4] = {};
-  for (int s = 0; s < n_split; ++s) {
-    const float w = __expf(mh[s] - m);
-    l += w * lh[s];
-    const float *oh = o_s + (static_cast<size_t>(head) * n_split + s) * hd;
+  const float my_m = lane < n_split ? mh[lane] : kNegBig;
+  const float my_l = lane < n_split ? lh[lane] : 0.f;
+  float m = my_m;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int d = lane + 64 * i;
-      if (d < hd) {
-        acc[i] += w * oh[d];
+  for (int off = 32; off > 0; off >>= 1) {
+    m = fmaxf(m, __shfl_xor(m, off, kWave));
+  }
+  const float my_w = __expf(my_m - m);  // weight of split `lane`
+  float l = my_w * my_l;
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    l += __shfl_xor(l, off, kWave);
+  }
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  const float *oh = o_s + static_cast<size_t>(head) * n_split * hd;
+  uint16_t *dst = out + static_cast<size_t>(head) * hd;
+  // Every lane runs every iteration (the shuffles below read other lanes);
+  // lanes past hd only skip the memory accesses.
+  for (int d0 = 0; d0 < hd; d0 += kWave) {
+    const int d = d0 + lane;
+    const bool on = d < hd;
+    float acc = 0.f;
+    int s = 0;
+    for (; s + 8 <= n_split; s += 8) {
+      float v[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        v[j] = on ? oh[static_cast<size_t>(s + j) * hd + d] : 0.f;
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        acc += __shfl(my_w, s + j, kWave) * v[j];
       }
     }
-  }
-  uint16_t *dst = out + static_cast<size_t>(head) * hd;
-  const float inv = l > 0.f ? 1.f / l : 0.f;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int d = lane + 64 * i;
-    if (d < hd) {
-      dst[d] = f32_to_bf16(l > 0.f ? acc[i] * inv : 0.f);
+    for (; s < n_split; ++s) {
+      const float v = on ? oh[static_cast<size_t>(s) * hd + d] : 0.f;
+      acc += __shfl(my_w, s, kWave) * v;
+    }
+    if (on) {
+      dst[d] = f32_to_bf16(l > 0.f ? acc * inv : 0.f);
     }
   }
 }

@@ -368,8 +368,22 @@ __global__ __launch_bounds__(kRmsBlock) void rms_vec(const uint16_t *__restrict_
                                                      const uint16_t *__restrict__ w,
                                                      uint16_t *__restrict__ y, int n, float eps) {
   __shared__ float part[kRmsBlock / kWave];
+  // Up to 8 elements per thread stay in registers (n <= 8192), so x and w are
+  // each read once and both loads are in flight before the reduction.
+  constexpr int kKeep = 8;
+  float xv[kKeep], wv[kKeep];
   float a = 0.f;
-  for (int i = threadIdx.x; i < n; i += kRmsBlock) {
+#pragma unroll
+  for (int j = 0; j < kKeep; ++j) {
+    const int i = threadIdx.x + j * kRmsBlock;
+    xv[j] = i < n ? bf16_to_f32(x[i]) : 0.f;
+    wv[j] = i < n ? bf16_to_f32(w[i]) : 0.f;
+  }
+#pragma unroll
+  for (int j = 0; j < kKeep; ++j) {
+    a = fmaf(xv[j], xv[j], a);
+  }
+  for (int i = threadIdx.x + kKeep * kRmsBlock; i < n; i += kRmsBlock) {
     const float v = bf16_to_f32(x[i]);
     a = fmaf(v, v, a);
   }
@@ -384,7 +398,14 @@ __global__ __launch_bounds__(kRmsBlock) void rms_vec(const uint16_t *__restrict_
     sum += part[i];
   }
   const float inv = rsqrtf(sum / static_cast<float>(n) + eps);
-  for (int i = threadIdx.x; i < n; i += kRmsBlock) {
+#pragma unroll
+  for (int j = 0; j < kKeep; ++j) {
+    const int i = threadIdx.x + j * kRmsBlock;
+    if (i < n) {
+      y[i] = f32_to_bf16((wv[j] * xv[j]) * inv);
+    }
+  }
+  for (int i = threadIdx.x + kKeep * kRmsBlock; i < n; i += kRmsBlock) {
     y[i] = f32_to_bf16((bf16_to_f32(w[i]) * bf16_to_f32(x[i])) * inv);
   }
 }

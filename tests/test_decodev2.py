@@ -197,3 +197,69 @@ def test_packed_embedding_rows_and_random_weights_step():
     dv2.greedy_decode(state, w)
     assert torch.isfinite(state.arena.logits.float()).all()
     assert 0 <= int(state.token.item()) < 1000 and int(state.position.item()) == 1
+
+
+LONGRUN = dv2.ArchSpec("longrun", "llama_swiglu", 4, 512, 8, 2, 64, 1536, 2048, 128, qkv_bias=False)
+
+
+def near_tie(logits: np.ndarray) -> bool:
+    """True when the two largest logits are closer than four bf16 steps of their
+    size: the GPU stores logits as bf16, so such a pick is a coin toss."""
+    top = np.sort(logits)[-2:]
+    return float(top[1] - top[0]) <= 4 * 2.0 ** (np.floor(np.log2(max(abs(top[1]), 1e-30))) - 7)
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2, 3])
+def test_greedy_64_tokens_identical_to_the_oracle(seed):
+    """64 generated tokens on random-init weights, ignore-EOS, eager and graph.
+    The stream must equal the oracle's; the only excuse for a first difference is
+    an oracle pick that is itself a near-tie at bf16 logit resolution."""
+    say("64 tokens seed", seed)
+    model, state, weights = session(LONGRUN, seed)
+    prompt = [11, 200, 37, 1999, 5, 640, 3, 77]
+    want, margins = so.greedy_ids(model, prompt, 64, ignore_eos=True, return_margins=True)
+    assert len(want) == 64
+    state.reset()
+    got = dv2.generate(state, weights, prompt, 64, ignore_eos=True)
+    say("  min / median top-1 margin", min(margins), float(np.median(margins)))
+    state.reset()
+    graph = dv2.capture_greedy(state, weights, warmup=1)
+    state.reset()
+    assert dv2.generate(state, weights, prompt, 64, step=graph, ignore_eos=True) == got
+    if got != want:
+        first = next(i for i, (a, b) in enumerate(zip(got, want)) if a != b)
+        logits = so.teacher_logits(model, prompt + want[:first])[-1]
+        say("  first difference at", first, "oracle margin", margins[first])
+        assert near_tie(logits), (first, margins[first])
+    IDENTICAL.append(got == want)
+
+
+IDENTICAL: list[bool] = []
+
+
+def test_some_seed_is_fully_identical():
+    # Random-init logits have a median top-1/top-2 gap of ~0.1 and a minimum over
+    # 64 picks that is usually below one bf16 step, so most streams hit a coin-toss
+    # pick somewhere; at least one of the four seeds must go all 64 tokens.
+    assert len(IDENTICAL) == 4 and sum(IDENTICAL) >= 1, IDENTICAL
+
+
+def test_teacher_forced_picks_agree_except_on_near_ties():
+    """Feed the oracle's own tokens: every GPU pick equals the oracle's pick unless
+    the oracle's top-1/top-2 logit gap is within bf16 resolution of the logit."""
+    model, state, weights = session(LONGRUN, 3)
+    rng = np.random.default_rng(5)
+    toks = rng.integers(0, LONGRUN.vocab, size=96).tolist()
+    want = so.teacher_logits(model, toks)
+    state.reset()
+    disagree = 0
+    for i, t in enumerate(toks):
+        dv2.teacher_force_token(state, weights, t)
+        pick = int(state.next_token.item())
+        ref = int(want[i].argmax())
+        if pick != ref:
+            top = np.sort(want[i])[-2:]
+            gap = float(top[1] - top[0])
+            assert gap <= 4 * 2.0 ** (np.floor(np.log2(abs(top[1]))) - 7), (i, gap)
+            disagree += 1
+    assert disagree <= 3
