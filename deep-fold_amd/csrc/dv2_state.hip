@@ -10,7 +10,77 @@
 #include "nf4_common.h"
 
 namespace chr {
+
+int gemv_add_norm_entry(const chr_nf4_dev_t *w, const void *x, void *y, const void *norm_w,
+                        float norm_eps, void *norm_out, float *scratch, int64_t scratch_floats,
+                        void *stream);
+int gemv_norm_blocks(int M);
+
 namespace {
+
+constexpr int kBeginBlock = 1024;
+
+// First launch of a fused decode step, one workgroup:
+//   valid_len = position + 1
+//   x   = bf16( LUT[code] * f32(scale) ) for row *token of the packed embedding
+//   h   = RMSNorm(x, norm_w, eps) rounded to bf16
+// i.e. GraphSafeKV.mark_written + the embedding gather + the first RMSNorm.
+__global__ __launch_bounds__(kBeginBlock) void begin_step(
+    const uint8_t *__restrict__ packed, const uint16_t *__restrict__ scale, int M, int K, int K_pad,
+    const int64_t *__restrict__ token, const int64_t *__restrict__ position,
+    int32_t *__restrict__ valid_len, uint16_t *__restrict__ x, const uint16_t *__restrict__ norm_w,
+    float eps, uint16_t *__restrict__ h) {
+  __shared__ float lut[16];
+  __shared__ float part[kBeginBlock / kWave];
+  if (threadIdx.x < 16) {
+    lut[threadIdx.x] = bits_to_f32(kLutBits[threadIdx.x]);
+  }
+  if (threadIdx.x == 0) {
+    *valid_len = static_cast<int32_t>(*position) + 1;
+  }
+  __syncthreads();
+  const int64_t id = *token;
+  const bool ok = id >= 0 && id < M;  // an id outside the table decodes to zeros
+  const uint32_t *prow =
+      reinterpret_cast<const uint32_t *>(packed + static_cast<size_t>(ok ? id : 0) * (K_pad >> 1));
+  const uint16_t *srow = scale + static_cast<size_t>(ok ? id : 0) * (K_pad >> 6);
+  float sq = 0.f;
+  for (int d = threadIdx.x; d < (K_pad >> 3); d += kBeginBlock) {
+    const uint32_t w = ok ? prow[d] : 0x77777777u;
+    const float s = ok ? f16_to_f32(srow[d >> 3]) : 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int k = (d << 3) + j;
+      if (k < K) {
+        const uint16_t b = f32_to_bf16(lut[(w >> (4 * j)) & 0xFu] * s);
+        x[k] = b;
+        const float v = bf16_to_f32(b);
+        sq = fmaf(v, v, sq);
+      }
+    }
+  }
+  sq = wave_sum(sq);
+  if ((threadIdx.x & (kWave - 1)) == 0) {
+    part[threadIdx.x >> 6] = sq;
+  }
+  __syncthreads();  // also orders this workgroup's x stores before the reads below
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < kBeginBlock / kWave; ++i) {
+    sum += part[i];
+  }
+  const float inv = rsqrtf(sum / static_cast<float>(K) + eps);
+  for (int d = threadIdx.x; d < (K_pad >> 3); d += kBeginBlock) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int k = (d << 3) + j;
+      if (k < K) {
+        // each thread re-reads only what it stored itself
+        h[k] = f32_to_bf16((bf16_to_f32(norm_w[k]) * bf16_to_f32(x[k])) * inv);
+      }
+    }
+  }
+}
 
 __global__ void mark_written(const int64_t *__restrict__ position, int32_t *__restrict__ valid_len) {
   if (threadIdx.x == 0) {
@@ -102,6 +172,40 @@ __global__ __launch_bounds__(kArgmaxBlock) void argmax_commit(
 }  // namespace chr
 
 using namespace chr;
+
+extern "C" int chr_dv2_begin_step(const chr_nf4_dev_t *table, const void *token,
+                                  const void *position, void *valid_len, void *x,
+                                  const void *norm_w, float eps, void *h, void *stream) {
+  if (table == nullptr || token == nullptr || position == nullptr || valid_len == nullptr ||
+      x == nullptr || norm_w == nullptr || h == nullptr) {
+    return -1;
+  }
+  if (table->M < 1 || table->K < 1 || table->packed == nullptr || table->scale == nullptr) {
+    return -3;
+  }
+  if (!k_pad_ok(table->K, table->K_pad)) {
+    return -4;
+  }
+  if ((reinterpret_cast<uintptr_t>(table->packed) & 3u) != 0 || !aligned2(table->scale)) {
+    return -5;
+  }
+  begin_step<<<dim3(1), dim3(kBeginBlock), 0, static_cast<hipStream_t>(stream)>>>(
+      table->packed, table->scale, table->M, table->K, table->K_pad,
+      static_cast<const int64_t *>(token), static_cast<const int64_t *>(position),
+      static_cast<int32_t *>(valid_len), static_cast<uint16_t *>(x),
+      static_cast<const uint16_t *>(norm_w), eps, static_cast<uint16_t *>(h));
+  return launch_rc();
+}
+
+extern "C" int chr_dv2_gemv_add_norm(const chr_nf4_dev_t *w, const void *x, void *y,
+                                     const void *norm_w, float norm_eps, void *norm_out,
+                                     float *scratch, int64_t scratch_floats, void *stream) {
+  return gemv_add_norm_entry(w, x, y, norm_w, norm_eps, norm_out, scratch, scratch_floats, stream);
+}
+
+extern "C" int64_t chr_dv2_gemv_add_norm_scratch(int32_t M) {
+  return M < 1 ? 0 : 16 + static_cast<int64_t>(gemv_norm_blocks(M));
+}
 
 extern "C" int chr_dv2_mark_written(const void *position, void *valid_len, void *stream) {
   if (position == nullptr || valid_len == nullptr) {

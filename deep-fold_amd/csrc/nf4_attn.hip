@@ -75,10 +75,107 @@ struct AttnArgs {
   const int64_t *position;
   int n_q, n_kv, hd, n_split, max_seq;
   float scale;
+  // fused merge (attn_flash<.., true>): the wavefront that finishes a head last
+  // folds that head's splits; head_count[n_q] is zero between launches
+  uint16_t *out;
+  unsigned int *head_count;
 };
 
+// Split partials that another wavefront of the same launch reads back travel at
+// device scope; the two-launch form uses ordinary accesses.
+template <bool COHERENT>
+__device__ __forceinline__ float ld_f32(const float *p) {
+  if constexpr (COHERENT) {
+    return load_coherent(p);
+  } else {
+    return *p;
+  }
+}
+template <bool COHERENT>
+__device__ __forceinline__ void st_f32(float *p, float v) {
+  if constexpr (COHERENT) {
+    store_coherent(p, v);
+  } else {
+    *p = v;
+  }
+}
+
+// out[head] = sum_s a_s o_s / sum_s a_s l_s with a_s = exp(m_s - max m); an
+// empty split has m = -1e30 and l = 0, so its weight underflows to zero.
+// One wavefront per head.  Lane s first takes split s's (m, l) so the maximum
+// and the denominator are wavefront reductions; then every lane owns dims
+// l, l+64, .. and walks the splits with all loads independent (unrolled), the
+// sum over splits running in split order.
+template <bool COHERENT>
+__device__ __forceinline__ void merge_head(const float *m_s, const float *l_s, const float *o_s,
+                                           uint16_t *out, int head, int hd, int n_split,
+                                           int lane) {
+  const float *mh = m_s + static_cast<size_t>(head) * n_split;
+  const float *lh = l_s + static_cast<size_t>(head) * n_split;
+  const float my_m = lane < n_split ? ld_f32<COHERENT>(mh + lane) : kNegBig;
+  const float my_l = lane < n_split ? ld_f32<COHERENT>(lh + lane) : 0.f;
+  float m = my_m;
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    m = fmaxf(m, __shfl_xor(m, off, kWave));
+  }
+  const float my_w = __expf(my_m - m);  // weight of split `lane`
+  float l = my_w * my_l;
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    l += __shfl_xor(l, off, kWave);
+  }
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  const float *oh = o_s + static_cast<size_t>(head) * n_split * hd;
+  uint16_t *dst = out + static_cast<size_t>(head) * hd;
+  // Every lane runs every iteration (the shuffles below read other lanes);
+  // lanes past hd only skip the memory accesses.
+  for (int d0 = 0; d0 < hd; d0 += kWave) {
+    const int d = d0 + lane;
+    const bool on = d < hd;
+    float acc = 0.f;
+    int s = 0;
+    for (; s + 8 <= n_split; s += 8) {
+      float v[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        v[j] = on ? ld_f32<COHERENT>(oh + static_cast<size_t>(s + j) * hd + d) : 0.f;
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        acc += __shfl(my_w, s + j, kWave) * v[j];
+      }
+    }
+    for (; s < n_split; ++s) {
+      const float v = on ? ld_f32<COHERENT>(oh + static_cast<size_t>(s) * hd + d) : 0.f;
+      acc += __shfl(my_w, s, kWave) * v;
+    }
+    if (on) {
+      dst[d] = f32_to_bf16(l > 0.f ? acc * inv : 0.f);
+    }
+  }
+}
+
+// After a wavefront has stored its split's partials: take a ticket for the head;
+// the wavefront holding the last ticket merges the head and re-arms the counter.
+__device__ __forceinline__ void merge_if_last(const AttnArgs &a, int head, int lane) {
+  unsigned int ticket = 0;
+  drain_stores();  // this wavefront's partials have landed before its ticket
+  if (lane == 0) {
+    ticket = atomicAdd(a.head_count + head, 1u);
+  }
+  ticket = static_cast<unsigned int>(__shfl(static_cast<int>(ticket), 0, kWave));
+  if (ticket != static_cast<unsigned int>(a.n_split - 1)) {
+    return;
+  }
+  merge_head<true>(a.m_s, a.l_s, a.o_s, a.out, head, a.hd, a.n_split, lane);
+  if (lane == 0) {
+    store_coherent(a.head_count + head, 0u);
+  }
+}
+
 // LPT lanes per time step, 8 dims per lane: hd == 8*LPT.
-template <int LPT>
+template <int LPT, bool FUSED>
 __global__ __launch_bounds__(kWave) void attn_flash(const AttnArgs a) {
   constexpr int TPW = kWave / LPT;  // time steps per wavefront iteration
   const int head = blockIdx.x / a.n_split;
@@ -193,18 +290,29 @@ __global__ __launch_bounds__(kWave) void attn_flash(const AttnArgs a) {
 
   const size_t slot = static_cast<size_t>(head) * a.n_split + split;
   if (lane == 0) {
-    a.m_s[slot] = m;
-    a.l_s[slot] = l;
+    st_f32<FUSED>(a.m_s + slot, m);
+    st_f32<FUSED>(a.l_s + slot, l);
   }
   if (grp == 0) {
     float *oh = a.o_s + slot * hd + d0;
-    *reinterpret_cast<float4 *>(oh) = make_float4(acc[0], acc[1], acc[2], acc[3]);
-    *reinterpret_cast<float4 *>(oh + 4) = make_float4(acc[4], acc[5], acc[6], acc[7]);
+    if constexpr (FUSED) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        store_coherent(oh + j, acc[j]);
+      }
+    } else {
+      *reinterpret_cast<float4 *>(oh) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+      *reinterpret_cast<float4 *>(oh + 4) = make_float4(acc[4], acc[5], acc[6], acc[7]);
+    }
+  }
+  if constexpr (FUSED) {
+    merge_if_last(a, head, lane);
   }
 }
 
 // Any hd <= 256: lane l owns dims l, l+64, l+128, l+192; one time step per
 // iteration.  Slow path for head sizes that are not 8 * 2^n.
+template <bool FUSED>
 __global__ __launch_bounds__(kWave) void attn_flash_generic(const AttnArgs a) {
   const int head = blockIdx.x / a.n_split;
   const int split = blockIdx.x % a.n_split;
@@ -297,75 +405,28 @@ __global__ __launch_bounds__(kWave) void attn_flash_generic(const AttnArgs a) {
   }
   const size_t slot = static_cast<size_t>(head) * a.n_split + split;
   if (lane == 0) {
-    a.m_s[slot] = m;
-    a.l_s[slot] = l;
+    st_f32<FUSED>(a.m_s + slot, m);
+    st_f32<FUSED>(a.l_s + slot, l);
   }
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int d = lane + 64 * i;
     if (d < hd) {
-      a.o_s[slot * hd + d] = acc[i];
+      st_f32<FUSED>(a.o_s + slot * hd + d, acc[i]);
     }
+  }
+  if constexpr (FUSED) {
+    merge_if_last(a, head, lane);
   }
 }
 
-// out[head] = sum_s a_s o_s / sum_s a_s l_s with a_s = exp(m_s - max m); an
-// empty split has m = -1e30 and l = 0, so its weight underflows to zero.
-// One wavefront per head.  Lane s first takes split s's (m, l) so the maximum
-// and the denominator are wavefront reductions; then every lane owns dims
-// l, l+64, .. and walks the splits with all loads independent (unrolled), the
-// sum over splits running in split order.
+// The split merge as its own launch (the two-launch form of chr_nf4_attn).
 __global__ __launch_bounds__(kWave) void attn_merge(const float *__restrict__ m_s,
                                                     const float *__restrict__ l_s,
                                                     const float *__restrict__ o_s,
                                                     uint16_t *__restrict__ out, int hd,
                                                     int n_split) {
-  const int head = blockIdx.x;
-  const int lane = threadIdx.x;
-  const float *mh = m_s + static_cast<size_t>(head) * n_split;
-  const float *lh = l_s + static_cast<size_t>(head) * n_split;
-  const float my_m = lane < n_split ? mh[lane] : kNegBig;
-  const float my_l = lane < n_split ? lh[lane] : 0.f;
-  float m = my_m;
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) {
-    m = fmaxf(m, __shfl_xor(m, off, kWave));
-  }
-  const float my_w = __expf(my_m - m);  // weight of split `lane`
-  float l = my_w * my_l;
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) {
-    l += __shfl_xor(l, off, kWave);
-  }
-  const float inv = l > 0.f ? 1.f / l : 0.f;
-  const float *oh = o_s + static_cast<size_t>(head) * n_split * hd;
-  uint16_t *dst = out + static_cast<size_t>(head) * hd;
-  // Every lane runs every iteration (the shuffles below read other lanes);
-  // lanes past hd only skip the memory accesses.
-  for (int d0 = 0; d0 < hd; d0 += kWave) {
-    const int d = d0 + lane;
-    const bool on = d < hd;
-    float acc = 0.f;
-    int s = 0;
-    for (; s + 8 <= n_split; s += 8) {
-      float v[8];
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        v[j] = on ? oh[static_cast<size_t>(s + j) * hd + d] : 0.f;
-      }
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        acc += __shfl(my_w, s + j, kWave) * v[j];
-      }
-    }
-    for (; s < n_split; ++s) {
-      const float v = on ? oh[static_cast<size_t>(s) * hd + d] : 0.f;
-      acc += __shfl(my_w, s, kWave) * v;
-    }
-    if (on) {
-      dst[d] = f32_to_bf16(l > 0.f ? acc * inv : 0.f);
-    }
-  }
+  merge_head<false>(m_s, l_s, o_s, out, blockIdx.x, hd, n_split, threadIdx.x);
 }
 
 // Standalone RoPE + cache write: one wavefront per head (q heads first, then kv).
@@ -443,11 +504,32 @@ extern "C" int chr_nf4_rope_kv(void *q, void *k, const void *v, void *k_cache, v
   return launch_rc();
 }
 
-extern "C" int chr_nf4_attn(const void *q, const void *k, const void *v, void *out,
-                            const void *valid_len, float *ws, int32_t n_q, int32_t n_kv,
-                            int32_t hd, int32_t n_split, float scale, void *stream,
-                            const void *k_act, const void *v_act, const void *cos,
-                            const void *sin, const void *position, int32_t max_seq) {
+namespace chr {
+namespace {
+
+template <bool FUSED>
+void launch_flash(const AttnArgs &a, bool vec_ok, hipStream_t st) {
+  const dim3 grid(static_cast<unsigned>(a.n_q * a.n_split));
+  const dim3 block(kWave);
+  if (vec_ok && a.hd == 128) {
+    attn_flash<16, FUSED><<<grid, block, 0, st>>>(a);
+  } else if (vec_ok && a.hd == 64) {
+    attn_flash<8, FUSED><<<grid, block, 0, st>>>(a);
+  } else if (vec_ok && a.hd == 256) {
+    attn_flash<32, FUSED><<<grid, block, 0, st>>>(a);
+  } else if (vec_ok && a.hd == 32) {
+    attn_flash<4, FUSED><<<grid, block, 0, st>>>(a);
+  } else if (vec_ok && a.hd == 16) {
+    attn_flash<2, FUSED><<<grid, block, 0, st>>>(a);
+  } else {
+    attn_flash_generic<FUSED><<<grid, block, 0, st>>>(a);
+  }
+}
+
+int attn_common(const void *q, const void *k, const void *v, void *out, const void *valid_len,
+                float *ws, int32_t n_q, int32_t n_kv, int32_t hd, int32_t n_split, float scale,
+                void *stream, const void *k_act, const void *v_act, const void *cos,
+                const void *sin, const void *position, int32_t max_seq, unsigned int *head_count) {
   if (q == nullptr || k == nullptr || v == nullptr || out == nullptr || valid_len == nullptr ||
       ws == nullptr) {
     return -1;
@@ -480,29 +562,45 @@ extern "C" int chr_nf4_attn(const void *q, const void *k, const void *v, void *o
   a.n_split = n_split;
   a.max_seq = max_seq;
   a.scale = scale;
+  a.out = static_cast<uint16_t *>(out);
+  a.head_count = head_count;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const dim3 grid(static_cast<unsigned>(nml));
-  const dim3 block(kWave);
   // The vector path needs 16-byte aligned rows and 16-byte aligned fp32 partials.
   const bool vec_ok = aligned16(q) && aligned16(k) && aligned16(v) &&
                       (k_act == nullptr || aligned16(k_act)) &&
                       (v_act == nullptr || aligned16(v_act)) &&
                       (cos == nullptr || aligned16(cos)) && (sin == nullptr || aligned16(sin)) &&
                       aligned16(a.o_s);
-  if (vec_ok && hd == 128) {
-    attn_flash<16><<<grid, block, 0, st>>>(a);
-  } else if (vec_ok && hd == 64) {
-    attn_flash<8><<<grid, block, 0, st>>>(a);
-  } else if (vec_ok && hd == 256) {
-    attn_flash<32><<<grid, block, 0, st>>>(a);
-  } else if (vec_ok && hd == 32) {
-    attn_flash<4><<<grid, block, 0, st>>>(a);
-  } else if (vec_ok && hd == 16) {
-    attn_flash<2><<<grid, block, 0, st>>>(a);
+  if (head_count != nullptr) {
+    launch_flash<true>(a, vec_ok, st);
   } else {
-    attn_flash_generic<<<grid, block, 0, st>>>(a);
+    launch_flash<false>(a, vec_ok, st);
+    attn_merge<<<dim3(static_cast<unsigned>(n_q)), dim3(kWave), 0, st>>>(a.m_s, a.l_s, a.o_s, a.out,
+                                                                         hd, n_split);
   }
-  attn_merge<<<dim3(static_cast<unsigned>(n_q)), block, 0, st>>>(
-      a.m_s, a.l_s, a.o_s, static_cast<uint16_t *>(out), hd, n_split);
   return launch_rc();
+}
+
+}  // namespace
+}  // namespace chr
+
+extern "C" int chr_nf4_attn(const void *q, const void *k, const void *v, void *out,
+                            const void *valid_len, float *ws, int32_t n_q, int32_t n_kv,
+                            int32_t hd, int32_t n_split, float scale, void *stream,
+                            const void *k_act, const void *v_act, const void *cos,
+                            const void *sin, const void *position, int32_t max_seq) {
+  return attn_common(q, k, v, out, valid_len, ws, n_q, n_kv, hd, n_split, scale, stream, k_act,
+                     v_act, cos, sin, position, max_seq, nullptr);
+}
+
+extern "C" int chr_dv2_attn(const void *q, const void *k, const void *v, void *out,
+                            const void *valid_len, float *ws, void *head_count, int32_t n_q,
+                            int32_t n_kv, int32_t hd, int32_t n_split, float scale, void *stream,
+                            const void *k_act, const void *v_act, const void *cos,
+                            const void *sin, const void *position, int32_t max_seq) {
+  if (head_count == nullptr) {
+    return -1;
+  }
+  return attn_common(q, k, v, out, valid_len, ws, n_q, n_kv, hd, n_split, scale, stream, k_act,
+                     v_act, cos, sin, position, max_seq, static_cast<unsigned int *>(head_count));
 }

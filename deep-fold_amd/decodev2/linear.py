@@ -149,7 +149,13 @@ class DeviceWeights:
             return DeviceLayer(vec(ly.norm1), vec(ly.norm2), up(ly.q), up(ly.k), up(ly.v),
                                up(ly.wqkv, order), up(ly.o), up(ly.gate), up(ly.up), up(ly.down))
 
-        return cls(spec, vec(model.embed), vec(model.final_norm), up(model.lm_head),
+        embed: torch.Tensor | PackedEmbed
+        if model.embed_nf4 is not None:
+            e = DeviceLinear.from_nf4(model.embed_nf4, device, dtype)
+            embed = PackedEmbed(e.packed, e.scale, spec.vocab, spec.hidden)
+        else:
+            embed = vec(model.embed)
+        return cls(spec, embed, vec(model.final_norm), up(model.lm_head),
                    [layer(ly) for ly in model.layers])
 
     @classmethod

@@ -8,18 +8,27 @@ Per layer: rms -> q/k/v GEMV -> attention (RoPE and the cache write fused) ->
 o GEMV accumulating into the residual -> rms -> fused SwiGLU GEMV -> down GEMV
 accumulating into the residual.  Then the final norm, lm_head and a device-side
 argmax that also feeds the id back.
+
+Two launch schedules compute that sequence.  The plain one issues it call by call
+(eight launches per layer) and is the default.  The fused one needs five: every
+RMSNorm rides on the launch that produces its input (the embedding gather, or the
+residual GEMV whose last workgroup normalises), and the attention launch merges
+its own splits.  On MI355X the hand-over between workgroups inside a launch costs
+more than the launches it saves (a device-scope round trip per stage), so the
+fused schedule is kept for comparison and only runs on request.
 """
 
 from __future__ import annotations
 
 import torch
 
-from ..nf4 import ATTN_SPLIT, nf4_attn, nf4_gemv, nf4_qkv, nf4_rms, nf4_swiglu
-from .embed import gather_embed
+from ..nf4 import (ATTN_SPLIT, dv2_attn, dv2_begin_step, dv2_gemv_add_norm, nf4_attn, nf4_gemv,
+                   nf4_qkv, nf4_rms, nf4_swiglu)
+from .embed import PackedEmbed, gather_embed
 from .linear import DeviceLayer, DeviceLinear, DeviceWeights
 from .state import DecodeState
 
-__all__ = ["forward_decode", "greedy_decode", "teacher_force_token"]
+__all__ = ["forward_decode", "greedy_decode", "teacher_force_token", "can_fuse"]
 
 
 def _gemv_accum(mat: DeviceLinear, src: torch.Tensor, dest: torch.Tensor) -> None:
@@ -47,9 +56,64 @@ def _qkv(state: DecodeState, layer: DeviceLayer, h: torch.Tensor):
     return ar.q.view(-1), ar.k.view(-1), ar.v.view(-1)
 
 
-def forward_decode(state: DecodeState, weights: DeviceWeights, *, commit: bool = False) -> None:
+def can_fuse(weights: DeviceWeights) -> bool:
+    """Whether the five-launch schedule applies: packed embedding rows, no bias on
+    the residual projections, and reduction lengths that are whole scale groups."""
+    spec = weights.spec
+    if not isinstance(weights.embed, PackedEmbed):
+        return False
+    if spec.q_dim % 64 or spec.intermediate % 64:
+        return False
+    return all(ly.o.bias is None and ly.down.bias is None for ly in weights.layers)
+
+
+def _gemv_accum_norm(state: DecodeState, mat: DeviceLinear, src: torch.Tensor, norm_w: torch.Tensor) -> None:
+    """``x += W @ src`` and ``h = RMSNorm(x, norm_w)`` in one launch."""
+    ar = state.arena
+    dv2_gemv_add_norm(mat.packed, mat.scale, src.view(-1), mat.M, mat.K, mat.K_pad, ar.x.view(-1),
+                      norm_w, state.spec.rms_eps, ar.h.view(-1), ar.norm_scratch)
+
+
+def _forward_fused(state: DecodeState, weights: DeviceWeights, commit: bool) -> None:
+    spec = state.spec
+    ar = state.arena
+    n_q, n_kv, hd = spec.n_q, spec.n_kv, spec.head_dim
+    layers = weights.layers
+    emb = weights.embed
+    dv2_begin_step(emb.packed, emb.scale, emb.hidden, state.token, state.position, state.valid_len,
+                   ar.x.view(-1), layers[0].norm1 if layers else weights.final_norm, spec.rms_eps,
+                   ar.h.view(-1))
+    for li, layer in enumerate(layers):
+        q, k, v = _qkv(state, layer, ar.h)
+        kc, vc = state.kv.layer(li)
+        dv2_attn(q.view(n_q, hd), kc, vc, ar.attn, state.valid_len, spec.attn_scale, ar.attn_ws,
+                 ar.head_count, ATTN_SPLIT, k.view(n_kv, hd), v.view(n_kv, hd), state.cos, state.sin,
+                 state.position)
+        _gemv_accum_norm(state, layer.o, ar.attn, layer.norm2)
+        g, u = layer.gate, layer.up
+        nf4_swiglu(g.packed, g.scale, u.packed, u.scale, ar.h.view(-1), g.M, g.K, g.K_pad,
+                   ar.down_in.view(-1))
+        nxt = layers[li + 1].norm1 if li + 1 < len(layers) else weights.final_norm
+        _gemv_accum_norm(state, layer.down, ar.down_in, nxt)
+    head = weights.lm_head
+    nf4_gemv(head.packed, head.scale, ar.h.view(-1), head.M, head.K, head.K_pad, ar.logits.view(-1),
+             None if head.bias is None else head.bias)
+    state.pick_next(commit)
+
+
+def forward_decode(state: DecodeState, weights: DeviceWeights, *, commit: bool = False,
+                   fused: bool | None = None) -> None:
     """Logits of ``state.token`` at ``state.position`` into the arena, its argmax
-    into ``state.next_token``; with ``commit`` the id is fed back on the device."""
+    into ``state.next_token``; with ``commit`` the id is fed back on the device.
+    ``fused`` picks the launch schedule (default: the plain one)."""
+    if fused is None:
+        fused = False
+    elif fused and not can_fuse(weights):
+        raise ValueError("the fused schedule needs packed embedding rows, bias-free o/down "
+                         "projections and reduction lengths that are multiples of 64")
+    if fused:
+        _forward_fused(state, weights, commit)
+        return
     spec = state.spec
     ar = state.arena
     n_q, n_kv, hd = spec.n_q, spec.n_kv, spec.head_dim
@@ -75,8 +139,8 @@ def forward_decode(state: DecodeState, weights: DeviceWeights, *, commit: bool =
     state.pick_next(commit)
 
 
-def greedy_decode(state: DecodeState, weights: DeviceWeights) -> None:
-    forward_decode(state, weights, commit=True)
+def greedy_decode(state: DecodeState, weights: DeviceWeights, *, fused: bool | None = None) -> None:
+    forward_decode(state, weights, commit=True, fused=fused)
 
 
 def teacher_force_token(state: DecodeState, weights: DeviceWeights, token_id: int) -> None:

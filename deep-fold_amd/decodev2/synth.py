@@ -54,6 +54,9 @@ class SynthModel:
     final_norm: np.ndarray
     lm_head: Nf4Matrix
     layers: list[SynthLayer]
+    #: packed form of ``embed`` when the model keeps its embedding rows in NF4;
+    #: ``embed`` then holds exactly the values those rows decode to (as bf16)
+    embed_nf4: Nf4Matrix | None = None
 
 
 def gpu_encode(w: np.ndarray) -> tuple[np.ndarray, np.ndarray]:
@@ -69,7 +72,22 @@ def gpu_encode(w: np.ndarray) -> tuple[np.ndarray, np.ndarray]:
     return packed.cpu().numpy(), scale.cpu().numpy()
 
 
-def build(spec: ArchSpec, seed: int, *, encode: Encoder | None = None) -> SynthModel:
+def gpu_decode_bf16(mat: Nf4Matrix) -> np.ndarray:
+    """The bf16 values (as float32) the library's row decoder gives for ``mat``."""
+    import torch
+
+    from ..nf4 import nf4_embed_rows
+
+    packed = torch.from_numpy(np.ascontiguousarray(mat.packed)).cuda()
+    scale = torch.from_numpy(np.ascontiguousarray(mat.scale).view(np.float16)).cuda()
+    ids = torch.arange(mat.M, device="cuda", dtype=torch.int64)
+    return nf4_embed_rows(packed, scale, ids, mat.K).float().cpu().numpy()
+
+
+def build(spec: ArchSpec, seed: int, *, encode: Encoder | None = None,
+          packed_embed: bool = False) -> SynthModel:
+    """``packed_embed`` keeps the embedding rows in NF4 as the large checkpoints do
+    (``gpu/decodev2/embed.py:17-94``); the draws are the same either way."""
     enc = gpu_encode if encode is None else encode
     rng = np.random.default_rng(int(seed))
 
@@ -99,4 +117,9 @@ def build(spec: ArchSpec, seed: int, *, encode: Encoder | None = None) -> SynthM
     embed = vector(spec.vocab * h).reshape(spec.vocab, h)
     final_norm = vector(h)
     lm_head = matrix(spec.vocab, h)
-    return SynthModel(spec, int(seed), embed, final_norm, lm_head, layers)
+    embed_nf4 = None
+    if packed_embed:
+        packed, scale = enc(embed)
+        embed_nf4 = Nf4Matrix(np.asarray(packed), np.asarray(scale), spec.vocab, h, k_pad(h))
+        embed = gpu_decode_bf16(embed_nf4)
+    return SynthModel(spec, int(seed), embed, final_norm, lm_head, layers, embed_nf4)

@@ -23,8 +23,8 @@ def say(*a):
     print(*a, flush=True)
 
 
-def session(spec, seed):
-    model = build(spec, seed)          # quantised by the library's GPU encoder
+def session(spec, seed, packed_embed=False):
+    model = build(spec, seed, packed_embed=packed_embed)   # quantised by the library's GPU encoder
     weights = dv2.DeviceWeights.from_synth(model, "cuda")
     state = dv2.DecodeState.allocate(spec, device="cuda")
     return model, state, weights
@@ -209,21 +209,26 @@ def near_tie(logits: np.ndarray) -> bool:
     return float(top[1] - top[0]) <= 4 * 2.0 ** (np.floor(np.log2(max(abs(top[1]), 1e-30))) - 7)
 
 
+@pytest.mark.parametrize("packed_embed", [False, True])
 @pytest.mark.parametrize("seed", [0, 1, 2, 3])
-def test_greedy_64_tokens_identical_to_the_oracle(seed):
+def test_greedy_64_tokens_identical_to_the_oracle(seed, packed_embed):
     """64 generated tokens on random-init weights, ignore-EOS, eager and graph.
     The stream must equal the oracle's; the only excuse for a first difference is
-    an oracle pick that is itself a near-tie at bf16 logit resolution."""
-    say("64 tokens seed", seed)
-    model, state, weights = session(LONGRUN, seed)
+    an oracle pick that is itself a near-tie at bf16 logit resolution.  Models with
+    packed embedding rows run the fused launch schedule."""
+    say("64 tokens seed", seed, "packed_embed", packed_embed)
+    model, state, weights = session(LONGRUN, seed, packed_embed)
+    assert dv2.can_fuse(weights) == packed_embed
+    fused = packed_embed
     prompt = [11, 200, 37, 1999, 5, 640, 3, 77]
     want, margins = so.greedy_ids(model, prompt, 64, ignore_eos=True, return_margins=True)
     assert len(want) == 64
     state.reset()
-    got = dv2.generate(state, weights, prompt, 64, ignore_eos=True)
+    step = (lambda s, w: dv2.greedy_decode(s, w, fused=True)) if fused else dv2.greedy_decode
+    got = dv2.generate(state, weights, prompt, 64, step=step, ignore_eos=True)
     say("  min / median top-1 margin", min(margins), float(np.median(margins)))
     state.reset()
-    graph = dv2.capture_greedy(state, weights, warmup=1)
+    graph = dv2.capture_greedy(state, weights, warmup=1, fused=fused)
     state.reset()
     assert dv2.generate(state, weights, prompt, 64, step=graph, ignore_eos=True) == got
     if got != want:
@@ -240,8 +245,8 @@ IDENTICAL: list[bool] = []
 def test_some_seed_is_fully_identical():
     # Random-init logits have a median top-1/top-2 gap of ~0.1 and a minimum over
     # 64 picks that is usually below one bf16 step, so most streams hit a coin-toss
-    # pick somewhere; at least one of the four seeds must go all 64 tokens.
-    assert len(IDENTICAL) == 4 and sum(IDENTICAL) >= 1, IDENTICAL
+    # pick somewhere; at least one of the eight runs must go all 64 tokens.
+    assert len(IDENTICAL) == 8 and sum(IDENTICAL) >= 1, IDENTICAL
 
 
 def test_teacher_forced_picks_agree_except_on_near_ties():
@@ -263,3 +268,56 @@ def test_teacher_forced_picks_agree_except_on_near_ties():
             assert gap <= 4 * 2.0 ** (np.floor(np.log2(abs(top[1]))) - 7), (i, gap)
             disagree += 1
     assert disagree <= 3
+
+
+# ---- the fused launch schedule ---------------------------------------------------
+
+@pytest.mark.parametrize("spec,seed", [(dv2.TINY_LLAMA, 0), (dv2.TINY_INTERNLM, 1), (dv2.MEDIUM_LLAMA, 0),
+                                       (LONGRUN, 2)])
+def test_fused_schedule_equals_plain_schedule(spec, seed):
+    """Same weights, same tokens: logits of the five-launch schedule against the
+    eight-launch one at every position, and both against the oracle's ids."""
+    say("fused vs plain", spec.name)
+    model, state, weights = session(spec, seed, packed_embed=True)
+    assert dv2.can_fuse(weights)
+    other = dv2.DecodeState.allocate(spec, device="cuda")
+    toks = np.random.default_rng(seed).integers(0, spec.vocab, size=min(24, spec.max_seq)).tolist()
+    for i, t in enumerate(toks):
+        for st, fused in ((state, True), (other, False)):
+            st.load_token(t)
+            dv2.forward_decode(st, weights, fused=fused)
+            st.position.add_(1)
+        a = state.arena.logits.float()
+        b = other.arena.logits.float()
+        # the two schedules differ only in the summation order of the RMS statistic
+        assert float((a - b).abs().max()) <= 0.02 * float(b.abs().max()) + 1e-3, i
+        assert int(state.valid_len.item()) == i + 1 == int(other.valid_len.item())
+        assert int(state.arena.head_count.abs().sum().item()) == 0
+        assert int(state.arena.norm_scratch.view(torch.int32)[0].item()) == 0   # the ticket is re-armed
+    kc, vc = state.kv.layer(0)
+    ko, vo = other.kv.layer(0)
+    assert float((kc.float() - ko.float()).abs().max()) <= 0.02 * float(ko.float().abs().max())
+    got = greedy_token_at_a_time(state, weights, SHORT, 10,
+                                 step=lambda s, w: dv2.greedy_decode(s, w, fused=True))
+    assert got == so.greedy_ids(model, SHORT, 10)
+    assert got == greedy_token_at_a_time(other, weights, SHORT, 10)
+
+
+def test_fused_schedule_in_a_graph():
+    model, state, weights = session(dv2.MEDIUM_LLAMA, 0, packed_embed=True)
+    eager = greedy_token_at_a_time(state, weights, SHORT, 12,
+                                   step=lambda s, w: dv2.greedy_decode(s, w, fused=True))
+    assert eager == so.greedy_ids(model, SHORT, 12)
+    state.reset()
+    graph = dv2.capture_greedy(state, weights, warmup=2, fused=True)
+    for rep in range(3):
+        assert greedy_token_at_a_time(state, weights, SHORT, 12, step=graph) == eager, rep
+        torch.cuda.synchronize()
+
+
+def test_fused_schedule_is_refused_when_it_does_not_apply():
+    _, state, weights = session(dv2.TINY_LLAMA, 0)          # dense embedding table
+    assert not dv2.can_fuse(weights)
+    state.load_token(1)
+    with pytest.raises(ValueError):
+        dv2.forward_decode(state, weights, fused=True)
