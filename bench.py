@@ -141,7 +141,7 @@ def bench_prefill(torch, nf4):
     return rows
 
 
-def bench_decode(torch, spec_name: str, prompt_len: int, new_tokens: int):
+def bench_decode(torch, spec_name: str, prompt_len: int, new_tokens: int, schedule: str | None = None):
     """Resident greedy decode on random-init weights: chunked prefill of a random
     prompt, then ``new_tokens`` graph replays with no host read in between."""
     from deepfold_amd import decodev2 as dv2
@@ -165,7 +165,7 @@ def bench_decode(torch, spec_name: str, prompt_len: int, new_tokens: int):
     prefill_ms = (time.perf_counter() - t0) * 1e3
     state.token.copy_(state.next_token)
     # graph capture advances the state by warmup+1 tokens; that is part of the run
-    graph = dv2.capture_greedy(state, weights, warmup=2)
+    graph = dv2.capture_greedy(state, weights, warmup=2, schedule=schedule)
     torch.cuda.synchronize()
     start_pos = int(state.position.item())
     e0 = torch.cuda.Event(enable_timing=True)
@@ -184,7 +184,7 @@ def bench_decode(torch, spec_name: str, prompt_len: int, new_tokens: int):
     # eager step for comparison (a few tokens)
     t0 = time.perf_counter()
     for _ in range(8):
-        dv2.greedy_decode(state, weights)
+        dv2.greedy_decode(state, weights, schedule=schedule)
     torch.cuda.synchronize()
     eager_ms = (time.perf_counter() - t0) * 1e3 / 8
     ms_tok = dev_ms / new_tokens
@@ -267,6 +267,7 @@ def main() -> int:
     ap.add_argument("--no-decode", action="store_true", help="skip the model decode leg")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill GEMM sweep")
     ap.add_argument("--decode-models", default="14b", help="comma list of 3b,14b,20b,32b")
+    ap.add_argument("--schedule", default=None, help="decode launch schedule: plain, fold_rms or handover")
     ap.add_argument("--prompt", type=int, default=512)
     ap.add_argument("--new-tokens", type=int, default=256)
     args = ap.parse_args()
@@ -317,7 +318,7 @@ def main() -> int:
         },
     }
     if not args.no_decode:
-        out["decode"] = [bench_decode(torch, name.strip(), args.prompt, args.new_tokens)
+        out["decode"] = [bench_decode(torch, name.strip(), args.prompt, args.new_tokens, args.schedule)
                          for name in args.decode_models.split(",") if name.strip()]
     if not args.no_prefill:
         out["prefill"] = bench_prefill(torch, nf4)

@@ -175,8 +175,28 @@ __device__ __forceinline__ void drain_stores() {
   __atomic_signal_fence(__ATOMIC_SEQ_CST);
 }
 
-inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
-inline bool aligned2(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 1u) == 0; }
+__host__ __device__ inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+__host__ __device__ inline bool aligned2(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 1u) == 0; }
+
+// Compute units of the current device (256 on an MI355X), cached after the first call.
+inline int device_cu_count() {
+  static int cached = [] {
+    constexpr int kDefault = 256;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) {
+      (void)hipGetLastError();
+      return kDefault;
+    }
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        n < 1) {
+      (void)hipGetLastError();
+      return kDefault;
+    }
+    return n;
+  }();
+  return cached;
+}
 
 inline int launch_rc() { return hipGetLastError() == hipSuccess ? 0 : -6; }
 

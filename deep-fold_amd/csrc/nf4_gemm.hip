@@ -83,25 +83,6 @@ Tuning &tuning() {
   return t;
 }
 
-constexpr int kDefaultOneWave = 256;  // compute units of an MI355X
-
-int device_cu_count() {
-  static int cached = [] {
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess) {
-      (void)hipGetLastError();
-      return kDefaultOneWave;
-    }
-    int n = 0;
-    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
-        n < 1) {
-      (void)hipGetLastError();
-      return kDefaultOneWave;
-    }
-    return n;
-  }();
-  return cached;
-}
 
 int resolved_one_wave() {
   const int w = tuning().one_wave;

@@ -120,7 +120,7 @@ struct StreamArgs {
   uint16_t *y[3];
   const uint16_t *add[3];  // optional residual / bias per segment, bf16 [M]
   int M[3];
-  int blocks[3];  // workgroups given to each segment
+  int groups[3];  // wavefront-sized row groups of each segment
   // second matrix of a SwiGLU pair (segment 0 only)
   const uint8_t *packed2;
   const uint16_t *scale2;
@@ -152,31 +152,113 @@ __device__ __forceinline__ float block_sum(float v, float *part) {
   return s;
 }
 
-// Activations of the workgroup in LDS as bf16, zero for k in [K, K_pad).  With
-// rms_w the value stored is bf16( (w*x) * rsqrt(mean(x^2)+eps) ), i.e. what a
-// separate RMSNorm launch would have handed over
-// (gpu/nf4/nf4_gemv.cu:264-289).  Only used when x cannot be read straight from
-// global memory: a ragged K, or the fused RMSNorm.
-__device__ __forceinline__ void stage_x(const StreamArgs &a, uint16_t *xh, float *part) {
-  float inv = 1.f;
-  if (a.rms_w != nullptr) {
-    float ss = 0.f;
-    for (int i = threadIdx.x; i < a.K; i += blockDim.x) {
-      const float v = bf16_to_f32(a.x[i]);
-      ss = fmaf(v, v, ss);
-    }
-    ss = block_sum(ss, part);
-    inv = rsqrtf(ss / static_cast<float>(a.K) + a.rms_eps);
+// ---- activations staged in LDS ------------------------------------------------------
+// A "piece" is 8 consecutive activations (16 bytes of bf16).  In the steps where every
+// lane holds a 16-byte chunk of weights, lane l of step j needs pieces 4c..4c+3 of chunk
+// c = 64j + l; they are stored as [j][q][l] so that one ds_read_b128 of the wavefront
+// covers 64 consecutive pieces (no bank conflicts).  The 8-byte tail chunks need two
+// pieces each and are stored as [step][q][l] the same way after the full steps.
+__host__ __device__ inline int x_pieces(int K_pad) {
+  const int chunks = K_pad >> 5;
+  const int nfull = chunks >> 6;
+  const int tail_half = (chunks & 63) * 2;
+  return nfull * 256 + ((tail_half + 63) >> 6) * 128;
+}
+
+__device__ __forceinline__ int x_slot(int piece, int nfull) {
+  const int full = nfull << 8;
+  if (piece < full) {
+    const int c = piece >> 2, q = piece & 3;
+    return ((c >> 6) << 8) + (q << 6) + (c & 63);
   }
-  for (int i = threadIdx.x; i < a.K_pad; i += blockDim.x) {
-    uint16_t v = 0;
-    if (i < a.K) {
-      v = a.x[i];
-      if (a.rms_w != nullptr) {
-        v = f32_to_bf16((bf16_to_f32(a.rms_w[i]) * bf16_to_f32(v)) * inv);
+  const int t = piece - full;
+  const int h = t >> 1, q = t & 1;
+  return full + ((h >> 6) << 7) + (q << 6) + (h & 63);
+}
+
+// Fill the LDS copy: zero for k in [K, K_pad) and for unused slots.  With rms_w the
+// value stored is bf16( (w*x) * rsqrt(mean(x^2)+eps) ), i.e. what a separate RMSNorm
+// launch would have handed over (gpu/nf4/nf4_gemv.cu:264-289).  Used for a ragged K
+// and for the fused RMSNorm.
+__device__ __forceinline__ void stage_x(const StreamArgs &a, uint4 *xs, float *part) {
+  constexpr int kKeep = 4;  // 16-byte vectors of x a thread keeps between the two passes
+  const int nfull = (a.K_pad >> 5) >> 6;
+  const int slots = x_pieces(a.K_pad);
+  const int nvec = a.K_pad >> 3;
+  const bool vec_ok = (a.K & 7) == 0 && aligned16(a.x) &&
+                      (a.rms_w == nullptr || aligned16(a.rms_w)) &&
+                      nvec <= kKeep * static_cast<int>(blockDim.x);
+  for (int i = nvec + threadIdx.x; i < slots; i += blockDim.x) {
+    xs[i] = make_uint4(0, 0, 0, 0);  // slots past the last piece (partial tail step)
+  }
+  if (vec_ok) {
+    uint4 v[kKeep];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < kKeep; ++j) {
+      const int i = threadIdx.x + j * blockDim.x;
+      v[j] = make_uint4(0, 0, 0, 0);
+      if (i * 8 < a.K) {
+        v[j] = reinterpret_cast<const uint4 *>(a.x)[i];
       }
     }
-    xh[i] = v;
+    float inv = 1.f;
+    if (a.rms_w != nullptr) {
+#pragma unroll
+      for (int j = 0; j < kKeep; ++j) {
+        const uint32_t u[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          ss = fmaf(bf16_lo(u[q]), bf16_lo(u[q]), ss);
+          ss = fmaf(bf16_hi(u[q]), bf16_hi(u[q]), ss);
+        }
+      }
+      ss = block_sum(ss, part);
+      inv = rsqrtf(ss / static_cast<float>(a.K) + a.rms_eps);
+    }
+#pragma unroll
+    for (int j = 0; j < kKeep; ++j) {
+      const int i = threadIdx.x + j * blockDim.x;
+      if (i < nvec) {
+        uint4 o = v[j];
+        if (a.rms_w != nullptr && i * 8 < a.K) {
+          const uint4 g = reinterpret_cast<const uint4 *>(a.rms_w)[i];
+          const uint32_t u[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+          const uint32_t gw[4] = {g.x, g.y, g.z, g.w};
+          uint32_t r[4];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const uint32_t lo = f32_to_bf16((bf16_lo(gw[q]) * bf16_lo(u[q])) * inv);
+            const uint32_t hi = f32_to_bf16((bf16_hi(gw[q]) * bf16_hi(u[q])) * inv);
+            r[q] = lo | (hi << 16);
+          }
+          o = make_uint4(r[0], r[1], r[2], r[3]);
+        }
+        xs[x_slot(i, nfull)] = o;
+      }
+    }
+  } else {
+    float inv = 1.f;
+    if (a.rms_w != nullptr) {
+      float ss = 0.f;
+      for (int i = threadIdx.x; i < a.K; i += blockDim.x) {
+        const float v = bf16_to_f32(a.x[i]);
+        ss = fmaf(v, v, ss);
+      }
+      ss = block_sum(ss, part);
+      inv = rsqrtf(ss / static_cast<float>(a.K) + a.rms_eps);
+    }
+    uint16_t *xh = reinterpret_cast<uint16_t *>(xs);
+    for (int i = threadIdx.x; i < a.K_pad; i += blockDim.x) {
+      uint16_t v = 0;
+      if (i < a.K) {
+        v = a.x[i];
+        if (a.rms_w != nullptr) {
+          v = f32_to_bf16((bf16_to_f32(a.rms_w[i]) * bf16_to_f32(v)) * inv);
+        }
+      }
+      xh[(x_slot(i >> 3, nfull) << 3) + (i & 7)] = v;
+    }
   }
   __syncthreads();
 }
@@ -217,11 +299,12 @@ __device__ __forceinline__ void rows_step(const uint32_t (&w)[R][NW], const floa
   }
 }
 
-// One wavefront, R weight rows sharing x.  x points at K_pad bf16 values
-// (global memory, or the LDS copy made by stage_x).
-template <int R>
+// One wavefront, R weight rows sharing x.  x4 points at the activations as 16-byte
+// pieces: K_pad/8 of them in global memory (XL == false), or the LDS copy made by
+// stage_x in its [step][q][lane] order (XL == true).
+template <int R, bool XL>
 __device__ __forceinline__ void rows_dot(const uint8_t *const (&prow)[R],
-                                         const uint16_t *const (&srow)[R], const uint16_t *x,
+                                         const uint16_t *const (&srow)[R], const uint4 *x4,
                                          int K_pad, const float *lut, int lane,
                                          float (&acc)[R]) {
   const int chunks = K_pad >> 5;            // 16-byte chunks per row
@@ -241,8 +324,9 @@ __device__ __forceinline__ void rows_dot(const uint8_t *const (&prow)[R],
       w[r][3] = v.w;
       sc[r] = srow[r][c >> 1];
     }
-    const uint4 *xp = reinterpret_cast<const uint4 *>(x) + (c << 2);
-    const uint4 x0 = xp[0], x1 = xp[1], x2 = xp[2], x3 = xp[3];
+    const uint4 *xp = XL ? x4 + (j << 8) + lane : x4 + (c << 2);
+    constexpr int xq = XL ? 64 : 1;
+    const uint4 x0 = xp[0], x1 = xp[xq], x2 = xp[2 * xq], x3 = xp[3 * xq];
     float xf[32];
     widen8(x0, xf);
     widen8(x1, xf + 8);
@@ -265,8 +349,8 @@ __device__ __forceinline__ void rows_dot(const uint8_t *const (&prow)[R],
         w[r][1] = v.y;
         sc[r] = srow[r][hc >> 2];
       }
-      const uint4 *xp = reinterpret_cast<const uint4 *>(x) + (hc << 1);
-      const uint4 x0 = xp[0], x1 = xp[1];
+      const uint4 *xp = XL ? x4 + (nfull << 8) + ((h0 >> 6) << 7) + lane : x4 + (hc << 1);
+      const uint4 x0 = xp[0], x1 = xp[XL ? 64 : 1];
       float xf[16];
       widen8(x0, xf);
       widen8(x1, xf + 8);
@@ -343,8 +427,8 @@ __device__ __forceinline__ void norm_tail(const StreamArgs &a, float sq, float *
 //       order (so the result does not depend on arrival order), then normalises
 //       all of y.  That replaces a separate one-workgroup RMSNorm launch.
 template <int R, bool SWIGLU, bool XLDS, bool NORM = false>
-__global__ __launch_bounds__(256) void gemv_stream(const StreamArgs a) {
-  extern __shared__ uint16_t xh[];
+__global__ __launch_bounds__(XLDS ? 1024 : 256) void gemv_stream(const StreamArgs a) {
+  extern __shared__ uint4 xs[];
   __shared__ GemvLds lds;
   constexpr int U = SWIGLU ? R / 2 : R;  // output rows per wavefront
   const int lane = threadIdx.x & (kWave - 1);
@@ -355,87 +439,95 @@ __global__ __launch_bounds__(256) void gemv_stream(const StreamArgs a) {
     lds.lut[threadIdx.x] = bits_to_f32(kLutBits[threadIdx.x]);
   }
   if constexpr (XLDS) {
-    stage_x(a, xh, lds.part);
+    stage_x(a, xs, lds.part);
   } else {
     __syncthreads();
   }
 
-  int b = blockIdx.x;
-  int seg = 0;
-  if (!SWIGLU) {
-    if (b >= a.blocks[0]) {
-      b -= a.blocks[0];
-      seg = 1;
-      if (b >= a.blocks[1]) {
-        b -= a.blocks[1];
-        seg = 2;
-      }
-    }
-  }
-  const int M = a.M[seg];
-  const int row0 = (b * waves + wave) * U;
-  if (!NORM && row0 >= M) {
-    return;
-  }
-
+  // Row groups (U rows each) are numbered through the segments.  Without the LDS
+  // copy a wavefront takes exactly one group; with it the grid is one workgroup per
+  // compute unit and a wavefront walks groups wave*grid + block, + grid*waves, ..,
+  // so the copy is made once per compute unit and units stay balanced to one group.
+  const int total = a.groups[0] + a.groups[1] + a.groups[2];
+  const int first = XLDS ? wave * static_cast<int>(gridDim.x) + static_cast<int>(blockIdx.x)
+                         : static_cast<int>(blockIdx.x) * waves + wave;
+  const int stride = XLDS ? static_cast<int>(gridDim.x) * waves : total;
   const size_t pstride = static_cast<size_t>(a.K_pad >> 1);
   const size_t sstride = static_cast<size_t>(a.K_pad >> 6);
-  const uint8_t *prow[R];
-  const uint16_t *srow[R];
+  float sq = 0.f;  // NORM: square of the value this lane stored
+
+  for (int grp = first; grp < total; grp += stride) {
+    int g = grp;
+    int seg = 0;
+    if (!SWIGLU) {
+      if (g >= a.groups[0]) {
+        g -= a.groups[0];
+        seg = 1;
+        if (g >= a.groups[1]) {
+          g -= a.groups[1];
+          seg = 2;
+        }
+      }
+    }
+    const int M = a.M[seg];
+    const int row0 = g * U;
+    const uint8_t *prow[R];
+    const uint16_t *srow[R];
 #pragma unroll
-  for (int u = 0; u < U; ++u) {
-    const int r = min(row0 + u, M - 1);  // rows past M are computed, never stored
-    prow[u] = a.packed[seg] + r * pstride;
-    srow[u] = a.scale[seg] + r * sstride;
+    for (int u = 0; u < U; ++u) {
+      const int r = min(row0 + u, M - 1);  // rows past M are computed, never stored
+      prow[u] = a.packed[seg] + r * pstride;
+      srow[u] = a.scale[seg] + r * sstride;
+      if constexpr (SWIGLU) {
+        prow[U + u] = a.packed2 + r * pstride;
+        srow[U + u] = a.scale2 + r * sstride;
+      }
+    }
+
+    float acc[R] = {};
+    if constexpr (XLDS) {
+      rows_dot<R, true>(prow, srow, static_cast<const uint4 *>(xs), a.K_pad, lds.lut, lane, acc);
+    } else {
+      rows_dot<R, false>(prow, srow, reinterpret_cast<const uint4 *>(a.x), a.K_pad, lds.lut, lane,
+                         acc);
+    }
+
     if constexpr (SWIGLU) {
-      prow[U + u] = a.packed2 + r * pstride;
-      srow[U + u] = a.scale2 + r * sstride;
-    }
-  }
-
-  float acc[R] = {};
-  if constexpr (XLDS) {
-    rows_dot<R>(prow, srow, static_cast<const uint16_t *>(xh), a.K_pad, lds.lut, lane, acc);
-  } else {
-    rows_dot<R>(prow, srow, a.x, a.K_pad, lds.lut, lane, acc);
-  }
-
-  if constexpr (SWIGLU) {
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const float gsum = wave_sum(acc[u]);
-      const float usum = wave_sum(acc[U + u]);
-      const int r = row0 + u;
-      if (lane == u && r < M) {
-        a.y[0][r] = f32_to_bf16(silu(gsum) * usum);
-      }
-    }
-  } else {
-    const uint16_t *add = a.add[seg];
-    uint16_t *y = a.y[seg];
-    float sq = 0.f;  // NORM: square of the value this lane stored
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const float s = wave_sum(acc[u]);
-      const int r = row0 + u;
-      if (lane == u && r < M) {
-        float v = s;
-        if (add != nullptr) {
-          v += bf16_to_f32(add[r]);
+      for (int u = 0; u < U; ++u) {
+        const float gsum = wave_sum(acc[u]);
+        const float usum = wave_sum(acc[U + u]);
+        const int r = row0 + u;
+        if (lane == u && r < M) {
+          a.y[0][r] = f32_to_bf16(silu(gsum) * usum);
         }
-        const uint16_t vb = f32_to_bf16(v);
-        if constexpr (NORM) {
-          store_coherent(y + r, vb);  // read back by the workgroup that normalises
-          const float vr = bf16_to_f32(vb);
-          sq = vr * vr;
-        } else {
-          y[r] = vb;
+      }
+    } else {
+      const uint16_t *add = a.add[seg];
+      uint16_t *y = a.y[seg];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const float s = wave_sum(acc[u]);
+        const int r = row0 + u;
+        if (lane == u && r < M) {
+          float v = s;
+          if (add != nullptr) {
+            v += bf16_to_f32(add[r]);
+          }
+          const uint16_t vb = f32_to_bf16(v);
+          if constexpr (NORM) {
+            store_coherent(y + r, vb);  // read back by the workgroup that normalises
+            const float vr = bf16_to_f32(vb);
+            sq = vr * vr;
+          } else {
+            y[r] = vb;
+          }
         }
       }
     }
-    if constexpr (NORM) {
-      norm_tail(a, sq, lds.part, M);
-    }
+  }
+  if constexpr (NORM) {
+    norm_tail(a, sq, lds.part, a.M[0]);
   }
 }
 
@@ -514,6 +606,7 @@ int rows_for_m(int M) {
 }
 
 constexpr int kThreads = 256;
+constexpr int kStagedThreads = 1024;  // workgroup of the kernels that stage x in LDS
 constexpr size_t kMaxDynLds = 150 * 1024;
 
 template <typename Kern>
@@ -534,30 +627,33 @@ int prep_lds(Kern kern, size_t dyn) {
 
 template <int R>
 int launch_stream_norm(StreamArgs &a, hipStream_t st) {
-  const int rows_per_wg = (kThreads / kWave) * R;
-  a.blocks[0] = (a.M[0] + rows_per_wg - 1) / rows_per_wg;
-  a.blocks[1] = a.blocks[2] = 0;
-  gemv_stream<R, false, false, true><<<dim3(a.blocks[0]), dim3(kThreads), 0, st>>>(a);
+  a.groups[0] = (a.M[0] + R - 1) / R;
+  a.groups[1] = a.groups[2] = 0;
+  const int waves = kThreads / kWave;
+  gemv_stream<R, false, false, true>
+      <<<dim3((a.groups[0] + waves - 1) / waves), dim3(kThreads), 0, st>>>(a);
   return launch_rc();
 }
 
 template <int R, bool SWIGLU>
 int launch_stream(StreamArgs &a, int n_seg, hipStream_t st) {
   constexpr int U = SWIGLU ? R / 2 : R;
-  const int rows_per_wg = (kThreads / kWave) * U;
   int total = 0;
   for (int i = 0; i < 3; ++i) {
-    a.blocks[i] = i < n_seg ? (a.M[i] + rows_per_wg - 1) / rows_per_wg : 0;
-    total += a.blocks[i];
+    a.groups[i] = i < n_seg ? (a.M[i] + U - 1) / U : 0;
+    total += a.groups[i];
   }
   if (a.rms_w != nullptr || a.K != a.K_pad) {
-    const size_t dyn = static_cast<size_t>(a.K_pad) * 2;
+    const size_t dyn = static_cast<size_t>(x_pieces(a.K_pad)) * 16;
     if (prep_lds(gemv_stream<R, SWIGLU, true>, dyn) != 0) {
       return -6;
     }
-    gemv_stream<R, SWIGLU, true><<<dim3(total), dim3(kThreads), dyn, st>>>(a);
+    const int waves = kStagedThreads / kWave;
+    const int grid = std::min(device_cu_count(), (total + waves - 1) / waves);
+    gemv_stream<R, SWIGLU, true><<<dim3(grid), dim3(kStagedThreads), dyn, st>>>(a);
   } else {
-    gemv_stream<R, SWIGLU, false><<<dim3(total), dim3(kThreads), 0, st>>>(a);
+    const int waves = kThreads / kWave;
+    gemv_stream<R, SWIGLU, false><<<dim3((total + waves - 1) / waves), dim3(kThreads), 0, st>>>(a);
   }
   return launch_rc();
 }
@@ -605,7 +701,10 @@ int gemv_entry(const chr_nf4_dev_t *w, const void *x, void *y, void *stream, con
 }
 
 // Workgroups a fused-norm GEMV over M rows launches (= partial sums it writes).
-int gemv_norm_blocks(int M) { return (M + (kThreads / kWave) * rows_for_m(M) - 1) / ((kThreads / kWave) * rows_for_m(M)); }
+int gemv_norm_blocks(int M) {
+  const int rows_per_wg = (kThreads / kWave) * rows_for_m(M);
+  return (M + rows_per_wg - 1) / rows_per_wg;
+}
 
 int gemv_add_norm_entry(const chr_nf4_dev_t *w, const void *x, void *y, const void *norm_w,
                         float norm_eps, void *norm_out, float *scratch, int64_t scratch_floats,

@@ -33,7 +33,7 @@ class GreedyGraph:
 
 
 def capture_greedy(state: DecodeState, weights: DeviceWeights, *, warmup: int = 3,
-                   fused: bool | None = None) -> GreedyGraph:
+                   schedule: str | None = None) -> GreedyGraph:
     """Warm up on a side stream (so one-time work such as kernel attribute calls
     stays out of the capture), then capture one ``greedy_decode``.
 
@@ -46,12 +46,12 @@ def capture_greedy(state: DecodeState, weights: DeviceWeights, *, warmup: int = 
     side.wait_stream(stream)
     with torch.cuda.stream(side):
         for _ in range(max(1, warmup)):
-            greedy_decode(state, weights, fused=fused)
+            greedy_decode(state, weights, schedule=schedule)
         side.synchronize()
         graph = torch.cuda.CUDAGraph()
         graph.capture_begin()
         try:
-            greedy_decode(state, weights, fused=fused)
+            greedy_decode(state, weights, schedule=schedule)
         finally:
             graph.capture_end()
     stream.wait_stream(side)

@@ -9,13 +9,16 @@ o GEMV accumulating into the residual -> rms -> fused SwiGLU GEMV -> down GEMV
 accumulating into the residual.  Then the final norm, lm_head and a device-side
 argmax that also feeds the id back.
 
-Two launch schedules compute that sequence.  The plain one issues it call by call
-(eight launches per layer) and is the default.  The fused one needs five: every
-RMSNorm rides on the launch that produces its input (the embedding gather, or the
-residual GEMV whose last workgroup normalises), and the attention launch merges
-its own splits.  On MI355X the hand-over between workgroups inside a launch costs
-more than the launches it saves (a device-scope round trip per stage), so the
-fused schedule is kept for comparison and only runs on request.
+Three launch schedules compute that sequence:
+
+``plain``     the call sequence above, eight launches per layer;
+``fold_rms``  every RMSNorm runs inside the GEMV that consumes it (six launches);
+``handover``  every RMSNorm rides on the launch that *produces* its input (the
+              embedding gather, or the residual GEMV whose last workgroup
+              normalises) and the attention launch merges its own splits (five).
+              On MI355X the hand-over between workgroups of one launch costs a
+              device-scope round trip per stage, more than the launches it
+              saves, so this one only runs on request.
 """
 
 from __future__ import annotations
@@ -28,7 +31,7 @@ from .embed import PackedEmbed, gather_embed
 from .linear import DeviceLayer, DeviceLinear, DeviceWeights
 from .state import DecodeState
 
-__all__ = ["forward_decode", "greedy_decode", "teacher_force_token", "can_fuse"]
+__all__ = ["forward_decode", "greedy_decode", "teacher_force_token", "can_fuse", "SCHEDULES"]
 
 
 def _gemv_accum(mat: DeviceLinear, src: torch.Tensor, dest: torch.Tensor) -> None:
@@ -39,20 +42,22 @@ def _gemv_accum(mat: DeviceLinear, src: torch.Tensor, dest: torch.Tensor) -> Non
         d.add_(mat.bias)
 
 
-def _qkv(state: DecodeState, layer: DeviceLayer, h: torch.Tensor):
-    """q, k, v of the current token as contiguous ``[heads*hd]`` views."""
+def _qkv(state: DecodeState, layer: DeviceLayer, h: torch.Tensor, rms_w: torch.Tensor | None = None):
+    """q, k, v of the current token as contiguous ``[heads*hd]`` views; with ``rms_w``
+    the GEMV normalises ``h`` itself."""
     ar = state.arena
     spec = state.spec
+    eps = spec.rms_eps
     if layer.wqkv is not None:
         m = layer.wqkv
         nf4_gemv(m.packed, m.scale, h.view(-1), m.M, m.K, m.K_pad, ar.qkv.view(-1),
-                 None if m.bias is None else m.bias)
+                 None if m.bias is None else m.bias, rms_w, eps)
         flat = ar.qkv.view(-1)
         return (flat[: spec.q_dim], flat[spec.q_dim: spec.q_dim + spec.kv_dim],
                 flat[spec.q_dim + spec.kv_dim:])
     q, k, v = layer.q, layer.k, layer.v
     nf4_qkv(q.packed, q.scale, k.packed, k.scale, v.packed, v.scale, h.view(-1), q.M, k.M, v.M, q.K,
-            q.K_pad, ar.q.view(-1), ar.k.view(-1), ar.v.view(-1), q.bias, k.bias, v.bias)
+            q.K_pad, ar.q.view(-1), ar.k.view(-1), ar.v.view(-1), q.bias, k.bias, v.bias, rms_w, eps)
     return ar.q.view(-1), ar.k.view(-1), ar.v.view(-1)
 
 
@@ -101,46 +106,73 @@ def _forward_fused(state: DecodeState, weights: DeviceWeights, commit: bool) -> 
     state.pick_next(commit)
 
 
-def forward_decode(state: DecodeState, weights: DeviceWeights, *, commit: bool = False,
-                   fused: bool | None = None) -> None:
-    """Logits of ``state.token`` at ``state.position`` into the arena, its argmax
-    into ``state.next_token``; with ``commit`` the id is fed back on the device.
-    ``fused`` picks the launch schedule (default: the plain one)."""
-    if fused is None:
-        fused = False
-    elif fused and not can_fuse(weights):
-        raise ValueError("the fused schedule needs packed embedding rows, bias-free o/down "
-                         "projections and reduction lengths that are multiples of 64")
-    if fused:
-        _forward_fused(state, weights, commit)
-        return
+SCHEDULES = ("plain", "fold_rms", "handover")
+#: schedule used when the caller does not name one
+DEFAULT_SCHEDULE = "fold_rms"
+
+
+def _forward_calls(state: DecodeState, weights: DeviceWeights, commit: bool, fold_rms: bool) -> None:
+    """The reference's call sequence.  With ``fold_rms`` every RMSNorm runs inside the
+    GEMV that consumes it (the ``rms_w`` argument of the GEMV entry points,
+    ``gpu/nf4/nf4_gemv.cu:264-289``): six launches per layer instead of eight."""
     spec = state.spec
     ar = state.arena
+    eps = spec.rms_eps
     n_q, n_kv, hd = spec.n_q, spec.n_kv, spec.head_dim
     gather_embed(weights.embed, state.token.reshape(1), out=ar.x)
     state.kv.mark_written(state.position)
     for li, layer in enumerate(weights.layers):
-        nf4_rms(ar.x, layer.norm1, ar.h, spec.rms_eps)
-        q, k, v = _qkv(state, layer, ar.h)
+        if fold_rms:
+            q, k, v = _qkv(state, layer, ar.x, layer.norm1)
+        else:
+            nf4_rms(ar.x, layer.norm1, ar.h, eps)
+            q, k, v = _qkv(state, layer, ar.h)
         kc, vc = state.kv.layer(li)
         nf4_attn(q.view(n_q, hd), kc, vc, ar.attn, state.valid_len, spec.attn_scale, ar.attn_ws,
                  ATTN_SPLIT, k.view(n_kv, hd), v.view(n_kv, hd), state.cos, state.sin,
                  state.position)
         _gemv_accum(layer.o, ar.attn, ar.x)
-        nf4_rms(ar.x, layer.norm2, ar.h, spec.rms_eps)
         g, u = layer.gate, layer.up
-        nf4_swiglu(g.packed, g.scale, u.packed, u.scale, ar.h.view(-1), g.M, g.K, g.K_pad,
-                   ar.down_in.view(-1))
+        if fold_rms:
+            nf4_swiglu(g.packed, g.scale, u.packed, u.scale, ar.x.view(-1), g.M, g.K, g.K_pad,
+                       ar.down_in.view(-1), layer.norm2, eps)
+        else:
+            nf4_rms(ar.x, layer.norm2, ar.h, eps)
+            nf4_swiglu(g.packed, g.scale, u.packed, u.scale, ar.h.view(-1), g.M, g.K, g.K_pad,
+                       ar.down_in.view(-1))
         _gemv_accum(layer.down, ar.down_in, ar.x)
-    nf4_rms(ar.x, weights.final_norm, ar.h, spec.rms_eps)
     head = weights.lm_head
-    nf4_gemv(head.packed, head.scale, ar.h.view(-1), head.M, head.K, head.K_pad, ar.logits.view(-1),
-             None if head.bias is None else head.bias)
+    bias = None if head.bias is None else head.bias
+    if fold_rms:
+        nf4_gemv(head.packed, head.scale, ar.x.view(-1), head.M, head.K, head.K_pad,
+                 ar.logits.view(-1), bias, weights.final_norm, eps)
+    else:
+        nf4_rms(ar.x, weights.final_norm, ar.h, eps)
+        nf4_gemv(head.packed, head.scale, ar.h.view(-1), head.M, head.K, head.K_pad,
+                 ar.logits.view(-1), bias)
     state.pick_next(commit)
 
 
-def greedy_decode(state: DecodeState, weights: DeviceWeights, *, fused: bool | None = None) -> None:
-    forward_decode(state, weights, commit=True, fused=fused)
+def forward_decode(state: DecodeState, weights: DeviceWeights, *, commit: bool = False,
+                   schedule: str | None = None) -> None:
+    """Logits of ``state.token`` at ``state.position`` into the arena, its argmax
+    into ``state.next_token``; with ``commit`` the id is fed back on the device.
+    ``schedule`` names the launch schedule (``SCHEDULES``; default ``DEFAULT_SCHEDULE``)."""
+    if schedule is None:
+        schedule = DEFAULT_SCHEDULE
+    if schedule not in SCHEDULES:
+        raise ValueError(f"schedule must be one of {SCHEDULES}, got {schedule!r}")
+    if schedule == "handover":
+        if not can_fuse(weights):
+            raise ValueError("the handover schedule needs packed embedding rows, bias-free o/down "
+                             "projections and reduction lengths that are multiples of 64")
+        _forward_fused(state, weights, commit)
+        return
+    _forward_calls(state, weights, commit, schedule == "fold_rms")
+
+
+def greedy_decode(state: DecodeState, weights: DeviceWeights, *, schedule: str | None = None) -> None:
+    forward_decode(state, weights, commit=True, schedule=schedule)
 
 
 def teacher_force_token(state: DecodeState, weights: DeviceWeights, token_id: int) -> None:

@@ -219,16 +219,16 @@ def test_greedy_64_tokens_identical_to_the_oracle(seed, packed_embed):
     say("64 tokens seed", seed, "packed_embed", packed_embed)
     model, state, weights = session(LONGRUN, seed, packed_embed)
     assert dv2.can_fuse(weights) == packed_embed
-    fused = packed_embed
+    sched = "handover" if packed_embed else None
     prompt = [11, 200, 37, 1999, 5, 640, 3, 77]
     want, margins = so.greedy_ids(model, prompt, 64, ignore_eos=True, return_margins=True)
     assert len(want) == 64
     state.reset()
-    step = (lambda s, w: dv2.greedy_decode(s, w, fused=True)) if fused else dv2.greedy_decode
+    step = lambda s, w: dv2.greedy_decode(s, w, schedule=sched)  # noqa: E731
     got = dv2.generate(state, weights, prompt, 64, step=step, ignore_eos=True)
     say("  min / median top-1 margin", min(margins), float(np.median(margins)))
     state.reset()
-    graph = dv2.capture_greedy(state, weights, warmup=1, fused=fused)
+    graph = dv2.capture_greedy(state, weights, warmup=1, schedule=sched)
     state.reset()
     assert dv2.generate(state, weights, prompt, 64, step=graph, ignore_eos=True) == got
     if got != want:
@@ -285,7 +285,7 @@ def test_fused_schedule_equals_plain_schedule(spec, seed):
     for i, t in enumerate(toks):
         for st, fused in ((state, True), (other, False)):
             st.load_token(t)
-            dv2.forward_decode(st, weights, fused=fused)
+            dv2.forward_decode(st, weights, schedule="handover" if fused else "plain")
             st.position.add_(1)
         a = state.arena.logits.float()
         b = other.arena.logits.float()
@@ -298,18 +298,38 @@ def test_fused_schedule_equals_plain_schedule(spec, seed):
     ko, vo = other.kv.layer(0)
     assert float((kc.float() - ko.float()).abs().max()) <= 0.02 * float(ko.float().abs().max())
     got = greedy_token_at_a_time(state, weights, SHORT, 10,
-                                 step=lambda s, w: dv2.greedy_decode(s, w, fused=True))
+                                 step=lambda s, w: dv2.greedy_decode(s, w, schedule="handover"))
     assert got == so.greedy_ids(model, SHORT, 10)
     assert got == greedy_token_at_a_time(other, weights, SHORT, 10)
+
+
+@pytest.mark.parametrize("spec,seed,packed", [(dv2.TINY_LLAMA, 0, False), (dv2.TINY_INTERNLM, 1, False),
+                                              (dv2.MEDIUM_LLAMA, 0, True), (LONGRUN, 1, True)])
+def test_rms_folded_into_the_gemvs_equals_separate_launches(spec, seed, packed):
+    """`fold_rms` against `plain`: the normalised activations are the same bf16 values up
+    to the summation order of the RMS statistic, so logits agree closely, position by
+    position, and the greedy ids equal the oracle's."""
+    model, state, weights = session(spec, seed, packed_embed=packed)
+    other = dv2.DecodeState.allocate(spec, device="cuda")
+    toks = np.random.default_rng(seed + 7).integers(0, spec.vocab, size=min(24, spec.max_seq)).tolist()
+    for i, t in enumerate(toks):
+        for st, sched in ((state, "fold_rms"), (other, "plain")):
+            st.load_token(t)
+            dv2.forward_decode(st, weights, schedule=sched)
+            st.position.add_(1)
+        a, b = state.arena.logits.float(), other.arena.logits.float()
+        assert float((a - b).abs().max()) <= 0.02 * float(b.abs().max()) + 1e-3, i
+    step = lambda s, w: dv2.greedy_decode(s, w, schedule="fold_rms")  # noqa: E731
+    assert greedy_token_at_a_time(state, weights, SHORT, 10, step=step) == so.greedy_ids(model, SHORT, 10)
 
 
 def test_fused_schedule_in_a_graph():
     model, state, weights = session(dv2.MEDIUM_LLAMA, 0, packed_embed=True)
     eager = greedy_token_at_a_time(state, weights, SHORT, 12,
-                                   step=lambda s, w: dv2.greedy_decode(s, w, fused=True))
+                                   step=lambda s, w: dv2.greedy_decode(s, w, schedule="handover"))
     assert eager == so.greedy_ids(model, SHORT, 12)
     state.reset()
-    graph = dv2.capture_greedy(state, weights, warmup=2, fused=True)
+    graph = dv2.capture_greedy(state, weights, warmup=2, schedule="handover")
     for rep in range(3):
         assert greedy_token_at_a_time(state, weights, SHORT, 12, step=graph) == eager, rep
         torch.cuda.synchronize()
@@ -320,4 +340,6 @@ def test_fused_schedule_is_refused_when_it_does_not_apply():
     assert not dv2.can_fuse(weights)
     state.load_token(1)
     with pytest.raises(ValueError):
-        dv2.forward_decode(state, weights, fused=True)
+        dv2.forward_decode(state, weights, schedule="handover")
+    with pytest.raises(ValueError):
+        dv2.forward_decode(state, weights, schedule="nope")
