@@ -602,7 +602,19 @@ int rows_for_m(int M) {
   if (f > 0) {
     return f;
   }
+  if (M >= 32768) {
+    return 4;  // long streams (lm_head): the x registers are shared by more rows
+  }
   return M >= 4096 ? 2 : 1;
+}
+
+// CHR_NF4_GEMV_STAGED=0|1 forces the kernel family (read on every launch); unset = automatic.
+int forced_staged() {
+  const char *e = std::getenv("CHR_NF4_GEMV_STAGED");
+  if (e != nullptr && (e[0] == '0' || e[0] == '1') && e[1] == '\0') {
+    return e[0] - '0';
+  }
+  return -1;
 }
 
 constexpr int kThreads = 256;
@@ -643,8 +655,11 @@ int launch_stream(StreamArgs &a, int n_seg, hipStream_t st) {
     a.groups[i] = i < n_seg ? (a.M[i] + U - 1) / U : 0;
     total += a.groups[i];
   }
-  if (a.rms_w != nullptr || a.K != a.K_pad) {
-    const size_t dyn = static_cast<size_t>(x_pieces(a.K_pad)) * 16;
+  const size_t dyn = static_cast<size_t>(x_pieces(a.K_pad)) * 16;
+  const bool must_stage = a.rms_w != nullptr || a.K != a.K_pad;
+  const int forced = forced_staged();
+  const bool staged = must_stage || (forced == 1 && dyn <= kMaxDynLds);
+  if (staged) {
     if (prep_lds(gemv_stream<R, SWIGLU, true>, dyn) != 0) {
       return -6;
     }

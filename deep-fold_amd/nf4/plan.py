@@ -72,6 +72,8 @@ def gemv_rows_per_wavefront(m: int, forced: int = 0) -> int:
     """Rows one wavefront of the GEMV walks together (they share x)."""
     if forced in (1, 2, 4):
         return forced
+    if m >= 32768:
+        return 4
     return 2 if m >= 4096 else 1
 
 
