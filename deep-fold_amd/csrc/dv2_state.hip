@@ -11,11 +11,6 @@
 
 namespace chr {
 
-int gemv_add_norm_entry(const chr_nf4_dev_t *w, const void *x, void *y, const void *norm_w,
-                        float norm_eps, void *norm_out, float *scratch, int64_t scratch_floats,
-                        void *stream);
-int gemv_norm_blocks(int M);
-
 namespace {
 
 constexpr int kBeginBlock = 1024;
@@ -23,8 +18,8 @@ constexpr int kBeginBlock = 1024;
 // First launch of a fused decode step, one workgroup:
 //   valid_len = position + 1
 //   x   = bf16( LUT[code] * f32(scale) ) for row *token of the packed embedding
-//   h   = RMSNorm(x, norm_w, eps) rounded to bf16
-// i.e. GraphSafeKV.mark_written + the embedding gather + the first RMSNorm.
+//   h   = RMSNorm(x, norm_w, eps) rounded to bf16, when norm_w is given
+// i.e. GraphSafeKV.mark_written + the embedding gather (+ the first RMSNorm).
 __global__ __launch_bounds__(kBeginBlock) void begin_step(
     const uint8_t *__restrict__ packed, const uint16_t *__restrict__ scale, int M, int K, int K_pad,
     const int64_t *__restrict__ token, const int64_t *__restrict__ position,
@@ -62,6 +57,9 @@ __global__ __launch_bounds__(kBeginBlock) void begin_step(
   sq = wave_sum(sq);
   if ((threadIdx.x & (kWave - 1)) == 0) {
     part[threadIdx.x >> 6] = sq;
+  }
+  if (norm_w == nullptr) {
+    return;
   }
   __syncthreads();  // also orders this workgroup's x stores before the reads below
   float sum = 0.f;
@@ -177,7 +175,7 @@ extern "C" int chr_dv2_begin_step(const chr_nf4_dev_t *table, const void *token,
                                   const void *position, void *valid_len, void *x,
                                   const void *norm_w, float eps, void *h, void *stream) {
   if (table == nullptr || token == nullptr || position == nullptr || valid_len == nullptr ||
-      x == nullptr || norm_w == nullptr || h == nullptr) {
+      x == nullptr || (norm_w != nullptr && h == nullptr)) {
     return -1;
   }
   if (table->M < 1 || table->K < 1 || table->packed == nullptr || table->scale == nullptr) {
@@ -195,16 +193,6 @@ extern "C" int chr_dv2_begin_step(const chr_nf4_dev_t *table, const void *token,
       static_cast<int32_t *>(valid_len), static_cast<uint16_t *>(x),
       static_cast<const uint16_t *>(norm_w), eps, static_cast<uint16_t *>(h));
   return launch_rc();
-}
-
-extern "C" int chr_dv2_gemv_add_norm(const chr_nf4_dev_t *w, const void *x, void *y,
-                                     const void *norm_w, float norm_eps, void *norm_out,
-                                     float *scratch, int64_t scratch_floats, void *stream) {
-  return gemv_add_norm_entry(w, x, y, norm_w, norm_eps, norm_out, scratch, scratch_floats, stream);
-}
-
-extern "C" int64_t chr_dv2_gemv_add_norm_scratch(int32_t M) {
-  return M < 1 ? 0 : 16 + static_cast<int64_t>(gemv_norm_blocks(M));
 }
 
 extern "C" int chr_dv2_mark_written(const void *position, void *valid_len, void *stream) {

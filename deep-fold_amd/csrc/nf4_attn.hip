@@ -75,30 +75,10 @@ struct AttnArgs {
   const int64_t *position;
   int n_q, n_kv, hd, n_split, max_seq;
   float scale;
-  // fused merge (attn_flash<.., true>): the wavefront that finishes a head last
-  // folds that head's splits; head_count[n_q] is zero between launches
-  uint16_t *out;
-  unsigned int *head_count;
+  uint16_t *out;  // merged heads, bf16 [n_q, hd]
 };
 
-// Split partials that another wavefront of the same launch reads back travel at
-// device scope; the two-launch form uses ordinary accesses.
-template <bool COHERENT>
-__device__ __forceinline__ float ld_f32(const float *p) {
-  if constexpr (COHERENT) {
-    return load_coherent(p);
-  } else {
-    return *p;
-  }
-}
-template <bool COHERENT>
-__device__ __forceinline__ void st_f32(float *p, float v) {
-  if constexpr (COHERENT) {
-    store_coherent(p, v);
-  } else {
-    *p = v;
-  }
-}
+constexpr int kMaxWgSplits = 16;  // wavefronts of a one-workgroup-per-head launch
 
 // out[head] = sum_s a_s o_s / sum_s a_s l_s with a_s = exp(m_s - max m); an
 // empty split has m = -1e30 and l = 0, so its weight underflows to zero.
@@ -106,14 +86,13 @@ __device__ __forceinline__ void st_f32(float *p, float v) {
 // and the denominator are wavefront reductions; then every lane owns dims
 // l, l+64, .. and walks the splits with all loads independent (unrolled), the
 // sum over splits running in split order.
-template <bool COHERENT>
 __device__ __forceinline__ void merge_head(const float *m_s, const float *l_s, const float *o_s,
                                            uint16_t *out, int head, int hd, int n_split,
                                            int lane) {
   const float *mh = m_s + static_cast<size_t>(head) * n_split;
   const float *lh = l_s + static_cast<size_t>(head) * n_split;
-  const float my_m = lane < n_split ? ld_f32<COHERENT>(mh + lane) : kNegBig;
-  const float my_l = lane < n_split ? ld_f32<COHERENT>(lh + lane) : 0.f;
+  const float my_m = lane < n_split ? *(mh + lane) : kNegBig;
+  const float my_l = lane < n_split ? *(lh + lane) : 0.f;
   float m = my_m;
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) {
@@ -139,7 +118,7 @@ __device__ __forceinline__ void merge_head(const float *m_s, const float *l_s, c
       float v[8];
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        v[j] = on ? ld_f32<COHERENT>(oh + static_cast<size_t>(s + j) * hd + d) : 0.f;
+        v[j] = on ? *(oh + static_cast<size_t>(s + j) * hd + d) : 0.f;
       }
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
@@ -147,7 +126,7 @@ __device__ __forceinline__ void merge_head(const float *m_s, const float *l_s, c
       }
     }
     for (; s < n_split; ++s) {
-      const float v = on ? ld_f32<COHERENT>(oh + static_cast<size_t>(s) * hd + d) : 0.f;
+      const float v = on ? *(oh + static_cast<size_t>(s) * hd + d) : 0.f;
       acc += __shfl(my_w, s, kWave) * v;
     }
     if (on) {
@@ -156,31 +135,18 @@ __device__ __forceinline__ void merge_head(const float *m_s, const float *l_s, c
   }
 }
 
-// After a wavefront has stored its split's partials: take a ticket for the head;
-// the wavefront holding the last ticket merges the head and re-arms the counter.
-__device__ __forceinline__ void merge_if_last(const AttnArgs &a, int head, int lane) {
-  unsigned int ticket = 0;
-  drain_stores();  // this wavefront's partials have landed before its ticket
-  if (lane == 0) {
-    ticket = atomicAdd(a.head_count + head, 1u);
-  }
-  ticket = static_cast<unsigned int>(__shfl(static_cast<int>(ticket), 0, kWave));
-  if (ticket != static_cast<unsigned int>(a.n_split - 1)) {
-    return;
-  }
-  merge_head<true>(a.m_s, a.l_s, a.o_s, a.out, head, a.hd, a.n_split, lane);
-  if (lane == 0) {
-    store_coherent(a.head_count + head, 0u);
-  }
-}
-
 // LPT lanes per time step, 8 dims per lane: hd == 8*LPT.
-template <int LPT, bool FUSED>
-__global__ __launch_bounds__(kWave) void attn_flash(const AttnArgs a) {
+// INWG == false: one wavefront per (head, split), partials to global memory, merged by a
+//                second launch (attn_merge).
+// INWG == true : one workgroup per head, wavefront w takes split w of n_split =
+//                blockDim.x/64 <= 16, partials meet in LDS and wavefront 0 merges them:
+//                no workspace and no second launch.
+template <int LPT, bool INWG>
+__global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flash(const AttnArgs a) {
   constexpr int TPW = kWave / LPT;  // time steps per wavefront iteration
-  const int head = blockIdx.x / a.n_split;
-  const int split = blockIdx.x % a.n_split;
-  const int lane = threadIdx.x;
+  const int head = INWG ? static_cast<int>(blockIdx.x) : static_cast<int>(blockIdx.x) / a.n_split;
+  const int split = INWG ? static_cast<int>(threadIdx.x >> 6) : static_cast<int>(blockIdx.x) % a.n_split;
+  const int lane = threadIdx.x & (kWave - 1);
   const int li = lane % LPT;  // which 8 dims of the head
   const int grp = lane / LPT; // which time step of the iteration
   const int hd = a.hd;
@@ -228,38 +194,49 @@ __global__ __launch_bounds__(kWave) void attn_flash(const AttnArgs a) {
   float l = 0.f;
   float acc[8] = {};
   const size_t row_stride = static_cast<size_t>(a.n_kv) * hd;
-  for (int t0 = split; t0 < vl; t0 += a.n_split * TPW) {
-    const int t = t0 + grp * a.n_split;
-    const bool live = t < vl;
-    const bool cur = fuse && t == pos;
-    float kf[8], vf[8];
-    if (live && !cur) {
-      const size_t off = static_cast<size_t>(t) * row_stride + static_cast<size_t>(kv_head) * hd + d0;
-      widen8(*reinterpret_cast<const uint4 *>(a.k_cache + off), kf);
-      widen8(*reinterpret_cast<const uint4 *>(a.v_cache + off), vf);
-    } else {
+  // Two time steps per lane group and iteration: their loads are independent, so the
+  // trip count (and with it the exposed memory latency) halves.
+  const int stride = a.n_split * TPW;
+  for (int t0 = split; t0 < vl; t0 += 2 * stride) {
+    float kf[2][8], vf[2][8];
+    bool live[2];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        kf[i] = cur ? kcur[i] : 0.f;
-        vf[i] = cur ? vcur[i] : 0.f;
+    for (int u = 0; u < 2; ++u) {
+      const int t = t0 + grp * a.n_split + u * stride;
+      live[u] = t < vl;
+      const bool cur = fuse && t == pos;
+      if (live[u] && !cur) {
+        const size_t off =
+            static_cast<size_t>(t) * row_stride + static_cast<size_t>(kv_head) * hd + d0;
+        widen8(*reinterpret_cast<const uint4 *>(a.k_cache + off), kf[u]);
+        widen8(*reinterpret_cast<const uint4 *>(a.v_cache + off), vf[u]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          kf[u][i] = cur ? kcur[i] : 0.f;
+          vf[u][i] = cur ? vcur[i] : 0.f;
+        }
       }
     }
-    float dot = 0.f;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      dot = fmaf(qf[i], kf[i], dot);
-    }
-    dot = group_sum<LPT>(dot) * a.scale;
-    if (live) {
-      const float m2 = fmaxf(m, dot);
-      const float alpha = __expf(m - m2);
-      const float e = __expf(dot - m2);
-      l = l * alpha + e;
+    for (int u = 0; u < 2; ++u) {
+      float dot = 0.f;
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        acc[i] = acc[i] * alpha + e * vf[i];
+        dot = fmaf(qf[i], kf[u][i], dot);
       }
-      m = m2;
+      dot = group_sum<LPT>(dot) * a.scale;
+      if (live[u]) {
+        const float m2 = fmaxf(m, dot);
+        const float alpha = __expf(m - m2);
+        const float e = __expf(dot - m2);
+        l = l * alpha + e;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          acc[i] = acc[i] * alpha + e * vf[u][i];
+        }
+        m = m2;
+      }
     }
   }
 
@@ -288,35 +265,44 @@ __global__ __launch_bounds__(kWave) void attn_flash(const AttnArgs a) {
     m = mg;
   }
 
-  const size_t slot = static_cast<size_t>(head) * a.n_split + split;
-  if (lane == 0) {
-    st_f32<FUSED>(a.m_s + slot, m);
-    st_f32<FUSED>(a.l_s + slot, l);
-  }
-  if (grp == 0) {
-    float *oh = a.o_s + slot * hd + d0;
-    if constexpr (FUSED) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        store_coherent(oh + j, acc[j]);
-      }
-    } else {
+  if constexpr (INWG) {
+    __shared__ float sm[kMaxWgSplits], sl[kMaxWgSplits];
+    __shared__ __align__(16) float so[kMaxWgSplits * 8 * LPT];
+    if (lane == 0) {
+      sm[split] = m;
+      sl[split] = l;
+    }
+    if (grp == 0) {
+      float *oh = so + split * hd + d0;
       *reinterpret_cast<float4 *>(oh) = make_float4(acc[0], acc[1], acc[2], acc[3]);
       *reinterpret_cast<float4 *>(oh + 4) = make_float4(acc[4], acc[5], acc[6], acc[7]);
     }
-  }
-  if constexpr (FUSED) {
-    merge_if_last(a, head, lane);
+    __syncthreads();
+    if (split == 0) {
+      merge_head(sm, sl, so, a.out + static_cast<size_t>(head) * hd, 0, hd, a.n_split, lane);
+    }
+  } else {
+    const size_t slot = static_cast<size_t>(head) * a.n_split + split;
+    if (lane == 0) {
+      a.m_s[slot] = m;
+      a.l_s[slot] = l;
+    }
+    if (grp == 0) {
+      float *oh = a.o_s + slot * hd + d0;
+      *reinterpret_cast<float4 *>(oh) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+      *reinterpret_cast<float4 *>(oh + 4) = make_float4(acc[4], acc[5], acc[6], acc[7]);
+    }
   }
 }
 
 // Any hd <= 256: lane l owns dims l, l+64, l+128, l+192; one time step per
 // iteration.  Slow path for head sizes that are not 8 * 2^n.
-template <bool FUSED>
-__global__ __launch_bounds__(kWave) void attn_flash_generic(const AttnArgs a) {
-  const int head = blockIdx.x / a.n_split;
-  const int split = blockIdx.x % a.n_split;
-  const int lane = threadIdx.x;
+template <bool INWG>
+__global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flash_generic(
+    const AttnArgs a) {
+  const int head = INWG ? static_cast<int>(blockIdx.x) : static_cast<int>(blockIdx.x) / a.n_split;
+  const int split = INWG ? static_cast<int>(threadIdx.x >> 6) : static_cast<int>(blockIdx.x) % a.n_split;
+  const int lane = threadIdx.x & (kWave - 1);
   const int hd = a.hd;
   const int half = hd / 2;
   const int n_rep = a.n_q / a.n_kv;
@@ -403,20 +389,37 @@ __global__ __launch_bounds__(kWave) void attn_flash_generic(const AttnArgs a) {
     }
     m = m2;
   }
-  const size_t slot = static_cast<size_t>(head) * a.n_split + split;
-  if (lane == 0) {
-    st_f32<FUSED>(a.m_s + slot, m);
-    st_f32<FUSED>(a.l_s + slot, l);
-  }
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int d = lane + 64 * i;
-    if (d < hd) {
-      st_f32<FUSED>(a.o_s + slot * hd + d, acc[i]);
+  if constexpr (INWG) {
+    __shared__ float sm[kMaxWgSplits], sl[kMaxWgSplits];
+    __shared__ float so[kMaxWgSplits * 256];
+    if (lane == 0) {
+      sm[split] = m;
+      sl[split] = l;
     }
-  }
-  if constexpr (FUSED) {
-    merge_if_last(a, head, lane);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int d = lane + 64 * i;
+      if (d < hd) {
+        so[split * hd + d] = acc[i];
+      }
+    }
+    __syncthreads();
+    if (split == 0) {
+      merge_head(sm, sl, so, a.out + static_cast<size_t>(head) * hd, 0, hd, a.n_split, lane);
+    }
+  } else {
+    const size_t slot = static_cast<size_t>(head) * a.n_split + split;
+    if (lane == 0) {
+      a.m_s[slot] = m;
+      a.l_s[slot] = l;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int d = lane + 64 * i;
+      if (d < hd) {
+        a.o_s[slot * hd + d] = acc[i];
+      }
+    }
   }
 }
 
@@ -426,7 +429,7 @@ __global__ __launch_bounds__(kWave) void attn_merge(const float *__restrict__ m_
                                                     const float *__restrict__ o_s,
                                                     uint16_t *__restrict__ out, int hd,
                                                     int n_split) {
-  merge_head<false>(m_s, l_s, o_s, out, blockIdx.x, hd, n_split, threadIdx.x);
+  merge_head(m_s, l_s, o_s, out, blockIdx.x, hd, n_split, threadIdx.x);
 }
 
 // Standalone RoPE + cache write: one wavefront per head (q heads first, then kv).
@@ -507,35 +510,36 @@ extern "C" int chr_nf4_rope_kv(void *q, void *k, const void *v, void *k_cache, v
 namespace chr {
 namespace {
 
-template <bool FUSED>
+template <bool INWG>
 void launch_flash(const AttnArgs &a, bool vec_ok, hipStream_t st) {
-  const dim3 grid(static_cast<unsigned>(a.n_q * a.n_split));
-  const dim3 block(kWave);
+  const dim3 grid(static_cast<unsigned>(INWG ? a.n_q : a.n_q * a.n_split));
+  const dim3 block(static_cast<unsigned>(INWG ? kWave * a.n_split : kWave));
   if (vec_ok && a.hd == 128) {
-    attn_flash<16, FUSED><<<grid, block, 0, st>>>(a);
+    attn_flash<16, INWG><<<grid, block, 0, st>>>(a);
   } else if (vec_ok && a.hd == 64) {
-    attn_flash<8, FUSED><<<grid, block, 0, st>>>(a);
+    attn_flash<8, INWG><<<grid, block, 0, st>>>(a);
   } else if (vec_ok && a.hd == 256) {
-    attn_flash<32, FUSED><<<grid, block, 0, st>>>(a);
+    attn_flash<32, INWG><<<grid, block, 0, st>>>(a);
   } else if (vec_ok && a.hd == 32) {
-    attn_flash<4, FUSED><<<grid, block, 0, st>>>(a);
+    attn_flash<4, INWG><<<grid, block, 0, st>>>(a);
   } else if (vec_ok && a.hd == 16) {
-    attn_flash<2, FUSED><<<grid, block, 0, st>>>(a);
+    attn_flash<2, INWG><<<grid, block, 0, st>>>(a);
   } else {
-    attn_flash_generic<FUSED><<<grid, block, 0, st>>>(a);
+    attn_flash_generic<INWG><<<grid, block, 0, st>>>(a);
   }
 }
 
+// ws == nullptr selects the one-workgroup-per-head form (n_split wavefronts, <= 16).
 int attn_common(const void *q, const void *k, const void *v, void *out, const void *valid_len,
                 float *ws, int32_t n_q, int32_t n_kv, int32_t hd, int32_t n_split, float scale,
                 void *stream, const void *k_act, const void *v_act, const void *cos,
-                const void *sin, const void *position, int32_t max_seq, unsigned int *head_count) {
+                const void *sin, const void *position, int32_t max_seq, bool in_wg) {
   if (q == nullptr || k == nullptr || v == nullptr || out == nullptr || valid_len == nullptr ||
-      ws == nullptr) {
+      (!in_wg && ws == nullptr)) {
     return -1;
   }
   if (n_q < 1 || n_kv < 1 || hd < 1 || hd > 256 || (n_q % n_kv) != 0 || n_split < 1 ||
-      n_split > 64 || max_seq < 1) {
+      n_split > (in_wg ? kMaxWgSplits : 64) || max_seq < 1) {
     return -3;
   }
   const bool rope = cos != nullptr && sin != nullptr && position != nullptr;
@@ -547,9 +551,11 @@ int attn_common(const void *q, const void *k, const void *v, void *out, const vo
   a.q = static_cast<const uint16_t *>(q);
   a.k_cache = static_cast<const uint16_t *>(k);
   a.v_cache = static_cast<const uint16_t *>(v);
-  a.m_s = ws;
-  a.l_s = ws + nml;
-  a.o_s = ws + 2 * static_cast<size_t>(nml);
+  if (!in_wg) {
+    a.m_s = ws;
+    a.l_s = ws + nml;
+    a.o_s = ws + 2 * static_cast<size_t>(nml);
+  }
   a.valid_len = static_cast<const int32_t *>(valid_len);
   a.k_act = static_cast<const uint16_t *>(k_act);
   a.v_act = static_cast<const uint16_t *>(v_act);
@@ -563,15 +569,14 @@ int attn_common(const void *q, const void *k, const void *v, void *out, const vo
   a.max_seq = max_seq;
   a.scale = scale;
   a.out = static_cast<uint16_t *>(out);
-  a.head_count = head_count;
   hipStream_t st = static_cast<hipStream_t>(stream);
   // The vector path needs 16-byte aligned rows and 16-byte aligned fp32 partials.
   const bool vec_ok = aligned16(q) && aligned16(k) && aligned16(v) &&
                       (k_act == nullptr || aligned16(k_act)) &&
                       (v_act == nullptr || aligned16(v_act)) &&
                       (cos == nullptr || aligned16(cos)) && (sin == nullptr || aligned16(sin)) &&
-                      aligned16(a.o_s);
-  if (head_count != nullptr) {
+                      (in_wg || aligned16(a.o_s));
+  if (in_wg) {
     launch_flash<true>(a, vec_ok, st);
   } else {
     launch_flash<false>(a, vec_ok, st);
@@ -590,17 +595,14 @@ extern "C" int chr_nf4_attn(const void *q, const void *k, const void *v, void *o
                             const void *k_act, const void *v_act, const void *cos,
                             const void *sin, const void *position, int32_t max_seq) {
   return attn_common(q, k, v, out, valid_len, ws, n_q, n_kv, hd, n_split, scale, stream, k_act,
-                     v_act, cos, sin, position, max_seq, nullptr);
+                     v_act, cos, sin, position, max_seq, false);
 }
 
 extern "C" int chr_dv2_attn(const void *q, const void *k, const void *v, void *out,
-                            const void *valid_len, float *ws, void *head_count, int32_t n_q,
-                            int32_t n_kv, int32_t hd, int32_t n_split, float scale, void *stream,
-                            const void *k_act, const void *v_act, const void *cos,
-                            const void *sin, const void *position, int32_t max_seq) {
-  if (head_count == nullptr) {
-    return -1;
-  }
-  return attn_common(q, k, v, out, valid_len, ws, n_q, n_kv, hd, n_split, scale, stream, k_act,
-                     v_act, cos, sin, position, max_seq, static_cast<unsigned int *>(head_count));
+                            const void *valid_len, int32_t n_q, int32_t n_kv, int32_t hd,
+                            int32_t n_waves, float scale, void *stream, const void *k_act,
+                            const void *v_act, const void *cos, const void *sin,
+                            const void *position, int32_t max_seq) {
+  return attn_common(q, k, v, out, valid_len, nullptr, n_q, n_kv, hd, n_waves, scale, stream,
+                     k_act, v_act, cos, sin, position, max_seq, true);
 }

@@ -154,27 +154,6 @@ inline bool k_pad_ok(int K, int K_pad) {
   return K_pad == kGroup * ((K + kGroup - 1) / kGroup);
 }
 
-// ---- hand-over between workgroups of one launch ------------------------------------
-// A producer stores its results with store_coherent, waits with drain_stores until the
-// memory system has acknowledged them, and only then takes a ticket with an atomic add;
-// whoever draws the last ticket reads everything back with load_coherent.  These
-// accesses are performed at device scope (they bypass the per-XCD caches that are
-// not kept coherent with each other), so no cache write-back or invalidate is needed:
-// a device-scope fence per wavefront costs a write-back of the whole L2 and serialises.
-template <typename T>
-__device__ __forceinline__ void store_coherent(T *p, T v) {
-  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-template <typename T>
-__device__ __forceinline__ T load_coherent(const T *p) {
-  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ void drain_stores() {
-  __atomic_signal_fence(__ATOMIC_SEQ_CST);
-  __builtin_amdgcn_s_waitcnt(0);  // vmcnt(0): every store of this wavefront has been acknowledged
-  __atomic_signal_fence(__ATOMIC_SEQ_CST);
-}
-
 __host__ __device__ inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 __host__ __device__ inline bool aligned2(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 1u) == 0; }
 

@@ -128,12 +128,6 @@ struct StreamArgs {
   const uint16_t *rms_w;  // optional, bf16 [K]
   int K, K_pad;
   float rms_eps;
-  // Fused "RMSNorm of the result" (segment 0 only, see gemv_stream<.., NORM>):
-  const uint16_t *norm_w;  // bf16 [M] weight of the norm applied to y
-  uint16_t *norm_out;      // bf16 [M] normalised y
-  float *norm_part;        // one partial sum of squares per workgroup
-  unsigned int *norm_count;  // arrival counter, zero between launches
-  float norm_eps;
 };
 
 // Sum of a value over the whole workgroup, the same in every thread.
@@ -361,72 +355,11 @@ __device__ __forceinline__ void rows_dot(const uint8_t *const (&prow)[R],
 
 __device__ __forceinline__ float silu(float v) { return v / (1.f + expf(-v)); }
 
-// Tail of a NORM launch.  sq is the squared value each storing lane wrote (0 for
-// every other lane).  Called by all threads of the workgroup.
-__device__ __forceinline__ void norm_tail(const StreamArgs &a, float sq, float *part, int M) {
-  __shared__ unsigned int last;
-  drain_stores();  // this wavefront's y rows have landed before the barrier below
-  const float mine = block_sum(sq, part);
-  if (threadIdx.x == 0) {
-    store_coherent(a.norm_part + blockIdx.x, mine);
-    drain_stores();
-    const unsigned int ticket = atomicAdd(a.norm_count, 1u);
-    last = (ticket == gridDim.x - 1) ? 1u : 0u;
-  }
-  __syncthreads();
-  if (last == 0u) {
-    return;
-  }
-  // Partials in index order: thread t adds t, t+T, ..; the block sum adds the
-  // per-thread values in a fixed order as well.
-  float tot = 0.f;
-  for (unsigned int i = threadIdx.x; i < gridDim.x; i += blockDim.x) {
-    tot += load_coherent(a.norm_part + i);
-  }
-  tot = block_sum(tot, part);
-  const float inv = rsqrtf(tot / static_cast<float>(M) + a.norm_eps);
-  const uint32_t *y2 = reinterpret_cast<const uint32_t *>(a.y[0]);
-  const uint32_t *w2 = reinterpret_cast<const uint32_t *>(a.norm_w);
-  uint32_t *o2 = reinterpret_cast<uint32_t *>(a.norm_out);
-  const int pairs = M >> 1;
-  constexpr int kBatch = 4;  // loads in flight per thread
-  for (int base = threadIdx.x; base < pairs; base += kBatch * blockDim.x) {
-    uint32_t yv[kBatch], wv[kBatch];
-#pragma unroll
-    for (int j = 0; j < kBatch; ++j) {
-      const int i = base + j * blockDim.x;
-      yv[j] = i < pairs ? load_coherent(y2 + i) : 0u;
-      wv[j] = i < pairs ? w2[i] : 0u;
-    }
-#pragma unroll
-    for (int j = 0; j < kBatch; ++j) {
-      const int i = base + j * blockDim.x;
-      if (i < pairs) {
-        const uint32_t lo = f32_to_bf16((bf16_lo(wv[j]) * bf16_lo(yv[j])) * inv);
-        const uint32_t hi = f32_to_bf16((bf16_hi(wv[j]) * bf16_hi(yv[j])) * inv);
-        o2[i] = lo | (hi << 16);
-      }
-    }
-  }
-  if ((M & 1) != 0 && threadIdx.x == 0) {
-    const uint16_t yv = load_coherent(a.y[0] + (M - 1));
-    a.norm_out[M - 1] = f32_to_bf16((bf16_to_f32(a.norm_w[M - 1]) * bf16_to_f32(yv)) * inv);
-  }
-  if (threadIdx.x == 0) {
-    store_coherent(a.norm_count, 0u);  // ready for the next launch on this stream
-  }
-}
-
 // SWIGLU == false: R rows of one segment per wavefront, epilogue y = acc (+ add).
 // SWIGLU == true : R/2 gate rows and the matching R/2 up rows per wavefront,
 //                  epilogue y = silu(gate) * up from the unrounded fp32 sums.
 // XLDS: x is first copied (and optionally RMS-normalised) into LDS.
-// NORM: after y is stored, the launch also produces norm_out = RMSNorm(y, norm_w):
-//       every workgroup leaves the sum of squares of its (rounded) rows in
-//       norm_part, and the workgroup that arrives last adds the partials in index
-//       order (so the result does not depend on arrival order), then normalises
-//       all of y.  That replaces a separate one-workgroup RMSNorm launch.
-template <int R, bool SWIGLU, bool XLDS, bool NORM = false>
+template <int R, bool SWIGLU, bool XLDS>
 __global__ __launch_bounds__(XLDS ? 1024 : 256) void gemv_stream(const StreamArgs a) {
   extern __shared__ uint4 xs[];
   __shared__ GemvLds lds;
@@ -454,7 +387,6 @@ __global__ __launch_bounds__(XLDS ? 1024 : 256) void gemv_stream(const StreamArg
   const int stride = XLDS ? static_cast<int>(gridDim.x) * waves : total;
   const size_t pstride = static_cast<size_t>(a.K_pad >> 1);
   const size_t sstride = static_cast<size_t>(a.K_pad >> 6);
-  float sq = 0.f;  // NORM: square of the value this lane stored
 
   for (int grp = first; grp < total; grp += stride) {
     int g = grp;
@@ -514,20 +446,10 @@ __global__ __launch_bounds__(XLDS ? 1024 : 256) void gemv_stream(const StreamArg
           if (add != nullptr) {
             v += bf16_to_f32(add[r]);
           }
-          const uint16_t vb = f32_to_bf16(v);
-          if constexpr (NORM) {
-            store_coherent(y + r, vb);  // read back by the workgroup that normalises
-            const float vr = bf16_to_f32(vb);
-            sq = vr * vr;
-          } else {
-            y[r] = vb;
-          }
+          y[r] = f32_to_bf16(v);
         }
       }
     }
-  }
-  if constexpr (NORM) {
-    norm_tail(a, sq, lds.part, a.M[0]);
   }
 }
 
@@ -637,16 +559,6 @@ int prep_lds(Kern kern, size_t dyn) {
   return 0;
 }
 
-template <int R>
-int launch_stream_norm(StreamArgs &a, hipStream_t st) {
-  a.groups[0] = (a.M[0] + R - 1) / R;
-  a.groups[1] = a.groups[2] = 0;
-  const int waves = kThreads / kWave;
-  gemv_stream<R, false, false, true>
-      <<<dim3((a.groups[0] + waves - 1) / waves), dim3(kThreads), 0, st>>>(a);
-  return launch_rc();
-}
-
 template <int R, bool SWIGLU>
 int launch_stream(StreamArgs &a, int n_seg, hipStream_t st) {
   constexpr int U = SWIGLU ? R / 2 : R;
@@ -713,58 +625,6 @@ int gemv_entry(const chr_nf4_dev_t *w, const void *x, void *y, void *stream, con
   a.K_pad = w->K_pad;
   a.rms_eps = rms_eps;
   return launch_rows(a, 1, w->M, static_cast<hipStream_t>(stream));
-}
-
-// Workgroups a fused-norm GEMV over M rows launches (= partial sums it writes).
-int gemv_norm_blocks(int M) {
-  const int rows_per_wg = (kThreads / kWave) * rows_for_m(M);
-  return (M + rows_per_wg - 1) / rows_per_wg;
-}
-
-int gemv_add_norm_entry(const chr_nf4_dev_t *w, const void *x, void *y, const void *norm_w,
-                        float norm_eps, void *norm_out, float *scratch, int64_t scratch_floats,
-                        void *stream) {
-  if (w == nullptr || x == nullptr || y == nullptr || norm_w == nullptr || norm_out == nullptr ||
-      scratch == nullptr) {
-    return -1;
-  }
-  if (w->M < 1 || w->K < 1 || w->packed == nullptr || w->scale == nullptr) {
-    return -3;
-  }
-  if (!k_pad_ok(w->K, w->K_pad) || w->K != w->K_pad) {
-    return -4;
-  }
-  if (!aligned16(w->packed) || !aligned16(x) || !aligned2(w->scale) ||
-      (reinterpret_cast<uintptr_t>(y) & 3u) != 0 || (reinterpret_cast<uintptr_t>(norm_w) & 3u) != 0 ||
-      (reinterpret_cast<uintptr_t>(norm_out) & 3u) != 0 || !aligned16(scratch)) {
-    return -5;
-  }
-  if (scratch_floats < 16 + gemv_norm_blocks(w->M)) {
-    return -7;
-  }
-  StreamArgs a{};
-  a.packed[0] = w->packed;
-  a.scale[0] = w->scale;
-  a.y[0] = static_cast<uint16_t *>(y);
-  a.add[0] = static_cast<const uint16_t *>(y);
-  a.M[0] = w->M;
-  a.x = static_cast<const uint16_t *>(x);
-  a.K = w->K;
-  a.K_pad = w->K_pad;
-  a.norm_w = static_cast<const uint16_t *>(norm_w);
-  a.norm_out = static_cast<uint16_t *>(norm_out);
-  a.norm_count = reinterpret_cast<unsigned int *>(scratch);
-  a.norm_part = scratch + 16;
-  a.norm_eps = norm_eps;
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  switch (rows_for_m(w->M)) {
-    case 4:
-      return launch_stream_norm<4>(a, st);
-    case 2:
-      return launch_stream_norm<2>(a, st);
-    default:
-      return launch_stream_norm<1>(a, st);
-  }
 }
 
 // Launch geometry of the N=1 path, reported by the planner.

@@ -12,14 +12,14 @@ from .prefill import forward_prefill, prefill_chunk_width
 from .rope import apply_rope_torch, rope_tables_numpy, rope_tables_torch
 from .runner import consume_prompt, generate
 from .state import DecodeState
-from .step import can_fuse, forward_decode, greedy_decode, teacher_force_token
+from .step import SCHEDULES, forward_decode, greedy_decode, teacher_force_token
 from .synth import Nf4Matrix, SynthLayer, SynthModel, build
 
 __all__ = [
     "ArchSpec", "Arena", "DecodeState", "DeviceLayer", "DeviceLinear", "DeviceWeights", "GraphSafeKV",
     "GreedyGraph", "PackedEmbed", "Nf4Matrix", "SynthLayer", "SynthModel", "TINY_LLAMA",
     "TINY_INTERNLM", "MEDIUM_LLAMA", "QWEN25_3B", "QWEN25_14B", "INTERNLM25_20B", "QWEN25_32B",
-    "apply_rope_torch", "build", "capture_greedy", "consume_prompt", "can_fuse", "forward_decode",
+    "apply_rope_torch", "build", "capture_greedy", "consume_prompt", "SCHEDULES", "forward_decode",
     "forward_prefill", "gather_embed", "generate", "greedy_decode", "nf4_linear",
     "prefill_chunk_width", "rope_tables_numpy", "rope_tables_torch", "teacher_force_token",
     "with_max_seq",

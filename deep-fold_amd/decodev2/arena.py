@@ -7,7 +7,7 @@ from dataclasses import dataclass
 
 import torch
 
-from ..nf4 import ATTN_SPLIT, dv2_gemv_add_norm_scratch
+from ..nf4 import ATTN_SPLIT
 from .plan import ArchSpec
 
 __all__ = ["Arena"]
@@ -26,8 +26,6 @@ class Arena:
     down_in: torch.Tensor
     logits: torch.Tensor
     attn_ws: torch.Tensor
-    head_count: torch.Tensor     # per-head tickets of the fused split merge, zero between launches
-    norm_scratch: torch.Tensor   # ticket + per-workgroup sums of the fused residual RMSNorm
 
     @classmethod
     def allocate(cls, spec: ArchSpec, *, device, dtype: torch.dtype = torch.bfloat16) -> "Arena":
@@ -47,7 +45,4 @@ class Arena:
             logits=z(1, spec.vocab),
             attn_ws=torch.zeros(spec.n_q * ATTN_SPLIT * (spec.head_dim + 2), dtype=torch.float32,
                                 device=device),
-            head_count=torch.zeros(spec.n_q, dtype=torch.int32, device=device),
-            norm_scratch=torch.zeros(dv2_gemv_add_norm_scratch(spec.hidden), dtype=torch.float32,
-                                     device=device),
         )

@@ -9,29 +9,27 @@ o GEMV accumulating into the residual -> rms -> fused SwiGLU GEMV -> down GEMV
 accumulating into the residual.  Then the final norm, lm_head and a device-side
 argmax that also feeds the id back.
 
-Three launch schedules compute that sequence:
+Two launch schedules compute that sequence:
 
-``plain``     the call sequence above, eight launches per layer;
-``fold_rms``  every RMSNorm runs inside the GEMV that consumes it (six launches);
-``handover``  every RMSNorm rides on the launch that *produces* its input (the
-              embedding gather, or the residual GEMV whose last workgroup
-              normalises) and the attention launch merges its own splits (five).
-              On MI355X the hand-over between workgroups of one launch costs a
-              device-scope round trip per stage, more than the launches it
-              saves, so this one only runs on request.
+``plain``     the reference's call sequence, eight launches per layer;
+``fold_rms``  every RMSNorm runs inside the GEMV that consumes it, attention is one
+              launch per layer while the cache is short enough for one workgroup
+              per head, and the embedding gather also sets the KV length: five
+              launches per layer.  A dependent launch costs about 5 us on an
+              MI355X whatever it does, so the launch count is what this buys.
 """
 
 from __future__ import annotations
 
 import torch
 
-from ..nf4 import (ATTN_SPLIT, dv2_attn, dv2_begin_step, dv2_gemv_add_norm, nf4_attn, nf4_gemv,
-                   nf4_qkv, nf4_rms, nf4_swiglu)
+from ..nf4 import (ATTN_SPLIT, ATTN_WG_WAVES, dv2_attn, dv2_begin_step, nf4_attn, nf4_gemv, nf4_qkv,
+                   nf4_rms, nf4_swiglu)
 from .embed import PackedEmbed, gather_embed
 from .linear import DeviceLayer, DeviceLinear, DeviceWeights
 from .state import DecodeState
 
-__all__ = ["forward_decode", "greedy_decode", "teacher_force_token", "can_fuse", "SCHEDULES"]
+__all__ = ["forward_decode", "greedy_decode", "teacher_force_token", "SCHEDULES", "ATTN_WG_MAX_SEQ"]
 
 
 def _gemv_accum(mat: DeviceLinear, src: torch.Tensor, dest: torch.Tensor) -> None:
@@ -61,79 +59,54 @@ def _qkv(state: DecodeState, layer: DeviceLayer, h: torch.Tensor, rms_w: torch.T
     return ar.q.view(-1), ar.k.view(-1), ar.v.view(-1)
 
 
-def can_fuse(weights: DeviceWeights) -> bool:
-    """Whether the five-launch schedule applies: packed embedding rows, no bias on
-    the residual projections, and reduction lengths that are whole scale groups."""
-    spec = weights.spec
-    if not isinstance(weights.embed, PackedEmbed):
-        return False
-    if spec.q_dim % 64 or spec.intermediate % 64:
-        return False
-    return all(ly.o.bias is None and ly.down.bias is None for ly in weights.layers)
+SCHEDULES = ("plain", "fold_rms")
+#: schedule used when the caller does not name one
+DEFAULT_SCHEDULE = "fold_rms"
+#: longest cache the one-launch attention (one workgroup per query head) is used for;
+#: longer caches go to the split kernel + merge, which spreads a head over many units
+ATTN_WG_MAX_SEQ = 4096
 
 
-def _gemv_accum_norm(state: DecodeState, mat: DeviceLinear, src: torch.Tensor, norm_w: torch.Tensor) -> None:
-    """``x += W @ src`` and ``h = RMSNorm(x, norm_w)`` in one launch."""
-    ar = state.arena
-    dv2_gemv_add_norm(mat.packed, mat.scale, src.view(-1), mat.M, mat.K, mat.K_pad, ar.x.view(-1),
-                      norm_w, state.spec.rms_eps, ar.h.view(-1), ar.norm_scratch)
-
-
-def _forward_fused(state: DecodeState, weights: DeviceWeights, commit: bool) -> None:
+def _attend(state: DecodeState, li: int, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+            one_launch: bool) -> None:
     spec = state.spec
     ar = state.arena
     n_q, n_kv, hd = spec.n_q, spec.n_kv, spec.head_dim
-    layers = weights.layers
-    emb = weights.embed
-    dv2_begin_step(emb.packed, emb.scale, emb.hidden, state.token, state.position, state.valid_len,
-                   ar.x.view(-1), layers[0].norm1 if layers else weights.final_norm, spec.rms_eps,
-                   ar.h.view(-1))
-    for li, layer in enumerate(layers):
-        q, k, v = _qkv(state, layer, ar.h)
-        kc, vc = state.kv.layer(li)
-        dv2_attn(q.view(n_q, hd), kc, vc, ar.attn, state.valid_len, spec.attn_scale, ar.attn_ws,
-                 ar.head_count, ATTN_SPLIT, k.view(n_kv, hd), v.view(n_kv, hd), state.cos, state.sin,
+    kc, vc = state.kv.layer(li)
+    if one_launch:
+        dv2_attn(q.view(n_q, hd), kc, vc, ar.attn, state.valid_len, spec.attn_scale, ATTN_WG_WAVES,
+                 k.view(n_kv, hd), v.view(n_kv, hd), state.cos, state.sin, state.position)
+    else:
+        nf4_attn(q.view(n_q, hd), kc, vc, ar.attn, state.valid_len, spec.attn_scale, ar.attn_ws,
+                 ATTN_SPLIT, k.view(n_kv, hd), v.view(n_kv, hd), state.cos, state.sin,
                  state.position)
-        _gemv_accum_norm(state, layer.o, ar.attn, layer.norm2)
-        g, u = layer.gate, layer.up
-        nf4_swiglu(g.packed, g.scale, u.packed, u.scale, ar.h.view(-1), g.M, g.K, g.K_pad,
-                   ar.down_in.view(-1))
-        nxt = layers[li + 1].norm1 if li + 1 < len(layers) else weights.final_norm
-        _gemv_accum_norm(state, layer.down, ar.down_in, nxt)
-    head = weights.lm_head
-    nf4_gemv(head.packed, head.scale, ar.h.view(-1), head.M, head.K, head.K_pad, ar.logits.view(-1),
-             None if head.bias is None else head.bias)
-    state.pick_next(commit)
 
 
-SCHEDULES = ("plain", "fold_rms", "handover")
-#: schedule used when the caller does not name one
-DEFAULT_SCHEDULE = "fold_rms"
-
-
-def _forward_calls(state: DecodeState, weights: DeviceWeights, commit: bool, fold_rms: bool) -> None:
-    """The reference's call sequence.  With ``fold_rms`` every RMSNorm runs inside the
-    GEMV that consumes it (the ``rms_w`` argument of the GEMV entry points,
-    ``gpu/nf4/nf4_gemv.cu:264-289``): six launches per layer instead of eight."""
+def _forward_calls(state: DecodeState, weights: DeviceWeights, commit: bool, fold: bool) -> None:
+    """``fold`` == False: the reference's call sequence.  ``fold`` == True: RMSNorm inside
+    the consuming GEMV (the ``rms_w`` argument of the GEMV entry points,
+    ``gpu/nf4/nf4_gemv.cu:264-289``), one-launch attention, one-launch step prologue."""
     spec = state.spec
     ar = state.arena
     eps = spec.rms_eps
-    n_q, n_kv, hd = spec.n_q, spec.n_kv, spec.head_dim
-    gather_embed(weights.embed, state.token.reshape(1), out=ar.x)
-    state.kv.mark_written(state.position)
+    emb = weights.embed
+    if fold and isinstance(emb, PackedEmbed):
+        dv2_begin_step(emb.packed, emb.scale, emb.hidden, state.token, state.position,
+                       state.valid_len, ar.x.view(-1))
+    else:
+        gather_embed(emb, state.token.reshape(1), out=ar.x)
+        state.kv.mark_written(state.position)
+    one_launch_attn = fold and spec.max_seq <= ATTN_WG_MAX_SEQ
     for li, layer in enumerate(weights.layers):
-        if fold_rms:
+        if fold:
             q, k, v = _qkv(state, layer, ar.x, layer.norm1)
         else:
             nf4_rms(ar.x, layer.norm1, ar.h, eps)
             q, k, v = _qkv(state, layer, ar.h)
-        kc, vc = state.kv.layer(li)
-        nf4_attn(q.view(n_q, hd), kc, vc, ar.attn, state.valid_len, spec.attn_scale, ar.attn_ws,
-                 ATTN_SPLIT, k.view(n_kv, hd), v.view(n_kv, hd), state.cos, state.sin,
-                 state.position)
+        _attend(state, li, q, k, v, one_launch_attn)
         _gemv_accum(layer.o, ar.attn, ar.x)
         g, u = layer.gate, layer.up
-        if fold_rms:
+        if fold:
             nf4_swiglu(g.packed, g.scale, u.packed, u.scale, ar.x.view(-1), g.M, g.K, g.K_pad,
                        ar.down_in.view(-1), layer.norm2, eps)
         else:
@@ -143,7 +116,7 @@ def _forward_calls(state: DecodeState, weights: DeviceWeights, commit: bool, fol
         _gemv_accum(layer.down, ar.down_in, ar.x)
     head = weights.lm_head
     bias = None if head.bias is None else head.bias
-    if fold_rms:
+    if fold:
         nf4_gemv(head.packed, head.scale, ar.x.view(-1), head.M, head.K, head.K_pad,
                  ar.logits.view(-1), bias, weights.final_norm, eps)
     else:
@@ -162,12 +135,6 @@ def forward_decode(state: DecodeState, weights: DeviceWeights, *, commit: bool =
         schedule = DEFAULT_SCHEDULE
     if schedule not in SCHEDULES:
         raise ValueError(f"schedule must be one of {SCHEDULES}, got {schedule!r}")
-    if schedule == "handover":
-        if not can_fuse(weights):
-            raise ValueError("the handover schedule needs packed embedding rows, bias-free o/down "
-                             "projections and reduction lengths that are multiples of 64")
-        _forward_fused(state, weights, commit)
-        return
     _forward_calls(state, weights, commit, schedule == "fold_rms")
 
 

@@ -40,8 +40,7 @@ __all__ = [
     "dv2_mark_written",
     "dv2_argmax_commit",
     "dv2_begin_step",
-    "dv2_gemv_add_norm",
-    "dv2_gemv_add_norm_scratch",
+    "ATTN_WG_WAVES",
     "dv2_attn",
     "library_path",
 ]
@@ -108,10 +107,8 @@ EXPORTS = (
     ("chr_nf4_embed_rows", ctypes.c_int, [_DP, _P, _I, _P, _P]),
     ("chr_nf4_quantize", ctypes.c_int, [_P, _DP, _P, _P]),
     ("chr_dv2_begin_step", ctypes.c_int, [_DP, _P, _P, _P, _P, _P, _F, _P, _P]),
-    ("chr_dv2_gemv_add_norm", ctypes.c_int, [_DP, _P, _P, _P, _F, _P, _P, ctypes.c_int64, _P]),
-    ("chr_dv2_gemv_add_norm_scratch", ctypes.c_int64, [_I]),
     ("chr_dv2_attn", ctypes.c_int,
-     [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _P, _P, _P, _P, _P, _P, _I]),
+     [_P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _P, _P, _P, _P, _P, _P, _I]),
     ("chr_dv2_mark_written", ctypes.c_int, [_P, _P, _P]),
     ("chr_dv2_argmax_commit", ctypes.c_int, [_P, _I, _P, _P, _P, _P, _P, _I, _P]),
     ("chr_nf4_abi_version", ctypes.c_int, []),
@@ -589,56 +586,36 @@ def dv2_argmax_commit(logits: torch.Tensor, next_token: torch.Tensor, token: tor
 
 def dv2_begin_step(packed: torch.Tensor, scale: torch.Tensor, K: int, token: torch.Tensor,  # noqa: N803
                    position: torch.Tensor, valid_len: torch.Tensor, x: torch.Tensor,
-                   norm_w: torch.Tensor, eps: float, h: torch.Tensor) -> None:
-    """First launch of a fused decode step: ``valid_len = position + 1``, ``x`` = the
-    packed embedding row ``token``, ``h = RMSNorm(x, norm_w, eps)``."""
+                   norm_w: torch.Tensor | None = None, eps: float = 1e-6,
+                   h: torch.Tensor | None = None) -> None:
+    """First launch of a decode step: ``valid_len = position + 1``, ``x`` = the packed
+    embedding row ``token`` and, with ``norm_w``, ``h = RMSNorm(x, norm_w, eps)``."""
     M, K, K_pad = int(packed.size(0)), int(K), int(packed.size(1)) * 2
     _check_packed(packed, scale, M, K, K_pad, "embed")
     _need(packed.is_contiguous() and scale.is_contiguous(), "embed blobs must be contiguous")
     for t, dt, name in ((token, torch.int64, "token"), (position, torch.int64, "position"),
                         (valid_len, torch.int32, "valid_len")):
         _need(t.is_cuda and t.dtype == dt and t.numel() == 1, f"{name} must be a CUDA {dt} scalar")
+    _need((norm_w is None) == (h is None), "norm_w and h go together")
     for t, name in ((x, "x"), (norm_w, "norm_w"), (h, "h")):
-        _need(t.is_cuda and t.dtype == torch.bfloat16 and t.is_contiguous() and t.numel() == K,
-              f"{name} must be contiguous CUDA bf16 with K elements")
+        _need(t is None or (t.is_cuda and t.dtype == torch.bfloat16 and t.is_contiguous()
+                            and t.numel() == K), f"{name} must be contiguous CUDA bf16 with K elements")
     w = _dev(packed, scale, M, K, K_pad)
     rc = _load_ext().chr_dv2_begin_step(ctypes.byref(w), token.data_ptr(), position.data_ptr(),
-                                        valid_len.data_ptr(), x.data_ptr(), norm_w.data_ptr(),
-                                        float(eps), h.data_ptr(), _stream())
+                                        valid_len.data_ptr(), x.data_ptr(),
+                                        None if norm_w is None else norm_w.data_ptr(), float(eps),
+                                        None if h is None else h.data_ptr(), _stream())
     _check_rc("chr_dv2_begin_step", rc)
 
 
-def dv2_gemv_add_norm_scratch(M: int) -> int:  # noqa: N803
-    """Floats of scratch ``dv2_gemv_add_norm`` needs for ``M`` output rows."""
-    return int(_load_ext().chr_dv2_gemv_add_norm_scratch(int(M)))
+#: wavefronts per head of the one-launch attention
+ATTN_WG_WAVES = 16
 
 
-def dv2_gemv_add_norm(packed: torch.Tensor, scale: torch.Tensor, x: torch.Tensor, M: int, K: int,  # noqa: N803
-                      K_pad: int, y: torch.Tensor, norm_w: torch.Tensor, norm_eps: float,  # noqa: N803
-                      norm_out: torch.Tensor, scratch: torch.Tensor) -> None:
-    """``y = bf16(W @ x + y)`` then ``norm_out = RMSNorm(y, norm_w, norm_eps)``, one launch.
-    ``scratch`` is fp32, zero before its first use, left zero."""
-    M, K, K_pad = int(M), int(K), int(K_pad)
-    _check_packed(packed, scale, M, K, K_pad)
-    _need(packed.is_contiguous() and scale.is_contiguous(), "blobs must be contiguous")
-    _need(x.is_cuda and x.dtype == torch.bfloat16 and x.is_contiguous() and x.numel() == K,
-          "x must be contiguous CUDA bf16 [K]")
-    for t, name in ((y, "y"), (norm_w, "norm_w"), (norm_out, "norm_out")):
-        _need(t.is_cuda and t.dtype == torch.bfloat16 and t.is_contiguous() and t.numel() == M,
-              f"{name} must be contiguous CUDA bf16 with M elements")
-    _need(scratch.is_cuda and scratch.dtype == torch.float32 and scratch.is_contiguous(),
-          "scratch must be contiguous CUDA fp32")
-    w = _dev(packed, scale, M, K, K_pad)
-    rc = _load_ext().chr_dv2_gemv_add_norm(ctypes.byref(w), x.data_ptr(), y.data_ptr(),
-                                           norm_w.data_ptr(), float(norm_eps), norm_out.data_ptr(),
-                                           scratch.data_ptr(), int(scratch.numel()), _stream())
-    _check_rc("chr_dv2_gemv_add_norm", rc)
-
-
-def dv2_attn(q, k, v, out, valid_len, scale: float, ws, head_count, n_split: int = ATTN_SPLIT,
+def dv2_attn(q, k, v, out, valid_len, scale: float, n_waves: int = ATTN_WG_WAVES,
              k_act=None, v_act=None, cos=None, sin=None, position=None) -> None:
-    """``nf4_attn`` with the split merge folded into the same launch.  ``head_count`` is
-    int32 ``[n_q]`` on the GPU, zero before its first use, left zero."""
+    """``nf4_attn`` as one launch: a workgroup of ``n_waves`` wavefronts per query head
+    merges its own partial softmax states in LDS (no workspace)."""
     _need(q.is_cuda and q.dtype == torch.bfloat16 and q.is_contiguous(), "q must be contiguous CUDA bf16")
     _need(k.is_contiguous() and v.is_contiguous() and k.dim() == 3, "caches must be contiguous [max_seq,n_kv,hd]")
     max_seq, n_kv, hd = (int(t) for t in k.shape)
@@ -646,10 +623,7 @@ def dv2_attn(q, k, v, out, valid_len, scale: float, ws, head_count, n_split: int
     _need(out.is_contiguous() and out.dtype == torch.bfloat16 and out.numel() >= n_q * hd, "out too small")
     _need(valid_len.is_cuda and valid_len.dtype == torch.int32 and valid_len.numel() == 1,
           "valid_len must be a CUDA int32 scalar")
-    _need(ws.is_cuda and ws.dtype == torch.float32 and ws.numel() >= n_q * int(n_split) * (hd + 2),
-          "attn workspace too small")
-    _need(head_count.is_cuda and head_count.dtype == torch.int32 and head_count.numel() >= n_q,
-          "head_count must be CUDA int32 [n_q]")
+    _need(1 <= int(n_waves) <= 16, "n_waves must be in 1..16")
 
     def ptr(t):
         return None if t is None else t.data_ptr()
@@ -657,7 +631,7 @@ def dv2_attn(q, k, v, out, valid_len, scale: float, ws, head_count, n_split: int
     for t in (k_act, v_act, cos, sin, position):
         _need(t is None or (t.is_cuda and t.is_contiguous()), "optional inputs must be contiguous CUDA")
     rc = _load_ext().chr_dv2_attn(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
-                                  valid_len.data_ptr(), ws.data_ptr(), head_count.data_ptr(), n_q,
-                                  n_kv, hd, int(n_split), float(scale), _stream(), ptr(k_act),
-                                  ptr(v_act), ptr(cos), ptr(sin), ptr(position), max_seq)
+                                  valid_len.data_ptr(), n_q, n_kv, hd, int(n_waves), float(scale),
+                                  _stream(), ptr(k_act), ptr(v_act), ptr(cos), ptr(sin),
+                                  ptr(position), max_seq)
     _check_rc("chr_dv2_attn", rc)

@@ -167,37 +167,27 @@ int chr_dv2_argmax_commit(const void *logits, int32_t n, void *next_token, void 
                           void *position, void *finished, const void *eos_id, int32_t commit,
                           void *stream);
 
-/* ---- fused decode step: fewer, fatter launches than the reference's eight per layer.
- * They compute what the cited sequences of reference calls compute.  Ticket counters
- * (head_count; the first 16 floats of a gemv_add_norm scratch) are caller-owned device
- * memory that must be zero before the first use; each call re-arms them to zero.  Two
- * calls sharing a scratch buffer must not overlap. */
+/* ---- decode step: fewer launches than the reference's call sequence.  These entry
+ * points have no single counterpart in the reference; each computes what the cited
+ * sequence of reference calls computes. */
 
-/* valid_len = *position + 1; x = packed embedding row *token as bf16; h = RMSNorm(x,
- * norm_w, eps).  One launch for GraphSafeKV.mark_written + gather_embed + the first
- * nf4_rms of forward_decode (gpu/decodev2/step.py:165-172, kv.py:118-120,
- * gpu/host/embedding.py:74-107). */
+/* valid_len = *position + 1; x = packed embedding row *token as bf16; and, when norm_w
+ * is not NULL, h = RMSNorm(x, norm_w, eps).  One launch for GraphSafeKV.mark_written +
+ * gather_embed (+ the first nf4_rms) of forward_decode (gpu/decodev2/step.py:165-172,
+ * kv.py:118-120, gpu/host/embedding.py:74-107). */
 int chr_dv2_begin_step(const chr_nf4_dev_t *table, const void *token, const void *position,
                        void *valid_len, void *x, const void *norm_w, float eps, void *h,
                        void *stream);
 
-/* y[M] = bf16(W @ x + y) (the residual GEMV of _gemv_accum, gpu/decodev2/step.py:119-137)
- * and then norm_out[M] = RMSNorm(y, norm_w, norm_eps) (the _rms_into that follows it,
- * step.py:20-26), in one launch: the workgroup that finishes last normalises.  K must be
- * a multiple of 64.  scratch: chr_dv2_gemv_add_norm_scratch(M) floats, 16-byte aligned. */
-int chr_dv2_gemv_add_norm(const chr_nf4_dev_t *w, const void *x, void *y, const void *norm_w,
-                          float norm_eps, void *norm_out, float *scratch, int64_t scratch_floats,
-                          void *stream);
-int64_t chr_dv2_gemv_add_norm_scratch(int32_t M);
-
-/* chr_nf4_attn with the split merge folded into the same launch: the wavefront that
- * finishes a head last merges it.  head_count: n_q uint32 on device, zero between calls.
- * Replaces the attn_flash + attn_merge pair (gpu/nf4/nf4_gemv.cu:952-994). */
+/* chr_nf4_attn as one launch: one workgroup of n_waves (1..16) wavefronts per query head,
+ * each wavefront takes every n_waves-th cache row, the partial softmax states meet in
+ * LDS and the workgroup writes the merged head.  No workspace.  Replaces the
+ * attn_flash + attn_merge pair (gpu/nf4/nf4_gemv.cu:952-994) for contexts short enough
+ * that n_q workgroups can stream the cache (a few thousand rows). */
 int chr_dv2_attn(const void *q, const void *k, const void *v, void *out, const void *valid_len,
-                 float *ws, void *head_count, int32_t n_q, int32_t n_kv, int32_t hd,
-                 int32_t n_split, float scale, void *stream, const void *k_act,
-                 const void *v_act, const void *cos, const void *sin, const void *position,
-                 int32_t max_seq);
+                 int32_t n_q, int32_t n_kv, int32_t hd, int32_t n_waves, float scale,
+                 void *stream, const void *k_act, const void *v_act, const void *cos,
+                 const void *sin, const void *position, int32_t max_seq);
 
 /* Library version, for the loader's sanity check. */
 int chr_nf4_abi_version(void);

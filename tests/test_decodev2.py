@@ -214,12 +214,11 @@ def near_tie(logits: np.ndarray) -> bool:
 def test_greedy_64_tokens_identical_to_the_oracle(seed, packed_embed):
     """64 generated tokens on random-init weights, ignore-EOS, eager and graph.
     The stream must equal the oracle's; the only excuse for a first difference is
-    an oracle pick that is itself a near-tie at bf16 logit resolution.  Models with
-    packed embedding rows run the fused launch schedule."""
+    an oracle pick that is itself a near-tie at bf16 logit resolution.  The dense-table
+    models run the reference's call sequence, the packed-table ones the folded one."""
     say("64 tokens seed", seed, "packed_embed", packed_embed)
     model, state, weights = session(LONGRUN, seed, packed_embed)
-    assert dv2.can_fuse(weights) == packed_embed
-    sched = "handover" if packed_embed else None
+    sched = "fold_rms" if packed_embed else "plain"
     prompt = [11, 200, 37, 1999, 5, 640, 3, 77]
     want, margins = so.greedy_ids(model, prompt, 64, ignore_eos=True, return_margins=True)
     assert len(want) == 64
@@ -270,38 +269,7 @@ def test_teacher_forced_picks_agree_except_on_near_ties():
     assert disagree <= 3
 
 
-# ---- the fused launch schedule ---------------------------------------------------
-
-@pytest.mark.parametrize("spec,seed", [(dv2.TINY_LLAMA, 0), (dv2.TINY_INTERNLM, 1), (dv2.MEDIUM_LLAMA, 0),
-                                       (LONGRUN, 2)])
-def test_fused_schedule_equals_plain_schedule(spec, seed):
-    """Same weights, same tokens: logits of the five-launch schedule against the
-    eight-launch one at every position, and both against the oracle's ids."""
-    say("fused vs plain", spec.name)
-    model, state, weights = session(spec, seed, packed_embed=True)
-    assert dv2.can_fuse(weights)
-    other = dv2.DecodeState.allocate(spec, device="cuda")
-    toks = np.random.default_rng(seed).integers(0, spec.vocab, size=min(24, spec.max_seq)).tolist()
-    for i, t in enumerate(toks):
-        for st, fused in ((state, True), (other, False)):
-            st.load_token(t)
-            dv2.forward_decode(st, weights, schedule="handover" if fused else "plain")
-            st.position.add_(1)
-        a = state.arena.logits.float()
-        b = other.arena.logits.float()
-        # the two schedules differ only in the summation order of the RMS statistic
-        assert float((a - b).abs().max()) <= 0.02 * float(b.abs().max()) + 1e-3, i
-        assert int(state.valid_len.item()) == i + 1 == int(other.valid_len.item())
-        assert int(state.arena.head_count.abs().sum().item()) == 0
-        assert int(state.arena.norm_scratch.view(torch.int32)[0].item()) == 0   # the ticket is re-armed
-    kc, vc = state.kv.layer(0)
-    ko, vo = other.kv.layer(0)
-    assert float((kc.float() - ko.float()).abs().max()) <= 0.02 * float(ko.float().abs().max())
-    got = greedy_token_at_a_time(state, weights, SHORT, 10,
-                                 step=lambda s, w: dv2.greedy_decode(s, w, schedule="handover"))
-    assert got == so.greedy_ids(model, SHORT, 10)
-    assert got == greedy_token_at_a_time(other, weights, SHORT, 10)
-
+# ---- launch schedules ------------------------------------------------------------------
 
 @pytest.mark.parametrize("spec,seed,packed", [(dv2.TINY_LLAMA, 0, False), (dv2.TINY_INTERNLM, 1, False),
                                               (dv2.MEDIUM_LLAMA, 0, True), (LONGRUN, 1, True)])
@@ -323,23 +291,31 @@ def test_rms_folded_into_the_gemvs_equals_separate_launches(spec, seed, packed):
     assert greedy_token_at_a_time(state, weights, SHORT, 10, step=step) == so.greedy_ids(model, SHORT, 10)
 
 
-def test_fused_schedule_in_a_graph():
+def test_folded_schedule_in_a_graph():
     model, state, weights = session(dv2.MEDIUM_LLAMA, 0, packed_embed=True)
-    eager = greedy_token_at_a_time(state, weights, SHORT, 12,
-                                   step=lambda s, w: dv2.greedy_decode(s, w, schedule="handover"))
+    step = lambda s, w: dv2.greedy_decode(s, w, schedule="fold_rms")  # noqa: E731
+    eager = greedy_token_at_a_time(state, weights, SHORT, 12, step=step)
     assert eager == so.greedy_ids(model, SHORT, 12)
     state.reset()
-    graph = dv2.capture_greedy(state, weights, warmup=2, schedule="handover")
+    graph = dv2.capture_greedy(state, weights, warmup=2, schedule="fold_rms")
     for rep in range(3):
         assert greedy_token_at_a_time(state, weights, SHORT, 12, step=graph) == eager, rep
         torch.cuda.synchronize()
 
 
-def test_fused_schedule_is_refused_when_it_does_not_apply():
-    _, state, weights = session(dv2.TINY_LLAMA, 0)          # dense embedding table
-    assert not dv2.can_fuse(weights)
+def test_long_cache_takes_the_split_attention(monkeypatch):
+    """Past ATTN_WG_MAX_SEQ the folded schedule uses the split kernel + merge; both give
+    the same ids."""
+    import deepfold_amd.decodev2.step as step_mod
+    model, state, weights = session(dv2.TINY_LLAMA, 0, packed_embed=True)
+    a = greedy_token_at_a_time(state, weights, SHORT, 10)
+    monkeypatch.setattr(step_mod, "ATTN_WG_MAX_SEQ", 0)
+    b = greedy_token_at_a_time(state, weights, SHORT, 10)
+    assert a == b == so.greedy_ids(model, SHORT, 10)
+
+
+def test_unknown_schedule_is_refused():
+    _, state, weights = session(dv2.TINY_LLAMA, 0)
     state.load_token(1)
-    with pytest.raises(ValueError):
-        dv2.forward_decode(state, weights, schedule="handover")
     with pytest.raises(ValueError):
         dv2.forward_decode(state, weights, schedule="nope")
