@@ -194,36 +194,44 @@ __global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flas
   float l = 0.f;
   float acc[8] = {};
   const size_t row_stride = static_cast<size_t>(a.n_kv) * hd;
-  // Two time steps per lane group and iteration: their loads are independent, so the
-  // trip count (and with it the exposed memory latency) halves.
+  // UNR time steps per lane group and iteration: their loads are independent and all in
+  // flight together, so the trip count (and with it the exposed memory latency) shrinks.
+  // The one-workgroup form has fewer wavefronts per head and unrolls further.
+  constexpr int UNR = INWG ? 8 : 2;
   const int stride = a.n_split * TPW;
-  for (int t0 = split; t0 < vl; t0 += 2 * stride) {
-    float kf[2][8], vf[2][8];
-    bool live[2];
+  for (int t0 = split; t0 < vl; t0 += UNR * stride) {
+    uint4 kraw[UNR], vraw[UNR];
+    bool live[UNR], cur[UNR];
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
+    for (int u = 0; u < UNR; ++u) {
       const int t = t0 + grp * a.n_split + u * stride;
       live[u] = t < vl;
-      const bool cur = fuse && t == pos;
-      if (live[u] && !cur) {
+      cur[u] = fuse && t == pos;
+      kraw[u] = make_uint4(0, 0, 0, 0);
+      vraw[u] = make_uint4(0, 0, 0, 0);
+      if (live[u] && !cur[u]) {
         const size_t off =
             static_cast<size_t>(t) * row_stride + static_cast<size_t>(kv_head) * hd + d0;
-        widen8(*reinterpret_cast<const uint4 *>(a.k_cache + off), kf[u]);
-        widen8(*reinterpret_cast<const uint4 *>(a.v_cache + off), vf[u]);
-      } else {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          kf[u][i] = cur ? kcur[i] : 0.f;
-          vf[u][i] = cur ? vcur[i] : 0.f;
-        }
+        kraw[u] = *reinterpret_cast<const uint4 *>(a.k_cache + off);
+        vraw[u] = *reinterpret_cast<const uint4 *>(a.v_cache + off);
       }
     }
 #pragma unroll
-    for (int u = 0; u < 2; ++u) {
+    for (int u = 0; u < UNR; ++u) {
+      float kf[8], vf[8];
+      widen8(kraw[u], kf);
+      widen8(vraw[u], vf);
+      if (cur[u]) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          kf[i] = kcur[i];
+          vf[i] = vcur[i];
+        }
+      }
       float dot = 0.f;
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        dot = fmaf(qf[i], kf[u][i], dot);
+        dot = fmaf(qf[i], kf[i], dot);
       }
       dot = group_sum<LPT>(dot) * a.scale;
       if (live[u]) {
@@ -233,7 +241,7 @@ __global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flas
         l = l * alpha + e;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-          acc[i] = acc[i] * alpha + e * vf[u][i];
+          acc[i] = acc[i] * alpha + e * vf[i];
         }
         m = m2;
       }
