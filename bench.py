@@ -32,6 +32,10 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes one GEMV launch of the primary workload moves, from FETCH_SIZE + WRITE_SIZE
+# hardware counters scaled by a plain device copy (profiles/gemv_stream_13824x5120_pmc.txt
+# has the runs and the arithmetic).  Hardware counters cannot be read inside this process.
+GEMV_TRAFFIC_BYTES = 37_827_972
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
 M, K = 13824, 5120  # headline layer: 14B gate/up projection
@@ -267,7 +271,10 @@ def main() -> int:
     ap.add_argument("--no-decode", action="store_true", help="skip the model decode leg")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill GEMM sweep")
     ap.add_argument("--decode-models", default="14b", help="comma list of 3b,14b,20b,32b")
-    ap.add_argument("--schedule", default=None, help="decode launch schedule: plain, fold_rms or handover")
+    ap.add_argument("--schedule", default=None, help="decode launch schedule: plain or fold_rms")
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
+                    help="first run four plain device copies of this size (a kernel of known "
+                         "traffic to scale hardware counters by)")
     ap.add_argument("--prompt", type=int, default=512)
     ap.add_argument("--new-tokens", type=int, default=256)
     args = ap.parse_args()
@@ -284,6 +291,14 @@ def main() -> int:
         print("bench.py: no GPU visible", file=sys.stderr)
         return 2
     torch.cuda.set_device(0)
+
+    if args.copy_calibration > 0:
+        src = torch.empty(args.copy_calibration << 20, dtype=torch.uint8, device="cuda").random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(4):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     ms, eager_ms, copies, by = bench_gemv(torch, nf4, args.steps, args.warmup, args.copies)
     achieved = by / (ms * 1e-3) / 1e9
@@ -312,7 +327,7 @@ def main() -> int:
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS,
-            "traffic": None,
+            "traffic": GEMV_TRAFFIC_BYTES if (M, K) == (13824, 5120) else None,
             "kernel": "gemv_stream",
             "algorithmic_bytes_per_launch": by,
         },
