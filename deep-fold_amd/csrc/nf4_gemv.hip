@@ -182,18 +182,31 @@ __device__ __forceinline__ void stage_x(const StreamArgs &a, uint4 *xs, float *p
   const bool vec_ok = (a.K & 7) == 0 && aligned16(a.x) &&
                       (a.rms_w == nullptr || aligned16(a.rms_w)) &&
                       nvec <= kKeep * static_cast<int>(blockDim.x);
-  for (int i = nvec + threadIdx.x; i < slots; i += blockDim.x) {
-    xs[i] = make_uint4(0, 0, 0, 0);  // slots past the last piece (partial tail step)
+  // Slots of the last tail step that no piece maps to (lanes past the end of the row).
+  {
+    const int full = nfull << 8;
+    const int tail_half = ((a.K_pad >> 5) & 63) * 2;
+    for (int i = full + threadIdx.x; i < slots; i += blockDim.x) {
+      const int h = (((i - full) >> 7) << 6) + (i & 63);
+      if (h >= tail_half) {
+        xs[i] = make_uint4(0, 0, 0, 0);
+      }
+    }
   }
   if (vec_ok) {
-    uint4 v[kKeep];
+    // x and the norm weights are requested together: one memory round trip, not two.
+    uint4 v[kKeep], g[kKeep];
     float ss = 0.f;
 #pragma unroll
     for (int j = 0; j < kKeep; ++j) {
       const int i = threadIdx.x + j * blockDim.x;
       v[j] = make_uint4(0, 0, 0, 0);
+      g[j] = make_uint4(0, 0, 0, 0);
       if (i * 8 < a.K) {
         v[j] = reinterpret_cast<const uint4 *>(a.x)[i];
+        if (a.rms_w != nullptr) {
+          g[j] = reinterpret_cast<const uint4 *>(a.rms_w)[i];
+        }
       }
     }
     float inv = 1.f;
@@ -216,9 +229,8 @@ __device__ __forceinline__ void stage_x(const StreamArgs &a, uint4 *xs, float *p
       if (i < nvec) {
         uint4 o = v[j];
         if (a.rms_w != nullptr && i * 8 < a.K) {
-          const uint4 g = reinterpret_cast<const uint4 *>(a.rms_w)[i];
           const uint32_t u[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
-          const uint32_t gw[4] = {g.x, g.y, g.z, g.w};
+          const uint32_t gw[4] = {g[j].x, g[j].y, g[j].z, g[j].w};
           uint32_t r[4];
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
@@ -371,12 +383,6 @@ __global__ __launch_bounds__(XLDS ? 1024 : 256) void gemv_stream(const StreamArg
   if (threadIdx.x < 16) {
     lds.lut[threadIdx.x] = bits_to_f32(kLutBits[threadIdx.x]);
   }
-  if constexpr (XLDS) {
-    stage_x(a, xs, lds.part);
-  } else {
-    __syncthreads();
-  }
-
   // Row groups (U rows each) are numbered through the segments.  Without the LDS
   // copy a wavefront takes exactly one group; with it the grid is one workgroup per
   // compute unit and a wavefront walks groups wave*grid + block, + grid*waves, ..,
@@ -387,6 +393,12 @@ __global__ __launch_bounds__(XLDS ? 1024 : 256) void gemv_stream(const StreamArg
   const int stride = XLDS ? static_cast<int>(gridDim.x) * waves : total;
   const size_t pstride = static_cast<size_t>(a.K_pad >> 1);
   const size_t sstride = static_cast<size_t>(a.K_pad >> 6);
+
+  if constexpr (XLDS) {
+    stage_x(a, xs, lds.part);
+  } else {
+    __syncthreads();
+  }
 
   for (int grp = first; grp < total; grp += stride) {
     int g = grp;

@@ -219,6 +219,27 @@ def test_gemv_fused_rms(m, k):
     check_linear(y, to_f32(y2), what="fused rms vs rms+gemv", ulps=1)
 
 
+@pytest.mark.parametrize("m,k", [(64, 512), (96, 1088), (40, 5120), (8, 13824)])
+def test_gemv_fused_rms_is_deterministic_with_a_partial_tail_step(m, k):
+    """K whose last step is only partly filled: the staged copy of x zero-fills the unused
+    slots and must never touch the used ones, whatever order the lanes run in."""
+    p, s, dp, ds = blobs(m, k, 77)
+    rng = np.random.default_rng(k)
+    x = bf16_tensor(oc.bf16_round(rng.standard_normal(k).astype(np.float32)))
+    g = bf16_tensor(oc.bf16_round(1 + 0.1 * rng.standard_normal(k).astype(np.float32)))
+    h = torch.empty(k, dtype=torch.bfloat16, device=DEV)
+    nf4.nf4_rms(x, g, h, 1e-6)
+    want = nf4.nf4_gemv(dp, ds, h, m, k, oc.k_pad(k))
+    first = None
+    for rep in range(25):
+        y = nf4.nf4_gemv(dp, ds, x, m, k, oc.k_pad(k), rms_w=g, rms_eps=1e-6)
+        bits = bf16_bits(y)
+        if first is None:
+            first = bits
+            check_linear(y, to_f32(want), what="fused rms, partial tail", ulps=1)
+        assert (bits == first).all(), rep
+
+
 def test_gemv_nan_behaviour():
     m, k = 256, 512
     p, s, dp, ds = blobs(m, k, 61)
