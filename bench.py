@@ -261,6 +261,50 @@ def cpu_baseline(m: int, k: int, budget_s: float = 12.0) -> dict:
     }
 
 
+def bench_ring(torch, nf4, n_matrices: int = 6, forwards: int = 10):
+    """Streaming variant (weights in pinned host memory, two device slots): a tape of
+    32B-architecture FFN matrices (27648x5120) through the ring, one GEMV each."""
+    from deepfold_amd import ring as rg
+
+    m, k = 27648, 5120
+    g = torch.Generator(device="cuda")
+    g.manual_seed(5)
+    tape = []
+    for i in range(n_matrices):
+        w = torch.randn((m, k), generator=g, device="cuda", dtype=torch.float32) * 0.02
+        packed, scale = nf4.nf4_quantize(w)
+        del w
+        tape.append(rg.StreamedMatrix.on_host(f"ffn{i}", rg.HostImage.from_blobs(packed.cpu(), scale.cpu(), k)))
+        del packed, scale
+    ring = rg.CopyRing(rg.SlotPair(tape[0].host_image.nbytes, "cuda"))
+    x = torch.randn(k, generator=g, device="cuda").to(torch.bfloat16)
+
+    def forward():
+        ring.arm(tape)
+        ring.prefetch()
+        for mat in tape:
+            rg.streamed_linear(ring, mat, x)
+        ring.prefetch_next()
+
+    forward()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(forwards):
+        forward()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / forwards
+    nbytes = n_matrices * tape[0].host_image.nbytes
+    return {
+        "workload": f"{n_matrices} x NF4 [{m},{k}] streamed from pinned host memory through 2 slots, "
+                    "one GEMV each",
+        "slot_bytes": tape[0].host_image.nbytes,
+        "ms_per_forward": dt * 1e3,
+        "h2d_gbps": nbytes / dt / 1e9,
+        "pinned": rg.is_pinned(tape[0].host_image.arena),
+        "copies_per_forward": n_matrices,
+    }
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -270,6 +314,7 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-decode", action="store_true", help="skip the model decode leg")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill GEMM sweep")
+    ap.add_argument("--no-ring", action="store_true", help="skip the host-streaming ring leg")
     ap.add_argument("--decode-models", default="14b", help="comma list of 3b,14b,20b,32b")
     ap.add_argument("--schedule", default=None, help="decode launch schedule: plain or fold_rms")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
@@ -337,6 +382,8 @@ def main() -> int:
                          for name in args.decode_models.split(",") if name.strip()]
     if not args.no_prefill:
         out["prefill"] = bench_prefill(torch, nf4)
+    if not args.no_ring:
+        out["ring"] = bench_ring(torch, nf4)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(M, K)
     print(json.dumps(out), flush=True)

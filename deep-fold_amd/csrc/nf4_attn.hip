@@ -145,7 +145,8 @@ template <int LPT, bool INWG>
 __global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flash(const AttnArgs a) {
   constexpr int TPW = kWave / LPT;  // time steps per wavefront iteration
   const int head = INWG ? static_cast<int>(blockIdx.x) : static_cast<int>(blockIdx.x) / a.n_split;
-  const int split = INWG ? static_cast<int>(threadIdx.x >> 6) : static_cast<int>(blockIdx.x) % a.n_split;
+  const int split = INWG ? __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6))
+                         : static_cast<int>(blockIdx.x) % a.n_split;
   const int lane = threadIdx.x & (kWave - 1);
   const int li = lane % LPT;  // which 8 dims of the head
   const int grp = lane / LPT; // which time step of the iteration
@@ -309,7 +310,8 @@ template <bool INWG>
 __global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flash_generic(
     const AttnArgs a) {
   const int head = INWG ? static_cast<int>(blockIdx.x) : static_cast<int>(blockIdx.x) / a.n_split;
-  const int split = INWG ? static_cast<int>(threadIdx.x >> 6) : static_cast<int>(blockIdx.x) % a.n_split;
+  const int split = INWG ? __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6))
+                         : static_cast<int>(blockIdx.x) % a.n_split;
   const int lane = threadIdx.x & (kWave - 1);
   const int hd = a.hd;
   const int half = hd / 2;

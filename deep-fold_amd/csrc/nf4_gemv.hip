@@ -377,7 +377,9 @@ __global__ __launch_bounds__(XLDS ? 1024 : 256) void gemv_stream(const StreamArg
   __shared__ GemvLds lds;
   constexpr int U = SWIGLU ? R / 2 : R;  // output rows per wavefront
   const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x >> 6;
+  // The wavefront index is the same in every lane: saying so keeps the row-group and
+  // segment arithmetic, and the kernel-argument reads indexed by it, on the scalar unit.
+  const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
   const int waves = blockDim.x >> 6;
 
   if (threadIdx.x < 16) {
@@ -390,7 +392,7 @@ __global__ __launch_bounds__(XLDS ? 1024 : 256) void gemv_stream(const StreamArg
   const int total = a.groups[0] + a.groups[1] + a.groups[2];
   const int first = XLDS ? wave * static_cast<int>(gridDim.x) + static_cast<int>(blockIdx.x)
                          : static_cast<int>(blockIdx.x) * waves + wave;
-  const int stride = XLDS ? static_cast<int>(gridDim.x) * waves : total;
+  const int stride = static_cast<int>(gridDim.x) * waves;
   const size_t pstride = static_cast<size_t>(a.K_pad >> 1);
   const size_t sstride = static_cast<size_t>(a.K_pad >> 6);
 
@@ -400,7 +402,7 @@ __global__ __launch_bounds__(XLDS ? 1024 : 256) void gemv_stream(const StreamArg
     __syncthreads();
   }
 
-  for (int grp = first; grp < total; grp += stride) {
+  auto run_group = [&](int grp) {
     int g = grp;
     int seg = 0;
     if (!SWIGLU) {
@@ -461,6 +463,15 @@ __global__ __launch_bounds__(XLDS ? 1024 : 256) void gemv_stream(const StreamArg
           y[r] = f32_to_bf16(v);
         }
       }
+    }
+  };
+  if constexpr (XLDS) {
+    for (int grp = first; grp < total; grp += stride) {
+      run_group(grp);
+    }
+  } else {
+    if (first < total) {
+      run_group(first);  // exactly one group per wavefront
     }
   }
 }
