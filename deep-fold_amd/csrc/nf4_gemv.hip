@@ -39,6 +39,7 @@ constexpr int kMaxWaves = 16;  // wavefronts per workgroup, upper bound
 struct GemvLds {
   float lut[16];
   float part[kMaxWaves];
+  float ksum[kMaxWaves][4];  // K-split: per-wavefront partial dot products of a row group
 };
 
 // lut is an LDS array of 16 floats; off is a byte offset in {0,4,..,60}.
@@ -121,6 +122,7 @@ struct StreamArgs {
   const uint16_t *add[3];  // optional residual / bias per segment, bf16 [M]
   int M[3];
   int groups[3];  // wavefront-sized row groups of each segment
+  int ksplit;     // 1, or > 1: the wavefronts of a workgroup share one row group along K
   // second matrix of a SwiGLU pair (segment 0 only)
   const uint8_t *packed2;
   const uint16_t *scale2;
@@ -312,55 +314,59 @@ template <int R, bool XL>
 __device__ __forceinline__ void rows_dot(const uint8_t *const (&prow)[R],
                                          const uint16_t *const (&srow)[R], const uint4 *x4,
                                          int K_pad, const float *lut, int lane,
-                                         float (&acc)[R]) {
+                                         float (&acc)[R], int t0 = 0, int tstep = 1) {
   const int chunks = K_pad >> 5;            // 16-byte chunks per row
   const int nfull = chunks >> 6;            // steps where all 64 lanes hold a chunk
   const int tail_half = (chunks & 63) * 2;  // 8-byte half chunks after them
+  const int nsteps = nfull + ((tail_half + kWave - 1) >> 6);
+  const int base_half = nfull << 7;         // first half chunk of the tail
 
-  for (int j = 0; j < nfull; ++j) {
-    const int c = (j << 6) + lane;
-    uint32_t w[R][4];
-    uint16_t sc[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const uint4 v = *(reinterpret_cast<const uint4 *>(prow[r]) + c);
-      w[r][0] = v.x;
-      w[r][1] = v.y;
-      w[r][2] = v.z;
-      w[r][3] = v.w;
-      sc[r] = srow[r][c >> 1];
-    }
-    const uint4 *xp = XL ? x4 + (j << 8) + lane : x4 + (c << 2);
-    constexpr int xq = XL ? 64 : 1;
-    const uint4 x0 = xp[0], x1 = xp[xq], x2 = xp[2 * xq], x3 = xp[3 * xq];
-    float xf[32];
-    widen8(x0, xf);
-    widen8(x1, xf + 8);
-    widen8(x2, xf + 16);
-    widen8(x3, xf + 24);
-    rows_step<R, 4>(w, xf, sc, lut, acc);
-  }
-
-  const int base_half = nfull << 7;  // first half chunk of the tail
-  for (int h0 = 0; h0 < tail_half; h0 += kWave) {
-    const int h = h0 + lane;
-    if (h < tail_half) {
-      const int hc = base_half + h;  // half-chunk index in the row: 16 weights
-      uint32_t w[R][2];
+  // Steps t0, t0 + tstep, ..: all of them for a wavefront that owns its rows, every
+  // tstep-th one when the wavefronts of a workgroup share a row group along K.
+  for (int t = t0; t < nsteps; t += tstep) {
+    if (t < nfull) {
+      const int c = (t << 6) + lane;
+      uint32_t w[R][4];
       uint16_t sc[R];
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        const uint2 v = *(reinterpret_cast<const uint2 *>(prow[r]) + hc);
+        const uint4 v = *(reinterpret_cast<const uint4 *>(prow[r]) + c);
         w[r][0] = v.x;
         w[r][1] = v.y;
-        sc[r] = srow[r][hc >> 2];
+        w[r][2] = v.z;
+        w[r][3] = v.w;
+        sc[r] = srow[r][c >> 1];
       }
-      const uint4 *xp = XL ? x4 + (nfull << 8) + ((h0 >> 6) << 7) + lane : x4 + (hc << 1);
-      const uint4 x0 = xp[0], x1 = xp[XL ? 64 : 1];
-      float xf[16];
+      const uint4 *xp = XL ? x4 + (t << 8) + lane : x4 + (c << 2);
+      constexpr int xq = XL ? 64 : 1;
+      const uint4 x0 = xp[0], x1 = xp[xq], x2 = xp[2 * xq], x3 = xp[3 * xq];
+      float xf[32];
       widen8(x0, xf);
       widen8(x1, xf + 8);
-      rows_step<R, 2>(w, xf, sc, lut, acc);
+      widen8(x2, xf + 16);
+      widen8(x3, xf + 24);
+      rows_step<R, 4>(w, xf, sc, lut, acc);
+    } else {
+      const int h0 = (t - nfull) << 6;
+      const int h = h0 + lane;
+      if (h < tail_half) {
+        const int hc = base_half + h;  // half-chunk index in the row: 16 weights
+        uint32_t w[R][2];
+        uint16_t sc[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          const uint2 v = *(reinterpret_cast<const uint2 *>(prow[r]) + hc);
+          w[r][0] = v.x;
+          w[r][1] = v.y;
+          sc[r] = srow[r][hc >> 2];
+        }
+        const uint4 *xp = XL ? x4 + (nfull << 8) + ((h0 >> 6) << 7) + lane : x4 + (hc << 1);
+        const uint4 x0 = xp[0], x1 = xp[XL ? 64 : 1];
+        float xf[16];
+        widen8(x0, xf);
+        widen8(x1, xf + 8);
+        rows_step<R, 2>(w, xf, sc, lut, acc);
+      }
     }
   }
 }
@@ -390,8 +396,10 @@ __global__ __launch_bounds__(XLDS ? 1024 : 256) void gemv_stream(const StreamArg
   // compute unit and a wavefront walks groups wave*grid + block, + grid*waves, ..,
   // so the copy is made once per compute unit and units stay balanced to one group.
   const int total = a.groups[0] + a.groups[1] + a.groups[2];
-  const int first = XLDS ? wave * static_cast<int>(gridDim.x) + static_cast<int>(blockIdx.x)
-                         : static_cast<int>(blockIdx.x) * waves + wave;
+  const bool ksplit = !XLDS && !SWIGLU && a.ksplit > 1;
+  const int first = XLDS     ? wave * static_cast<int>(gridDim.x) + static_cast<int>(blockIdx.x)
+                    : ksplit ? static_cast<int>(blockIdx.x)
+                             : static_cast<int>(blockIdx.x) * waves + wave;
   const int stride = static_cast<int>(gridDim.x) * waves;
   const size_t pstride = static_cast<size_t>(a.K_pad >> 1);
   const size_t sstride = static_cast<size_t>(a.K_pad >> 6);
@@ -435,7 +443,7 @@ __global__ __launch_bounds__(XLDS ? 1024 : 256) void gemv_stream(const StreamArg
       rows_dot<R, true>(prow, srow, static_cast<const uint4 *>(xs), a.K_pad, lds.lut, lane, acc);
     } else {
       rows_dot<R, false>(prow, srow, reinterpret_cast<const uint4 *>(a.x), a.K_pad, lds.lut, lane,
-                         acc);
+                         acc, ksplit ? wave : 0, ksplit ? waves : 1);
     }
 
     if constexpr (SWIGLU) {
@@ -451,11 +459,37 @@ __global__ __launch_bounds__(XLDS ? 1024 : 256) void gemv_stream(const StreamArg
     } else {
       const uint16_t *add = a.add[seg];
       uint16_t *y = a.y[seg];
+      float sums[U];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const float s = wave_sum(acc[u]);
+        sums[u] = wave_sum(acc[u]);
+      }
+      bool writer = true;
+      if (ksplit) {
+        // every wavefront of the workgroup holds a partial of the same rows: add them in
+        // wavefront order, wavefront 0 finishes
+        if (lane == 0) {
+#pragma unroll
+          for (int u = 0; u < U; ++u) {
+            lds.ksum[wave][u] = sums[u];
+          }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          float t = 0.f;
+          for (int w = 0; w < waves; ++w) {
+            t += lds.ksum[w][u];
+          }
+          sums[u] = t;
+        }
+        writer = wave == 0;
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const float s = sums[u];
         const int r = row0 + u;
-        if (lane == u && r < M) {
+        if (writer && lane == u && r < M) {
           float v = s;
           if (add != nullptr) {
             v += bf16_to_f32(add[r]);
@@ -603,7 +637,14 @@ int launch_stream(StreamArgs &a, int n_seg, hipStream_t st) {
     gemv_stream<R, SWIGLU, true><<<dim3(grid), dim3(kStagedThreads), dyn, st>>>(a);
   } else {
     const int waves = kThreads / kWave;
-    gemv_stream<R, SWIGLU, false><<<dim3((total + waves - 1) / waves), dim3(kThreads), 0, st>>>(a);
+    // Long rows and few of them (a down projection): a wavefront walking a whole row pays
+    // the memory latency once per step, so the four wavefronts of a workgroup split the
+    // steps of one row group instead.
+    const int nsteps = (a.K_pad + 2047) / 2048;
+    const bool split = !SWIGLU && nsteps >= 4 && total * 4 <= 16 * device_cu_count() * 4;
+    a.ksplit = split ? waves : 1;
+    const int grid = split ? total : (total + waves - 1) / waves;
+    gemv_stream<R, SWIGLU, false><<<dim3(grid), dim3(kThreads), 0, st>>>(a);
   }
   return launch_rc();
 }
