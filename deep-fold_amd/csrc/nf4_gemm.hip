@@ -9,15 +9,22 @@
 // tile with v_mfma_f32_32x32x16_bf16.  For that instruction lane l supplies
 // A[row l%32][k 8*(l/32) .. +8) and B[k 8*(l/32) .. +8)][col l%32], eight
 // consecutive k each, i.e. exactly one packed dword of codes on the A side.
-// A lane therefore loads 16 bytes (32 codes) of its own row per 64-wide K
-// step, rebuilds bf16(LUT*scale) pairs in registers and feeds four MFMAs;
-// lanes l and l+32 read adjacent 16-byte pieces of the same row.
 //
-// The activation tile [BK=256, N] is staged once per workgroup in LDS,
-// transposed to [32][BK+8] bf16 (token-major, padded so the 16-byte B reads of
-// 32 lanes fall in distinct banks), and shared by the four wavefronts.
-// Columns >= N and rows >= K are zero-filled, so padding codes and the unused
-// MFMA columns contribute nothing.
+// Weights.  The MFMA layout wants 32 different rows per instruction, which read
+// straight from global memory would be a 64-line gather.  Instead a wavefront
+// fetches its 32 rows x 128 bytes of a K tile with four fully coalesced loads
+// (eight rows of one 128-byte line each), one tile ahead of the arithmetic, and
+// passes them through a private LDS area (row stride 144 bytes, conflict-free for
+// the 16-byte reads); the group scales of the tile travel the same way.  A lane
+// then takes 16 bytes (32 codes) of its row per 64-wide K step, rebuilds
+// bf16(LUT*scale) in registers (one byte-select AND and one LDS lookup per code,
+// the 16 levels at LDS address 0) and feeds four MFMAs.
+//
+// Activations.  The tile [BK=256, N] is contiguous in x; every thread fetches its
+// 16-byte vectors of the next tile while the current one is multiplied, then
+// scatters them into LDS transposed to [32][BK+8] bf16 (token-major, padded so the
+// 16-byte B reads of 32 lanes fall in distinct banks).  Columns >= N and rows >= K
+// are zero, so padding codes and unused MFMA columns contribute nothing.
 //
 // Split-K over grid.y writes fp32 partials [split][M][N] to the caller's
 // workspace; a second kernel adds them in split order (deterministic) and
@@ -47,10 +54,21 @@ constexpr int kPlanMaxN = 64;
 constexpr int kBM = 128;      // rows per workgroup
 constexpr int kBK = 256;      // K per staged activation tile
 constexpr int kBN = 32;       // token columns of the MFMA tile
-constexpr int kGemmBlock = 256;
+// Wavefront groups of a workgroup that take alternate K tiles and add their results
+// through LDS.  Two groups were measured slower than one at the 14B shapes (72 KB of LDS
+// leaves two workgroups per compute unit and the grid no longer fits one round).
+constexpr int kKHalves = 1;
+constexpr int kGroupThreads = 256;                    // four wavefronts x 32 rows
+constexpr int kGemmBlock = kKHalves * kGroupThreads;
 constexpr int kXPad = 8;      // bf16 elements of row padding in LDS
 constexpr int kXStride = kBK + kXPad;
-constexpr int kGemmLds = kBN * kXStride * 2;
+constexpr int kWRow = kBK / 2 + 16;             // bytes of one staged weight row (padded)
+constexpr int kWStage = 32 * kWRow;             // bytes of a wavefront's weight area
+constexpr int kGroupsPerTile = kBK / 64;
+// codebook + activation tile + per-wavefront weight and scale areas (= sizeof(GemmLds))
+constexpr int kGemmWaves = kGemmBlock / 64;
+constexpr int kGemmLds = 64 + kKHalves * kBN * kXStride * 2 + kGemmWaves * kWStage +
+                         kGemmWaves * 32 * kGroupsPerTile * 2;
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -91,16 +109,21 @@ int resolved_one_wave() {
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
-// split so that grid_x * split reaches two workgroups per compute unit, capped
-// at the number of K tiles; split is recomputed from tiles_per_split so the
+// split so that grid_x * split reaches three workgroups per compute unit, capped at
+// kMaxAutoSplit (more splits cost more in fp32 partials than they win in occupancy)
+// and at the number of K tiles; split is recomputed from tiles_per_split so the
 // pair always agrees with what the kernel indexes
 // (gpu/nf4/nf4_gemm.cu:1526-1543).
+constexpr int kMaxAutoSplit = 8;
+
 void pick_split(int grid_x, int n_ktiles, int have_ws, int *split, int *tiles_per_split) {
   const Tuning &t = tuning();
   int want = 1;
   if (have_ws) {
-    const int target = resolved_one_wave() * 2;
-    want = t.split_k > 0 ? t.split_k : ceil_div(target, grid_x);
+    // three workgroups of four wavefronts per compute unit keep its SIMDs busy through the
+    // LDS and MFMA latencies of a tile (measured: 2 is 10-15 % slower, 4 no faster)
+    const int target = resolved_one_wave() * 3;
+    want = t.split_k > 0 ? t.split_k : std::min(kMaxAutoSplit, ceil_div(target, grid_x));
   }
   want = std::max(1, std::min(want, n_ktiles));
   const int tps = ceil_div(n_ktiles, want);
@@ -162,107 +185,242 @@ int check_args(const chr_nf4_dev_t *w, int32_t N, bool need_ptrs, chr_nf4_dev_t 
   return 0;
 }
 
-// Stage x[k0 .. k0+kBK) x [0, N) into LDS as xs[n][k - k0] (bf16), zero where
-// k >= K or n >= N.  x is [K, N] row-major.
-__device__ __forceinline__ void stage_x(const uint16_t *__restrict__ x, uint16_t *xs, int k0,
-                                        int K, int N) {
-  // 256 threads walk (k, n) with n fastest: consecutive threads read
-  // consecutive global elements.
-  for (int i = threadIdx.x; i < kBK * kBN; i += kGemmBlock) {
-    const int kk = i / kBN;
-    const int n = i - kk * kBN;
-    const int k = k0 + kk;
-    uint16_t v = 0;
-    if (n < N && k < K) {
-      v = x[static_cast<size_t>(k) * N + n];
+struct GemmLds {
+  float lut[16];                                  // at LDS address 0 (lookup8)
+  __attribute__((aligned(16))) uint16_t xs[kKHalves][kBN * kXStride];
+  __attribute__((aligned(16))) uint8_t w[kGemmWaves][kWStage];
+  uint16_t sc[kGemmWaves][32 * kGroupsPerTile];
+};
+static_assert(sizeof(GemmLds) == kGemmLds, "the planner reports this size");
+static_assert(kKHalves == 1 || kKHalves * kBN * kXStride * 2 >= 4 * 32 * 32 * 4,
+              "the final reduction reuses xs");
+
+// Activation vectors of one K tile held by a thread between fetch and scatter.  The tile
+// x[k0 .. k0+kBK) x [0, N) is kBK*N contiguous bf16; vector v of a thread holds flat
+// elements 8v .. 8v+7, element f being (k0 + f / N, f % N).
+struct XRegs {
+  uint32_t d[16];  // up to four 16-byte vectors (N = 32), as plain dwords
+};
+
+template <bool VEC>
+__device__ __forceinline__ void fetch_x(XRegs &r, const uint16_t *__restrict__ x, int k0, int K,
+                                        int N, int tid) {
+  const int n_elem = min(kBK, K - k0) * N;  // valid elements of the tile (rows >= K are zero)
+  const uint16_t *base = x + static_cast<size_t>(k0) * N;
+  if constexpr (VEC) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int v = tid + j * kGroupThreads;
+      uint4 t = make_uint4(0, 0, 0, 0);
+      if (v * 8 < n_elem) {  // N % 8 == 0 here, so a vector never straddles the end
+        t = *reinterpret_cast<const uint4 *>(base + v * 8);
+      }
+      r.d[4 * j + 0] = t.x;
+      r.d[4 * j + 1] = t.y;
+      r.d[4 * j + 2] = t.z;
+      r.d[4 * j + 3] = t.w;
     }
-    xs[n * kXStride + kk] = v;
+  } else {
+    (void)r;
   }
 }
 
-// Vector variant for N == 32 with a 16-byte aligned x: one thread moves eight
-// consecutive tokens of one k.
-__device__ __forceinline__ void stage_x_n32(const uint16_t *__restrict__ x, uint16_t *xs, int k0,
-                                            int K) {
-  for (int i = threadIdx.x; i < kBK * 4; i += kGemmBlock) {
-    const int kk = i >> 2;
-    const int n0 = (i & 3) * 8;
-    const int k = k0 + kk;
-    uint4 v = make_uint4(0, 0, 0, 0);
-    if (k < K) {
-      v = *reinterpret_cast<const uint4 *>(x + static_cast<size_t>(k) * 32 + n0);
-    }
-    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+template <bool VEC>
+__device__ __forceinline__ void scatter_x(const XRegs &r, const uint16_t *__restrict__ x,
+                                          uint16_t *xs, int k0, int K, int N, int tid) {
+  if constexpr (VEC) {
+    const int shift = N == 32 ? 5 : (N == 16 ? 4 : 3);  // VEC: N in {8, 16, 32}
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      xs[(n0 + 2 * j) * kXStride + kk] = static_cast<uint16_t>(w[j] & 0xFFFFu);
-      xs[(n0 + 2 * j + 1) * kXStride + kk] = static_cast<uint16_t>(w[j] >> 16);
+      const int v = tid + j * kGroupThreads;
+      if (v * 8 < kBK * N) {
+        const int f = v * 8;
+        const int kk = f >> shift;
+        const int n0 = f & (N - 1);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const uint32_t w = r.d[4 * j + e];
+          xs[(n0 + 2 * e) * kXStride + kk] = static_cast<uint16_t>(w & 0xFFFFu);
+          xs[(n0 + 2 * e + 1) * kXStride + kk] = static_cast<uint16_t>(w >> 16);
+        }
+      }
+    }
+  } else {
+    // any N, any alignment: element by element
+    for (int i = tid; i < kBK * N; i += kGroupThreads) {
+      const int kk = i / N;
+      const int n = i - kk * N;
+      const int k = k0 + kk;
+      xs[n * kXStride + kk] = k < K ? x[static_cast<size_t>(k) * N + n] : static_cast<uint16_t>(0);
     }
   }
+}
+
+// The 32 rows x 128 bytes of one K tile that a wavefront multiplies, as fetched: load j
+// covers rows 8j .. 8j+7, lane l the 16 bytes at offset 16*(l%8) of row 8j + l/8.
+struct WRegs {
+  uint32_t d[16];
+  uint32_t sc;  // two adjacent group scales of row l/2 (groups 2*(l%2), +1 of the tile)
+};
+
+__device__ __forceinline__ void fetch_w(WRegs &r, const uint8_t *__restrict__ packed,
+                                        const uint16_t *__restrict__ scale, int row_base, int M,
+                                        int K_pad, int k0, int lane) {
+  const int row_bytes = K_pad >> 1;
+  const int col = (k0 >> 1) + ((lane & 7) << 4);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int row = min(row_base + 8 * j + (lane >> 3), M - 1);
+    uint4 t = make_uint4(0x77777777u, 0x77777777u, 0x77777777u, 0x77777777u);
+    if (col < row_bytes) {
+      t = *reinterpret_cast<const uint4 *>(packed + static_cast<size_t>(row) * row_bytes + col);
+    }
+    r.d[4 * j + 0] = t.x;
+    r.d[4 * j + 1] = t.y;
+    r.d[4 * j + 2] = t.z;
+    r.d[4 * j + 3] = t.w;
+  }
+  const int srow = min(row_base + (lane >> 1), M - 1);
+  const int g = (k0 >> 6) + ((lane & 1) << 1);
+  const int groups = K_pad >> 6;
+  const uint16_t *sp = scale + static_cast<size_t>(srow) * groups;
+  const uint32_t s0 = g < groups ? sp[g] : 0u;
+  const uint32_t s1 = g + 1 < groups ? sp[g + 1] : 0u;
+  r.sc = s0 | (s1 << 16);
+}
+
+__device__ __forceinline__ void stash_w(const WRegs &r, uint8_t *wst, uint16_t *sst, int lane) {
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    uint8_t *dst = wst + (8 * j + (lane >> 3)) * kWRow + ((lane & 7) << 4);
+    *reinterpret_cast<uint4 *>(dst) =
+        make_uint4(r.d[4 * j + 0], r.d[4 * j + 1], r.d[4 * j + 2], r.d[4 * j + 3]);
+  }
+  *reinterpret_cast<uint32_t *>(sst + (lane >> 1) * kGroupsPerTile + ((lane & 1) << 1)) = r.sc;
 }
 
 __device__ __forceinline__ bf16x8 dequant8(uint32_t w, float s, const float *lut) {
+  const Levels8 v = lookup8(w, lut);
   bf16x8 a;
 #pragma unroll
   for (int j = 0; j < 8; ++j) {
-    a[j] = static_cast<__bf16>(lut[(w >> (4 * j)) & 0xFu] * s);
+    a[j] = static_cast<__bf16>(v.l[j] * s);
   }
   return a;
 }
 
+template <bool VEC>
 __global__ __launch_bounds__(kGemmBlock) void gemm_mfma(const uint8_t *__restrict__ packed,
                                                         const uint16_t *__restrict__ scale,
                                                         const uint16_t *__restrict__ x,
                                                         uint16_t *__restrict__ y,
                                                         float *__restrict__ partial, int M, int K,
                                                         int K_pad, int N, int n_ktiles,
-                                                        int tiles_per_split, int x_vec) {
-  __shared__ float lut[16];
-  __shared__ __attribute__((aligned(16))) uint16_t xs[kBN * kXStride];
+                                                        int tiles_per_split) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  GemmLds &lds = *reinterpret_cast<GemmLds *>(lds_raw);
   if (threadIdx.x < 16) {
-    lut[threadIdx.x] = bits_to_f32(kLutBits[threadIdx.x]);
+    lds.lut[threadIdx.x] = bits_to_f32(kLutBits[threadIdx.x]);
+  }
+  // columns >= N of the activation tiles are never written by the scatter: zero them once
+  for (int i = threadIdx.x; i < kKHalves * kBN * kXStride / 2; i += kGemmBlock) {
+    reinterpret_cast<uint32_t *>(&lds.xs[0][0])[i] = 0u;
   }
   const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x >> 6;
-  const int row = blockIdx.x * kBM + wave * 32 + (lane & 31);
-  const int rowc = min(row, M - 1);  // clamp: rows past M compute but never store
-  const int khalf = lane >> 5;       // which 32-wide half of a 64-wide K step
-  const uint8_t *prow = packed + static_cast<size_t>(rowc) * (K_pad >> 1);
-  const uint16_t *srow = scale + static_cast<size_t>(rowc) * (K_pad >> 6);
+  const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
+  const int rt = wave & 3;        // which 32 rows of the workgroup's 128
+  const int kgrp = wave >> 2;     // which K tiles: tile0 + kgrp, + 2, ..
+  const int tid = threadIdx.x & (kGroupThreads - 1);
+  const int row_base = blockIdx.x * kBM + rt * 32;
+  const int khalf = lane >> 5;  // which 32-wide half of a 64-wide K step
+  uint8_t *wst = lds.w[wave];
+  uint16_t *sst = lds.sc[wave];
+  uint16_t *xs = lds.xs[kgrp];
 
   const int tile0 = blockIdx.y * tiles_per_split;
   const int tile1 = min(tile0 + tiles_per_split, n_ktiles);
 
   f32x16 acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   const uint16_t *xl = xs + (lane & 31) * kXStride + khalf * 32;
+  const uint8_t *wl = wst + (lane & 31) * kWRow + khalf * 16;
+  const uint16_t *sl = sst + (lane & 31) * kGroupsPerTile;
 
-  for (int tile = tile0; tile < tile1; ++tile) {
+  WRegs wr;
+  XRegs xr;
+  if (tile0 + kgrp < tile1) {
+    fetch_w(wr, packed, scale, row_base, M, K_pad, (tile0 + kgrp) * kBK, lane);
+    fetch_x<VEC>(xr, x, (tile0 + kgrp) * kBK, K, N, tid);
+  }
+  // Both wavefront groups run the same number of rounds (the barriers are workgroup-wide);
+  // a group without a tile in the last round only keeps step.
+  for (int base = tile0; base < tile1; base += kKHalves) {
+    const int tile = base + kgrp;
+    const bool mine = tile < tile1;
     const int k0 = tile * kBK;
-    __syncthreads();  // previous tile's readers are done (and the LUT is visible)
-    if (x_vec) {
-      stage_x_n32(x, xs, k0, K);
-    } else {
-      stage_x(x, xs, k0, K, N);
+    __syncthreads();  // the previous round's readers are done (and the LUT / zero fill is visible)
+    if (mine) {
+      scatter_x<VEC>(xr, x, xs, k0, K, N, tid);
+      stash_w(wr, wst, sst, lane);
     }
     __syncthreads();
+    if (!mine) {
+      continue;
+    }
+    if (tile + kKHalves < tile1) {  // next tile's trip to memory overlaps this tile's arithmetic
+      fetch_w(wr, packed, scale, row_base, M, K_pad, k0 + kKHalves * kBK, lane);
+      fetch_x<VEC>(xr, x, k0 + kKHalves * kBK, K, N, tid);
+    }
     const int kend = min(kBK, K_pad - k0);
     for (int kk = 0; kk < kend; kk += 64) {
-      const int k = k0 + kk + khalf * 32;
-      const uint4 pk = *reinterpret_cast<const uint4 *>(prow + (k >> 1));
-      const float s = f16_to_f32(srow[k >> 6]);
+      const uint4 pk = *reinterpret_cast<const uint4 *>(wl + (kk >> 1));
+      const float s = f16_to_f32(sl[kk >> 6]);
       const uint32_t w[4] = {pk.x, pk.y, pk.z, pk.w};
+      // all 32 lookups and the four B reads of the step are issued before the first
+      // conversion, so their LDS latency is paid once per step
+      Levels8 lv[4];
+      bf16x8 b[4];
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
-        const bf16x8 a = dequant8(w[t], s, lut);
-        const bf16x8 b = *reinterpret_cast<const bf16x8 *>(xl + kk + 8 * t);
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
+        lv[t] = lookup8(w[t], lds.lut);
+        b[t] = *reinterpret_cast<const bf16x8 *>(xl + kk + 8 * t);
       }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        bf16x8 a;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          a[j] = static_cast<__bf16>(lv[t].l[j] * s);
+        }
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b[t], acc, 0, 0, 0);
+      }
+    }
+  }
+
+  if constexpr (kKHalves > 1) {
+    // Add the second group's tile to the first's through LDS (the activation area is free
+    // now), in a fixed order, then the first group stores.
+    __syncthreads();
+    float *red = reinterpret_cast<float *>(&lds.xs[0][0]) + rt * (16 * kWave);
+    if (kgrp == 1) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        red[i * kWave + lane] = acc[i];
+      }
+    }
+    __syncthreads();
+    if (kgrp != 0) {
+      return;
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      acc[i] += red[i * kWave + lane];
     }
   }
 
   // acc[i] is C[row 8*(i/4) + 4*(lane/32) + i%4][col lane%32] of the 32x32 tile.
   const int n = lane & 31;
-  const int rbase = blockIdx.x * kBM + wave * 32 + 4 * (lane >> 5);
+  const int rbase = row_base + 4 * (lane >> 5);
   if (n < N) {
     if (partial == nullptr) {
 #pragma unroll
@@ -298,6 +456,24 @@ __global__ __launch_bounds__(256) void reduce_splitk(const float *__restrict__ p
     s += partial[static_cast<size_t>(j) * rows + i];
   }
   y[i] = f32_to_bf16(s);
+}
+
+// The kernels use more than the default 64 KB of LDS: raise the limit once per process
+// (on the first launch, which a caller warming up before graph capture makes eagerly).
+int gemm_lds_ready() {
+  static const int rc = [] {
+    const void *kernels[2] = {reinterpret_cast<const void *>(gemm_mfma<true>),
+                              reinterpret_cast<const void *>(gemm_mfma<false>)};
+    for (const void *k : kernels) {
+      if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLds) !=
+          hipSuccess) {
+        (void)hipGetLastError();
+        return -6;
+      }
+    }
+    return 0;
+  }();
+  return rc;
 }
 
 }  // namespace
@@ -356,11 +532,20 @@ extern "C" int chr_nf4_gemm_ws_max(const chr_nf4_dev_t *w, const void *x, void *
   float *partial = p.grid_y > 1 ? ws : nullptr;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const dim3 grid(static_cast<unsigned>(p.grid_x), static_cast<unsigned>(p.grid_y));
-  const int x_vec = (N == 32) ? 1 : 0;
-  gemm_mfma<<<grid, dim3(kGemmBlock), 0, st>>>(h.packed, h.scale,
-                                               static_cast<const uint16_t *>(x),
-                                               static_cast<uint16_t *>(y), partial, h.M, h.K,
-                                               h.K_pad, N, p.n_ktiles, p.tiles_per_split, x_vec);
+  // 16-byte activation vectors need N in {8, 16, 32}; x is 16-byte aligned (checked above)
+  const bool vec = N == 8 || N == 16 || N == 32;
+  if (gemm_lds_ready() != 0) {
+    return -6;
+  }
+  if (vec) {
+    gemm_mfma<true><<<grid, dim3(kGemmBlock), kGemmLds, st>>>(
+        h.packed, h.scale, static_cast<const uint16_t *>(x), static_cast<uint16_t *>(y), partial,
+        h.M, h.K, h.K_pad, N, p.n_ktiles, p.tiles_per_split);
+  } else {
+    gemm_mfma<false><<<grid, dim3(kGemmBlock), kGemmLds, st>>>(
+        h.packed, h.scale, static_cast<const uint16_t *>(x), static_cast<uint16_t *>(y), partial,
+        h.M, h.K, h.K_pad, N, p.n_ktiles, p.tiles_per_split);
+  }
   if (partial != nullptr) {
     const int rows = h.M * N;
     reduce_splitk<<<dim3(static_cast<unsigned>(ceil_div(rows, 256))), dim3(256), 0, st>>>(

@@ -42,63 +42,6 @@ struct GemvLds {
   float ksum[kMaxWaves][4];  // K-split: per-wavefront partial dot products of a row group
 };
 
-// lut is an LDS array of 16 floats; off is a byte offset in {0,4,..,60}.
-__device__ __forceinline__ float lut_at(const float *lut, uint32_t off) {
-  return *reinterpret_cast<const float *>(reinterpret_cast<const char *>(lut) + off);
-}
-
-// (byte J of w) & mask in one VALU op: the sub-dword source select of gfx9
-// SDWA picks the byte, so no separate shift or bit-field extract is needed.
-template <int J>
-__device__ __forceinline__ uint32_t and_byte(uint32_t w, uint32_t mask) {
-  uint32_t r;
-  if constexpr (J == 0) {
-    asm("v_and_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_0 "
-        "src1_sel:DWORD"
-        : "=v"(r)
-        : "v"(w), "v"(mask));
-  } else if constexpr (J == 1) {
-    asm("v_and_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_1 "
-        "src1_sel:DWORD"
-        : "=v"(r)
-        : "v"(w), "v"(mask));
-  } else if constexpr (J == 2) {
-    asm("v_and_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_2 "
-        "src1_sel:DWORD"
-        : "=v"(r)
-        : "v"(w), "v"(mask));
-  } else {
-    asm("v_and_b32_sdwa %0, %1, %2 dst_sel:DWORD dst_unused:UNUSED_PAD src0_sel:BYTE_3 "
-        "src1_sel:DWORD"
-        : "=v"(r)
-        : "v"(w), "v"(mask));
-  }
-  return r;
-}
-
-// Eight codes of one dword -> eight codebook levels.  In (w << 2) byte j
-// carries 4*code(2j) in bits 2..5; in (w >> 2) byte j carries 4*code(2j+1)
-// there.  Masking a selected byte with 0x3C is the LDS byte offset of the level.
-struct Levels8 {
-  float l[8];
-};
-
-__device__ __forceinline__ Levels8 lookup8(uint32_t w, const float *lut) {
-  const uint32_t ev = w << 2;
-  const uint32_t od = w >> 2;
-  const uint32_t mask = 0x3Cu;
-  Levels8 r;
-  r.l[0] = lut_at(lut, and_byte<0>(ev, mask));
-  r.l[1] = lut_at(lut, and_byte<0>(od, mask));
-  r.l[2] = lut_at(lut, and_byte<1>(ev, mask));
-  r.l[3] = lut_at(lut, and_byte<1>(od, mask));
-  r.l[4] = lut_at(lut, and_byte<2>(ev, mask));
-  r.l[5] = lut_at(lut, and_byte<2>(od, mask));
-  r.l[6] = lut_at(lut, and_byte<3>(ev, mask));
-  r.l[7] = lut_at(lut, and_byte<3>(od, mask));
-  return r;
-}
-
 __device__ __forceinline__ float fma8(const Levels8 &v, const float *xf, float acc) {
 #pragma unroll
   for (int j = 0; j < 8; ++j) {

@@ -53,7 +53,10 @@ PLAN_MAX_N = 64
 _BM = 128
 _BK = 256
 _BLOCK = 256
-_X_LDS = 32 * (_BK + 8) * 2  # staged activation tile, bf16, padded rows
+_MAX_AUTO_SPLIT = 8
+# codebook, staged activation tile (bf16, padded rows), and per wavefront (4) a weight area
+# (32 rows of BK/2 + 16 bytes) and the tile's group scales
+_X_LDS = 64 + 32 * (_BK + 8) * 2 + 4 * 32 * (_BK // 2 + 16) + 4 * 32 * (_BK // 64) * 2
 
 _PATH_NAME = {GEMV: "gemv", PREFILL: "prefill", PREFILL_N32: "prefill_n32",
               PREFILL_N64: "prefill_n64"}
@@ -104,8 +107,8 @@ def _pick_split(grid_x: int, n_ktiles: int, have_ws: bool, force_split: int,
                 one_wave: int) -> tuple[int, int]:
     want = 1
     if have_ws:
-        target = max(1, int(one_wave) * 2)
-        want = force_split if force_split > 0 else _ceil_div(target, grid_x)
+        target = max(1, int(one_wave) * 3)
+        want = force_split if force_split > 0 else min(_MAX_AUTO_SPLIT, _ceil_div(target, grid_x))
     want = max(1, min(want, n_ktiles))
     tiles_per_split = _ceil_div(n_ktiles, want)
     return _ceil_div(n_ktiles, tiles_per_split), tiles_per_split
@@ -125,7 +128,7 @@ def plan(M: int, K: int, N: int = 1, *, K_pad: int | None = None, have_ws: bool 
         bm = 4 * gemv_rows_per_wavefront(M, gemv_rows)
         n_ktiles = _ceil_div(kp, 2048)
         grid_x = _ceil_div(M, bm)
-        lds = (16 + 16) * 4  # codebook + reduction partials
+        lds = (16 + 16 + 16 * 4) * 4  # codebook + reduction partials + K-split partials
         return Plan(GEMV, grid_x, 1, 256, bm, 2048, n_ktiles, n_ktiles, grid_x, lds, 0)
     path = PREFILL if N <= 16 else (PREFILL_N32 if N <= 32 else PREFILL_N64)
     grid_x = _ceil_div(M, _BM)
