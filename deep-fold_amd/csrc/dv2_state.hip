@@ -11,6 +11,9 @@
 
 namespace chr {
 
+int gemv_attn_entry(const chr_nf4_dev_t *w, const float *state, int n_q, int hd, int n_parts,
+                    void *y, const void *add, void *stream);
+
 namespace {
 
 constexpr int kBeginBlock = 1024;
@@ -193,6 +196,12 @@ extern "C" int chr_dv2_begin_step(const chr_nf4_dev_t *table, const void *token,
       static_cast<int32_t *>(valid_len), static_cast<uint16_t *>(x),
       static_cast<const uint16_t *>(norm_w), eps, static_cast<uint16_t *>(h));
   return launch_rc();
+}
+
+extern "C" int chr_dv2_gemv_attn(const chr_nf4_dev_t *w, const float *state, int32_t n_q,
+                                 int32_t hd, int32_t n_parts, void *y, const void *add,
+                                 void *stream) {
+  return gemv_attn_entry(w, state, n_q, hd, n_parts, y, add, stream);
 }
 
 extern "C" int chr_dv2_mark_written(const void *position, void *valid_len, void *stream) {

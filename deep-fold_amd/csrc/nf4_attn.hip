@@ -76,6 +76,11 @@ struct AttnArgs {
   int n_q, n_kv, hd, n_split, max_seq;
   float scale;
   uint16_t *out;  // merged heads, bf16 [n_q, hd]
+  // one-workgroup forms: n_parts workgroups per head (>= 1); with state != nullptr each
+  // leaves its unnormalised softmax state {m, l, 0, 0, o[hd]} at state[(head*n_parts+part)]
+  // for a later merge instead of writing out
+  int n_parts;
+  float *state;
 };
 
 constexpr int kMaxWgSplits = 16;  // wavefronts of a one-workgroup-per-head launch
@@ -88,7 +93,7 @@ constexpr int kMaxWgSplits = 16;  // wavefronts of a one-workgroup-per-head laun
 // sum over splits running in split order.
 __device__ __forceinline__ void merge_head(const float *m_s, const float *l_s, const float *o_s,
                                            uint16_t *out, int head, int hd, int n_split,
-                                           int lane) {
+                                           int lane, float *state = nullptr) {
   const float *mh = m_s + static_cast<size_t>(head) * n_split;
   const float *lh = l_s + static_cast<size_t>(head) * n_split;
   const float my_m = lane < n_split ? *(mh + lane) : kNegBig;
@@ -107,6 +112,10 @@ __device__ __forceinline__ void merge_head(const float *m_s, const float *l_s, c
   const float inv = l > 0.f ? 1.f / l : 0.f;
   const float *oh = o_s + static_cast<size_t>(head) * n_split * hd;
   uint16_t *dst = out + static_cast<size_t>(head) * hd;
+  if (state != nullptr && lane == 0) {
+    state[0] = m;
+    state[1] = l;
+  }
   // Every lane runs every iteration (the shuffles below read other lanes);
   // lanes past hd only skip the memory accesses.
   for (int d0 = 0; d0 < hd; d0 += kWave) {
@@ -130,7 +139,11 @@ __device__ __forceinline__ void merge_head(const float *m_s, const float *l_s, c
       acc += __shfl(my_w, s, kWave) * v;
     }
     if (on) {
-      dst[d] = f32_to_bf16(l > 0.f ? acc * inv : 0.f);
+      if (state != nullptr) {
+        state[4 + d] = acc;  // unnormalised: the later merge divides
+      } else {
+        dst[d] = f32_to_bf16(l > 0.f ? acc * inv : 0.f);
+      }
     }
   }
 }
@@ -144,9 +157,12 @@ __device__ __forceinline__ void merge_head(const float *m_s, const float *l_s, c
 template <int LPT, bool INWG>
 __global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flash(const AttnArgs a) {
   constexpr int TPW = kWave / LPT;  // time steps per wavefront iteration
-  const int head = INWG ? static_cast<int>(blockIdx.x) : static_cast<int>(blockIdx.x) / a.n_split;
-  const int split = INWG ? __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6))
-                         : static_cast<int>(blockIdx.x) % a.n_split;
+  const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
+  const int wg_waves = static_cast<int>(blockDim.x >> 6);
+  const int part = INWG ? static_cast<int>(blockIdx.x) % a.n_parts : 0;
+  const int head = INWG ? static_cast<int>(blockIdx.x) / a.n_parts
+                        : static_cast<int>(blockIdx.x) / a.n_split;
+  const int split = INWG ? part * wg_waves + wave : static_cast<int>(blockIdx.x) % a.n_split;
   const int lane = threadIdx.x & (kWave - 1);
   const int li = lane % LPT;  // which 8 dims of the head
   const int grp = lane / LPT; // which time step of the iteration
@@ -155,6 +171,39 @@ __global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flas
   const int n_rep = a.n_q / a.n_kv;
   const int kv_head = head / n_rep;
   const int vl = min(*a.valid_len, a.max_seq);
+
+  // The first block of cache rows is requested before anything else (RoPE tables, q, the
+  // current k/v): its trip to memory overlaps that prologue.  UNR time steps per lane group
+  // and iteration: their loads are independent and all in flight together, so the trip count
+  // (and with it the exposed memory latency) shrinks; the one-workgroup form has fewer
+  // wavefronts per head and unrolls further.
+  constexpr int UNR = INWG ? 4 : 2;
+  const int stride = a.n_split * TPW;
+  const size_t row_stride = static_cast<size_t>(a.n_kv) * hd;
+  // plain dwords: arrays of vector structs would not stay in registers
+  uint32_t kraw[UNR][4], vraw[UNR][4];
+  auto load_block = [&](int t0) {
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      const int t = t0 + grp * a.n_split + u * stride;
+      uint4 kv = make_uint4(0, 0, 0, 0), vv = make_uint4(0, 0, 0, 0);
+      if (t < vl) {  // the row at *position may be mid-write: it is replaced below
+        const size_t off =
+            static_cast<size_t>(t) * row_stride + static_cast<size_t>(kv_head) * hd + d0;
+        kv = *reinterpret_cast<const uint4 *>(a.k_cache + off);
+        vv = *reinterpret_cast<const uint4 *>(a.v_cache + off);
+      }
+      kraw[u][0] = kv.x;
+      kraw[u][1] = kv.y;
+      kraw[u][2] = kv.z;
+      kraw[u][3] = kv.w;
+      vraw[u][0] = vv.x;
+      vraw[u][1] = vv.y;
+      vraw[u][2] = vv.z;
+      vraw[u][3] = vv.w;
+    }
+  };
+  load_block(split);
 
   float qf[8];
   float kcur[8];
@@ -194,34 +243,22 @@ __global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flas
   float m = kNegBig;
   float l = 0.f;
   float acc[8] = {};
-  const size_t row_stride = static_cast<size_t>(a.n_kv) * hd;
-  // UNR time steps per lane group and iteration: their loads are independent and all in
-  // flight together, so the trip count (and with it the exposed memory latency) shrinks.
-  // The one-workgroup form has fewer wavefronts per head and unrolls further.
-  constexpr int UNR = INWG ? 8 : 2;
-  const int stride = a.n_split * TPW;
   for (int t0 = split; t0 < vl; t0 += UNR * stride) {
-    uint4 kraw[UNR], vraw[UNR];
+    if (t0 != split) {
+      load_block(t0);
+    }
     bool live[UNR], cur[UNR];
 #pragma unroll
     for (int u = 0; u < UNR; ++u) {
       const int t = t0 + grp * a.n_split + u * stride;
       live[u] = t < vl;
       cur[u] = fuse && t == pos;
-      kraw[u] = make_uint4(0, 0, 0, 0);
-      vraw[u] = make_uint4(0, 0, 0, 0);
-      if (live[u] && !cur[u]) {
-        const size_t off =
-            static_cast<size_t>(t) * row_stride + static_cast<size_t>(kv_head) * hd + d0;
-        kraw[u] = *reinterpret_cast<const uint4 *>(a.k_cache + off);
-        vraw[u] = *reinterpret_cast<const uint4 *>(a.v_cache + off);
-      }
     }
 #pragma unroll
     for (int u = 0; u < UNR; ++u) {
       float kf[8], vf[8];
-      widen8(kraw[u], kf);
-      widen8(vraw[u], vf);
+      widen8(make_uint4(kraw[u][0], kraw[u][1], kraw[u][2], kraw[u][3]), kf);
+      widen8(make_uint4(vraw[u][0], vraw[u][1], vraw[u][2], vraw[u][3]), vf);
       if (cur[u]) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
@@ -278,17 +315,20 @@ __global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flas
     __shared__ float sm[kMaxWgSplits], sl[kMaxWgSplits];
     __shared__ __align__(16) float so[kMaxWgSplits * 8 * LPT];
     if (lane == 0) {
-      sm[split] = m;
-      sl[split] = l;
+      sm[wave] = m;
+      sl[wave] = l;
     }
     if (grp == 0) {
-      float *oh = so + split * hd + d0;
+      float *oh = so + wave * hd + d0;
       *reinterpret_cast<float4 *>(oh) = make_float4(acc[0], acc[1], acc[2], acc[3]);
       *reinterpret_cast<float4 *>(oh + 4) = make_float4(acc[4], acc[5], acc[6], acc[7]);
     }
     __syncthreads();
-    if (split == 0) {
-      merge_head(sm, sl, so, a.out + static_cast<size_t>(head) * hd, 0, hd, a.n_split, lane);
+    if (wave == 0) {
+      float *st = a.state == nullptr
+                      ? nullptr
+                      : a.state + (static_cast<size_t>(head) * a.n_parts + part) * (hd + 4);
+      merge_head(sm, sl, so, a.out + static_cast<size_t>(head) * hd, 0, hd, wg_waves, lane, st);
     }
   } else {
     const size_t slot = static_cast<size_t>(head) * a.n_split + split;
@@ -309,9 +349,12 @@ __global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flas
 template <bool INWG>
 __global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flash_generic(
     const AttnArgs a) {
-  const int head = INWG ? static_cast<int>(blockIdx.x) : static_cast<int>(blockIdx.x) / a.n_split;
-  const int split = INWG ? __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6))
-                         : static_cast<int>(blockIdx.x) % a.n_split;
+  const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
+  const int wg_waves = static_cast<int>(blockDim.x >> 6);
+  const int part = INWG ? static_cast<int>(blockIdx.x) % a.n_parts : 0;
+  const int head = INWG ? static_cast<int>(blockIdx.x) / a.n_parts
+                        : static_cast<int>(blockIdx.x) / a.n_split;
+  const int split = INWG ? part * wg_waves + wave : static_cast<int>(blockIdx.x) % a.n_split;
   const int lane = threadIdx.x & (kWave - 1);
   const int hd = a.hd;
   const int half = hd / 2;
@@ -403,19 +446,22 @@ __global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flas
     __shared__ float sm[kMaxWgSplits], sl[kMaxWgSplits];
     __shared__ float so[kMaxWgSplits * 256];
     if (lane == 0) {
-      sm[split] = m;
-      sl[split] = l;
+      sm[wave] = m;
+      sl[wave] = l;
     }
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int d = lane + 64 * i;
       if (d < hd) {
-        so[split * hd + d] = acc[i];
+        so[wave * hd + d] = acc[i];
       }
     }
     __syncthreads();
-    if (split == 0) {
-      merge_head(sm, sl, so, a.out + static_cast<size_t>(head) * hd, 0, hd, a.n_split, lane);
+    if (wave == 0) {
+      float *st = a.state == nullptr
+                      ? nullptr
+                      : a.state + (static_cast<size_t>(head) * a.n_parts + part) * (hd + 4);
+      merge_head(sm, sl, so, a.out + static_cast<size_t>(head) * hd, 0, hd, wg_waves, lane, st);
     }
   } else {
     const size_t slot = static_cast<size_t>(head) * a.n_split + split;
@@ -522,8 +568,9 @@ namespace {
 
 template <bool INWG>
 void launch_flash(const AttnArgs &a, bool vec_ok, hipStream_t st) {
-  const dim3 grid(static_cast<unsigned>(INWG ? a.n_q : a.n_q * a.n_split));
-  const dim3 block(static_cast<unsigned>(INWG ? kWave * a.n_split : kWave));
+  // one-workgroup forms: a.n_split counts all wavefronts of a head (parts x wavefronts)
+  const dim3 grid(static_cast<unsigned>(INWG ? a.n_q * a.n_parts : a.n_q * a.n_split));
+  const dim3 block(static_cast<unsigned>(INWG ? kWave * (a.n_split / a.n_parts) : kWave));
   if (vec_ok && a.hd == 128) {
     attn_flash<16, INWG><<<grid, block, 0, st>>>(a);
   } else if (vec_ok && a.hd == 64) {
@@ -539,32 +586,44 @@ void launch_flash(const AttnArgs &a, bool vec_ok, hipStream_t st) {
   }
 }
 
-// ws == nullptr selects the one-workgroup-per-head form (n_split wavefronts, <= 16).
+// mode 0: one wavefront per (head, split) + merge launch (ws = partials).
+// mode 1: one workgroup of n_split wavefronts per head, merged in LDS, writes out.
+// mode 2: n_parts workgroups of n_split wavefronts per head; each leaves its softmax state
+//         in ws (n_q * n_parts * (hd + 4) floats) for the consumer to merge.
 int attn_common(const void *q, const void *k, const void *v, void *out, const void *valid_len,
                 float *ws, int32_t n_q, int32_t n_kv, int32_t hd, int32_t n_split, float scale,
                 void *stream, const void *k_act, const void *v_act, const void *cos,
-                const void *sin, const void *position, int32_t max_seq, bool in_wg) {
-  if (q == nullptr || k == nullptr || v == nullptr || out == nullptr || valid_len == nullptr ||
-      (!in_wg && ws == nullptr)) {
+                const void *sin, const void *position, int32_t max_seq, int mode,
+                int32_t n_parts) {
+  if (q == nullptr || k == nullptr || v == nullptr || valid_len == nullptr ||
+      (mode != 2 && out == nullptr) || (mode != 1 && ws == nullptr)) {
     return -1;
   }
   if (n_q < 1 || n_kv < 1 || hd < 1 || hd > 256 || (n_q % n_kv) != 0 || n_split < 1 ||
-      n_split > (in_wg ? kMaxWgSplits : 64) || max_seq < 1) {
+      n_split > (mode == 0 ? 64 : kMaxWgSplits) || max_seq < 1 ||
+      (mode == 2 && (n_parts < 1 || n_parts > 64))) {
     return -3;
   }
   const bool rope = cos != nullptr && sin != nullptr && position != nullptr;
   if (rope && (hd & 1) != 0) {
     return -3;
   }
+  if (mode == 2 && !aligned16(ws)) {
+    return -5;
+  }
   AttnArgs a{};
-  const int nml = n_q * n_split;
   a.q = static_cast<const uint16_t *>(q);
   a.k_cache = static_cast<const uint16_t *>(k);
   a.v_cache = static_cast<const uint16_t *>(v);
-  if (!in_wg) {
+  a.n_parts = mode == 2 ? n_parts : 1;
+  a.n_split = mode == 2 ? n_split * n_parts : n_split;  // wavefronts that share a head
+  if (mode == 0) {
+    const int nml = n_q * n_split;
     a.m_s = ws;
     a.l_s = ws + nml;
     a.o_s = ws + 2 * static_cast<size_t>(nml);
+  } else if (mode == 2) {
+    a.state = ws;
   }
   a.valid_len = static_cast<const int32_t *>(valid_len);
   a.k_act = static_cast<const uint16_t *>(k_act);
@@ -575,7 +634,6 @@ int attn_common(const void *q, const void *k, const void *v, void *out, const vo
   a.n_q = n_q;
   a.n_kv = n_kv;
   a.hd = hd;
-  a.n_split = n_split;
   a.max_seq = max_seq;
   a.scale = scale;
   a.out = static_cast<uint16_t *>(out);
@@ -585,8 +643,8 @@ int attn_common(const void *q, const void *k, const void *v, void *out, const vo
                       (k_act == nullptr || aligned16(k_act)) &&
                       (v_act == nullptr || aligned16(v_act)) &&
                       (cos == nullptr || aligned16(cos)) && (sin == nullptr || aligned16(sin)) &&
-                      (in_wg || aligned16(a.o_s));
-  if (in_wg) {
+                      (mode != 0 || aligned16(a.o_s));
+  if (mode != 0) {
     launch_flash<true>(a, vec_ok, st);
   } else {
     launch_flash<false>(a, vec_ok, st);
@@ -605,7 +663,7 @@ extern "C" int chr_nf4_attn(const void *q, const void *k, const void *v, void *o
                             const void *k_act, const void *v_act, const void *cos,
                             const void *sin, const void *position, int32_t max_seq) {
   return attn_common(q, k, v, out, valid_len, ws, n_q, n_kv, hd, n_split, scale, stream, k_act,
-                     v_act, cos, sin, position, max_seq, false);
+                     v_act, cos, sin, position, max_seq, 0, 1);
 }
 
 extern "C" int chr_dv2_attn(const void *q, const void *k, const void *v, void *out,
@@ -614,5 +672,22 @@ extern "C" int chr_dv2_attn(const void *q, const void *k, const void *v, void *o
                             const void *v_act, const void *cos, const void *sin,
                             const void *position, int32_t max_seq) {
   return attn_common(q, k, v, out, valid_len, nullptr, n_q, n_kv, hd, n_waves, scale, stream,
-                     k_act, v_act, cos, sin, position, max_seq, true);
+                     k_act, v_act, cos, sin, position, max_seq, 1, 1);
+}
+
+extern "C" int64_t chr_dv2_attn_state_floats(int32_t n_q, int32_t hd, int32_t n_parts) {
+  if (n_q < 1 || hd < 1 || n_parts < 1) {
+    return 0;
+  }
+  return static_cast<int64_t>(n_q) * n_parts * (hd + 4);
+}
+
+extern "C" int chr_dv2_attn_parts(const void *q, const void *k, const void *v,
+                                  const void *valid_len, float *state, int32_t n_q, int32_t n_kv,
+                                  int32_t hd, int32_t n_parts, int32_t n_waves, float scale,
+                                  void *stream, const void *k_act, const void *v_act,
+                                  const void *cos, const void *sin, const void *position,
+                                  int32_t max_seq) {
+  return attn_common(q, k, v, nullptr, valid_len, state, n_q, n_kv, hd, n_waves, scale, stream,
+                     k_act, v_act, cos, sin, position, max_seq, 2, n_parts);
 }

@@ -66,6 +66,10 @@ struct StreamArgs {
   int M[3];
   int groups[3];  // wavefront-sized row groups of each segment
   int ksplit;     // 1, or > 1: the wavefronts of a workgroup share one row group along K
+  // x is not given but merged, while it is staged, from the softmax states that
+  // attn_parts workgroups per head left: {m, l, 0, 0, o[attn_hd]} each (K = heads*attn_hd)
+  const float *attn_state;
+  int attn_parts, attn_hd;
   // second matrix of a SwiGLU pair (segment 0 only)
   const uint8_t *packed2;
   const uint16_t *scale2;
@@ -119,7 +123,87 @@ __device__ __forceinline__ int x_slot(int piece, int nfull) {
 // value stored is bf16( (w*x) * rsqrt(mean(x^2)+eps) ), i.e. what a separate RMSNorm
 // launch would have handed over (gpu/nf4/nf4_gemv.cu:264-289).  Used for a ragged K
 // and for the fused RMSNorm.
+// x piece i (8 consecutive dims of one head) merged from the per-part softmax states:
+// x = sum_p e^{m_p - M} o_p / sum_p e^{m_p - M} l_p, rounded to bf16 as the attention
+// launch itself would have stored it.  An empty part has m = -1e30, l = 0: weight zero.
+__device__ __forceinline__ uint4 merged_attn_piece(const StreamArgs &a, int i) {
+  constexpr int kBatch = 8;  // parts whose states are fetched together (one memory round trip)
+  const int hd = a.attn_hd;
+  const int k = i << 3;
+  const int head = k / hd;
+  const int d = k - head * hd;
+  const float *st = a.attn_state + static_cast<size_t>(head) * a.attn_parts * (hd + 4);
+  float mx = -1e30f;
+  float l = 0.f;
+  float o[8] = {};
+  for (int p0 = 0; p0 < a.attn_parts; p0 += kBatch) {
+    float2 ml[kBatch];
+    float4 lo[kBatch], hi[kBatch];
+#pragma unroll
+    for (int j = 0; j < kBatch; ++j) {
+      const bool on = p0 + j < a.attn_parts;
+      const float *sp = st + (on ? p0 + j : p0) * (hd + 4);
+      ml[j] = *reinterpret_cast<const float2 *>(sp);
+      lo[j] = *reinterpret_cast<const float4 *>(sp + 4 + d);
+      hi[j] = *reinterpret_cast<const float4 *>(sp + 8 + d);
+      if (!on) {
+        ml[j] = make_float2(-1e30f, 0.f);
+      }
+    }
+    float bm = mx;
+#pragma unroll
+    for (int j = 0; j < kBatch; ++j) {
+      bm = fmaxf(bm, ml[j].x);
+    }
+    const float keep = __expf(mx - bm);  // rescale what earlier batches added
+    l *= keep;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      o[e] *= keep;
+    }
+    mx = bm;
+#pragma unroll
+    for (int j = 0; j < kBatch; ++j) {
+      const float w = __expf(ml[j].x - mx);
+      l = fmaf(w, ml[j].y, l);
+      o[0] = fmaf(w, lo[j].x, o[0]);
+      o[1] = fmaf(w, lo[j].y, o[1]);
+      o[2] = fmaf(w, lo[j].z, o[2]);
+      o[3] = fmaf(w, lo[j].w, o[3]);
+      o[4] = fmaf(w, hi[j].x, o[4]);
+      o[5] = fmaf(w, hi[j].y, o[5]);
+      o[6] = fmaf(w, hi[j].z, o[6]);
+      o[7] = fmaf(w, hi[j].w, o[7]);
+    }
+  }
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  uint32_t r[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const uint32_t lo16 = f32_to_bf16(o[2 * q] * inv);
+    const uint32_t hi16 = f32_to_bf16(o[2 * q + 1] * inv);
+    r[q] = lo16 | (hi16 << 16);
+  }
+  return make_uint4(r[0], r[1], r[2], r[3]);
+}
+
 __device__ __forceinline__ void stage_x(const StreamArgs &a, uint4 *xs, float *part) {
+  if (a.attn_state != nullptr) {
+    const int nfull_a = (a.K_pad >> 5) >> 6;
+    for (int i = threadIdx.x; i < (a.K_pad >> 3); i += blockDim.x) {
+      xs[x_slot(i, nfull_a)] = merged_attn_piece(a, i);
+    }
+    const int full = nfull_a << 8;
+    const int tail_half = ((a.K_pad >> 5) & 63) * 2;
+    for (int i = full + threadIdx.x; i < x_pieces(a.K_pad); i += blockDim.x) {
+      const int h = (((i - full) >> 7) << 6) + (i & 63);
+      if (h >= tail_half) {
+        xs[i] = make_uint4(0, 0, 0, 0);
+      }
+    }
+    __syncthreads();
+    return;
+  }
   constexpr int kKeep = 4;  // 16-byte vectors of x a thread keeps between the two passes
   const int nfull = (a.K_pad >> 5) >> 6;
   const int slots = x_pieces(a.K_pad);
@@ -568,7 +652,7 @@ int launch_stream(StreamArgs &a, int n_seg, hipStream_t st) {
     total += a.groups[i];
   }
   const size_t dyn = static_cast<size_t>(x_pieces(a.K_pad)) * 16;
-  const bool must_stage = a.rms_w != nullptr || a.K != a.K_pad;
+  const bool must_stage = a.rms_w != nullptr || a.K != a.K_pad || a.attn_state != nullptr;
   const int forced = forced_staged();
   const bool staged = must_stage || (forced == 1 && dyn <= kMaxDynLds);
   if (staged) {
@@ -631,6 +715,36 @@ int gemv_entry(const chr_nf4_dev_t *w, const void *x, void *y, void *stream, con
   a.K = w->K;
   a.K_pad = w->K_pad;
   a.rms_eps = rms_eps;
+  return launch_rows(a, 1, w->M, static_cast<hipStream_t>(stream));
+}
+
+// y = W @ merge(states) (+ add): the o projection consuming what chr_dv2_attn_parts left.
+int gemv_attn_entry(const chr_nf4_dev_t *w, const float *state, int n_q, int hd, int n_parts,
+                    void *y, const void *add, void *stream) {
+  if (w == nullptr || state == nullptr || y == nullptr) {
+    return -1;
+  }
+  if (w->M < 1 || w->K < 1 || w->packed == nullptr || w->scale == nullptr || n_q < 1 || hd < 8 ||
+      (hd & 7) != 0 || n_parts < 1 || n_parts > 64 || w->K != n_q * hd) {
+    return -3;
+  }
+  if (!k_pad_ok(w->K, w->K_pad) || w->K != w->K_pad) {
+    return -4;
+  }
+  if (!aligned16(w->packed) || !aligned16(state) || !aligned2(w->scale)) {
+    return -5;
+  }
+  StreamArgs a{};
+  a.packed[0] = w->packed;
+  a.scale[0] = w->scale;
+  a.y[0] = static_cast<uint16_t *>(y);
+  a.add[0] = static_cast<const uint16_t *>(add);
+  a.M[0] = w->M;
+  a.K = w->K;
+  a.K_pad = w->K_pad;
+  a.attn_state = state;
+  a.attn_parts = n_parts;
+  a.attn_hd = hd;
   return launch_rows(a, 1, w->M, static_cast<hipStream_t>(stream));
 }
 

@@ -7,7 +7,7 @@ from dataclasses import dataclass
 
 import torch
 
-from ..nf4 import ATTN_SPLIT
+from ..nf4 import ATTN_SPLIT, dv2_attn_state_floats
 from .plan import ArchSpec
 
 __all__ = ["Arena"]
@@ -26,6 +26,7 @@ class Arena:
     down_in: torch.Tensor
     logits: torch.Tensor
     attn_ws: torch.Tensor
+    attn_state: torch.Tensor     # softmax states of the attention whose merge the o projection does
 
     @classmethod
     def allocate(cls, spec: ArchSpec, *, device, dtype: torch.dtype = torch.bfloat16) -> "Arena":
@@ -45,4 +46,6 @@ class Arena:
             logits=z(1, spec.vocab),
             attn_ws=torch.zeros(spec.n_q * ATTN_SPLIT * (spec.head_dim + 2), dtype=torch.float32,
                                 device=device),
+            attn_state=torch.zeros(dv2_attn_state_floats(spec.n_q, spec.head_dim), dtype=torch.float32,
+                                   device=device),
         )

@@ -12,24 +12,24 @@ argmax that also feeds the id back.
 Two launch schedules compute that sequence:
 
 ``plain``     the reference's call sequence, eight launches per layer;
-``fold_rms``  every RMSNorm runs inside the GEMV that consumes it, attention is one
-              launch per layer while the cache is short enough for one workgroup
-              per head, and the embedding gather also sets the KV length: five
-              launches per layer.  A dependent launch costs about 5 us on an
-              MI355X whatever it does, so the launch count is what this buys.
+``fold_rms``  every RMSNorm runs inside the GEMV that consumes it, the merge of the
+              attention splits runs inside the o projection, and the embedding
+              gather also sets the KV length: five launches per layer.  A
+              dependent launch costs about 5 us on an MI355X whatever it does, so
+              the launch count is what this buys.
 """
 
 from __future__ import annotations
 
 import torch
 
-from ..nf4 import (ATTN_SPLIT, ATTN_WG_WAVES, dv2_attn, dv2_begin_step, nf4_attn, nf4_gemv, nf4_qkv,
-                   nf4_rms, nf4_swiglu)
+from ..nf4 import (ATTN_SPLIT, dv2_attn_parts, dv2_begin_step, dv2_gemv_attn, nf4_attn, nf4_gemv,
+                   nf4_qkv, nf4_rms, nf4_swiglu)
 from .embed import PackedEmbed, gather_embed
 from .linear import DeviceLayer, DeviceLinear, DeviceWeights
 from .state import DecodeState
 
-__all__ = ["forward_decode", "greedy_decode", "teacher_force_token", "SCHEDULES", "ATTN_WG_MAX_SEQ"]
+__all__ = ["forward_decode", "greedy_decode", "teacher_force_token", "SCHEDULES"]
 
 
 def _gemv_accum(mat: DeviceLinear, src: torch.Tensor, dest: torch.Tensor) -> None:
@@ -62,24 +62,33 @@ def _qkv(state: DecodeState, layer: DeviceLayer, h: torch.Tensor, rms_w: torch.T
 SCHEDULES = ("plain", "fold_rms")
 #: schedule used when the caller does not name one
 DEFAULT_SCHEDULE = "fold_rms"
-#: longest cache the one-launch attention (one workgroup per query head) is used for;
-#: longer caches go to the split kernel + merge, which spreads a head over many units
-ATTN_WG_MAX_SEQ = 4096
 
 
-def _attend(state: DecodeState, li: int, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
-            one_launch: bool) -> None:
+def _attend_into_o(state: DecodeState, li: int, layer: DeviceLayer, q, k, v) -> None:
+    """Attention + o projection + residual as two launches: the attention workgroups (several
+    per head, so a head's cache rows stream through several compute units) leave their
+    softmax states, and the o GEMV merges them while it stages its activations."""
     spec = state.spec
     ar = state.arena
     n_q, n_kv, hd = spec.n_q, spec.n_kv, spec.head_dim
     kc, vc = state.kv.layer(li)
-    if one_launch:
-        dv2_attn(q.view(n_q, hd), kc, vc, ar.attn, state.valid_len, spec.attn_scale, ATTN_WG_WAVES,
-                 k.view(n_kv, hd), v.view(n_kv, hd), state.cos, state.sin, state.position)
-    else:
-        nf4_attn(q.view(n_q, hd), kc, vc, ar.attn, state.valid_len, spec.attn_scale, ar.attn_ws,
-                 ATTN_SPLIT, k.view(n_kv, hd), v.view(n_kv, hd), state.cos, state.sin,
-                 state.position)
+    dv2_attn_parts(q.view(n_q, hd), kc, vc, state.valid_len, spec.attn_scale, ar.attn_state,
+                   k_act=k.view(n_kv, hd), v_act=v.view(n_kv, hd), cos=state.cos, sin=state.sin,
+                   position=state.position)
+    o = layer.o
+    d = ar.x.view(-1)
+    dv2_gemv_attn(o.packed, o.scale, ar.attn_state, n_q, hd, o.M, o.K, o.K_pad, d, d)
+    if o.bias is not None:
+        d.add_(o.bias)
+
+
+def _attend(state: DecodeState, li: int, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> None:
+    spec = state.spec
+    ar = state.arena
+    n_q, n_kv, hd = spec.n_q, spec.n_kv, spec.head_dim
+    kc, vc = state.kv.layer(li)
+    nf4_attn(q.view(n_q, hd), kc, vc, ar.attn, state.valid_len, spec.attn_scale, ar.attn_ws,
+             ATTN_SPLIT, k.view(n_kv, hd), v.view(n_kv, hd), state.cos, state.sin, state.position)
 
 
 def _forward_calls(state: DecodeState, weights: DeviceWeights, commit: bool, fold: bool) -> None:
@@ -96,15 +105,18 @@ def _forward_calls(state: DecodeState, weights: DeviceWeights, commit: bool, fol
     else:
         gather_embed(emb, state.token.reshape(1), out=ar.x)
         state.kv.mark_written(state.position)
-    one_launch_attn = fold and spec.max_seq <= ATTN_WG_MAX_SEQ
+    merge_in_o = fold and spec.head_dim % 8 == 0
     for li, layer in enumerate(weights.layers):
         if fold:
             q, k, v = _qkv(state, layer, ar.x, layer.norm1)
         else:
             nf4_rms(ar.x, layer.norm1, ar.h, eps)
             q, k, v = _qkv(state, layer, ar.h)
-        _attend(state, li, q, k, v, one_launch_attn)
-        _gemv_accum(layer.o, ar.attn, ar.x)
+        if merge_in_o:
+            _attend_into_o(state, li, layer, q, k, v)
+        else:
+            _attend(state, li, q, k, v)
+            _gemv_accum(layer.o, ar.attn, ar.x)
         g, u = layer.gate, layer.up
         if fold:
             nf4_swiglu(g.packed, g.scale, u.packed, u.scale, ar.x.view(-1), g.M, g.K, g.K_pad,

@@ -41,6 +41,11 @@ __all__ = [
     "dv2_argmax_commit",
     "dv2_begin_step",
     "ATTN_WG_WAVES",
+    "ATTN_PARTS",
+    "ATTN_PART_WAVES",
+    "dv2_attn_state_floats",
+    "dv2_attn_parts",
+    "dv2_gemv_attn",
     "dv2_attn",
     "library_path",
 ]
@@ -109,6 +114,10 @@ EXPORTS = (
     ("chr_dv2_begin_step", ctypes.c_int, [_DP, _P, _P, _P, _P, _P, _F, _P, _P]),
     ("chr_dv2_attn", ctypes.c_int,
      [_P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _P, _P, _P, _P, _P, _P, _I]),
+    ("chr_dv2_attn_state_floats", ctypes.c_int64, [_I, _I, _I]),
+    ("chr_dv2_attn_parts", ctypes.c_int,
+     [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _P, _P, _P, _P, _P, _P, _I]),
+    ("chr_dv2_gemv_attn", ctypes.c_int, [_DP, _P, _I, _I, _I, _P, _P, _P]),
     ("chr_dv2_mark_written", ctypes.c_int, [_P, _P, _P]),
     ("chr_dv2_argmax_commit", ctypes.c_int, [_P, _I, _P, _P, _P, _P, _P, _I, _P]),
     ("chr_nf4_abi_version", ctypes.c_int, []),
@@ -635,3 +644,64 @@ def dv2_attn(q, k, v, out, valid_len, scale: float, n_waves: int = ATTN_WG_WAVES
                                   _stream(), ptr(k_act), ptr(v_act), ptr(cos), ptr(sin),
                                   ptr(position), max_seq)
     _check_rc("chr_dv2_attn", rc)
+
+
+#: workgroups per head and wavefronts per workgroup of the attention that leaves its merge
+#: to the o projection
+ATTN_PARTS = 4
+ATTN_PART_WAVES = 8
+
+
+def dv2_attn_state_floats(n_q: int, hd: int, n_parts: int = ATTN_PARTS) -> int:
+    """fp32 elements ``dv2_attn_parts`` writes for ``n_q`` heads of ``hd`` dims."""
+    return int(_load_ext().chr_dv2_attn_state_floats(int(n_q), int(hd), int(n_parts)))
+
+
+def dv2_attn_parts(q, k, v, valid_len, scale: float, state, n_parts: int = ATTN_PARTS,
+                   n_waves: int = ATTN_PART_WAVES, k_act=None, v_act=None, cos=None, sin=None,
+                   position=None) -> None:
+    """Attention that stops before the merge: ``n_parts`` workgroups per query head leave
+    their softmax states in ``state`` (fp32); ``dv2_gemv_attn`` merges them."""
+    _need(q.is_cuda and q.dtype == torch.bfloat16 and q.is_contiguous(), "q must be contiguous CUDA bf16")
+    _need(k.is_contiguous() and v.is_contiguous() and k.dim() == 3, "caches must be contiguous [max_seq,n_kv,hd]")
+    max_seq, n_kv, hd = (int(t) for t in k.shape)
+    n_q = _heads(q, hd)
+    _need(valid_len.is_cuda and valid_len.dtype == torch.int32 and valid_len.numel() == 1,
+          "valid_len must be a CUDA int32 scalar")
+    _need(1 <= int(n_waves) <= 16 and 1 <= int(n_parts) <= 64, "n_waves in 1..16, n_parts in 1..64")
+    _need(state.is_cuda and state.dtype == torch.float32 and state.is_contiguous()
+          and state.numel() >= n_q * int(n_parts) * (hd + 4), "attention state buffer too small")
+
+    def ptr(t):
+        return None if t is None else t.data_ptr()
+
+    for t in (k_act, v_act, cos, sin, position):
+        _need(t is None or (t.is_cuda and t.is_contiguous()), "optional inputs must be contiguous CUDA")
+    rc = _load_ext().chr_dv2_attn_parts(q.data_ptr(), k.data_ptr(), v.data_ptr(), valid_len.data_ptr(),
+                                        state.data_ptr(), n_q, n_kv, hd, int(n_parts), int(n_waves),
+                                        float(scale), _stream(), ptr(k_act), ptr(v_act), ptr(cos),
+                                        ptr(sin), ptr(position), max_seq)
+    _check_rc("chr_dv2_attn_parts", rc)
+
+
+def dv2_gemv_attn(packed: torch.Tensor, scale: torch.Tensor, state: torch.Tensor, n_q: int, hd: int,
+                  M: int, K: int, K_pad: int, out: torch.Tensor, add: torch.Tensor | None = None,  # noqa: N803
+                  n_parts: int = ATTN_PARTS) -> torch.Tensor:
+    """``out = W @ merge(state) (+ add)``: the o projection that also merges the softmax
+    states of ``dv2_attn_parts``.  ``K == n_q * hd`` and a multiple of 64; ``hd % 8 == 0``."""
+    M, K, K_pad = int(M), int(K), int(K_pad)
+    _check_packed(packed, scale, M, K, K_pad)
+    _need(packed.is_contiguous() and scale.is_contiguous(), "blobs must be contiguous")
+    _need(K == int(n_q) * int(hd) and K == K_pad and int(hd) % 8 == 0,
+          "K must equal n_q*hd, be a multiple of 64, and hd a multiple of 8")
+    _need(state.is_cuda and state.dtype == torch.float32 and state.is_contiguous()
+          and state.numel() >= int(n_q) * int(n_parts) * (int(hd) + 4), "attention state buffer too small")
+    for t, name in ((out, "out"), (add, "add")):
+        _need(t is None or (t.is_cuda and t.dtype == torch.bfloat16 and t.is_contiguous()
+                            and t.numel() >= M), f"{name} must be contiguous CUDA bf16 with M elements")
+    w = _dev(packed, scale, M, K, K_pad)
+    rc = _load_ext().chr_dv2_gemv_attn(ctypes.byref(w), state.data_ptr(), int(n_q), int(hd),
+                                       int(n_parts), out.data_ptr(),
+                                       None if add is None else add.data_ptr(), _stream())
+    _check_rc("chr_dv2_gemv_attn", rc)
+    return out

@@ -189,6 +189,23 @@ int chr_dv2_attn(const void *q, const void *k, const void *v, void *out, const v
                  void *stream, const void *k_act, const void *v_act, const void *cos,
                  const void *sin, const void *position, int32_t max_seq);
 
+/* Attention whose merge is left to the o projection: n_parts workgroups of n_waves (<= 16)
+ * wavefronts per query head each leave an unnormalised softmax state {m, l, 0, 0, o[hd]} in
+ * `state` (chr_dv2_attn_state_floats(n_q, hd, n_parts) floats, 16-byte aligned); RoPE and the
+ * cache write are fused as in chr_nf4_attn.  chr_dv2_gemv_attn then computes
+ * y = W @ merge(state) (+ add), merging while it stages its activations: hd % 8 == 0,
+ * W.K == n_q*hd == W.K_pad.  Together they replace attn_flash + attn_merge + the o GEMV
+ * (gpu/nf4/nf4_gemv.cu:952-994, gpu/decodev2/step.py:119-137) with two launches that spread
+ * a head over several compute units.  No reference counterpart. */
+int64_t chr_dv2_attn_state_floats(int32_t n_q, int32_t hd, int32_t n_parts);
+int chr_dv2_attn_parts(const void *q, const void *k, const void *v, const void *valid_len,
+                       float *state, int32_t n_q, int32_t n_kv, int32_t hd, int32_t n_parts,
+                       int32_t n_waves, float scale, void *stream, const void *k_act,
+                       const void *v_act, const void *cos, const void *sin,
+                       const void *position, int32_t max_seq);
+int chr_dv2_gemv_attn(const chr_nf4_dev_t *w, const float *state, int32_t n_q, int32_t hd,
+                      int32_t n_parts, void *y, const void *add, void *stream);
+
 /* Library version, for the loader's sanity check. */
 int chr_nf4_abi_version(void);
 

@@ -303,17 +303,6 @@ def test_folded_schedule_in_a_graph():
         torch.cuda.synchronize()
 
 
-def test_long_cache_takes_the_split_attention(monkeypatch):
-    """Past ATTN_WG_MAX_SEQ the folded schedule uses the split kernel + merge; both give
-    the same ids."""
-    import deepfold_amd.decodev2.step as step_mod
-    model, state, weights = session(dv2.TINY_LLAMA, 0, packed_embed=True)
-    a = greedy_token_at_a_time(state, weights, SHORT, 10)
-    monkeypatch.setattr(step_mod, "ATTN_WG_MAX_SEQ", 0)
-    b = greedy_token_at_a_time(state, weights, SHORT, 10)
-    assert a == b == so.greedy_ids(model, SHORT, 10)
-
-
 def test_unknown_schedule_is_refused():
     _, state, weights = session(dv2.TINY_LLAMA, 0)
     state.load_token(1)

@@ -602,3 +602,61 @@ def test_begin_step(vocab, k):
         xv = to_f32(row).astype(np.float64)
         ref = to_f32(g).astype(np.float64) * xv / np.sqrt((xv ** 2).mean() + eps)
         assert (np.abs(a - ref) <= ulp_bf16(ref)).all()
+
+
+@pytest.mark.parametrize("n_q,n_kv,hd,max_seq,pos,parts,waves", [
+    (4, 2, 16, 16, 0, 8, 4), (16, 2, 128, 128, 100, 8, 4), (40, 8, 128, 2048, 1500, 8, 4),
+    (4, 2, 48, 32, 9, 3, 2), (40, 8, 128, 2048, 2047, 5, 16), (8, 8, 64, 64, 33, 1, 1)])
+def test_attention_merged_by_the_o_projection(n_q, n_kv, hd, max_seq, pos, parts, waves):
+    """dv2_attn_parts + dv2_gemv_attn against nf4_attn + nf4_gemv(add) (each checked against
+    float64 above): the same softmax over another partition of the rows, merged inside the
+    GEMV's staging."""
+    say("attn parts", n_q, n_kv, hd, max_seq, pos, parts, waves)
+    rng = np.random.default_rng(hd + pos + parts)
+    cos, sin = rope_tables(max_seq, hd)
+    q = bf16_tensor(rng.standard_normal((n_q, hd)).astype(np.float32))
+    k_act = bf16_tensor(rng.standard_normal((n_kv, hd)).astype(np.float32))
+    v_act = bf16_tensor(rng.standard_normal((n_kv, hd)).astype(np.float32))
+    kc0 = bf16_tensor(rng.standard_normal((max_seq, n_kv, hd)).astype(np.float32))
+    vc0 = bf16_tensor(rng.standard_normal((max_seq, n_kv, hd)).astype(np.float32))
+    kc0[pos + 1:] = 1e4      # a dirty tail must be ignored
+    vc0[pos + 1:] = -1e4
+    tcos, tsin = bf16_tensor(cos), bf16_tensor(sin)
+    vl = torch.tensor(pos + 1, dtype=torch.int32, device=DEV)
+    position = torch.tensor(pos, dtype=torch.int64, device=DEV)
+    scale = hd ** -0.5
+    hidden = n_q * hd
+    m = 192
+    p, s, dp, ds = blobs(m, hidden, 91)
+    res = bf16_tensor(rng.standard_normal(m).astype(np.float32))
+    # reference sequence
+    kc_a, vc_a = kc0.clone(), vc0.clone()
+    attn = torch.zeros(hidden, dtype=torch.bfloat16, device=DEV)
+    nf4.nf4_attn(q, kc_a, vc_a, attn, vl, scale, None, nf4.ATTN_SPLIT, k_act, v_act, tcos, tsin, position)
+    want = res.clone()
+    nf4.nf4_gemv(dp, ds, attn, m, hidden, hidden, want, want)
+    # two launches
+    state = torch.full((nf4.dv2_attn_state_floats(n_q, hd, parts),), float("nan"), dtype=torch.float32,
+                       device=DEV)
+    for rep in range(2):
+        kc_b, vc_b = kc0.clone(), vc0.clone()
+        nf4.dv2_attn_parts(q, kc_b, vc_b, vl, scale, state, parts, waves, k_act, v_act, tcos, tsin, position)
+        got = res.clone()
+        nf4.dv2_gemv_attn(dp, ds, state, n_q, hd, m, hidden, hidden, got, got, parts)
+        assert (bf16_bits(kc_a) == bf16_bits(kc_b)).all() and (bf16_bits(vc_a) == bf16_bits(vc_b)).all()
+        assert torch.isfinite(got.float()).all()
+        # the merged activations differ from the two-launch ones by bf16 rounding at most
+        err = np.abs(to_f32(got) - to_f32(want)).max()
+        assert err <= 0.02 * max(1.0, float(np.abs(to_f32(want)).max())), (rep, err)
+
+
+def test_gemv_attn_rejects_bad_arguments():
+    p, s, dp, ds = blobs(64, 128, 5)
+    state = torch.zeros(nf4.dv2_attn_state_floats(2, 64, 4), dtype=torch.float32, device=DEV)
+    y = torch.zeros(64, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(RuntimeError):
+        nf4.dv2_gemv_attn(dp, ds, state, 3, 64, 64, 128, 128, y, None, 4)      # K != n_q*hd
+    with pytest.raises(RuntimeError):
+        nf4.dv2_gemv_attn(dp, ds, state[:10], 2, 64, 64, 128, 128, y, None, 4)  # state too small
+    nf4.dv2_gemv_attn(dp, ds, state, 2, 64, 64, 128, 128, y, None, 4)           # zero states -> zeros
+    assert float(y.float().abs().max()) == 0.0
