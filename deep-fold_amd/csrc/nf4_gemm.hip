@@ -109,9 +109,8 @@ int resolved_one_wave() {
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
-// split so that grid_x * split reaches three workgroups per compute unit, capped at
-// kMaxAutoSplit (more splits cost more in fp32 partials than they win in occupancy)
-// and at the number of K tiles; split is recomputed from tiles_per_split so the
+// split so that grid_x * split reaches two workgroups per compute unit, capped at
+// kMaxAutoSplit and at the number of K tiles; split is recomputed from tiles_per_split so the
 // pair always agrees with what the kernel indexes
 // (gpu/nf4/nf4_gemm.cu:1526-1543).
 constexpr int kMaxAutoSplit = 8;
@@ -120,9 +119,9 @@ void pick_split(int grid_x, int n_ktiles, int have_ws, int *split, int *tiles_pe
   const Tuning &t = tuning();
   int want = 1;
   if (have_ws) {
-    // three workgroups of four wavefronts per compute unit keep its SIMDs busy through the
-    // LDS and MFMA latencies of a tile (measured: 2 is 10-15 % slower, 4 no faster)
-    const int target = resolved_one_wave() * 3;
+    // two workgroups per compute unit: more splits were measured to cost as much in fp32
+    // partials (long-K shapes) as they win in occupancy
+    const int target = resolved_one_wave() * 2;
     want = t.split_k > 0 ? t.split_k : std::min(kMaxAutoSplit, ceil_div(target, grid_x));
   }
   want = std::max(1, std::min(want, n_ktiles));

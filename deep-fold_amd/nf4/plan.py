@@ -107,7 +107,7 @@ def _pick_split(grid_x: int, n_ktiles: int, have_ws: bool, force_split: int,
                 one_wave: int) -> tuple[int, int]:
     want = 1
     if have_ws:
-        target = max(1, int(one_wave) * 3)
+        target = max(1, int(one_wave) * 2)
         want = force_split if force_split > 0 else min(_MAX_AUTO_SPLIT, _ceil_div(target, grid_x))
     want = max(1, min(want, n_ktiles))
     tiles_per_split = _ceil_div(n_ktiles, want)
