@@ -13,7 +13,8 @@ import sys
 
 CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 LIB = os.path.join(CSRC, "libchr_nf4_amd.so")
-SOURCES = ("nf4_gemv.hip", "nf4_codec.hip", "nf4_attn.hip", "nf4_gemm.hip", "dv2_state.hip")
+SOURCES = ("nf4_gemv.hip", "nf4_codec.hip", "nf4_attn.hip", "nf4_gemm.hip", "dv2_state.hip",
+           "dv2_prefill.hip")
 HEADERS = ("nf4_common.h", os.path.join("..", "..", "include", "chr_nf4_amd.h"))
 
 #: -packed-fp32-ops is switched off on purpose: the kernels are written for

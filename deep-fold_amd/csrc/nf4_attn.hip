@@ -81,6 +81,10 @@ struct AttnArgs {
   // for a later merge instead of writing out
   int n_parts;
   float *state;
+  // several query tokens in one launch (blockIdx.y = token): token t reads its q at
+  // q + t*q_tok_stride, sees *valid_len + t cache rows, and writes dim d of a head to
+  // out[t*out_tok_stride + (head*hd + d)*out_dim_stride]
+  int q_tok_stride, out_tok_stride, out_dim_stride;
 };
 
 constexpr int kMaxWgSplits = 16;  // wavefronts of a one-workgroup-per-head launch
@@ -93,7 +97,7 @@ constexpr int kMaxWgSplits = 16;  // wavefronts of a one-workgroup-per-head laun
 // sum over splits running in split order.
 __device__ __forceinline__ void merge_head(const float *m_s, const float *l_s, const float *o_s,
                                            uint16_t *out, int head, int hd, int n_split,
-                                           int lane, float *state = nullptr) {
+                                           int lane, float *state = nullptr, int dstride = 1) {
   const float *mh = m_s + static_cast<size_t>(head) * n_split;
   const float *lh = l_s + static_cast<size_t>(head) * n_split;
   const float my_m = lane < n_split ? *(mh + lane) : kNegBig;
@@ -142,7 +146,7 @@ __device__ __forceinline__ void merge_head(const float *m_s, const float *l_s, c
       if (state != nullptr) {
         state[4 + d] = acc;  // unnormalised: the later merge divides
       } else {
-        dst[d] = f32_to_bf16(l > 0.f ? acc * inv : 0.f);
+        dst[static_cast<size_t>(d) * dstride] = f32_to_bf16(l > 0.f ? acc * inv : 0.f);
       }
     }
   }
@@ -170,7 +174,8 @@ __global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flas
   const int d0 = li * 8;
   const int n_rep = a.n_q / a.n_kv;
   const int kv_head = head / n_rep;
-  const int vl = min(*a.valid_len, a.max_seq);
+  const int tok = INWG ? static_cast<int>(blockIdx.y) : 0;
+  const int vl = min(*a.valid_len + tok, a.max_seq);
 
   // The first block of cache rows is requested before anything else (RoPE tables, q, the
   // current k/v): its trip to memory overlaps that prologue.  UNR time steps per lane group
@@ -210,7 +215,7 @@ __global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flas
   float vcur[8];
   int pos = -1;
   bool fuse = false;
-  const uint16_t *qh = a.q + static_cast<size_t>(head) * hd;
+  const uint16_t *qh = a.q + static_cast<size_t>(tok) * a.q_tok_stride + static_cast<size_t>(head) * hd;
   bool rotated = false;
   if (a.cos != nullptr && a.sin != nullptr && a.position != nullptr) {
     const long long p = *a.position;
@@ -328,7 +333,9 @@ __global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flas
       float *st = a.state == nullptr
                       ? nullptr
                       : a.state + (static_cast<size_t>(head) * a.n_parts + part) * (hd + 4);
-      merge_head(sm, sl, so, a.out + static_cast<size_t>(head) * hd, 0, hd, wg_waves, lane, st);
+      uint16_t *dst = a.out + static_cast<size_t>(tok) * a.out_tok_stride +
+                      static_cast<size_t>(head) * hd * a.out_dim_stride;
+      merge_head(sm, sl, so, dst, 0, hd, wg_waves, lane, st, a.out_dim_stride);
     }
   } else {
     const size_t slot = static_cast<size_t>(head) * a.n_split + split;
@@ -360,8 +367,9 @@ __global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flas
   const int half = hd / 2;
   const int n_rep = a.n_q / a.n_kv;
   const int kv_head = head / n_rep;
-  const int vl = min(*a.valid_len, a.max_seq);
-  const uint16_t *qh = a.q + static_cast<size_t>(head) * hd;
+  const int tok = INWG ? static_cast<int>(blockIdx.y) : 0;
+  const int vl = min(*a.valid_len + tok, a.max_seq);
+  const uint16_t *qh = a.q + static_cast<size_t>(tok) * a.q_tok_stride + static_cast<size_t>(head) * hd;
 
   float qf[4] = {}, kcur[4] = {}, vcur[4] = {};
   int pos = -1;
@@ -461,7 +469,9 @@ __global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flas
       float *st = a.state == nullptr
                       ? nullptr
                       : a.state + (static_cast<size_t>(head) * a.n_parts + part) * (hd + 4);
-      merge_head(sm, sl, so, a.out + static_cast<size_t>(head) * hd, 0, hd, wg_waves, lane, st);
+      uint16_t *dst = a.out + static_cast<size_t>(tok) * a.out_tok_stride +
+                      static_cast<size_t>(head) * hd * a.out_dim_stride;
+      merge_head(sm, sl, so, dst, 0, hd, wg_waves, lane, st, a.out_dim_stride);
     }
   } else {
     const size_t slot = static_cast<size_t>(head) * a.n_split + split;
@@ -567,9 +577,10 @@ namespace chr {
 namespace {
 
 template <bool INWG>
-void launch_flash(const AttnArgs &a, bool vec_ok, hipStream_t st) {
+void launch_flash(const AttnArgs &a, bool vec_ok, hipStream_t st, int n_tok = 1) {
   // one-workgroup forms: a.n_split counts all wavefronts of a head (parts x wavefronts)
-  const dim3 grid(static_cast<unsigned>(INWG ? a.n_q * a.n_parts : a.n_q * a.n_split));
+  const dim3 grid(static_cast<unsigned>(INWG ? a.n_q * a.n_parts : a.n_q * a.n_split),
+                  static_cast<unsigned>(INWG ? n_tok : 1));
   const dim3 block(static_cast<unsigned>(INWG ? kWave * (a.n_split / a.n_parts) : kWave));
   if (vec_ok && a.hd == 128) {
     attn_flash<16, INWG><<<grid, block, 0, st>>>(a);
@@ -594,14 +605,16 @@ int attn_common(const void *q, const void *k, const void *v, void *out, const vo
                 float *ws, int32_t n_q, int32_t n_kv, int32_t hd, int32_t n_split, float scale,
                 void *stream, const void *k_act, const void *v_act, const void *cos,
                 const void *sin, const void *position, int32_t max_seq, int mode,
-                int32_t n_parts) {
+                int32_t n_parts, int32_t n_tok = 1, int32_t out_tok_stride = 0,
+                int32_t out_dim_stride = 1) {
   if (q == nullptr || k == nullptr || v == nullptr || valid_len == nullptr ||
       (mode != 2 && out == nullptr) || (mode != 1 && ws == nullptr)) {
     return -1;
   }
   if (n_q < 1 || n_kv < 1 || hd < 1 || hd > 256 || (n_q % n_kv) != 0 || n_split < 1 ||
       n_split > (mode == 0 ? 64 : kMaxWgSplits) || max_seq < 1 ||
-      (mode == 2 && (n_parts < 1 || n_parts > 64))) {
+      (mode == 2 && (n_parts < 1 || n_parts > 64)) || n_tok < 1 || n_tok > 65535 ||
+      (n_tok > 1 && mode != 1)) {
     return -3;
   }
   const bool rope = cos != nullptr && sin != nullptr && position != nullptr;
@@ -637,6 +650,9 @@ int attn_common(const void *q, const void *k, const void *v, void *out, const vo
   a.max_seq = max_seq;
   a.scale = scale;
   a.out = static_cast<uint16_t *>(out);
+  a.q_tok_stride = n_q * hd;
+  a.out_tok_stride = out_tok_stride;
+  a.out_dim_stride = out_dim_stride;
   hipStream_t st = static_cast<hipStream_t>(stream);
   // The vector path needs 16-byte aligned rows and 16-byte aligned fp32 partials.
   const bool vec_ok = aligned16(q) && aligned16(k) && aligned16(v) &&
@@ -645,7 +661,7 @@ int attn_common(const void *q, const void *k, const void *v, void *out, const vo
                       (cos == nullptr || aligned16(cos)) && (sin == nullptr || aligned16(sin)) &&
                       (mode != 0 || aligned16(a.o_s));
   if (mode != 0) {
-    launch_flash<true>(a, vec_ok, st);
+    launch_flash<true>(a, vec_ok, st, n_tok);
   } else {
     launch_flash<false>(a, vec_ok, st);
     attn_merge<<<dim3(static_cast<unsigned>(n_q)), dim3(kWave), 0, st>>>(a.m_s, a.l_s, a.o_s, a.out,
@@ -690,4 +706,17 @@ extern "C" int chr_dv2_attn_parts(const void *q, const void *k, const void *v,
                                   int32_t max_seq) {
   return attn_common(q, k, v, nullptr, valid_len, state, n_q, n_kv, hd, n_waves, scale, stream,
                      k_act, v_act, cos, sin, position, max_seq, 2, n_parts);
+}
+
+extern "C" int chr_dv2_attn_chunk(const void *q, const void *k, const void *v, void *out,
+                                  const void *first_len, int32_t n_tok, int32_t n_q, int32_t n_kv,
+                                  int32_t hd, int32_t n_waves, float scale, void *stream,
+                                  int32_t max_seq, int32_t out_tok_stride,
+                                  int32_t out_dim_stride) {
+  if (out_dim_stride < 1 || out_tok_stride < 0) {
+    return -3;
+  }
+  return attn_common(q, k, v, out, first_len, nullptr, n_q, n_kv, hd, n_waves, scale, stream,
+                     nullptr, nullptr, nullptr, nullptr, nullptr, max_seq, 1, 1, n_tok,
+                     out_tok_stride, out_dim_stride);
 }

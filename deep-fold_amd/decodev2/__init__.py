@@ -8,7 +8,7 @@ from .kv import GraphSafeKV
 from .linear import DeviceLayer, DeviceLinear, DeviceWeights, nf4_linear
 from .plan import (INTERNLM25_20B, MEDIUM_LLAMA, QWEN25_3B, QWEN25_14B, QWEN25_32B, TINY_INTERNLM,
                    TINY_LLAMA, ArchSpec, with_max_seq)
-from .prefill import forward_prefill, prefill_chunk_width
+from .prefill import ChunkPrefill, forward_prefill, prefill_chunk_width
 from .rope import apply_rope_torch, rope_tables_numpy, rope_tables_torch
 from .runner import consume_prompt, generate
 from .state import DecodeState
@@ -16,7 +16,7 @@ from .step import SCHEDULES, forward_decode, greedy_decode, teacher_force_token
 from .synth import Nf4Matrix, SynthLayer, SynthModel, build
 
 __all__ = [
-    "ArchSpec", "Arena", "DecodeState", "DeviceLayer", "DeviceLinear", "DeviceWeights", "GraphSafeKV",
+    "ArchSpec", "Arena", "ChunkPrefill", "DecodeState", "DeviceLayer", "DeviceLinear", "DeviceWeights", "GraphSafeKV",
     "GreedyGraph", "PackedEmbed", "Nf4Matrix", "SynthLayer", "SynthModel", "TINY_LLAMA",
     "TINY_INTERNLM", "MEDIUM_LLAMA", "QWEN25_3B", "QWEN25_14B", "INTERNLM25_20B", "QWEN25_32B",
     "apply_rope_torch", "build", "capture_greedy", "consume_prompt", "SCHEDULES", "forward_decode",

@@ -1,18 +1,26 @@
 """Chunked prompt prefill (``gpu/decodev2/prefill.py:26-141``): at most 32 prompt
-positions per pass, linears on the MFMA GEMM, never captured into the graph."""
+positions per pass, linears on the MFMA GEMM.
+
+Two forms.  ``forward_prefill`` is the reference's sequence: token-major torch glue
+around the GEMMs, never captured.  ``ChunkPrefill`` keeps every activation in the
+GEMM's own feature-major ``[features, N]`` layout, runs the glue (RMSNorm, RoPE + cache
+write, causal attention, SwiGLU, bias/residual) as library launches, and replays each
+chunk width as a captured graph, so a layer costs its kernels and not the host's
+dispatch."""
 
 from __future__ import annotations
 
 import torch
 
-from ..nf4 import LIVE_MAX_N
+from ..nf4 import (LIVE_MAX_N, dv2_add_cols, dv2_attn_chunk, dv2_rms_cols, dv2_rope_kv_cols,
+                   dv2_swiglu_elems, nf4_gemm)
 from .embed import gather_embed
-from .linear import DeviceWeights, nf4_linear
+from .linear import DeviceLinear, DeviceWeights, nf4_linear
 from .ops import causal_attend, rms, split_qkv, swiglu
 from .rope import apply_rope_torch
 from .state import DecodeState
 
-__all__ = ["forward_prefill", "prefill_chunk_width"]
+__all__ = ["forward_prefill", "prefill_chunk_width", "ChunkPrefill"]
 
 
 def prefill_chunk_width(state: DecodeState, chunk: int | None = None) -> int:
@@ -53,3 +61,92 @@ def forward_prefill(state: DecodeState, weights: DeviceWeights, token_ids: torch
     hidden = rms(x[-1:], weights.final_norm, spec.rms_eps)
     state.arena.logits.copy_(nf4_linear(weights.lm_head, hidden).reshape(1, -1))
     state.pick_next(commit=False)
+
+
+def _gemm_cols(mat: DeviceLinear, x: torch.Tensor) -> torch.Tensor:
+    """``[K, N] -> [M, N]`` with the bias, if any, added per row."""
+    y = nf4_gemm(mat.packed, mat.scale, x, mat.M, mat.K, mat.K_pad)
+    if mat.bias is not None:
+        dv2_add_cols(y, bias=mat.bias)
+    return y
+
+
+class ChunkPrefill:
+    """Feature-major prefill of one request's prompt chunks.
+
+    ``run(ids, start, logits)`` has ``forward_prefill``'s contract.  All launches of a
+    chunk read the chunk's ids, its first cache slot and the prefix length of its first
+    token from fixed device buffers, so one captured graph per chunk width serves every
+    position (``use_graph``); without graphs the same launches are issued eagerly."""
+
+    def __init__(self, state: DecodeState, weights: DeviceWeights, *, use_graph: bool = True) -> None:
+        self.state = state
+        self.weights = weights
+        self.use_graph = bool(use_graph)
+        dev = state.device
+        spec = state.spec
+        self.ids = torch.zeros(int(LIVE_MAX_N), dtype=torch.long, device=dev)
+        self.start = torch.zeros((), dtype=torch.int64, device=dev)
+        self.first_len = torch.zeros((), dtype=torch.int32, device=dev)
+        self.last_hidden = torch.zeros(spec.hidden, dtype=torch.bfloat16, device=dev)
+        self._graphs: dict[int, torch.cuda.CUDAGraph] = {}
+
+    def _chunk(self, n: int) -> None:
+        state, weights, spec = self.state, self.weights, self.state.spec
+        x = gather_embed(weights.embed, self.ids[:n]).t().contiguous()  # [hidden, n]
+        q_rows = torch.empty((n, spec.q_dim), dtype=torch.bfloat16, device=x.device)
+        attn = torch.empty((spec.q_dim, n), dtype=torch.bfloat16, device=x.device)
+        for li, layer in enumerate(weights.layers):
+            h = dv2_rms_cols(x, layer.norm1, spec.rms_eps)
+            if layer.wqkv is not None:
+                y = _gemm_cols(layer.wqkv, h)  # rows are [Q | K | V]
+                q, k, v = y[:spec.q_dim], y[spec.q_dim:spec.q_dim + spec.kv_dim], y[spec.q_dim + spec.kv_dim:]
+            else:
+                q, k, v = _gemm_cols(layer.q, h), _gemm_cols(layer.k, h), _gemm_cols(layer.v, h)
+            k_cache, v_cache = state.kv.layer(li)
+            dv2_rope_kv_cols(q, k, v, q_rows, k_cache, v_cache, state.cos, state.sin, self.start)
+            dv2_attn_chunk(q_rows, k_cache, v_cache, attn, self.first_len, spec.attn_scale)
+            dv2_add_cols(x, _gemm_cols(layer.o, attn))
+            h = dv2_rms_cols(x, layer.norm2, spec.rms_eps)
+            act = dv2_swiglu_elems(_gemm_cols(layer.gate, h), _gemm_cols(layer.up, h))
+            dv2_add_cols(x, _gemm_cols(layer.down, act))
+        self.last_hidden.copy_(x[:, n - 1])
+
+    def _replay(self, n: int) -> None:
+        if not self.use_graph:
+            self._chunk(n)
+            return
+        g = self._graphs.get(n)
+        if g is None:
+            # one eager pass first: it sizes the GEMM's dynamic LDS and warms the allocator
+            self._chunk(n)
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                self._chunk(n)
+            self._graphs[n] = g
+            return  # the capture pass does not run; the eager pass above already did the work
+        g.replay()
+
+    def run(self, token_ids: torch.Tensor, start: int, *, logits: bool = True) -> None:
+        state, spec = self.state, self.state.spec
+        ids = token_ids.reshape(-1).to(device=state.device, dtype=torch.long)
+        n = int(ids.numel())
+        if n < 1:
+            raise ValueError("prefill chunk must be non-empty")
+        if n > int(LIVE_MAX_N):
+            raise ValueError(f"prefill chunk of {n} tokens exceeds {int(LIVE_MAX_N)}")
+        start = int(start)
+        seq = start + n
+        if start < 0 or seq > spec.max_seq:
+            raise ValueError(f"prefill {start}..{seq} exceeds max_seq={spec.max_seq}")
+        self.ids[:n].copy_(ids)
+        self.start.fill_(start)
+        self.first_len.fill_(start + 1)
+        self._replay(n)
+        state.position.fill_(seq)
+        state.valid_len.fill_(seq)
+        if not logits:
+            return
+        hidden = rms(self.last_hidden.view(1, -1), self.weights.final_norm, spec.rms_eps)
+        state.arena.logits.copy_(nf4_linear(self.weights.lm_head, hidden).reshape(1, -1))
+        state.pick_next(commit=False)

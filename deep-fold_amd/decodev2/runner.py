@@ -8,7 +8,7 @@ from collections.abc import Sequence
 import torch
 
 from .linear import DeviceWeights
-from .prefill import forward_prefill, prefill_chunk_width
+from .prefill import ChunkPrefill, forward_prefill, prefill_chunk_width
 from .state import DecodeState
 from .step import greedy_decode
 
@@ -16,9 +16,12 @@ __all__ = ["consume_prompt", "generate"]
 
 
 def consume_prompt(state: DecodeState, weights: DeviceWeights, token_ids: Sequence[int], *,
-                   chunk: int | None = None, start: int = 0) -> None:
+                   chunk: int | None = None, start: int = 0,
+                   prefill: ChunkPrefill | None = None) -> None:
     """Fill KV for ``token_ids`` starting at slot ``start`` (0 = a cold prompt after
-    ``reset``; a positive value appends a suffix to an existing prefix)."""
+    ``reset``; a positive value appends a suffix to an existing prefix).  With
+    ``prefill`` the chunks go through its feature-major launches (and graphs)
+    instead of the token-major torch glue."""
     if not len(token_ids):
         raise ValueError("prompt must be non-empty")
     ids = [int(t) for t in token_ids]
@@ -32,13 +35,17 @@ def consume_prompt(state: DecodeState, weights: DeviceWeights, token_ids: Sequen
     buf = torch.tensor(ids, dtype=torch.long, device=state.device)
     for lo in range(0, n, width):
         hi = min(lo + width, n)
-        forward_prefill(state, weights, buf[lo:hi], start=pos + lo, logits=(hi == n))
+        if prefill is not None:
+            prefill.run(buf[lo:hi], pos + lo, logits=(hi == n))
+        else:
+            forward_prefill(state, weights, buf[lo:hi], start=pos + lo, logits=(hi == n))
 
 
 def generate(state: DecodeState, weights: DeviceWeights, prompt_ids: Sequence[int], n_new: int, *,
-             step=None, ignore_eos: bool = False, chunk: int | None = None) -> list[int]:
+             step=None, ignore_eos: bool = False, chunk: int | None = None,
+             prefill: ChunkPrefill | None = None) -> list[int]:
     """Host list of new ids.  ``step`` is ``greedy_decode`` or a captured graph."""
-    consume_prompt(state, weights, prompt_ids, chunk=chunk)
+    consume_prompt(state, weights, prompt_ids, chunk=chunk, prefill=prefill)
     decode = greedy_decode if step is None else step
     out = [int(state.next_token.item())]
     if not ignore_eos:

@@ -47,6 +47,11 @@ __all__ = [
     "dv2_attn_parts",
     "dv2_gemv_attn",
     "dv2_attn",
+    "dv2_rms_cols",
+    "dv2_rope_kv_cols",
+    "dv2_attn_chunk",
+    "dv2_swiglu_elems",
+    "dv2_add_cols",
     "library_path",
 ]
 
@@ -118,6 +123,11 @@ EXPORTS = (
     ("chr_dv2_attn_parts", ctypes.c_int,
      [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _P, _P, _P, _P, _P, _P, _I]),
     ("chr_dv2_gemv_attn", ctypes.c_int, [_DP, _P, _I, _I, _I, _P, _P, _P]),
+    ("chr_dv2_rms_cols", ctypes.c_int, [_P, _P, _P, _I, _I, _F, _P]),
+    ("chr_dv2_rope_kv_cols", ctypes.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]),
+    ("chr_dv2_attn_chunk", ctypes.c_int, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _P, _I, _I, _I]),
+    ("chr_dv2_swiglu_elems", ctypes.c_int, [_P, _P, _P, ctypes.c_int64, _P]),
+    ("chr_dv2_add_cols", ctypes.c_int, [_P, _P, _P, _I, _I, _P]),
     ("chr_dv2_mark_written", ctypes.c_int, [_P, _P, _P]),
     ("chr_dv2_argmax_commit", ctypes.c_int, [_P, _I, _P, _P, _P, _P, _P, _I, _P]),
     ("chr_nf4_abi_version", ctypes.c_int, []),
@@ -705,3 +715,105 @@ def dv2_gemv_attn(packed: torch.Tensor, scale: torch.Tensor, state: torch.Tensor
                                        None if add is None else add.data_ptr(), _stream())
     _check_rc("chr_dv2_gemv_attn", rc)
     return out
+
+
+def _bf16_cuda(t: torch.Tensor, what: str) -> None:
+    _need(t.is_cuda and t.dtype == torch.bfloat16 and t.is_contiguous(),
+          f"{what} must be a contiguous CUDA bfloat16 tensor")
+
+
+def dv2_rms_cols(x: torch.Tensor, w: torch.Tensor, eps: float, out: torch.Tensor | None = None) -> torch.Tensor:
+    """RMSNorm of every column of feature-major ``x [rows, N]`` (N <= 32)."""
+    _bf16_cuda(x, "x")
+    _bf16_cuda(w, "w")
+    _need(x.dim() == 2 and w.numel() == x.size(0), "x must be [rows, N] and w hold rows elements")
+    if out is None:
+        out = torch.empty_like(x)
+    _bf16_cuda(out, "out")
+    _need(out.shape == x.shape, "out must have x's shape")
+    rc = _load_ext().chr_dv2_rms_cols(x.data_ptr(), w.data_ptr(), out.data_ptr(), int(x.size(0)),
+                                      int(x.size(1)), float(eps), _stream())
+    _check_rc("chr_dv2_rms_cols", rc)
+    return out
+
+
+def dv2_rope_kv_cols(q, k, v, q_out, k_cache, v_cache, cos, sin, start) -> None:
+    """RoPE of feature-major ``q [n_q*hd, N]`` / ``k [n_kv*hd, N]`` at positions
+    ``start + n`` (``start``: CUDA int64 scalar); rotated q goes token-major to
+    ``q_out [N, n_q*hd]``, rotated k and ``v`` to the cache rows."""
+    for t, name in ((q, "q"), (k, "k"), (v, "v"), (q_out, "q_out"), (k_cache, "k_cache"),
+                    (v_cache, "v_cache"), (cos, "cos"), (sin, "sin")):
+        _bf16_cuda(t, name)
+    _need(k_cache.dim() == 3 and v_cache.shape == k_cache.shape, "caches must be [max_seq, n_kv, hd]")
+    max_seq, n_kv, hd = (int(t) for t in k_cache.shape)
+    _need(q.dim() == 2 and k.dim() == 2 and v.shape == k.shape, "q, k, v must be [features, N]")
+    n = int(q.size(1))
+    _need(int(k.size(1)) == n and int(k.size(0)) == n_kv * hd and int(q.size(0)) % hd == 0,
+          "q, k, v feature counts must match the caches")
+    n_q = int(q.size(0)) // hd
+    _need(q_out.numel() >= n * n_q * hd, "q_out too small")
+    _need(cos.dim() == 2 and cos.size(1) == hd and cos.size(0) >= max_seq and sin.shape == cos.shape,
+          "cos/sin must be [>= max_seq, hd]")
+    _need(start.is_cuda and start.dtype == torch.int64 and start.numel() == 1,
+          "start must be a CUDA int64 scalar")
+    rc = _load_ext().chr_dv2_rope_kv_cols(q.data_ptr(), k.data_ptr(), v.data_ptr(), q_out.data_ptr(),
+                                          k_cache.data_ptr(), v_cache.data_ptr(), cos.data_ptr(),
+                                          sin.data_ptr(), start.data_ptr(), n, n_q, n_kv, hd,
+                                          max_seq, _stream())
+    _check_rc("chr_dv2_rope_kv_cols", rc)
+
+
+def dv2_attn_chunk(q, k, v, out, first_len, scale: float, n_waves: int = ATTN_WG_WAVES,
+                   feature_major: bool = True) -> None:
+    """Causal attention of a chunk: token ``t`` of ``q [N, n_q*hd]`` sees cache rows
+    ``0 .. first_len + t - 1``.  ``out`` is ``[n_q*hd, N]`` when ``feature_major`` else
+    ``[N, n_q*hd]``."""
+    _bf16_cuda(q, "q")
+    _bf16_cuda(out, "out")
+    _need(k.is_contiguous() and v.is_contiguous() and k.dim() == 3 and k.dtype == torch.bfloat16
+          and v.dtype == torch.bfloat16 and v.shape == k.shape, "caches must be contiguous bf16 [max_seq,n_kv,hd]")
+    max_seq, n_kv, hd = (int(t) for t in k.shape)
+    _need(q.dim() == 2 and int(q.size(1)) % hd == 0, "q must be [N, n_q*hd]")
+    n, n_q = int(q.size(0)), int(q.size(1)) // hd
+    _need(out.numel() == n * n_q * hd, "out must hold N*n_q*hd elements")
+    _need(first_len.is_cuda and first_len.dtype == torch.int32 and first_len.numel() == 1,
+          "first_len must be a CUDA int32 scalar")
+    _need(1 <= int(n_waves) <= 16, "n_waves must be in 1..16")
+    strides = (1, n) if feature_major else (n_q * hd, 1)
+    rc = _load_ext().chr_dv2_attn_chunk(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+                                        first_len.data_ptr(), n, n_q, n_kv, hd, int(n_waves),
+                                        float(scale), _stream(), max_seq, strides[0], strides[1])
+    _check_rc("chr_dv2_attn_chunk", rc)
+
+
+def dv2_swiglu_elems(gate: torch.Tensor, up: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """``silu(gate) * up`` elementwise on bf16 tensors of one shape."""
+    _bf16_cuda(gate, "gate")
+    _bf16_cuda(up, "up")
+    _need(gate.shape == up.shape, "gate and up must have one shape")
+    if out is None:
+        out = torch.empty_like(gate)
+    _bf16_cuda(out, "out")
+    _need(out.numel() == gate.numel(), "out must have gate's size")
+    rc = _load_ext().chr_dv2_swiglu_elems(gate.data_ptr(), up.data_ptr(), out.data_ptr(),
+                                          int(gate.numel()), _stream())
+    _check_rc("chr_dv2_swiglu_elems", rc)
+    return out
+
+
+def dv2_add_cols(y: torch.Tensor, a: torch.Tensor | None = None, bias: torch.Tensor | None = None) -> torch.Tensor:
+    """In place on feature-major ``y [rows, N]``: ``y += a (+ bias[row])`` or ``y += bias[row]``."""
+    _bf16_cuda(y, "y")
+    _need(y.dim() == 2, "y must be [rows, N]")
+    _need(a is not None or bias is not None, "give a, bias or both")
+    if a is not None:
+        _bf16_cuda(a, "a")
+        _need(a.shape == y.shape, "a must have y's shape")
+    if bias is not None:
+        _bf16_cuda(bias, "bias")
+        _need(bias.numel() == y.size(0), "bias must hold rows elements")
+    rc = _load_ext().chr_dv2_add_cols(y.data_ptr(), None if a is None else a.data_ptr(),
+                                      None if bias is None else bias.data_ptr(), int(y.size(0)),
+                                      int(y.size(1)), _stream())
+    _check_rc("chr_dv2_add_cols", rc)
+    return y

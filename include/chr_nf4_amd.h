@@ -206,6 +206,47 @@ int chr_dv2_attn_parts(const void *q, const void *k, const void *v, const void *
 int chr_dv2_gemv_attn(const chr_nf4_dev_t *w, const float *state, int32_t n_q, int32_t hd,
                       int32_t n_parts, void *y, const void *add, void *stream);
 
+/* ---- Chunked prefill glue on the GEMM's own layout -----------------------------------------
+ * The reference's prefill (gpu/decodev2/prefill.py:58-133) runs everything but its linears as
+ * stock torch ops on token-major [N, features] tensors and transposes around every GEMM
+ * (gpu/decodev2/linear.py:96-113).  These entries do the same arithmetic directly on the
+ * feature-major [features, N] bf16 tiles chr_nf4_gemm reads and writes (N <= 32 tokens of one
+ * chunk, token index fastest), so a prefill layer is a straight sequence of launches that can
+ * be captured in a graph.  None has a counterpart in the reference's C-ABI. */
+
+/* y[k][n] = (w[k] * x[k][n]) * rsqrt(mean_k x[k][n]^2 + eps) per column n
+ * (gpu/decodev2/ops.py:18-20).  -2 when N is outside 1..32. */
+int chr_dv2_rms_cols(const void *x, const void *w, void *y, int32_t rows, int32_t N, float eps,
+                     void *stream);
+
+/* Rotate-half RoPE of q [n_q*hd, N] and k [n_kv*hd, N] at positions *start + n
+ * (start: device int64), writing rotated q token-major to q_out [N, n_q*hd] and rotated k
+ * and v to cache rows *start + n of [max_seq, n_kv, hd] (gpu/decodev2/prefill.py:100-108).
+ * Tokens whose row would fall outside the cache are skipped. */
+int chr_dv2_rope_kv_cols(const void *q, const void *k, const void *v, void *q_out,
+                         void *k_cache, void *v_cache, const void *cos, const void *sin,
+                         const void *start, int32_t N, int32_t n_q, int32_t n_kv, int32_t hd,
+                         int32_t max_seq, void *stream);
+
+/* Causal attention of a chunk (gpu/decodev2/ops.py:31-44): token t of q [n_tok, n_q*hd]
+ * attends to cache rows 0 .. *first_len + t - 1 (first_len: device int32, the prefix length
+ * token 0 sees, itself included), one workgroup of n_waves (<= 16) wavefronts per
+ * (head, token).  out[t*out_tok_stride + (head*hd + d)*out_dim_stride]: strides (n_q*hd, 1)
+ * give token-major output, (1, N) feature-major. */
+int chr_dv2_attn_chunk(const void *q, const void *k, const void *v, void *out,
+                       const void *first_len, int32_t n_tok, int32_t n_q, int32_t n_kv,
+                       int32_t hd, int32_t n_waves, float scale, void *stream, int32_t max_seq,
+                       int32_t out_tok_stride, int32_t out_dim_stride);
+
+/* y = silu(gate) * up over `count` bf16 elements, the activation rounded to bf16 before the
+ * product as torch's two ops round (gpu/decodev2/ops.py:23-24). */
+int chr_dv2_swiglu_elems(const void *gate, const void *up, void *y, int64_t count, void *stream);
+
+/* Feature-major residual/bias: with a, y = y + (a [+ bias[row]]); with a NULL, y += bias[row];
+ * every sum rounded to bf16 (gpu/decodev2/linear.py:114-116, prefill.py:113,133). */
+int chr_dv2_add_cols(void *y, const void *a, const void *bias, int32_t rows, int32_t N,
+                     void *stream);
+
 /* Library version, for the loader's sanity check. */
 int chr_nf4_abi_version(void);
 

@@ -1,0 +1,240 @@
+"""GPU parity of the feature-major prefill glue (RMSNorm, RoPE + cache write, chunk
+attention, SwiGLU, bias/residual) and of the chunked prefill built from it."""
+
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from deepfold_amd import decodev2 as dv2
+from deepfold_amd import nf4
+from deepfold_amd.decodev2.synth import build
+from oracle import nf4_oracle as oc
+from oracle import step_oracle as so
+
+from helpers import DEV, bf16_bits, bf16_tensor, to_f32
+from test_nf4_kernels import attn_ref, rope_tables, rot_half
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+def rnd(shape, seed, scale=1.0):
+    rng = np.random.default_rng(seed)
+    return oc.bf16_round((rng.standard_normal(shape) * scale).astype(np.float32))
+
+
+@pytest.mark.parametrize("rows,n", [(64, 1), (256, 7), (5120, 32), (1000, 16), (2050, 31)])
+def test_rms_cols(rows, n):
+    say("rms_cols", rows, n)
+    x = rnd((rows, n), rows + n, 1.5)
+    w = rnd((rows,), 3, 1.0)
+    eps = 1e-6
+    got = to_f32(nf4.dv2_rms_cols(bf16_tensor(x), bf16_tensor(w), eps))
+    x64 = x.astype(np.float64)
+    ref = x64 * w.astype(np.float64)[:, None] / np.sqrt((x64 ** 2).mean(axis=0, keepdims=True) + eps)
+    assert np.abs(got - ref).max() <= 2 ** -7 * max(1.0, np.abs(ref).max())
+    # the N=1 kernel of the decode step is the same arithmetic, column by column
+    for c in (0, n - 1):
+        y = torch.empty(rows, dtype=torch.bfloat16, device=DEV)
+        nf4.nf4_rms(bf16_tensor(np.ascontiguousarray(x[:, c])), bf16_tensor(w), y, eps)
+        assert np.abs(to_f32(y) - got[:, c]).max() <= 2 ** -7 * max(1.0, np.abs(ref).max())
+    # library cross-check
+    t = F.rms_norm(bf16_tensor(np.ascontiguousarray(x.T)).float(), (rows,), bf16_tensor(w).float(), eps)
+    assert np.abs(got - t.cpu().numpy().T).max() <= 2 ** -7 * max(1.0, np.abs(ref).max())
+
+
+def test_rms_cols_rejects_wide_chunks():
+    x = torch.zeros((64, 33), dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(RuntimeError):
+        nf4.dv2_rms_cols(x, torch.ones(64, dtype=torch.bfloat16, device=DEV), 1e-6)
+
+
+@pytest.mark.parametrize("n_q,n_kv,hd,n,start", [(4, 2, 16, 5, 0), (16, 2, 128, 32, 40),
+                                                 (6, 3, 256, 3, 61), (8, 8, 64, 32, 0)])
+def test_rope_kv_cols(n_q, n_kv, hd, n, start):
+    say("rope_kv_cols", n_q, n_kv, hd, n, start)
+    max_seq = 96
+    cos, sin = rope_tables(max_seq, hd)
+    q = rnd((n_q * hd, n), 1)
+    k = rnd((n_kv * hd, n), 2)
+    v = rnd((n_kv * hd, n), 3)
+    kc = torch.zeros((max_seq, n_kv, hd), dtype=torch.bfloat16, device=DEV)
+    vc = torch.zeros_like(kc)
+    q_rows = torch.zeros((n, n_q * hd), dtype=torch.bfloat16, device=DEV)
+    dcos, dsin = bf16_tensor(cos), bf16_tensor(sin)
+    nf4.dv2_rope_kv_cols(bf16_tensor(q), bf16_tensor(k), bf16_tensor(v), q_rows, kc, vc, dcos, dsin,
+                         torch.tensor(start, dtype=torch.int64, device=DEV))
+    for t in range(n):
+        c, s = cos[start + t], sin[start + t]
+        qr = rot_half(q[:, t].reshape(n_q, hd).astype(np.float64), c, s)
+        kr = rot_half(k[:, t].reshape(n_kv, hd).astype(np.float64), c, s)
+        assert np.abs(to_f32(q_rows[t]).reshape(n_q, hd) - qr).max() <= 2 ** -6
+        assert np.abs(to_f32(kc[start + t]) - kr).max() <= 2 ** -6
+        assert (to_f32(vc[start + t]) == v[:, t].reshape(n_kv, hd)).all()
+        # bit for bit the decode step's one-token kernel
+        dq = bf16_tensor(np.ascontiguousarray(q[:, t]).reshape(n_q, hd))
+        dk = bf16_tensor(np.ascontiguousarray(k[:, t]).reshape(n_kv, hd))
+        dv = bf16_tensor(np.ascontiguousarray(v[:, t]).reshape(n_kv, hd))
+        kc1 = torch.zeros_like(kc)
+        vc1 = torch.zeros_like(kc)
+        nf4.nf4_rope_kv(dq, dk, dv, kc1, vc1, dcos, dsin,
+                        torch.tensor(start + t, dtype=torch.int64, device=DEV))
+        assert (bf16_bits(dq).reshape(-1) == bf16_bits(q_rows[t]).reshape(-1)).all()
+        assert (bf16_bits(kc1[start + t]) == bf16_bits(kc[start + t])).all()
+    assert (to_f32(kc[:start]) == 0).all() and (to_f32(kc[start + n:]) == 0).all()
+    assert (to_f32(vc[:start]) == 0).all() and (to_f32(vc[start + n:]) == 0).all()
+
+
+def test_rope_kv_cols_skips_rows_past_the_cache():
+    n_q, n_kv, hd, n, max_seq = 2, 1, 16, 4, 8
+    cos, sin = rope_tables(max_seq, hd)
+    kc = torch.zeros((max_seq, n_kv, hd), dtype=torch.bfloat16, device=DEV)
+    vc = torch.zeros_like(kc)
+    q_rows = torch.zeros((n, n_q * hd), dtype=torch.bfloat16, device=DEV)
+    nf4.dv2_rope_kv_cols(bf16_tensor(rnd((n_q * hd, n), 1)), bf16_tensor(rnd((n_kv * hd, n), 2)),
+                         bf16_tensor(rnd((n_kv * hd, n), 3)), q_rows, kc, vc, bf16_tensor(cos),
+                         bf16_tensor(sin), torch.tensor(6, dtype=torch.int64, device=DEV))
+    torch.cuda.synchronize()
+    assert (to_f32(kc[:6]) == 0).all() and (to_f32(kc[6:]) != 0).any()
+    assert (to_f32(q_rows[2:]) == 0).all()
+
+
+@pytest.mark.parametrize("n_q,n_kv,hd,max_seq,first,n,waves", [
+    (4, 2, 16, 64, 1, 8, 16), (16, 2, 128, 256, 100, 32, 16), (40, 8, 128, 600, 481, 32, 16),
+    (6, 3, 256, 80, 40, 5, 4), (4, 2, 48, 64, 1, 32, 1), (8, 8, 64, 40, 9, 32, 16)])
+def test_attn_chunk(n_q, n_kv, hd, max_seq, first, n, waves):
+    say("attn_chunk", n_q, n_kv, hd, max_seq, first, n, waves)
+    q = rnd((n, n_q * hd), 11)
+    kc = rnd((max_seq, n_kv, hd), 12)
+    vc = rnd((max_seq, n_kv, hd), 13)
+    last = first + n - 1
+    kc[last:] = 1e4  # rows no token of the chunk may see
+    vc[last:] = -1e4
+    scale = hd ** -0.5
+    dq, dk, dv = bf16_tensor(q), bf16_tensor(kc), bf16_tensor(vc)
+    fl = torch.tensor(first, dtype=torch.int32, device=DEV)
+    out_f = torch.zeros((n_q * hd, n), dtype=torch.bfloat16, device=DEV)
+    out_t = torch.zeros((n, n_q * hd), dtype=torch.bfloat16, device=DEV)
+    nf4.dv2_attn_chunk(dq, dk, dv, out_f, fl, scale, n_waves=waves)
+    nf4.dv2_attn_chunk(dq, dk, dv, out_t, fl, scale, n_waves=waves, feature_major=False)
+    assert (bf16_bits(out_f.t().contiguous()) == bf16_bits(out_t)).all()
+    got = to_f32(out_t)
+    one = torch.zeros(n_q * hd, dtype=torch.bfloat16, device=DEV)
+    for t in range(n):
+        ref = attn_ref(q[t].reshape(n_q, hd).astype(np.float64), kc.astype(np.float64),
+                       vc.astype(np.float64), first + t, scale, n_q // n_kv)
+        assert np.abs(got[t].reshape(n_q, hd) - ref).max() <= 0.02, t
+        # bit for bit the decode step's attention at the same prefix length
+        nf4.dv2_attn(dq[t].view(n_q, hd), dk, dv, one, torch.tensor(first + t, dtype=torch.int32, device=DEV), scale,
+                     n_waves=waves)
+        assert (bf16_bits(one) == bf16_bits(out_t[t])).all(), t
+
+
+def test_attn_chunk_clamps_to_the_cache():
+    n_q, n_kv, hd, max_seq, n = 2, 1, 16, 8, 4
+    q, kc, vc = rnd((n, n_q * hd), 1), rnd((max_seq, n_kv, hd), 2), rnd((max_seq, n_kv, hd), 3)
+    out = torch.zeros((n, n_q * hd), dtype=torch.bfloat16, device=DEV)
+    nf4.dv2_attn_chunk(bf16_tensor(q), bf16_tensor(kc), bf16_tensor(vc), out,
+                       torch.tensor(7, dtype=torch.int32, device=DEV), hd ** -0.5, feature_major=False)
+    ref = attn_ref(q[3].reshape(n_q, hd).astype(np.float64), kc.astype(np.float64),
+                   vc.astype(np.float64), max_seq, hd ** -0.5, 2)
+    assert np.abs(to_f32(out[3]).reshape(n_q, hd) - ref).max() <= 0.02
+
+
+@pytest.mark.parametrize("shape", [(13824, 32), (100, 3), (1, 1)])
+def test_swiglu_elems(shape):
+    g, u = rnd(shape, 5, 2.0), rnd(shape, 6, 1.0)
+    got = nf4.dv2_swiglu_elems(bf16_tensor(g), bf16_tensor(u))
+    want = F.silu(bf16_tensor(g)) * bf16_tensor(u)
+    d = np.abs(to_f32(got) - to_f32(want))
+    # expf against torch's exponential: at most one bf16 step of the result
+    assert (d <= 2 ** -7 * np.maximum(np.abs(to_f32(want)), 2 ** -20)).all()
+    g64 = g.astype(np.float64)
+    ref = g64 / (1 + np.exp(-g64)) * u
+    assert np.abs(to_f32(got) - ref).max() <= 2 ** -6 * max(1.0, np.abs(ref).max())
+
+
+def test_add_cols():
+    rows, n = 300, 17
+    y, a, b = rnd((rows, n), 1), rnd((rows, n), 2), rnd((rows,), 3)
+    dy, da, db = bf16_tensor(y), bf16_tensor(a), bf16_tensor(b)
+    want = dy + (da + db[:, None])
+    nf4.dv2_add_cols(dy, da, db)
+    assert (bf16_bits(dy) == bf16_bits(want)).all()
+    dy = bf16_tensor(y)
+    nf4.dv2_add_cols(dy, da)
+    assert (bf16_bits(dy) == bf16_bits(bf16_tensor(y) + da)).all()
+    dy = bf16_tensor(y)
+    nf4.dv2_add_cols(dy, bias=db)
+    assert (bf16_bits(dy) == bf16_bits(bf16_tensor(y) + db[:, None])).all()
+    with pytest.raises(RuntimeError):
+        nf4.dv2_add_cols(dy)
+
+
+# ---- the chunked prefill built from them ------------------------------------------------
+
+LONG = [4, 5, 6, 7, 1, 2, 3, 4]
+
+
+def session(spec, seed, packed_embed=False):
+    model = build(spec, seed, packed_embed=packed_embed)
+    weights = dv2.DeviceWeights.from_synth(model, "cuda")
+    state = dv2.DecodeState.allocate(spec, device="cuda")
+    return model, state, weights
+
+
+@pytest.mark.parametrize("spec,seed", [(dv2.TINY_LLAMA, 0), (dv2.TINY_INTERNLM, 1), (dv2.MEDIUM_LLAMA, 0)])
+@pytest.mark.parametrize("use_graph", [False, True])
+def test_feature_major_prefill_gives_the_oracle_ids(spec, seed, use_graph):
+    say("chunk prefill", spec.name, use_graph)
+    model, state, weights = session(spec, seed)
+    want = so.greedy_ids(model, LONG, 6)
+    pre = dv2.ChunkPrefill(state, weights, use_graph=use_graph)
+    for chunk in (2, 3, 8, None):
+        for _ in range(2):  # the second pass replays the graphs the first one captured
+            state.reset()
+            got = dv2.generate(state, weights, LONG, 6, chunk=chunk, prefill=pre)
+            assert got == want, chunk
+            assert int(state.valid_len.item()) == len(LONG) + len(got) - 1
+
+
+def test_feature_major_prefill_tracks_the_torch_glue():
+    spec = dv2.MEDIUM_LLAMA
+    rng = np.random.default_rng(0)
+    prompt = [int(t) for t in rng.integers(0, spec.vocab, size=min(70, spec.max_seq - 8))]
+    _, a, w = session(spec, 2, packed_embed=True)
+    b = dv2.DecodeState.allocate(spec, device="cuda")
+    dv2.consume_prompt(a, w, prompt)
+    pre = dv2.ChunkPrefill(b, w)
+    dv2.consume_prompt(b, w, prompt, prefill=pre)
+    n = len(prompt)
+    assert int(a.valid_len.item()) == int(b.valid_len.item()) == n
+    ka, kb = a.kv.k[:, :n].float(), b.kv.k[:, :n].float()
+    va, vb = a.kv.v[:, :n].float(), b.kv.v[:, :n].float()
+    assert (ka - kb).abs().max().item() <= 0.03 * max(1.0, ka.abs().max().item())
+    assert (va - vb).abs().max().item() <= 0.03 * max(1.0, va.abs().max().item())
+    la, lb = a.arena.logits.float().view(-1), b.arena.logits.float().view(-1)
+    assert (la - lb).abs().max().item() <= 0.03 * max(1.0, la.abs().max().item())
+    # a replay of the captured graphs on a fresh request gives the same bits as its first run
+    first = b.kv.k[:, :n].clone(), b.arena.logits.clone()
+    b.reset()
+    dv2.consume_prompt(b, w, prompt, prefill=pre)
+    assert torch.equal(first[0], b.kv.k[:, :n]) and torch.equal(first[1], b.arena.logits)
+
+
+def test_chunk_prefill_errors():
+    spec = dv2.TINY_LLAMA
+    _, state, w = session(spec, 0)
+    pre = dv2.ChunkPrefill(state, w, use_graph=False)
+    with pytest.raises(ValueError):
+        pre.run(torch.zeros(0, dtype=torch.long), 0)
+    with pytest.raises(ValueError):
+        pre.run(torch.zeros(33, dtype=torch.long), 0)
+    with pytest.raises(ValueError):
+        pre.run(torch.zeros(4, dtype=torch.long), spec.max_seq - 2)
