@@ -215,6 +215,29 @@ __device__ __forceinline__ Levels8 lookup8(uint32_t w, const float *lut) {
   return r;
 }
 
+// lookup8 for a kernel whose 16 levels sit at LDS address 0 and whose LDS is all dynamic
+// (the compiler then does not know the base and would add it to every offset): the byte
+// offset is the whole address.
+__device__ __forceinline__ float lds0_at(uint32_t off) {
+  return *reinterpret_cast<const __attribute__((address_space(3))) float *>(off);
+}
+
+__device__ __forceinline__ Levels8 lookup8_lds0(uint32_t w) {
+  const uint32_t ev = w << 2;
+  const uint32_t od = w >> 2;
+  const uint32_t mask = 0x3Cu;
+  Levels8 r;
+  r.l[0] = lds0_at(and_byte<0>(ev, mask));
+  r.l[1] = lds0_at(and_byte<0>(od, mask));
+  r.l[2] = lds0_at(and_byte<1>(ev, mask));
+  r.l[3] = lds0_at(and_byte<1>(od, mask));
+  r.l[4] = lds0_at(and_byte<2>(ev, mask));
+  r.l[5] = lds0_at(and_byte<2>(od, mask));
+  r.l[6] = lds0_at(and_byte<3>(ev, mask));
+  r.l[7] = lds0_at(and_byte<3>(od, mask));
+  return r;
+}
+
 // Compute units of the current device (256 on an MI355X), cached after the first call.
 inline int device_cu_count() {
   static int cached = [] {

@@ -109,20 +109,22 @@ int resolved_one_wave() {
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
-// split so that grid_x * split reaches two workgroups per compute unit, capped at
-// kMaxAutoSplit and at the number of K tiles; split is recomputed from tiles_per_split so the
-// pair always agrees with what the kernel indexes
-// (gpu/nf4/nf4_gemm.cu:1526-1543).
-constexpr int kMaxAutoSplit = 8;
+// Split-K.  A workgroup is quickest with about three K tiles (measured at every 14B linear
+// shape, N = 8 and 32: fewer tiles leave the fetch latency uncovered, more leave compute units
+// idle), so split = ceil(n_ktiles / 3), as long as the grid stays within the four workgroups
+// a compute unit holds at once; split is recomputed from tiles_per_split so the pair always
+// agrees with what the kernel indexes (gpu/nf4/nf4_gemm.cu:1526-1543).
+constexpr int kTilesPerSplit = 3;
+constexpr int kResidentPerCu = 4;
+constexpr int kMaxAutoSplit = 32;
 
 void pick_split(int grid_x, int n_ktiles, int have_ws, int *split, int *tiles_per_split) {
   const Tuning &t = tuning();
   int want = 1;
   if (have_ws) {
-    // two workgroups per compute unit: more splits were measured to cost as much in fp32
-    // partials (long-K shapes) as they win in occupancy
-    const int target = resolved_one_wave() * 2;
-    want = t.split_k > 0 ? t.split_k : std::min(kMaxAutoSplit, ceil_div(target, grid_x));
+    const int room = (resolved_one_wave() * kResidentPerCu) / grid_x;
+    const int by_tiles = ceil_div(n_ktiles, kTilesPerSplit);
+    want = t.split_k > 0 ? t.split_k : std::min(kMaxAutoSplit, std::min(by_tiles, room));
   }
   want = std::max(1, std::min(want, n_ktiles));
   const int tps = ceil_div(n_ktiles, want);
@@ -315,7 +317,9 @@ __global__ __launch_bounds__(kGemmBlock) void gemm_mfma(const uint8_t *__restric
                                                         uint16_t *__restrict__ y,
                                                         float *__restrict__ partial, int M, int K,
                                                         int K_pad, int N, int n_ktiles,
-                                                        int tiles_per_split) {
+                                                        int tiles_per_split,
+                                                        const uint16_t *__restrict__ bias,
+                                                        const uint16_t *res) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   GemmLds &lds = *reinterpret_cast<GemmLds *>(lds_raw);
   if (threadIdx.x < 16) {
@@ -380,7 +384,7 @@ __global__ __launch_bounds__(kGemmBlock) void gemm_mfma(const uint8_t *__restric
       bf16x8 b[4];
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
-        lv[t] = lookup8(w[t], lds.lut);
+        lv[t] = lookup8_lds0(w[t]);  // lds.lut is at LDS address 0
         b[t] = *reinterpret_cast<const bf16x8 *>(xl + kk + 8 * t);
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -426,7 +430,17 @@ __global__ __launch_bounds__(kGemmBlock) void gemm_mfma(const uint8_t *__restric
       for (int i = 0; i < 16; ++i) {
         const int r = rbase + 8 * (i >> 2) + (i & 3);
         if (r < M) {
-          y[static_cast<size_t>(r) * N + n] = f32_to_bf16(acc[i]);
+          // unsplit: the epilogue of reduce_splitk, here (res may alias y: same thread,
+          // same element)
+          const size_t at = static_cast<size_t>(r) * N + n;
+          uint16_t v = f32_to_bf16(acc[i]);
+          if (bias != nullptr) {
+            v = f32_to_bf16(bf16_to_f32(v) + bf16_to_f32(bias[r]));
+          }
+          if (res != nullptr) {
+            v = f32_to_bf16(bf16_to_f32(res[at]) + bf16_to_f32(v));
+          }
+          y[at] = v;
         }
       }
     } else {
@@ -442,10 +456,13 @@ __global__ __launch_bounds__(kGemmBlock) void gemm_mfma(const uint8_t *__restric
   }
 }
 
-// y[i] = bf16( sum over splits, in split order, of partial[s][i] ).
+// y[i] = bf16( sum over splits, in split order, of partial[s][i] ), then optionally
+// bf16(y + bias[row]) and bf16(res[i] + y): the roundings of separate bias and residual adds.
 __global__ __launch_bounds__(256) void reduce_splitk(const float *__restrict__ partial,
                                                      uint16_t *__restrict__ y, int rows,
-                                                     int split) {
+                                                     int split, int N,
+                                                     const uint16_t *__restrict__ bias,
+                                                     const uint16_t *res) {
   const int i = blockIdx.x * 256 + threadIdx.x;
   if (i >= rows) {
     return;
@@ -454,7 +471,14 @@ __global__ __launch_bounds__(256) void reduce_splitk(const float *__restrict__ p
   for (int j = 0; j < split; ++j) {
     s += partial[static_cast<size_t>(j) * rows + i];
   }
-  y[i] = f32_to_bf16(s);
+  uint16_t v = f32_to_bf16(s);
+  if (bias != nullptr) {
+    v = f32_to_bf16(bf16_to_f32(v) + bf16_to_f32(bias[i / N]));
+  }
+  if (res != nullptr) {
+    v = f32_to_bf16(bf16_to_f32(res[i]) + bf16_to_f32(v));
+  }
+  y[i] = v;
 }
 
 // The kernels use more than the default 64 KB of LDS: raise the limit once per process
@@ -500,8 +524,12 @@ extern "C" int chr_nf4_gemm_plan(const chr_nf4_dev_t *w, int32_t N, int32_t have
   return plan_impl(h, N, have_ws, out);
 }
 
-extern "C" int chr_nf4_gemm_ws_max(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N,
-                                   float *ws, int64_t ws_floats, void *stream, int32_t max_n) {
+namespace chr {
+namespace {
+
+int gemm_launch(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N, float *ws,
+                int64_t ws_floats, void *stream, int32_t max_n, const void *bias,
+                const void *res) {
   if (x == nullptr || y == nullptr) {
     return -1;
   }
@@ -520,6 +548,9 @@ extern "C" int chr_nf4_gemm_ws_max(const chr_nf4_dev_t *w, const void *x, void *
     return -5;
   }
   if (N == 1) {
+    if (bias != nullptr || res != nullptr) {
+      return -2;  // the fused epilogue belongs to the tiles (N >= 2)
+    }
     return gemv_entry(&h, x, y, stream, nullptr, nullptr, 0.f);
   }
   const int have_ws = (ws != nullptr && ws_floats > 0) ? 1 : 0;
@@ -539,18 +570,35 @@ extern "C" int chr_nf4_gemm_ws_max(const chr_nf4_dev_t *w, const void *x, void *
   if (vec) {
     gemm_mfma<true><<<grid, dim3(kGemmBlock), kGemmLds, st>>>(
         h.packed, h.scale, static_cast<const uint16_t *>(x), static_cast<uint16_t *>(y), partial,
-        h.M, h.K, h.K_pad, N, p.n_ktiles, p.tiles_per_split);
+        h.M, h.K, h.K_pad, N, p.n_ktiles, p.tiles_per_split,
+        static_cast<const uint16_t *>(bias), static_cast<const uint16_t *>(res));
   } else {
     gemm_mfma<false><<<grid, dim3(kGemmBlock), kGemmLds, st>>>(
         h.packed, h.scale, static_cast<const uint16_t *>(x), static_cast<uint16_t *>(y), partial,
-        h.M, h.K, h.K_pad, N, p.n_ktiles, p.tiles_per_split);
+        h.M, h.K, h.K_pad, N, p.n_ktiles, p.tiles_per_split,
+        static_cast<const uint16_t *>(bias), static_cast<const uint16_t *>(res));
   }
   if (partial != nullptr) {
     const int rows = h.M * N;
     reduce_splitk<<<dim3(static_cast<unsigned>(ceil_div(rows, 256))), dim3(256), 0, st>>>(
-        partial, static_cast<uint16_t *>(y), rows, p.grid_y);
+        partial, static_cast<uint16_t *>(y), rows, p.grid_y, N,
+        static_cast<const uint16_t *>(bias), static_cast<const uint16_t *>(res));
   }
   return launch_rc();
+}
+
+}  // namespace
+}  // namespace chr
+
+extern "C" int chr_nf4_gemm_ws_max(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N,
+                                   float *ws, int64_t ws_floats, void *stream, int32_t max_n) {
+  return gemm_launch(w, x, y, N, ws, ws_floats, stream, max_n, nullptr, nullptr);
+}
+
+extern "C" int chr_dv2_gemm_add(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N,
+                                float *ws, int64_t ws_floats, const void *bias,
+                                const void *residual, void *stream) {
+  return gemm_launch(w, x, y, N, ws, ws_floats, stream, kLiveMaxN, bias, residual);
 }
 
 extern "C" int chr_nf4_gemm_ws(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N,

@@ -63,11 +63,19 @@ def forward_prefill(state: DecodeState, weights: DeviceWeights, token_ids: torch
     state.pick_next(commit=False)
 
 
-def _gemm_cols(mat: DeviceLinear, x: torch.Tensor) -> torch.Tensor:
-    """``[K, N] -> [M, N]`` with the bias, if any, added per row."""
+def _gemm_cols(mat: DeviceLinear, x: torch.Tensor, residual: torch.Tensor | None = None) -> torch.Tensor:
+    """``[K, N] -> [M, N]`` with the bias, if any, added per row; with ``residual`` the
+    result is added to it in place.  One column (a one-token chunk) goes to the GEMV and
+    takes its bias and residual from separate launches."""
+    if x.size(1) >= 2:
+        return nf4_gemm(mat.packed, mat.scale, x, mat.M, mat.K, mat.K_pad, bias=mat.bias,
+                        residual=residual)
     y = nf4_gemm(mat.packed, mat.scale, x, mat.M, mat.K, mat.K_pad)
     if mat.bias is not None:
         dv2_add_cols(y, bias=mat.bias)
+    if residual is not None:
+        dv2_add_cols(residual, y)
+        return residual
     return y
 
 
@@ -106,10 +114,10 @@ class ChunkPrefill:
             k_cache, v_cache = state.kv.layer(li)
             dv2_rope_kv_cols(q, k, v, q_rows, k_cache, v_cache, state.cos, state.sin, self.start)
             dv2_attn_chunk(q_rows, k_cache, v_cache, attn, self.first_len, spec.attn_scale)
-            dv2_add_cols(x, _gemm_cols(layer.o, attn))
+            _gemm_cols(layer.o, attn, residual=x)
             h = dv2_rms_cols(x, layer.norm2, spec.rms_eps)
             act = dv2_swiglu_elems(_gemm_cols(layer.gate, h), _gemm_cols(layer.up, h))
-            dv2_add_cols(x, _gemm_cols(layer.down, act))
+            _gemm_cols(layer.down, act, residual=x)
         self.last_hidden.copy_(x[:, n - 1])
 
     def _replay(self, n: int) -> None:

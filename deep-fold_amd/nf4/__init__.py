@@ -128,6 +128,7 @@ EXPORTS = (
     ("chr_dv2_attn_chunk", ctypes.c_int, [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _P, _I, _I, _I]),
     ("chr_dv2_swiglu_elems", ctypes.c_int, [_P, _P, _P, ctypes.c_int64, _P]),
     ("chr_dv2_add_cols", ctypes.c_int, [_P, _P, _P, _I, _I, _P]),
+    ("chr_dv2_gemm_add", ctypes.c_int, [_DP, _P, _P, _I, _P, ctypes.c_int64, _P, _P, _P]),
     ("chr_dv2_mark_written", ctypes.c_int, [_P, _P, _P]),
     ("chr_dv2_argmax_commit", ctypes.c_int, [_P, _I, _P, _P, _P, _P, _P, _I, _P]),
     ("chr_nf4_abi_version", ctypes.c_int, []),
@@ -261,9 +262,12 @@ def nf4_set_tuning(path: int = 0, split_k: int = 0, one_wave: int = 0) -> None:
 
 
 def nf4_gemm(packed: torch.Tensor, scale: torch.Tensor, x: torch.Tensor, M: int, K: int,  # noqa: N803
-             K_pad: int, max_n: int = LIVE_MAX_N) -> torch.Tensor:  # noqa: N803
+             K_pad: int, max_n: int = LIVE_MAX_N, *, bias: torch.Tensor | None = None,  # noqa: N803
+             residual: torch.Tensor | None = None) -> torch.Tensor:
     """Fused NF4 dequant-MFMA GEMM.  ``x`` is bf16 ``[K, N]`` or ``[K]``; returns
-    ``y [M, N]`` (``gpu/nf4/__init__.py:151-176``, ``bindings.cpp:35-97``)."""
+    ``y [M, N]`` (``gpu/nf4/__init__.py:151-176``, ``bindings.cpp:35-97``).  With
+    ``bias`` (bf16 ``[M]``) and/or ``residual`` (bf16 ``[M, N]``, N >= 2) the result is
+    ``residual + (y + bias)``, written over ``residual``, in the same launches."""
     n = 1 if x.dim() == 1 else int(x.size(-1))
     cap = int(max_n)
     if cap < 1 or cap > PLAN_MAX_N:
@@ -291,9 +295,21 @@ def nf4_gemm(packed: torch.Tensor, scale: torch.Tensor, x: torch.Tensor, M: int,
     if p.ws_floats > 0:
         ws = torch.empty(int(p.ws_floats), dtype=torch.float32, device=x.device)
         ws_ptr = ws.data_ptr()
-    rc = lib.chr_nf4_gemm_ws_max(ctypes.byref(w), x.data_ptr(), y.data_ptr(), n, ws_ptr,
-                                 int(p.ws_floats), _stream(), cap)
-    _check_rc("chr_nf4_gemm", rc)
+    if bias is None and residual is None:
+        rc = lib.chr_nf4_gemm_ws_max(ctypes.byref(w), x.data_ptr(), y.data_ptr(), n, ws_ptr,
+                                     int(p.ws_floats), _stream(), cap)
+        _check_rc("chr_nf4_gemm", rc)
+        return y
+    _need(n >= 2 and n <= LIVE_MAX_N, "bias/residual ride on the N = 2..32 tiles")
+    for t, numel, name in ((bias, M, "bias"), (residual, M * n, "residual")):
+        _need(t is None or (t.is_cuda and t.dtype == torch.bfloat16 and t.is_contiguous()
+                            and t.numel() == numel), f"{name} must be contiguous CUDA bf16 of {numel} elements")
+    if residual is not None:
+        y = residual.view(M, n)
+    rc = lib.chr_dv2_gemm_add(ctypes.byref(w), x.data_ptr(), y.data_ptr(), n, ws_ptr, int(p.ws_floats),
+                              None if bias is None else bias.data_ptr(),
+                              None if residual is None else residual.data_ptr(), _stream())
+    _check_rc("chr_dv2_gemm_add", rc)
     return y
 
 

@@ -11,7 +11,8 @@ are ``M``, in features ``K``):
 
 * ``N == 1``  row-streaming GEMV, no split-K (path ``GEMV``).
 * ``N = 2..16`` / ``17..32``  MFMA tile, 128 rows x 32 columns per workgroup,
-  split-K over ``grid_y`` (paths ``PREFILL`` / ``PREFILL_N32``).
+  split-K over ``grid_y`` at about three K tiles per workgroup while the grid fits
+  the four workgroups a compute unit holds (paths ``PREFILL`` / ``PREFILL_N32``).
 * ``N = 33..64``  described by the planner, never launched (``PREFILL_N64``).
 """
 
@@ -53,7 +54,9 @@ PLAN_MAX_N = 64
 _BM = 128
 _BK = 256
 _BLOCK = 256
-_MAX_AUTO_SPLIT = 8
+_MAX_AUTO_SPLIT = 32
+_TILES_PER_SPLIT = 3
+_RESIDENT_PER_CU = 4
 # codebook, staged activation tile (bf16, padded rows), and per wavefront (4) a weight area
 # (32 rows of BK/2 + 16 bytes) and the tile's group scales
 _X_LDS = 64 + 32 * (_BK + 8) * 2 + 4 * 32 * (_BK // 2 + 16) + 4 * 32 * (_BK // 64) * 2
@@ -107,8 +110,9 @@ def _pick_split(grid_x: int, n_ktiles: int, have_ws: bool, force_split: int,
                 one_wave: int) -> tuple[int, int]:
     want = 1
     if have_ws:
-        target = max(1, int(one_wave) * 2)
-        want = force_split if force_split > 0 else min(_MAX_AUTO_SPLIT, _ceil_div(target, grid_x))
+        room = (int(one_wave) * _RESIDENT_PER_CU) // grid_x
+        by_tiles = _ceil_div(n_ktiles, _TILES_PER_SPLIT)
+        want = force_split if force_split > 0 else min(_MAX_AUTO_SPLIT, by_tiles, room)
     want = max(1, min(want, n_ktiles))
     tiles_per_split = _ceil_div(n_ktiles, want)
     return _ceil_div(n_ktiles, tiles_per_split), tiles_per_split

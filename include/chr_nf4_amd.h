@@ -247,6 +247,14 @@ int chr_dv2_swiglu_elems(const void *gate, const void *up, void *y, int64_t coun
 int chr_dv2_add_cols(void *y, const void *a, const void *bias, int32_t rows, int32_t N,
                      void *stream);
 
+/* chr_nf4_gemm_ws with the epilogue of the reference's linear + residual
+ * (gpu/decodev2/linear.py:114-116, prefill.py:113,133) folded into the split-K reduction:
+ * y = residual + (bf16(W x) + bias[row]), each step rounded to bf16 as the separate torch
+ * adds round; bias (bf16 [M]) and residual (bf16 [M, N]) may each be NULL, residual may alias
+ * y.  N = 2..32 (-2 for N = 1: the GEMV has its own residual argument). */
+int chr_dv2_gemm_add(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N, float *ws,
+                     int64_t ws_floats, const void *bias, const void *residual, void *stream);
+
 /* Library version, for the loader's sanity check. */
 int chr_nf4_abi_version(void);
 

@@ -14,7 +14,7 @@ from deepfold_amd.decodev2.synth import build
 from oracle import nf4_oracle as oc
 from oracle import step_oracle as so
 
-from helpers import DEV, bf16_bits, bf16_tensor, to_f32
+from helpers import DEV, bf16_bits, bf16_tensor, to_f32, up, up_scale
 from test_nf4_kernels import attn_ref, rope_tables, rot_half
 
 pytestmark = pytest.mark.gpu
@@ -175,6 +175,33 @@ def test_add_cols():
     assert (bf16_bits(dy) == bf16_bits(bf16_tensor(y) + db[:, None])).all()
     with pytest.raises(RuntimeError):
         nf4.dv2_add_cols(dy)
+
+
+@pytest.mark.parametrize("m,k,n", [(256, 512, 8), (130, 1088, 5), (5120, 5120, 32), (384, 256, 2)])
+def test_gemm_with_bias_and_residual_in_its_reduction(m, k, n):
+    say("gemm_add", m, k, n)
+    rng = np.random.default_rng(m + n)
+    p, s_ = oc.c_encode((rng.standard_normal((m, k)) * 0.05).astype(np.float32))
+    dp, ds = up(p), up_scale(s_)
+    kp = p.shape[1] * 2
+    x = bf16_tensor(rnd((k, n), 1))
+    bias = bf16_tensor(rnd((m,), 2))
+    res = rnd((m, n), 3)
+    plain = nf4.nf4_gemm(dp, ds, x, m, k, kp)
+    for use_bias, use_res in ((True, False), (False, True), (True, True)):
+        want = plain
+        if use_bias:
+            want = want + bias[:, None]
+        r = bf16_tensor(res)
+        if use_res:
+            want = r + want
+        got = nf4.nf4_gemm(dp, ds, x, m, k, kp, bias=bias if use_bias else None,
+                           residual=r if use_res else None)
+        assert (bf16_bits(got) == bf16_bits(want)).all(), (use_bias, use_res)
+        if use_res:
+            assert got.data_ptr() == r.data_ptr()  # added in place
+    with pytest.raises(RuntimeError):
+        nf4.nf4_gemm(dp, ds, x[:, :1].contiguous(), m, k, kp, bias=bias)
 
 
 # ---- the chunked prefill built from them ------------------------------------------------
