@@ -2,6 +2,7 @@
 arena and KV, eager step, HIP-graph replay, chunked prefill."""
 
 from .arena import Arena
+from .chr import weights_from_chr, write_synth_chr
 from .embed import PackedEmbed, gather_embed
 from .graph import GreedyGraph, capture_greedy
 from .kv import GraphSafeKV
@@ -22,5 +23,5 @@ __all__ = [
     "apply_rope_torch", "build", "capture_greedy", "consume_prompt", "SCHEDULES", "forward_decode",
     "forward_prefill", "gather_embed", "generate", "greedy_decode", "nf4_linear",
     "prefill_chunk_width", "rope_tables_numpy", "rope_tables_torch", "teacher_force_token",
-    "with_max_seq",
+    "weights_from_chr", "with_max_seq", "write_synth_chr",
 ]
