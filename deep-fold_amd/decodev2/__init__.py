@@ -12,12 +12,13 @@ from .plan import (INTERNLM25_20B, MEDIUM_LLAMA, QWEN25_3B, QWEN25_14B, QWEN25_3
 from .prefill import ChunkPrefill, forward_prefill, prefill_chunk_width
 from .rope import apply_rope_torch, rope_tables_numpy, rope_tables_torch
 from .runner import consume_prompt, generate
+from .session import DecodeV2Loop, Generation
 from .state import DecodeState
 from .step import SCHEDULES, forward_decode, greedy_decode, teacher_force_token
 from .synth import Nf4Matrix, SynthLayer, SynthModel, build
 
 __all__ = [
-    "ArchSpec", "Arena", "ChunkPrefill", "DecodeState", "DeviceLayer", "DeviceLinear", "DeviceWeights", "GraphSafeKV",
+    "ArchSpec", "Arena", "ChunkPrefill", "DecodeState", "DecodeV2Loop", "Generation", "DeviceLayer", "DeviceLinear", "DeviceWeights", "GraphSafeKV",
     "GreedyGraph", "PackedEmbed", "Nf4Matrix", "SynthLayer", "SynthModel", "TINY_LLAMA",
     "TINY_INTERNLM", "MEDIUM_LLAMA", "QWEN25_3B", "QWEN25_14B", "INTERNLM25_20B", "QWEN25_32B",
     "apply_rope_torch", "build", "capture_greedy", "consume_prompt", "SCHEDULES", "forward_decode",
