@@ -1,7 +1,7 @@
 // Glue kernels of the chunked prefill for gfx950 (MI355X), all on the layout the prefill GEMM
-// reads and writes: feature-major [features, N] bf16 with the N <= 32 tokens of the chunk
-// fastest.  With them a prefill layer needs no transposes between its GEMMs.  They stand in
-// for the stock torch ops of the reference's prefill (gpu/decodev2/prefill.py:58-133,
+// reads and writes: feature-major [features, N] bf16 with the N tokens of the chunk fastest
+// (N <= 64, the widest chunk chr_dv2_gemm_add multiplies).  With them a prefill layer needs no
+// transposes between its GEMMs.  They stand in for the stock torch ops of the reference's prefill (gpu/decodev2/prefill.py:58-133,
 // gpu/decodev2/ops.py:18-44): RMSNorm, rotate-half RoPE + cache write, SwiGLU, bias/residual.
 
 #include "nf4_common.h"
@@ -11,7 +11,7 @@ namespace {
 
 constexpr int kColsBlock = 1024;
 constexpr int kColsWaves = kColsBlock / kWave;
-constexpr int kMaxCols = 32;
+constexpr int kMaxCols = 64;
 
 // y[k][n] = bf16( (w[k] * x[k][n]) * rsqrt(mean_k x[k][n]^2 + eps) ).  Every workgroup sums the
 // squares of the whole tile itself (it is a few hundred KB and sits in L2; all workgroups add in
@@ -19,7 +19,7 @@ constexpr int kMaxCols = 32;
 // no cross-workgroup hand-over.
 //
 // Thread t owns column t % CP of rows t / CP, t / CP + 1024 / CP, ..; CP is N rounded up to a
-// power of two, threads whose column is >= N idle.  VEC: N is 8, 16 or 32 and rows are 16-byte
+// power of two, threads whose column is >= N idle.  VEC: N is 8, 16, 32 or 64 and rows are 16-byte
 // aligned, a thread then owns the eight columns of one 16-byte piece.
 template <bool VEC>
 __global__ __launch_bounds__(kColsBlock) void rms_cols(const uint16_t *__restrict__ x,
@@ -206,10 +206,10 @@ extern "C" int chr_dv2_rms_cols(const void *x, const void *w, void *y, int32_t r
   if (rows < 1) {
     return -3;
   }
-  if (N < 1 || N > 32) {
+  if (N < 1 || N > kMaxCols) {
     return -2;
   }
-  const bool vec = (N == 8 || N == 16 || N == 32) && aligned16(x) && aligned16(y);
+  const bool vec = (N == 8 || N == 16 || N == 32 || N == 64) && aligned16(x) && aligned16(y);
   int cp = 1;
   while (cp < N) {
     cp <<= 1;
@@ -242,7 +242,7 @@ extern "C" int chr_dv2_rope_kv_cols(const void *q, const void *k, const void *v,
   if (n_q < 1 || n_kv < 1 || hd < 2 || (hd & 1) != 0 || max_seq < 1) {
     return -3;
   }
-  if (N < 1 || N > 32) {
+  if (N < 1 || N > kMaxCols) {
     return -2;
   }
   rope_kv_cols<<<dim3(static_cast<unsigned>(n_q + n_kv)), dim3(256), 0,

@@ -37,6 +37,7 @@
 
 #include <algorithm>
 #include <cstdlib>
+#include <utility>
 
 namespace chr {
 
@@ -65,10 +66,14 @@ constexpr int kXStride = kBK + kXPad;
 constexpr int kWRow = kBK / 2 + 16;             // bytes of one staged weight row (padded)
 constexpr int kWStage = 32 * kWRow;             // bytes of a wavefront's weight area
 constexpr int kGroupsPerTile = kBK / 64;
-// codebook + activation tile + per-wavefront weight and scale areas (= sizeof(GemmLds))
+// codebook + activation tile (NB blocks of 32 columns) + per-wavefront weight and scale
+// areas (= sizeof(GemmLds<NB>))
 constexpr int kGemmWaves = kGemmBlock / 64;
-constexpr int kGemmLds = 64 + kKHalves * kBN * kXStride * 2 + kGemmWaves * kWStage +
-                         kGemmWaves * 32 * kGroupsPerTile * 2;
+constexpr int gemm_lds_bytes(int nb) {
+  return 64 + kKHalves * nb * kBN * kXStride * 2 + kGemmWaves * kWStage +
+         kGemmWaves * 32 * kGroupsPerTile * 2;
+}
+constexpr int kGemmLds = gemm_lds_bytes(1);
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -154,7 +159,7 @@ int plan_impl(const chr_nf4_dev_t &h, int32_t N, int32_t have_ws, chr_nf4_plan_t
     p.grid_x = ceil_div(h.M, kBM);
     p.n_ktiles = ceil_div(h.K_pad, kBK);
     pick_split(p.grid_x, p.n_ktiles, have_ws, &p.grid_y, &p.tiles_per_split);
-    p.smem_bytes = (N <= 32 ? 1 : 2) * kGemmLds;
+    p.smem_bytes = gemm_lds_bytes(N <= 32 ? 1 : 2);
     if (p.grid_y > 1) {
       p.ws_floats = static_cast<int64_t>(p.grid_y) * h.M * N;
     }
@@ -186,31 +191,33 @@ int check_args(const chr_nf4_dev_t *w, int32_t N, bool need_ptrs, chr_nf4_dev_t 
   return 0;
 }
 
+template <int NB>
 struct GemmLds {
   float lut[16];                                  // at LDS address 0 (lookup8)
-  __attribute__((aligned(16))) uint16_t xs[kKHalves][kBN * kXStride];
+  __attribute__((aligned(16))) uint16_t xs[kKHalves][NB * kBN * kXStride];
   __attribute__((aligned(16))) uint8_t w[kGemmWaves][kWStage];
   uint16_t sc[kGemmWaves][32 * kGroupsPerTile];
 };
-static_assert(sizeof(GemmLds) == kGemmLds, "the planner reports this size");
-static_assert(kKHalves == 1 || kKHalves * kBN * kXStride * 2 >= 4 * 32 * 32 * 4,
-              "the final reduction reuses xs");
+static_assert(sizeof(GemmLds<1>) == gemm_lds_bytes(1) && sizeof(GemmLds<2>) == gemm_lds_bytes(2),
+              "the planner reports these sizes");
+static_assert(kKHalves == 1, "the two-group reduction was written for one column block");
 
 // Activation vectors of one K tile held by a thread between fetch and scatter.  The tile
 // x[k0 .. k0+kBK) x [0, N) is kBK*N contiguous bf16; vector v of a thread holds flat
 // elements 8v .. 8v+7, element f being (k0 + f / N, f % N).
+template <int NB>
 struct XRegs {
-  uint32_t d[16];  // up to four 16-byte vectors (N = 32), as plain dwords
+  uint32_t d[16 * NB];  // up to 4 NB 16-byte vectors (N = 32 NB), as plain dwords
 };
 
-template <bool VEC>
-__device__ __forceinline__ void fetch_x(XRegs &r, const uint16_t *__restrict__ x, int k0, int K,
+template <bool VEC, int NB>
+__device__ __forceinline__ void fetch_x(XRegs<NB> &r, const uint16_t *__restrict__ x, int k0, int K,
                                         int N, int tid) {
   const int n_elem = min(kBK, K - k0) * N;  // valid elements of the tile (rows >= K are zero)
   const uint16_t *base = x + static_cast<size_t>(k0) * N;
   if constexpr (VEC) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < 4 * NB; ++j) {
       const int v = tid + j * kGroupThreads;
       uint4 t = make_uint4(0, 0, 0, 0);
       if (v * 8 < n_elem) {  // N % 8 == 0 here, so a vector never straddles the end
@@ -226,13 +233,13 @@ __device__ __forceinline__ void fetch_x(XRegs &r, const uint16_t *__restrict__ x
   }
 }
 
-template <bool VEC>
-__device__ __forceinline__ void scatter_x(const XRegs &r, const uint16_t *__restrict__ x,
+template <bool VEC, int NB>
+__device__ __forceinline__ void scatter_x(const XRegs<NB> &r, const uint16_t *__restrict__ x,
                                           uint16_t *xs, int k0, int K, int N, int tid) {
   if constexpr (VEC) {
-    const int shift = N == 32 ? 5 : (N == 16 ? 4 : 3);  // VEC: N in {8, 16, 32}
+    const int shift = N == 64 ? 6 : (N == 32 ? 5 : (N == 16 ? 4 : 3));  // VEC: N in {8, 16, 32, 64}
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < 4 * NB; ++j) {
       const int v = tid + j * kGroupThreads;
       if (v * 8 < kBK * N) {
         const int f = v * 8;
@@ -310,7 +317,9 @@ __device__ __forceinline__ bf16x8 dequant8(uint32_t w, float s, const float *lut
   return a;
 }
 
-template <bool VEC>
+// NB: 32-column blocks of the activation tile (1 for N <= 32, 2 for N <= 64); one
+// dequantised weight fragment feeds NB MFMAs.
+template <bool VEC, int NB>
 __global__ __launch_bounds__(kGemmBlock) void gemm_mfma(const uint8_t *__restrict__ packed,
                                                         const uint16_t *__restrict__ scale,
                                                         const uint16_t *__restrict__ x,
@@ -321,71 +330,67 @@ __global__ __launch_bounds__(kGemmBlock) void gemm_mfma(const uint8_t *__restric
                                                         const uint16_t *__restrict__ bias,
                                                         const uint16_t *res) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-  GemmLds &lds = *reinterpret_cast<GemmLds *>(lds_raw);
+  GemmLds<NB> &lds = *reinterpret_cast<GemmLds<NB> *>(lds_raw);
   if (threadIdx.x < 16) {
     lds.lut[threadIdx.x] = bits_to_f32(kLutBits[threadIdx.x]);
   }
   // columns >= N of the activation tiles are never written by the scatter: zero them once
-  for (int i = threadIdx.x; i < kKHalves * kBN * kXStride / 2; i += kGemmBlock) {
+  for (int i = threadIdx.x; i < NB * kBN * kXStride / 2; i += kGemmBlock) {
     reinterpret_cast<uint32_t *>(&lds.xs[0][0])[i] = 0u;
   }
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
-  const int rt = wave & 3;        // which 32 rows of the workgroup's 128
-  const int kgrp = wave >> 2;     // which K tiles: tile0 + kgrp, + 2, ..
-  const int tid = threadIdx.x & (kGroupThreads - 1);
-  const int row_base = blockIdx.x * kBM + rt * 32;
+  const int tid = threadIdx.x;
+  const int row_base = blockIdx.x * kBM + wave * 32;
   const int khalf = lane >> 5;  // which 32-wide half of a 64-wide K step
   uint8_t *wst = lds.w[wave];
   uint16_t *sst = lds.sc[wave];
-  uint16_t *xs = lds.xs[kgrp];
+  uint16_t *xs = lds.xs[0];
 
   const int tile0 = blockIdx.y * tiles_per_split;
   const int tile1 = min(tile0 + tiles_per_split, n_ktiles);
 
-  f32x16 acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  f32x16 acc[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    acc[nb] = f32x16{0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  }
   const uint16_t *xl = xs + (lane & 31) * kXStride + khalf * 32;
   const uint8_t *wl = wst + (lane & 31) * kWRow + khalf * 16;
   const uint16_t *sl = sst + (lane & 31) * kGroupsPerTile;
 
   WRegs wr;
-  XRegs xr;
-  if (tile0 + kgrp < tile1) {
-    fetch_w(wr, packed, scale, row_base, M, K_pad, (tile0 + kgrp) * kBK, lane);
-    fetch_x<VEC>(xr, x, (tile0 + kgrp) * kBK, K, N, tid);
+  XRegs<NB> xr;
+  if (tile0 < tile1) {
+    fetch_w(wr, packed, scale, row_base, M, K_pad, tile0 * kBK, lane);
+    fetch_x<VEC, NB>(xr, x, tile0 * kBK, K, N, tid);
   }
-  // Both wavefront groups run the same number of rounds (the barriers are workgroup-wide);
-  // a group without a tile in the last round only keeps step.
-  for (int base = tile0; base < tile1; base += kKHalves) {
-    const int tile = base + kgrp;
-    const bool mine = tile < tile1;
+  for (int tile = tile0; tile < tile1; ++tile) {
     const int k0 = tile * kBK;
     __syncthreads();  // the previous round's readers are done (and the LUT / zero fill is visible)
-    if (mine) {
-      scatter_x<VEC>(xr, x, xs, k0, K, N, tid);
-      stash_w(wr, wst, sst, lane);
-    }
+    scatter_x<VEC, NB>(xr, x, xs, k0, K, N, tid);
+    stash_w(wr, wst, sst, lane);
     __syncthreads();
-    if (!mine) {
-      continue;
-    }
-    if (tile + kKHalves < tile1) {  // next tile's trip to memory overlaps this tile's arithmetic
-      fetch_w(wr, packed, scale, row_base, M, K_pad, k0 + kKHalves * kBK, lane);
-      fetch_x<VEC>(xr, x, k0 + kKHalves * kBK, K, N, tid);
+    if (tile + 1 < tile1) {  // next tile's trip to memory overlaps this tile's arithmetic
+      fetch_w(wr, packed, scale, row_base, M, K_pad, k0 + kBK, lane);
+      fetch_x<VEC, NB>(xr, x, k0 + kBK, K, N, tid);
     }
     const int kend = min(kBK, K_pad - k0);
     for (int kk = 0; kk < kend; kk += 64) {
       const uint4 pk = *reinterpret_cast<const uint4 *>(wl + (kk >> 1));
       const float s = f16_to_f32(sl[kk >> 6]);
       const uint32_t w[4] = {pk.x, pk.y, pk.z, pk.w};
-      // all 32 lookups and the four B reads of the step are issued before the first
+      // all 32 lookups and the B reads of the step are issued before the first
       // conversion, so their LDS latency is paid once per step
       Levels8 lv[4];
-      bf16x8 b[4];
+      bf16x8 b[4][NB];
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
         lv[t] = lookup8_lds0(w[t]);  // lds.lut is at LDS address 0
-        b[t] = *reinterpret_cast<const bf16x8 *>(xl + kk + 8 * t);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+          b[t][nb] = *reinterpret_cast<const bf16x8 *>(xl + nb * kBN * kXStride + kk + 8 * t);
+        }
       }
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -395,61 +400,46 @@ __global__ __launch_bounds__(kGemmBlock) void gemm_mfma(const uint8_t *__restric
         for (int j = 0; j < 8; ++j) {
           a[j] = static_cast<__bf16>(lv[t].l[j] * s);
         }
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b[t], acc, 0, 0, 0);
-      }
-    }
-  }
-
-  if constexpr (kKHalves > 1) {
-    // Add the second group's tile to the first's through LDS (the activation area is free
-    // now), in a fixed order, then the first group stores.
-    __syncthreads();
-    float *red = reinterpret_cast<float *>(&lds.xs[0][0]) + rt * (16 * kWave);
-    if (kgrp == 1) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        red[i * kWave + lane] = acc[i];
-      }
-    }
-    __syncthreads();
-    if (kgrp != 0) {
-      return;
-    }
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      acc[i] += red[i * kWave + lane];
-    }
-  }
-
-  // acc[i] is C[row 8*(i/4) + 4*(lane/32) + i%4][col lane%32] of the 32x32 tile.
-  const int n = lane & 31;
-  const int rbase = row_base + 4 * (lane >> 5);
-  if (n < N) {
-    if (partial == nullptr) {
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int r = rbase + 8 * (i >> 2) + (i & 3);
-        if (r < M) {
-          // unsplit: the epilogue of reduce_splitk, here (res may alias y: same thread,
-          // same element)
-          const size_t at = static_cast<size_t>(r) * N + n;
-          uint16_t v = f32_to_bf16(acc[i]);
-          if (bias != nullptr) {
-            v = f32_to_bf16(bf16_to_f32(v) + bf16_to_f32(bias[r]));
-          }
-          if (res != nullptr) {
-            v = f32_to_bf16(bf16_to_f32(res[at]) + bf16_to_f32(v));
-          }
-          y[at] = v;
+        for (int nb = 0; nb < NB; ++nb) {
+          acc[nb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b[t][nb], acc[nb], 0, 0, 0);
         }
       }
-    } else {
-      float *p = partial + static_cast<size_t>(blockIdx.y) * M * N;
+    }
+  }
+
+  // acc[nb][i] is C[row 8*(i/4) + 4*(lane/32) + i%4][col 32 nb + lane%32] of the 32-row tile.
+  const int rbase = row_base + 4 * (lane >> 5);
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int r = rbase + 8 * (i >> 2) + (i & 3);
-        if (r < M) {
-          p[static_cast<size_t>(r) * N + n] = acc[i];
+  for (int nb = 0; nb < NB; ++nb) {
+    const int n = nb * kBN + (lane & 31);
+    if (n < N) {
+      if (partial == nullptr) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int r = rbase + 8 * (i >> 2) + (i & 3);
+          if (r < M) {
+            // unsplit: the epilogue of reduce_splitk, here (res may alias y: same thread,
+            // same element)
+            const size_t at = static_cast<size_t>(r) * N + n;
+            uint16_t v = f32_to_bf16(acc[nb][i]);
+            if (bias != nullptr) {
+              v = f32_to_bf16(bf16_to_f32(v) + bf16_to_f32(bias[r]));
+            }
+            if (res != nullptr) {
+              v = f32_to_bf16(bf16_to_f32(res[at]) + bf16_to_f32(v));
+            }
+            y[at] = v;
+          }
+        }
+      } else {
+        float *p = partial + static_cast<size_t>(blockIdx.y) * M * N;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int r = rbase + 8 * (i >> 2) + (i & 3);
+          if (r < M) {
+            p[static_cast<size_t>(r) * N + n] = acc[nb][i];
+          }
         }
       }
     }
@@ -485,10 +475,13 @@ __global__ __launch_bounds__(256) void reduce_splitk(const float *__restrict__ p
 // (on the first launch, which a caller warming up before graph capture makes eagerly).
 int gemm_lds_ready() {
   static const int rc = [] {
-    const void *kernels[2] = {reinterpret_cast<const void *>(gemm_mfma<true>),
-                              reinterpret_cast<const void *>(gemm_mfma<false>)};
-    for (const void *k : kernels) {
-      if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, kGemmLds) !=
+    const std::pair<const void *, int> kernels[4] = {
+        {reinterpret_cast<const void *>(gemm_mfma<true, 1>), gemm_lds_bytes(1)},
+        {reinterpret_cast<const void *>(gemm_mfma<false, 1>), gemm_lds_bytes(1)},
+        {reinterpret_cast<const void *>(gemm_mfma<true, 2>), gemm_lds_bytes(2)},
+        {reinterpret_cast<const void *>(gemm_mfma<false, 2>), gemm_lds_bytes(2)}};
+    for (const auto &k : kernels) {
+      if (hipFuncSetAttribute(k.first, hipFuncAttributeMaxDynamicSharedMemorySize, k.second) !=
           hipSuccess) {
         (void)hipGetLastError();
         return -6;
@@ -527,9 +520,11 @@ extern "C" int chr_nf4_gemm_plan(const chr_nf4_dev_t *w, int32_t N, int32_t have
 namespace chr {
 namespace {
 
+// live_max: widest chunk the entry launches.  The reference's entries stop at 32 columns
+// (wider ones are described by the planner only); chr_dv2_gemm_add goes to 64.
 int gemm_launch(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N, float *ws,
                 int64_t ws_floats, void *stream, int32_t max_n, const void *bias,
-                const void *res) {
+                const void *res, int32_t live_max = kLiveMaxN) {
   if (x == nullptr || y == nullptr) {
     return -1;
   }
@@ -541,8 +536,8 @@ int gemm_launch(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N, float
   if (rc != 0) {
     return rc;
   }
-  if (N > kLiveMaxN) {
-    return -2;  // no 64-column tile is built
+  if (N > live_max) {
+    return -2;
   }
   if (!aligned16(h.packed) || !aligned16(x) || !aligned2(h.scale)) {
     return -5;
@@ -562,21 +557,36 @@ int gemm_launch(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N, float
   float *partial = p.grid_y > 1 ? ws : nullptr;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const dim3 grid(static_cast<unsigned>(p.grid_x), static_cast<unsigned>(p.grid_y));
-  // 16-byte activation vectors need N in {8, 16, 32}; x is 16-byte aligned (checked above)
-  const bool vec = N == 8 || N == 16 || N == 32;
+  // 16-byte activation vectors need N in {8, 16, 32, 64}; x is 16-byte aligned (checked above)
+  const bool vec = N == 8 || N == 16 || N == 32 || N == 64;
   if (gemm_lds_ready() != 0) {
     return -6;
   }
-  if (vec) {
-    gemm_mfma<true><<<grid, dim3(kGemmBlock), kGemmLds, st>>>(
-        h.packed, h.scale, static_cast<const uint16_t *>(x), static_cast<uint16_t *>(y), partial,
-        h.M, h.K, h.K_pad, N, p.n_ktiles, p.tiles_per_split,
-        static_cast<const uint16_t *>(bias), static_cast<const uint16_t *>(res));
+  const auto *xp = static_cast<const uint16_t *>(x);
+  auto *yp = static_cast<uint16_t *>(y);
+  const auto *bp = static_cast<const uint16_t *>(bias);
+  const auto *rp = static_cast<const uint16_t *>(res);
+  const dim3 block(kGemmBlock);
+  if (N <= kBN) {
+    if (vec) {
+      gemm_mfma<true, 1><<<grid, block, gemm_lds_bytes(1), st>>>(
+          h.packed, h.scale, xp, yp, partial, h.M, h.K, h.K_pad, N, p.n_ktiles, p.tiles_per_split,
+          bp, rp);
+    } else {
+      gemm_mfma<false, 1><<<grid, block, gemm_lds_bytes(1), st>>>(
+          h.packed, h.scale, xp, yp, partial, h.M, h.K, h.K_pad, N, p.n_ktiles, p.tiles_per_split,
+          bp, rp);
+    }
   } else {
-    gemm_mfma<false><<<grid, dim3(kGemmBlock), kGemmLds, st>>>(
-        h.packed, h.scale, static_cast<const uint16_t *>(x), static_cast<uint16_t *>(y), partial,
-        h.M, h.K, h.K_pad, N, p.n_ktiles, p.tiles_per_split,
-        static_cast<const uint16_t *>(bias), static_cast<const uint16_t *>(res));
+    if (vec) {
+      gemm_mfma<true, 2><<<grid, block, gemm_lds_bytes(2), st>>>(
+          h.packed, h.scale, xp, yp, partial, h.M, h.K, h.K_pad, N, p.n_ktiles, p.tiles_per_split,
+          bp, rp);
+    } else {
+      gemm_mfma<false, 2><<<grid, block, gemm_lds_bytes(2), st>>>(
+          h.packed, h.scale, xp, yp, partial, h.M, h.K, h.K_pad, N, p.n_ktiles, p.tiles_per_split,
+          bp, rp);
+    }
   }
   if (partial != nullptr) {
     const int rows = h.M * N;
@@ -598,7 +608,7 @@ extern "C" int chr_nf4_gemm_ws_max(const chr_nf4_dev_t *w, const void *x, void *
 extern "C" int chr_dv2_gemm_add(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N,
                                 float *ws, int64_t ws_floats, const void *bias,
                                 const void *residual, void *stream) {
-  return gemm_launch(w, x, y, N, ws, ws_floats, stream, kLiveMaxN, bias, residual);
+  return gemm_launch(w, x, y, N, ws, ws_floats, stream, kPlanMaxN, bias, residual, kPlanMaxN);
 }
 
 extern "C" int chr_nf4_gemm_ws(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N,

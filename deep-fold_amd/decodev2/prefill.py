@@ -12,7 +12,7 @@ from __future__ import annotations
 
 import torch
 
-from ..nf4 import (LIVE_MAX_N, dv2_add_cols, dv2_attn_chunk, dv2_rms_cols, dv2_rope_kv_cols,
+from ..nf4 import (LIVE_MAX_N, PLAN_MAX_N, dv2_add_cols, dv2_attn_chunk, dv2_rms_cols, dv2_rope_kv_cols,
                    dv2_swiglu_elems, nf4_gemm)
 from .embed import gather_embed
 from .linear import DeviceLinear, DeviceWeights, nf4_linear
@@ -68,8 +68,8 @@ def _gemm_cols(mat: DeviceLinear, x: torch.Tensor, residual: torch.Tensor | None
     result is added to it in place.  One column (a one-token chunk) goes to the GEMV and
     takes its bias and residual from separate launches."""
     if x.size(1) >= 2:
-        return nf4_gemm(mat.packed, mat.scale, x, mat.M, mat.K, mat.K_pad, bias=mat.bias,
-                        residual=residual)
+        return nf4_gemm(mat.packed, mat.scale, x, mat.M, mat.K, mat.K_pad, int(PLAN_MAX_N),
+                        bias=mat.bias, residual=residual)
     y = nf4_gemm(mat.packed, mat.scale, x, mat.M, mat.K, mat.K_pad)
     if mat.bias is not None:
         dv2_add_cols(y, bias=mat.bias)
@@ -85,15 +85,24 @@ class ChunkPrefill:
     ``run(ids, start, logits)`` has ``forward_prefill``'s contract.  All launches of a
     chunk read the chunk's ids, its first cache slot and the prefix length of its first
     token from fixed device buffers, so one captured graph per chunk width serves every
-    position (``use_graph``); without graphs the same launches are issued eagerly."""
+    position (``use_graph``); without graphs the same launches are issued eagerly.
 
-    def __init__(self, state: DecodeState, weights: DeviceWeights, *, use_graph: bool = True) -> None:
+    ``width`` is the chunk ``consume_prompt`` cuts prompts into: up to 64 tokens, twice the
+    reference's 32, so the weights are streamed half as often (the 33..64-column GEMM tile
+    dequantises each weight once for both 32-column blocks)."""
+
+    MAX_WIDTH = int(PLAN_MAX_N)
+
+    def __init__(self, state: DecodeState, weights: DeviceWeights, *, use_graph: bool = True,
+                 width: int | None = None) -> None:
         self.state = state
         self.weights = weights
         self.use_graph = bool(use_graph)
         dev = state.device
         spec = state.spec
-        self.ids = torch.zeros(int(LIVE_MAX_N), dtype=torch.long, device=dev)
+        cap = min(self.MAX_WIDTH, int(spec.max_seq))
+        self.width = cap if width is None else max(1, min(int(width), cap))
+        self.ids = torch.zeros(self.MAX_WIDTH, dtype=torch.long, device=dev)
         self.start = torch.zeros((), dtype=torch.int64, device=dev)
         self.first_len = torch.zeros((), dtype=torch.int32, device=dev)
         self.last_hidden = torch.zeros(spec.hidden, dtype=torch.bfloat16, device=dev)
@@ -141,8 +150,8 @@ class ChunkPrefill:
         n = int(ids.numel())
         if n < 1:
             raise ValueError("prefill chunk must be non-empty")
-        if n > int(LIVE_MAX_N):
-            raise ValueError(f"prefill chunk of {n} tokens exceeds {int(LIVE_MAX_N)}")
+        if n > self.MAX_WIDTH:
+            raise ValueError(f"prefill chunk of {n} tokens exceeds {self.MAX_WIDTH}")
         start = int(start)
         seq = start + n
         if start < 0 or seq > spec.max_seq:

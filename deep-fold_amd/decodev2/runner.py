@@ -32,6 +32,8 @@ def consume_prompt(state: DecodeState, weights: DeviceWeights, token_ids: Sequen
     if pos + n > state.spec.max_seq:
         raise ValueError(f"prompt {pos}+{n} exceeds max_seq={state.spec.max_seq}")
     width = prefill_chunk_width(state, chunk)
+    if prefill is not None:  # its own, wider chunks unless the caller asked for a width
+        width = prefill.width if chunk is None else max(1, min(int(chunk), prefill.MAX_WIDTH))
     buf = torch.tensor(ids, dtype=torch.long, device=state.device)
     for lo in range(0, n, width):
         hi = min(lo + width, n)

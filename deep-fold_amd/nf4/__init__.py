@@ -267,13 +267,15 @@ def nf4_gemm(packed: torch.Tensor, scale: torch.Tensor, x: torch.Tensor, M: int,
     """Fused NF4 dequant-MFMA GEMM.  ``x`` is bf16 ``[K, N]`` or ``[K]``; returns
     ``y [M, N]`` (``gpu/nf4/__init__.py:151-176``, ``bindings.cpp:35-97``).  With
     ``bias`` (bf16 ``[M]``) and/or ``residual`` (bf16 ``[M, N]``, N >= 2) the result is
-    ``residual + (y + bias)``, written over ``residual``, in the same launches."""
+    ``residual + (y + bias)``, written over ``residual``, in the same launches.  With
+    ``max_n=64`` chunks of 33..64 columns run too (one pass over the weights)."""
     n = 1 if x.dim() == 1 else int(x.size(-1))
     cap = int(max_n)
     if cap < 1 or cap > PLAN_MAX_N:
         raise RuntimeError(f"chr_nf4_gemm: max_n={cap} not in 1..{PLAN_MAX_N}")
     if n < 1 or n > cap:
         raise RuntimeError(f"chr_nf4_gemm: N={n} not in 1..{cap} (host must chunk N>{LIVE_MAX_N})")
+    wide = n > LIVE_MAX_N  # the 33..64-column tile: launched by chr_dv2_gemm_add only
     _need(packed.is_cuda and scale.is_cuda and x.is_cuda, "packed, scale, and x must be CUDA tensors")
     _need(x.dtype == torch.bfloat16, "x must be bfloat16")
     M, K, K_pad = int(M), int(K), int(K_pad)
@@ -295,12 +297,12 @@ def nf4_gemm(packed: torch.Tensor, scale: torch.Tensor, x: torch.Tensor, M: int,
     if p.ws_floats > 0:
         ws = torch.empty(int(p.ws_floats), dtype=torch.float32, device=x.device)
         ws_ptr = ws.data_ptr()
-    if bias is None and residual is None:
+    if bias is None and residual is None and not wide:
         rc = lib.chr_nf4_gemm_ws_max(ctypes.byref(w), x.data_ptr(), y.data_ptr(), n, ws_ptr,
                                      int(p.ws_floats), _stream(), cap)
         _check_rc("chr_nf4_gemm", rc)
         return y
-    _need(n >= 2 and n <= LIVE_MAX_N, "bias/residual ride on the N = 2..32 tiles")
+    _need(n >= 2, "bias/residual ride on the N >= 2 tiles")
     for t, numel, name in ((bias, M, "bias"), (residual, M * n, "residual")):
         _need(t is None or (t.is_cuda and t.dtype == torch.bfloat16 and t.is_contiguous()
                             and t.numel() == numel), f"{name} must be contiguous CUDA bf16 of {numel} elements")
@@ -739,7 +741,7 @@ def _bf16_cuda(t: torch.Tensor, what: str) -> None:
 
 
 def dv2_rms_cols(x: torch.Tensor, w: torch.Tensor, eps: float, out: torch.Tensor | None = None) -> torch.Tensor:
-    """RMSNorm of every column of feature-major ``x [rows, N]`` (N <= 32)."""
+    """RMSNorm of every column of feature-major ``x [rows, N]`` (N <= 64)."""
     _bf16_cuda(x, "x")
     _bf16_cuda(w, "w")
     _need(x.dim() == 2 and w.numel() == x.size(0), "x must be [rows, N] and w hold rows elements")

@@ -13,7 +13,9 @@ are ``M``, in features ``K``):
 * ``N = 2..16`` / ``17..32``  MFMA tile, 128 rows x 32 columns per workgroup,
   split-K over ``grid_y`` at about three K tiles per workgroup while the grid fits
   the four workgroups a compute unit holds (paths ``PREFILL`` / ``PREFILL_N32``).
-* ``N = 33..64``  described by the planner, never launched (``PREFILL_N64``).
+* ``N = 33..64``  the same tile with two 32-column blocks per weight fragment
+  (``PREFILL_N64``); launched only through ``chr_nf4_gemm_ws_max`` with ``max_n`` > 32,
+  the plain entries keep the reference's ceiling of 32.
 """
 
 from __future__ import annotations
@@ -57,9 +59,14 @@ _BLOCK = 256
 _MAX_AUTO_SPLIT = 32
 _TILES_PER_SPLIT = 3
 _RESIDENT_PER_CU = 4
-# codebook, staged activation tile (bf16, padded rows), and per wavefront (4) a weight area
-# (32 rows of BK/2 + 16 bytes) and the tile's group scales
-_X_LDS = 64 + 32 * (_BK + 8) * 2 + 4 * 32 * (_BK // 2 + 16) + 4 * 32 * (_BK // 64) * 2
+
+
+def _gemm_lds(col_blocks: int) -> int:
+    """codebook, staged activation tile (bf16, padded rows, ``col_blocks`` x 32 columns), and
+    per wavefront (4) a weight area (32 rows of BK/2 + 16 bytes) and the tile's group scales"""
+    return (64 + col_blocks * 32 * (_BK + 8) * 2 + 4 * 32 * (_BK // 2 + 16)
+            + 4 * 32 * (_BK // 64) * 2)
+
 
 _PATH_NAME = {GEMV: "gemv", PREFILL: "prefill", PREFILL_N32: "prefill_n32",
               PREFILL_N64: "prefill_n64"}
@@ -103,6 +110,7 @@ class Plan:
 
     @property
     def live(self) -> bool:
+        """Launched by the entries that keep the reference's ceiling of 32 columns."""
         return self.path != PREFILL_N64
 
 
@@ -139,5 +147,5 @@ def plan(M: int, K: int, N: int = 1, *, K_pad: int | None = None, have_ws: bool 
     n_ktiles = _ceil_div(kp, _BK)
     split, tps = _pick_split(grid_x, n_ktiles, have_ws, force_split, one_wave)
     ws = split * M * N if split > 1 else 0
-    smem = (1 if N <= 32 else 2) * _X_LDS
+    smem = _gemm_lds(1 if N <= 32 else 2)
     return Plan(path, grid_x, split, _BLOCK, _BM, _BK, n_ktiles, tps, grid_x * split, smem, ws)

@@ -210,12 +210,12 @@ int chr_dv2_gemv_attn(const chr_nf4_dev_t *w, const float *state, int32_t n_q, i
  * The reference's prefill (gpu/decodev2/prefill.py:58-133) runs everything but its linears as
  * stock torch ops on token-major [N, features] tensors and transposes around every GEMM
  * (gpu/decodev2/linear.py:96-113).  These entries do the same arithmetic directly on the
- * feature-major [features, N] bf16 tiles chr_nf4_gemm reads and writes (N <= 32 tokens of one
+ * feature-major [features, N] bf16 tiles chr_nf4_gemm reads and writes (N <= 64 tokens of one
  * chunk, token index fastest), so a prefill layer is a straight sequence of launches that can
  * be captured in a graph.  None has a counterpart in the reference's C-ABI. */
 
 /* y[k][n] = (w[k] * x[k][n]) * rsqrt(mean_k x[k][n]^2 + eps) per column n
- * (gpu/decodev2/ops.py:18-20).  -2 when N is outside 1..32. */
+ * (gpu/decodev2/ops.py:18-20).  -2 when N is outside 1..64. */
 int chr_dv2_rms_cols(const void *x, const void *w, void *y, int32_t rows, int32_t N, float eps,
                      void *stream);
 
@@ -251,7 +251,11 @@ int chr_dv2_add_cols(void *y, const void *a, const void *bias, int32_t rows, int
  * (gpu/decodev2/linear.py:114-116, prefill.py:113,133) folded into the split-K reduction:
  * y = residual + (bf16(W x) + bias[row]), each step rounded to bf16 as the separate torch
  * adds round; bias (bf16 [M]) and residual (bf16 [M, N]) may each be NULL, residual may alias
- * y.  N = 2..32 (-2 for N = 1: the GEMV has its own residual argument). */
+ * y.  N = 2..64 (-2 for N = 1: the GEMV has its own residual argument).  Beyond the 32
+ * columns of the reference's live entries this one also launches the 33..64-column tile that
+ * chr_nf4_gemm_plan describes: two 32-column blocks per dequantised weight fragment, so a
+ * 64-token chunk costs one pass over the weights, not two.  Workspace as the plan says.
+ * No reference counterpart. */
 int chr_dv2_gemm_add(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N, float *ws,
                      int64_t ws_floats, const void *bias, const void *residual, void *stream);
 

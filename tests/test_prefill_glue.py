@@ -29,7 +29,7 @@ def rnd(shape, seed, scale=1.0):
     return oc.bf16_round((rng.standard_normal(shape) * scale).astype(np.float32))
 
 
-@pytest.mark.parametrize("rows,n", [(64, 1), (256, 7), (5120, 32), (1000, 16), (2050, 31)])
+@pytest.mark.parametrize("rows,n", [(64, 1), (256, 7), (5120, 32), (1000, 16), (2050, 31), (5120, 64), (300, 40)])
 def test_rms_cols(rows, n):
     say("rms_cols", rows, n)
     x = rnd((rows, n), rows + n, 1.5)
@@ -50,13 +50,13 @@ def test_rms_cols(rows, n):
 
 
 def test_rms_cols_rejects_wide_chunks():
-    x = torch.zeros((64, 33), dtype=torch.bfloat16, device=DEV)
+    x = torch.zeros((64, 65), dtype=torch.bfloat16, device=DEV)
     with pytest.raises(RuntimeError):
         nf4.dv2_rms_cols(x, torch.ones(64, dtype=torch.bfloat16, device=DEV), 1e-6)
 
 
 @pytest.mark.parametrize("n_q,n_kv,hd,n,start", [(4, 2, 16, 5, 0), (16, 2, 128, 32, 40),
-                                                 (6, 3, 256, 3, 61), (8, 8, 64, 32, 0)])
+                                                 (6, 3, 256, 3, 61), (8, 8, 64, 32, 0), (8, 2, 64, 64, 17)])
 def test_rope_kv_cols(n_q, n_kv, hd, n, start):
     say("rope_kv_cols", n_q, n_kv, hd, n, start)
     max_seq = 96
@@ -204,6 +204,32 @@ def test_gemm_with_bias_and_residual_in_its_reduction(m, k, n):
         nf4.nf4_gemm(dp, ds, x[:, :1].contiguous(), m, k, kp, bias=bias)
 
 
+@pytest.mark.parametrize("m,k,n", [(256, 512, 64), (130, 1088, 33), (5120, 5120, 64), (384, 256, 40),
+                                   (13824, 5120, 48)])
+def test_wide_chunk_equals_two_narrow_ones(m, k, n):
+    """33..64 columns in one pass over the weights: every column must come out as it does
+    from the 32-column tile (same K order, same split)."""
+    say("gemm wide", m, k, n)
+    rng = np.random.default_rng(m + n)
+    p, s_ = oc.c_encode((rng.standard_normal((m, k)) * 0.05).astype(np.float32))
+    dp, ds = up(p), up_scale(s_)
+    kp = p.shape[1] * 2
+    x = bf16_tensor(rnd((k, n), 1))
+    wide = nf4.nf4_gemm(dp, ds, x, m, k, kp, max_n=64)
+    lo = nf4.nf4_gemm(dp, ds, x[:, :32].contiguous(), m, k, kp)
+    first = min(32, n - 2)  # at least two columns: one alone would go to the GEMV
+    hi = nf4.nf4_gemm(dp, ds, x[:, first:].contiguous(), m, k, kp)
+    assert tuple(wide.shape) == (m, n)
+    assert (bf16_bits(wide[:, :32].contiguous()) == bf16_bits(lo)).all()
+    assert (bf16_bits(wide[:, first:].contiguous()) == bf16_bits(hi.view(m, n - first))).all()
+    bias, res = bf16_tensor(rnd((m,), 2)), bf16_tensor(rnd((m, n), 3))
+    want = res + (wide + bias[:, None])
+    got = nf4.nf4_gemm(dp, ds, x, m, k, kp, max_n=64, bias=bias, residual=res)
+    assert (bf16_bits(got) == bf16_bits(want)).all()
+    with pytest.raises(RuntimeError):
+        nf4.nf4_gemm(dp, ds, x, m, k, kp)  # the reference's ceiling without max_n
+
+
 # ---- the chunked prefill built from them ------------------------------------------------
 
 LONG = [4, 5, 6, 7, 1, 2, 3, 4]
@@ -255,6 +281,32 @@ def test_feature_major_prefill_tracks_the_torch_glue():
     assert torch.equal(first[0], b.kv.k[:, :n]) and torch.equal(first[1], b.arena.logits)
 
 
+def test_sixty_four_token_chunks():
+    spec = dv2.with_max_seq(dv2.MEDIUM_LLAMA, 256)
+    rng = np.random.default_rng(1)
+    prompt = [int(t) for t in rng.integers(0, spec.vocab, size=150)]
+    model, a, w = session(spec, 4, packed_embed=True)
+    b = dv2.DecodeState.allocate(spec, device="cuda")
+    pre32 = dv2.ChunkPrefill(a, w, width=32)
+    pre64 = dv2.ChunkPrefill(b, w)
+    assert (pre32.width, pre64.width) == (32, 64)
+    dv2.consume_prompt(a, w, prompt, prefill=pre32)   # 32+32+32+32+22
+    dv2.consume_prompt(b, w, prompt, prefill=pre64)   # 64+64+22
+    n = len(prompt)
+    assert int(a.valid_len.item()) == int(b.valid_len.item()) == n
+    # per column the wide GEMM tile computes what the narrow one does, but the RMSNorm sums
+    # its squares in an order that depends on the chunk width: equal up to bf16 rounding
+    for ta, tb in ((a.kv.k[:, :n], b.kv.k[:, :n]), (a.kv.v[:, :n], b.kv.v[:, :n]),
+                   (a.arena.logits, b.arena.logits)):
+        ta, tb = ta.float(), tb.float()
+        assert (ta - tb).abs().max().item() <= 0.03 * max(1.0, ta.abs().max().item())
+    # greedy ids follow the oracle until a pick whose top-two logits are nearly tied
+    want, margins = so.greedy_ids(model, prompt[:70], 5, return_margins=True)
+    thin = next((i for i, m in enumerate(margins) if m < 0.02), len(want))
+    got = dv2.generate(b, w, prompt[:70], 5, prefill=pre64)
+    assert thin >= 3 and got[:thin] == want[:thin]
+
+
 def test_chunk_prefill_errors():
     spec = dv2.TINY_LLAMA
     _, state, w = session(spec, 0)
@@ -262,6 +314,6 @@ def test_chunk_prefill_errors():
     with pytest.raises(ValueError):
         pre.run(torch.zeros(0, dtype=torch.long), 0)
     with pytest.raises(ValueError):
-        pre.run(torch.zeros(33, dtype=torch.long), 0)
+        pre.run(torch.zeros(65, dtype=torch.long), 0)
     with pytest.raises(ValueError):
         pre.run(torch.zeros(4, dtype=torch.long), spec.max_seq - 2)
