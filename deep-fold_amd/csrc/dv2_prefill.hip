@@ -112,8 +112,12 @@ __global__ __launch_bounds__(kColsBlock) void rms_cols(const uint16_t *__restric
 
 // Rotate-half RoPE of the chunk's q and k at positions *start + n, and the cache write.
 // q, k, v are feature-major [heads*hd, N]; q_out is token-major [N, n_q*hd] (what the
-// attention reads); the caches are [max_seq, n_kv, hd].  One workgroup per head (q heads
-// first, then kv heads); thread t takes token t % N, dims t / N, + 256 / N, ..
+// attention reads); the caches are [max_seq, n_kv, hd].  grid.x = head (q heads first, then
+// kv heads); a thread takes one token and eight consecutive dims d0 .. d0+7 of the lower
+// half plus their partners d0+half ..: lanes run along the tokens, so the reads of a row are
+// contiguous, and every store is a 16-byte vector of one token's row.  VEC needs hd % 16 == 0
+// and 16-byte aligned outputs; otherwise one pair of dims per thread.
+template <bool VEC>
 __global__ __launch_bounds__(256) void rope_kv_cols(const uint16_t *__restrict__ q,
                                                     const uint16_t *__restrict__ k,
                                                     const uint16_t *__restrict__ v,
@@ -131,29 +135,49 @@ __global__ __launch_bounds__(256) void rope_kv_cols(const uint16_t *__restrict__
   const uint16_t *src = (is_q ? q : k) + static_cast<size_t>(head) * hd * N;
   const uint16_t *vsrc = v + static_cast<size_t>(head) * hd * N;
   const int half = hd / 2;
-  for (int i = threadIdx.x; i < half * N; i += blockDim.x) {
-    const int d = i / N;
-    const int n = i - d * N;
+  constexpr int W = VEC ? 8 : 1;  // dims of each half a thread rotates
+  const int items = (half / W) * N;
+  for (int i = blockIdx.y * blockDim.x + threadIdx.x; i < items; i += gridDim.y * blockDim.x) {
+    const int d0 = (i / N) * W;
+    const int n = i % N;
     const long long p = s0 + n;
     if (p < 0 || p >= max_seq) {
       continue;
     }
-    const float t0 = bf16_to_f32(src[static_cast<size_t>(d) * N + n]);
-    const float t1 = bf16_to_f32(src[static_cast<size_t>(d + half) * N + n]);
     const uint16_t *c = cos + static_cast<size_t>(p) * hd;
     const uint16_t *sn = sin + static_cast<size_t>(p) * hd;
-    const uint16_t lo = f32_to_bf16(t0 * bf16_to_f32(c[d]) + (-t1) * bf16_to_f32(sn[d]));
-    const uint16_t hi = f32_to_bf16(t1 * bf16_to_f32(c[d + half]) + t0 * bf16_to_f32(sn[d + half]));
+    uint16_t lo[W], hi[W], vlo[W], vhi[W];
+#pragma unroll
+    for (int e = 0; e < W; ++e) {
+      const int d = d0 + e;
+      const float t0 = bf16_to_f32(src[static_cast<size_t>(d) * N + n]);
+      const float t1 = bf16_to_f32(src[static_cast<size_t>(d + half) * N + n]);
+      lo[e] = f32_to_bf16(t0 * bf16_to_f32(c[d]) + (-t1) * bf16_to_f32(sn[d]));
+      hi[e] = f32_to_bf16(t1 * bf16_to_f32(c[d + half]) + t0 * bf16_to_f32(sn[d + half]));
+      if (!is_q) {
+        vlo[e] = vsrc[static_cast<size_t>(d) * N + n];
+        vhi[e] = vsrc[static_cast<size_t>(d + half) * N + n];
+      }
+    }
+    auto put = [](uint16_t *dst, const uint16_t (&val)[W]) {
+      if constexpr (VEC) {
+        *reinterpret_cast<uint4 *>(dst) = make_uint4(
+            val[0] | (static_cast<uint32_t>(val[1]) << 16), val[2] | (static_cast<uint32_t>(val[3]) << 16),
+            val[4] | (static_cast<uint32_t>(val[5]) << 16), val[6] | (static_cast<uint32_t>(val[7]) << 16));
+      } else {
+        dst[0] = val[0];
+      }
+    };
     if (is_q) {
       uint16_t *dst = q_out + (static_cast<size_t>(n) * n_q + head) * hd;
-      dst[d] = lo;
-      dst[d + half] = hi;
+      put(dst + d0, lo);
+      put(dst + d0 + half, hi);
     } else {
       const size_t off = (static_cast<size_t>(p) * n_kv + head) * hd;
-      k_cache[off + d] = lo;
-      k_cache[off + d + half] = hi;
-      v_cache[off + d] = vsrc[static_cast<size_t>(d) * N + n];
-      v_cache[off + d + half] = vsrc[static_cast<size_t>(d + half) * N + n];
+      put(k_cache + off + d0, lo);
+      put(k_cache + off + d0 + half, hi);
+      put(v_cache + off + d0, vlo);
+      put(v_cache + off + d0 + half, vhi);
     }
   }
 }
@@ -245,13 +269,25 @@ extern "C" int chr_dv2_rope_kv_cols(const void *q, const void *k, const void *v,
   if (N < 1 || N > kMaxCols) {
     return -2;
   }
-  rope_kv_cols<<<dim3(static_cast<unsigned>(n_q + n_kv)), dim3(256), 0,
-                 static_cast<hipStream_t>(stream)>>>(
-      static_cast<const uint16_t *>(q), static_cast<const uint16_t *>(k),
-      static_cast<const uint16_t *>(v), static_cast<uint16_t *>(q_out),
-      static_cast<uint16_t *>(k_cache), static_cast<uint16_t *>(v_cache),
-      static_cast<const uint16_t *>(cos), static_cast<const uint16_t *>(sin),
-      static_cast<const int64_t *>(start), N, n_q, n_kv, hd, max_seq);
+  const bool vec = (hd % 16) == 0 && aligned16(q_out) && aligned16(k_cache) && aligned16(v_cache);
+  const int items = (hd / 2 / (vec ? 8 : 1)) * N;
+  const dim3 grid(static_cast<unsigned>(n_q + n_kv), static_cast<unsigned>((items + 255) / 256));
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (vec) {
+    rope_kv_cols<true><<<grid, dim3(256), 0, st>>>(
+        static_cast<const uint16_t *>(q), static_cast<const uint16_t *>(k),
+        static_cast<const uint16_t *>(v), static_cast<uint16_t *>(q_out),
+        static_cast<uint16_t *>(k_cache), static_cast<uint16_t *>(v_cache),
+        static_cast<const uint16_t *>(cos), static_cast<const uint16_t *>(sin),
+        static_cast<const int64_t *>(start), N, n_q, n_kv, hd, max_seq);
+  } else {
+    rope_kv_cols<false><<<grid, dim3(256), 0, st>>>(
+        static_cast<const uint16_t *>(q), static_cast<const uint16_t *>(k),
+        static_cast<const uint16_t *>(v), static_cast<uint16_t *>(q_out),
+        static_cast<uint16_t *>(k_cache), static_cast<uint16_t *>(v_cache),
+        static_cast<const uint16_t *>(cos), static_cast<const uint16_t *>(sin),
+        static_cast<const int64_t *>(start), N, n_q, n_kv, hd, max_seq);
+  }
   return launch_rc();
 }
 

@@ -191,6 +191,16 @@ int check_args(const chr_nf4_dev_t *w, int32_t N, bool need_ptrs, chr_nf4_dev_t 
   return 0;
 }
 
+// Up to three matrices that share x, K and the chunk (q, k and v of one layer): their row
+// blocks are numbered through on grid.x, their outputs stacked in y and in the partials.
+struct GemmSegs {
+  const uint8_t *packed[3];
+  const uint16_t *scale[3];
+  int M[3];       // rows of each matrix
+  int blocks[3];  // row blocks (of kBM rows) of each
+  int row0[3];    // first output row of each
+};
+
 template <int NB>
 struct GemmLds {
   float lut[16];                                  // at LDS address 0 (lookup8)
@@ -320,12 +330,11 @@ __device__ __forceinline__ bf16x8 dequant8(uint32_t w, float s, const float *lut
 // NB: 32-column blocks of the activation tile (1 for N <= 32, 2 for N <= 64); one
 // dequantised weight fragment feeds NB MFMAs.
 template <bool VEC, int NB>
-__global__ __launch_bounds__(kGemmBlock) void gemm_mfma(const uint8_t *__restrict__ packed,
-                                                        const uint16_t *__restrict__ scale,
+__global__ __launch_bounds__(kGemmBlock) void gemm_mfma(const GemmSegs segs,
                                                         const uint16_t *__restrict__ x,
                                                         uint16_t *__restrict__ y,
-                                                        float *__restrict__ partial, int M, int K,
-                                                        int K_pad, int N, int n_ktiles,
+                                                        float *__restrict__ partial, int M_all,
+                                                        int K, int K_pad, int N, int n_ktiles,
                                                         int tiles_per_split,
                                                         const uint16_t *__restrict__ bias,
                                                         const uint16_t *res) {
@@ -341,7 +350,22 @@ __global__ __launch_bounds__(kGemmBlock) void gemm_mfma(const uint8_t *__restric
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
   const int tid = threadIdx.x;
-  const int row_base = blockIdx.x * kBM + wave * 32;
+  // which matrix this row block belongs to, and the block's number inside it
+  int bx = static_cast<int>(blockIdx.x);
+  int seg = 0;
+  if (bx >= segs.blocks[0]) {
+    bx -= segs.blocks[0];
+    seg = 1;
+    if (bx >= segs.blocks[1]) {
+      bx -= segs.blocks[1];
+      seg = 2;
+    }
+  }
+  const uint8_t *__restrict__ packed = segs.packed[seg];
+  const uint16_t *__restrict__ scale = segs.scale[seg];
+  const int M = segs.M[seg];
+  const int out0 = segs.row0[seg];
+  const int row_base = bx * kBM + wave * 32;
   const int khalf = lane >> 5;  // which 32-wide half of a 64-wide K step
   uint8_t *wst = lds.w[wave];
   uint16_t *sst = lds.sc[wave];
@@ -421,10 +445,10 @@ __global__ __launch_bounds__(kGemmBlock) void gemm_mfma(const uint8_t *__restric
           if (r < M) {
             // unsplit: the epilogue of reduce_splitk, here (res may alias y: same thread,
             // same element)
-            const size_t at = static_cast<size_t>(r) * N + n;
+            const size_t at = static_cast<size_t>(out0 + r) * N + n;
             uint16_t v = f32_to_bf16(acc[nb][i]);
             if (bias != nullptr) {
-              v = f32_to_bf16(bf16_to_f32(v) + bf16_to_f32(bias[r]));
+              v = f32_to_bf16(bf16_to_f32(v) + bf16_to_f32(bias[out0 + r]));
             }
             if (res != nullptr) {
               v = f32_to_bf16(bf16_to_f32(res[at]) + bf16_to_f32(v));
@@ -433,12 +457,12 @@ __global__ __launch_bounds__(kGemmBlock) void gemm_mfma(const uint8_t *__restric
           }
         }
       } else {
-        float *p = partial + static_cast<size_t>(blockIdx.y) * M * N;
+        float *p = partial + static_cast<size_t>(blockIdx.y) * M_all * N;
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
           const int r = rbase + 8 * (i >> 2) + (i & 3);
           if (r < M) {
-            p[static_cast<size_t>(r) * N + n] = acc[nb][i];
+            p[static_cast<size_t>(out0 + r) * N + n] = acc[nb][i];
           }
         }
       }
@@ -520,10 +544,36 @@ extern "C" int chr_nf4_gemm_plan(const chr_nf4_dev_t *w, int32_t N, int32_t have
 namespace chr {
 namespace {
 
+// Grid, split and workspace of a launch over nseg stacked matrices (nseg == 1: plan_impl).
+struct StackPlan {
+  GemmSegs segs;
+  int M_all, grid_x, grid_y, n_ktiles, tiles_per_split;
+  int64_t ws_floats;
+};
+
+StackPlan plan_stack(const chr_nf4_dev_t *h, int nseg, int N, int have_ws) {
+  StackPlan sp{};
+  for (int i = 0; i < 3; ++i) {
+    const bool on = i < nseg;
+    sp.segs.packed[i] = on ? h[i].packed : nullptr;
+    sp.segs.scale[i] = on ? h[i].scale : nullptr;
+    sp.segs.M[i] = on ? h[i].M : 0;
+    sp.segs.blocks[i] = on ? ceil_div(h[i].M, kBM) : 0;
+    sp.segs.row0[i] = sp.M_all;
+    sp.M_all += sp.segs.M[i];
+    sp.grid_x += sp.segs.blocks[i];
+  }
+  sp.n_ktiles = ceil_div(h[0].K_pad, kBK);
+  pick_split(sp.grid_x, sp.n_ktiles, have_ws, &sp.grid_y, &sp.tiles_per_split);
+  sp.ws_floats = sp.grid_y > 1 ? static_cast<int64_t>(sp.grid_y) * sp.M_all * N : 0;
+  return sp;
+}
+
 // live_max: widest chunk the entry launches.  The reference's entries stop at 32 columns
-// (wider ones are described by the planner only); chr_dv2_gemm_add goes to 64.
-int gemm_launch(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N, float *ws,
-                int64_t ws_floats, void *stream, int32_t max_n, const void *bias,
+// (wider ones are described by the planner only); the chr_dv2_gemm_* entries go to 64.
+// w[0..nseg) share K and x; y, bias and res cover the stacked rows.
+int gemm_launch(const chr_nf4_dev_t *const *w, int nseg, const void *x, void *y, int32_t N,
+                float *ws, int64_t ws_floats, void *stream, int32_t max_n, const void *bias,
                 const void *res, int32_t live_max = kLiveMaxN) {
   if (x == nullptr || y == nullptr) {
     return -1;
@@ -531,32 +581,41 @@ int gemm_launch(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N, float
   if (max_n < 1 || max_n > kPlanMaxN) {
     return -2;
   }
-  chr_nf4_dev_t h{};
-  const int rc = check_args(w, N, /*need_ptrs=*/true, &h, max_n);
-  if (rc != 0) {
-    return rc;
+  chr_nf4_dev_t h[3] = {};
+  for (int i = 0; i < nseg; ++i) {
+    const int rc = check_args(w[i], N, /*need_ptrs=*/true, &h[i], max_n);
+    if (rc != 0) {
+      return rc;
+    }
+    if (h[i].K != h[0].K || h[i].K_pad != h[0].K_pad) {
+      return -3;  // stacked matrices multiply the same x
+    }
   }
   if (N > live_max) {
     return -2;
   }
-  if (!aligned16(h.packed) || !aligned16(x) || !aligned2(h.scale)) {
+  for (int i = 0; i < nseg; ++i) {
+    if (!aligned16(h[i].packed) || !aligned2(h[i].scale)) {
+      return -5;
+    }
+  }
+  if (!aligned16(x)) {
     return -5;
   }
   if (N == 1) {
-    if (bias != nullptr || res != nullptr) {
-      return -2;  // the fused epilogue belongs to the tiles (N >= 2)
+    if (bias != nullptr || res != nullptr || nseg != 1) {
+      return -2;  // the fused epilogue and the stacking belong to the tiles (N >= 2)
     }
-    return gemv_entry(&h, x, y, stream, nullptr, nullptr, 0.f);
+    return gemv_entry(&h[0], x, y, stream, nullptr, nullptr, 0.f);
   }
   const int have_ws = (ws != nullptr && ws_floats > 0) ? 1 : 0;
-  chr_nf4_plan_t p{};
-  plan_impl(h, N, have_ws, &p);
-  if (p.ws_floats > 0 && (!have_ws || ws_floats < p.ws_floats)) {
+  const StackPlan sp = plan_stack(h, nseg, N, have_ws);
+  if (sp.ws_floats > 0 && (!have_ws || ws_floats < sp.ws_floats)) {
     return -7;
   }
-  float *partial = p.grid_y > 1 ? ws : nullptr;
+  float *partial = sp.grid_y > 1 ? ws : nullptr;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  const dim3 grid(static_cast<unsigned>(p.grid_x), static_cast<unsigned>(p.grid_y));
+  const dim3 grid(static_cast<unsigned>(sp.grid_x), static_cast<unsigned>(sp.grid_y));
   // 16-byte activation vectors need N in {8, 16, 32, 64}; x is 16-byte aligned (checked above)
   const bool vec = N == 8 || N == 16 || N == 32 || N == 64;
   if (gemm_lds_ready() != 0) {
@@ -567,32 +626,28 @@ int gemm_launch(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N, float
   const auto *bp = static_cast<const uint16_t *>(bias);
   const auto *rp = static_cast<const uint16_t *>(res);
   const dim3 block(kGemmBlock);
+  const int K = h[0].K, K_pad = h[0].K_pad;
   if (N <= kBN) {
     if (vec) {
       gemm_mfma<true, 1><<<grid, block, gemm_lds_bytes(1), st>>>(
-          h.packed, h.scale, xp, yp, partial, h.M, h.K, h.K_pad, N, p.n_ktiles, p.tiles_per_split,
-          bp, rp);
+          sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, sp.n_ktiles, sp.tiles_per_split, bp, rp);
     } else {
       gemm_mfma<false, 1><<<grid, block, gemm_lds_bytes(1), st>>>(
-          h.packed, h.scale, xp, yp, partial, h.M, h.K, h.K_pad, N, p.n_ktiles, p.tiles_per_split,
-          bp, rp);
+          sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, sp.n_ktiles, sp.tiles_per_split, bp, rp);
     }
   } else {
     if (vec) {
       gemm_mfma<true, 2><<<grid, block, gemm_lds_bytes(2), st>>>(
-          h.packed, h.scale, xp, yp, partial, h.M, h.K, h.K_pad, N, p.n_ktiles, p.tiles_per_split,
-          bp, rp);
+          sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, sp.n_ktiles, sp.tiles_per_split, bp, rp);
     } else {
       gemm_mfma<false, 2><<<grid, block, gemm_lds_bytes(2), st>>>(
-          h.packed, h.scale, xp, yp, partial, h.M, h.K, h.K_pad, N, p.n_ktiles, p.tiles_per_split,
-          bp, rp);
+          sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, sp.n_ktiles, sp.tiles_per_split, bp, rp);
     }
   }
   if (partial != nullptr) {
-    const int rows = h.M * N;
+    const int rows = sp.M_all * N;
     reduce_splitk<<<dim3(static_cast<unsigned>(ceil_div(rows, 256))), dim3(256), 0, st>>>(
-        partial, static_cast<uint16_t *>(y), rows, p.grid_y, N,
-        static_cast<const uint16_t *>(bias), static_cast<const uint16_t *>(res));
+        partial, yp, rows, sp.grid_y, N, bp, rp);
   }
   return launch_rc();
 }
@@ -602,13 +657,35 @@ int gemm_launch(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N, float
 
 extern "C" int chr_nf4_gemm_ws_max(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N,
                                    float *ws, int64_t ws_floats, void *stream, int32_t max_n) {
-  return gemm_launch(w, x, y, N, ws, ws_floats, stream, max_n, nullptr, nullptr);
+  return gemm_launch(&w, 1, x, y, N, ws, ws_floats, stream, max_n, nullptr, nullptr);
 }
 
 extern "C" int chr_dv2_gemm_add(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N,
                                 float *ws, int64_t ws_floats, const void *bias,
                                 const void *residual, void *stream) {
-  return gemm_launch(w, x, y, N, ws, ws_floats, stream, kPlanMaxN, bias, residual, kPlanMaxN);
+  return gemm_launch(&w, 1, x, y, N, ws, ws_floats, stream, kPlanMaxN, bias, residual, kPlanMaxN);
+}
+
+extern "C" int64_t chr_dv2_gemm_qkv_ws(const chr_nf4_dev_t *q, const chr_nf4_dev_t *k,
+                                       const chr_nf4_dev_t *v, int32_t N) {
+  if (q == nullptr || k == nullptr || v == nullptr || N < 2 || N > kPlanMaxN) {
+    return -1;
+  }
+  const chr_nf4_dev_t h[3] = {*q, *k, *v};
+  if (h[0].M < 1 || h[1].M < 1 || h[2].M < 1 || h[0].K < 1 || !k_pad_ok(h[0].K, h[0].K_pad)) {
+    return -1;
+  }
+  return plan_stack(h, 3, N, 1).ws_floats;
+}
+
+extern "C" int chr_dv2_gemm_qkv(const chr_nf4_dev_t *q, const chr_nf4_dev_t *k,
+                                const chr_nf4_dev_t *v, const void *x, void *y, int32_t N,
+                                float *ws, int64_t ws_floats, const void *bias, void *stream) {
+  if (q == nullptr || k == nullptr || v == nullptr) {
+    return -1;
+  }
+  const chr_nf4_dev_t *w[3] = {q, k, v};
+  return gemm_launch(w, 3, x, y, N, ws, ws_floats, stream, kPlanMaxN, bias, nullptr, kPlanMaxN);
 }
 
 extern "C" int chr_nf4_gemm_ws(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N,

@@ -12,8 +12,8 @@ from __future__ import annotations
 
 import torch
 
-from ..nf4 import (LIVE_MAX_N, PLAN_MAX_N, dv2_add_cols, dv2_attn_chunk, dv2_rms_cols, dv2_rope_kv_cols,
-                   dv2_swiglu_elems, nf4_gemm)
+from ..nf4 import (LIVE_MAX_N, PLAN_MAX_N, dv2_add_cols, dv2_attn_chunk, dv2_gemm_qkv, dv2_rms_cols,
+                   dv2_rope_kv_cols, dv2_swiglu_elems, nf4_gemm)
 from .embed import gather_embed
 from .linear import DeviceLinear, DeviceWeights, nf4_linear
 from .ops import causal_attend, rms, split_qkv, swiglu
@@ -107,6 +107,16 @@ class ChunkPrefill:
         self.first_len = torch.zeros((), dtype=torch.int32, device=dev)
         self.last_hidden = torch.zeros(spec.hidden, dtype=torch.bfloat16, device=dev)
         self._graphs: dict[int, torch.cuda.CUDAGraph] = {}
+        # stacked q/k/v biases for the one-launch q/k/v GEMM (zeros where a matrix has none)
+        self._qkv_bias: list[torch.Tensor | None] = []
+        for layer in weights.layers:
+            mats = (layer.q, layer.k, layer.v)
+            if layer.wqkv is not None or all(m.bias is None for m in mats):
+                self._qkv_bias.append(None)
+            else:
+                self._qkv_bias.append(torch.cat([
+                    m.bias if m.bias is not None else torch.zeros(m.M, dtype=torch.bfloat16, device=dev)
+                    for m in mats]).contiguous())
 
     def _chunk(self, n: int) -> None:
         state, weights, spec = self.state, self.weights, self.state.spec
@@ -117,6 +127,10 @@ class ChunkPrefill:
             h = dv2_rms_cols(x, layer.norm1, spec.rms_eps)
             if layer.wqkv is not None:
                 y = _gemm_cols(layer.wqkv, h)  # rows are [Q | K | V]
+                q, k, v = y[:spec.q_dim], y[spec.q_dim:spec.q_dim + spec.kv_dim], y[spec.q_dim + spec.kv_dim:]
+            elif n >= 2:
+                y = dv2_gemm_qkv(*((m.packed, m.scale, m.M) for m in (layer.q, layer.k, layer.v)), h,
+                                 bias=self._qkv_bias[li])
                 q, k, v = y[:spec.q_dim], y[spec.q_dim:spec.q_dim + spec.kv_dim], y[spec.q_dim + spec.kv_dim:]
             else:
                 q, k, v = _gemm_cols(layer.q, h), _gemm_cols(layer.k, h), _gemm_cols(layer.v, h)

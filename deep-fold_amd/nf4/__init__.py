@@ -52,6 +52,7 @@ __all__ = [
     "dv2_attn_chunk",
     "dv2_swiglu_elems",
     "dv2_add_cols",
+    "dv2_gemm_qkv",
     "library_path",
 ]
 
@@ -129,6 +130,8 @@ EXPORTS = (
     ("chr_dv2_swiglu_elems", ctypes.c_int, [_P, _P, _P, ctypes.c_int64, _P]),
     ("chr_dv2_add_cols", ctypes.c_int, [_P, _P, _P, _I, _I, _P]),
     ("chr_dv2_gemm_add", ctypes.c_int, [_DP, _P, _P, _I, _P, ctypes.c_int64, _P, _P, _P]),
+    ("chr_dv2_gemm_qkv_ws", ctypes.c_int64, [_DP, _DP, _DP, _I]),
+    ("chr_dv2_gemm_qkv", ctypes.c_int, [_DP, _DP, _DP, _P, _P, _I, _P, ctypes.c_int64, _P, _P]),
     ("chr_dv2_mark_written", ctypes.c_int, [_P, _P, _P]),
     ("chr_dv2_argmax_commit", ctypes.c_int, [_P, _I, _P, _P, _P, _P, _P, _I, _P]),
     ("chr_nf4_abi_version", ctypes.c_int, []),
@@ -834,4 +837,33 @@ def dv2_add_cols(y: torch.Tensor, a: torch.Tensor | None = None, bias: torch.Ten
                                       None if bias is None else bias.data_ptr(), int(y.size(0)),
                                       int(y.size(1)), _stream())
     _check_rc("chr_dv2_add_cols", rc)
+    return y
+
+
+def dv2_gemm_qkv(q, k, v, x: torch.Tensor, bias: torch.Tensor | None = None) -> torch.Tensor:
+    """One launch for q, k and v of a layer: ``q``, ``k``, ``v`` are ``(packed, scale, M)``
+    triples over the same ``K``; ``x`` is bf16 ``[K, N]``, N = 2..64.  Returns
+    ``[Mq + Mk + Mv, N]`` (q's rows first) with ``bias`` (stacked, bf16) added per row."""
+    _bf16_cuda(x, "x")
+    _need(x.dim() == 2 and 2 <= x.size(1) <= PLAN_MAX_N, f"x must be [K, N] with N in 2..{PLAN_MAX_N}")
+    K, n = int(x.size(0)), int(x.size(1))
+    kp = _k_pad(K)
+    devs = []
+    for name, (packed, scale, M) in (("q", q), ("k", k), ("v", v)):
+        _check_packed(packed, scale, int(M), K, kp, name)
+        _need(packed.is_contiguous() and scale.is_contiguous(), f"{name} blobs must be contiguous")
+        devs.append(_dev(packed, scale, int(M), K, kp))
+    m_all = sum(d.M for d in devs)
+    if bias is not None:
+        _bf16_cuda(bias, "bias")
+        _need(bias.numel() == m_all, f"bias must hold {m_all} elements")
+    lib = _load_ext()
+    need = int(lib.chr_dv2_gemm_qkv_ws(ctypes.byref(devs[0]), ctypes.byref(devs[1]), ctypes.byref(devs[2]), n))
+    _need(need >= 0, "chr_dv2_gemm_qkv_ws refused the shapes")
+    ws = torch.empty(max(need, 1), dtype=torch.float32, device=x.device)
+    y = torch.empty((m_all, n), dtype=torch.bfloat16, device=x.device)
+    rc = lib.chr_dv2_gemm_qkv(ctypes.byref(devs[0]), ctypes.byref(devs[1]), ctypes.byref(devs[2]),
+                              x.data_ptr(), y.data_ptr(), n, ws.data_ptr() if need else None, need,
+                              None if bias is None else bias.data_ptr(), _stream())
+    _check_rc("chr_dv2_gemm_qkv", rc)
     return y

@@ -259,6 +259,17 @@ int chr_dv2_add_cols(void *y, const void *a, const void *bias, int32_t rows, int
 int chr_dv2_gemm_add(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N, float *ws,
                      int64_t ws_floats, const void *bias, const void *residual, void *stream);
 
+/* q, k and v of one layer in one launch (the prefill twin of chr_nf4_gemv_qkv,
+ * gpu/decodev2/ops.py:27-35 calls three GEMMs): the three matrices share x [K, N] and K; y is
+ * [Mq + Mk + Mv, N] with q's rows first, bias (bf16 [Mq + Mk + Mv], or NULL) is added per row
+ * as chr_dv2_gemm_add adds it.  N = 2..64.  chr_dv2_gemm_qkv_ws gives the fp32 workspace
+ * elements the launch needs (0: none; -1: bad arguments).  No reference counterpart. */
+int64_t chr_dv2_gemm_qkv_ws(const chr_nf4_dev_t *q, const chr_nf4_dev_t *k,
+                            const chr_nf4_dev_t *v, int32_t N);
+int chr_dv2_gemm_qkv(const chr_nf4_dev_t *q, const chr_nf4_dev_t *k, const chr_nf4_dev_t *v,
+                     const void *x, void *y, int32_t N, float *ws, int64_t ws_floats,
+                     const void *bias, void *stream);
+
 /* Library version, for the loader's sanity check. */
 int chr_nf4_abi_version(void);
 

@@ -230,6 +230,34 @@ def test_wide_chunk_equals_two_narrow_ones(m, k, n):
         nf4.nf4_gemm(dp, ds, x, m, k, kp)  # the reference's ceiling without max_n
 
 
+@pytest.mark.parametrize("mq,mk,k,n,bias", [(256, 64, 512, 8, True), (5120, 1024, 5120, 64, True),
+                                            (130, 70, 1088, 5, False), (2048, 256, 2048, 32, False)])
+def test_stacked_qkv_equals_three_gemms(mq, mk, k, n, bias):
+    say("gemm_qkv", mq, mk, k, n, bias)
+    rng = np.random.default_rng(mq + n)
+    mats = []
+    for m in (mq, mk, mk):
+        p, s_ = oc.c_encode((rng.standard_normal((m, k)) * 0.05).astype(np.float32))
+        mats.append((up(p), up_scale(s_), m))
+    kp = mats[0][0].shape[1] * 2
+    x = bf16_tensor(rnd((k, n), 1))
+    b = bf16_tensor(rnd((mq + 2 * mk,), 2)) if bias else None
+    got = nf4.dv2_gemm_qkv(*mats, x, bias=b)
+    assert tuple(got.shape) == (mq + 2 * mk, n)
+    row = 0
+    for packed, scale, m in mats:
+        want = nf4.nf4_gemm(packed, scale, x, m, k, kp, max_n=64)
+        if bias:
+            want = want + b[row:row + m, None]
+        # the stack has its own split-K (more row blocks, fewer splits): equal up to the
+        # fp32 summation order
+        d = (got[row:row + m].float() - want.float()).abs().max().item()
+        assert d <= 2 ** -7 * max(1.0, want.float().abs().max().item()), (row, d)
+        row += m
+    with pytest.raises(RuntimeError):
+        nf4.dv2_gemm_qkv(mats[0], mats[1], (mats[2][0], mats[2][1], mk + 1), x)
+
+
 # ---- the chunked prefill built from them ------------------------------------------------
 
 LONG = [4, 5, 6, 7, 1, 2, 3, 4]
