@@ -495,6 +495,26 @@ __global__ __launch_bounds__(256) void reduce_splitk(const float *__restrict__ p
   y[i] = v;
 }
 
+// Gate rows stacked over up rows: y[i] = silu(bf16 gate) * bf16 up with the roundings of the
+// reference's separate ops (F.silu on bf16, then a bf16 product; gpu/decodev2/ops.py:23-24).
+__global__ __launch_bounds__(256) void reduce_swiglu(const float *__restrict__ partial,
+                                                     uint16_t *__restrict__ y, int half_rows,
+                                                     int split) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= half_rows) {
+    return;
+  }
+  float g = 0.f, u = 0.f;
+  for (int j = 0; j < split; ++j) {
+    const float *p = partial + static_cast<size_t>(j) * 2 * half_rows;
+    g += p[i];
+    u += p[half_rows + i];
+  }
+  const float a = bf16_to_f32(f32_to_bf16(g));
+  const float act = bf16_to_f32(f32_to_bf16(a / (1.f + expf(-a))));
+  y[i] = f32_to_bf16(act * bf16_to_f32(f32_to_bf16(u)));
+}
+
 // The kernels use more than the default 64 KB of LDS: raise the limit once per process
 // (on the first launch, which a caller warming up before graph capture makes eagerly).
 int gemm_lds_ready() {
@@ -574,7 +594,7 @@ StackPlan plan_stack(const chr_nf4_dev_t *h, int nseg, int N, int have_ws) {
 // w[0..nseg) share K and x; y, bias and res cover the stacked rows.
 int gemm_launch(const chr_nf4_dev_t *const *w, int nseg, const void *x, void *y, int32_t N,
                 float *ws, int64_t ws_floats, void *stream, int32_t max_n, const void *bias,
-                const void *res, int32_t live_max = kLiveMaxN) {
+                const void *res, int32_t live_max = kLiveMaxN, bool swiglu = false) {
   if (x == nullptr || y == nullptr) {
     return -1;
   }
@@ -609,11 +629,18 @@ int gemm_launch(const chr_nf4_dev_t *const *w, int nseg, const void *x, void *y,
     return gemv_entry(&h[0], x, y, stream, nullptr, nullptr, 0.f);
   }
   const int have_ws = (ws != nullptr && ws_floats > 0) ? 1 : 0;
-  const StackPlan sp = plan_stack(h, nseg, N, have_ws);
+  StackPlan sp = plan_stack(h, nseg, N, have_ws);
+  if (swiglu) {
+    // the activation lives in the reduce, so this launch always goes through fp32 partials
+    if (nseg != 2 || h[0].M != h[1].M || bias != nullptr || res != nullptr) {
+      return -3;
+    }
+    sp.ws_floats = static_cast<int64_t>(sp.grid_y) * sp.M_all * N;
+  }
   if (sp.ws_floats > 0 && (!have_ws || ws_floats < sp.ws_floats)) {
     return -7;
   }
-  float *partial = sp.grid_y > 1 ? ws : nullptr;
+  float *partial = (sp.grid_y > 1 || swiglu) ? ws : nullptr;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const dim3 grid(static_cast<unsigned>(sp.grid_x), static_cast<unsigned>(sp.grid_y));
   // 16-byte activation vectors need N in {8, 16, 32, 64}; x is 16-byte aligned (checked above)
@@ -644,7 +671,11 @@ int gemm_launch(const chr_nf4_dev_t *const *w, int nseg, const void *x, void *y,
           sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, sp.n_ktiles, sp.tiles_per_split, bp, rp);
     }
   }
-  if (partial != nullptr) {
+  if (swiglu) {
+    const int half_rows = h[0].M * N;
+    reduce_swiglu<<<dim3(static_cast<unsigned>(ceil_div(half_rows, 256))), dim3(256), 0, st>>>(
+        partial, yp, half_rows, sp.grid_y);
+  } else if (partial != nullptr) {
     const int rows = sp.M_all * N;
     reduce_splitk<<<dim3(static_cast<unsigned>(ceil_div(rows, 256))), dim3(256), 0, st>>>(
         partial, yp, rows, sp.grid_y, N, bp, rp);
@@ -696,4 +727,28 @@ extern "C" int chr_nf4_gemm_ws(const chr_nf4_dev_t *w, const void *x, void *y, i
 extern "C" int chr_nf4_gemm(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N,
                             void *stream) {
   return chr_nf4_gemm_ws(w, x, y, N, nullptr, 0, stream);
+}
+
+extern "C" int64_t chr_dv2_gemm_swiglu_ws(const chr_nf4_dev_t *gate, const chr_nf4_dev_t *up,
+                                          int32_t N) {
+  if (gate == nullptr || up == nullptr || N < 2 || N > kPlanMaxN) {
+    return -1;
+  }
+  const chr_nf4_dev_t h[2] = {*gate, *up};
+  if (h[0].M < 1 || h[0].M != h[1].M || h[0].K < 1 || !k_pad_ok(h[0].K, h[0].K_pad)) {
+    return -1;
+  }
+  const StackPlan sp = plan_stack(h, 2, N, 1);
+  return static_cast<int64_t>(sp.grid_y) * sp.M_all * N;
+}
+
+extern "C" int chr_dv2_gemm_swiglu(const chr_nf4_dev_t *gate, const chr_nf4_dev_t *up,
+                                   const void *x, void *y, int32_t N, float *ws,
+                                   int64_t ws_floats, void *stream) {
+  if (gate == nullptr || up == nullptr) {
+    return -1;
+  }
+  const chr_nf4_dev_t *w[2] = {gate, up};
+  return gemm_launch(w, 2, x, y, N, ws, ws_floats, stream, kPlanMaxN, nullptr, nullptr, kPlanMaxN,
+                     /*swiglu=*/true);
 }

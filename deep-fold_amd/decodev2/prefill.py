@@ -12,8 +12,8 @@ from __future__ import annotations
 
 import torch
 
-from ..nf4 import (LIVE_MAX_N, PLAN_MAX_N, dv2_add_cols, dv2_attn_chunk, dv2_gemm_qkv, dv2_rms_cols,
-                   dv2_rope_kv_cols, dv2_swiglu_elems, nf4_gemm)
+from ..nf4 import (LIVE_MAX_N, PLAN_MAX_N, dv2_add_cols, dv2_attn_chunk, dv2_gemm_qkv, dv2_gemm_swiglu,
+                   dv2_rms_cols, dv2_rope_kv_cols, dv2_swiglu_elems, nf4_gemm)
 from .embed import gather_embed
 from .linear import DeviceLinear, DeviceWeights, nf4_linear
 from .ops import causal_attend, rms, split_qkv, swiglu
@@ -139,7 +139,11 @@ class ChunkPrefill:
             dv2_attn_chunk(q_rows, k_cache, v_cache, attn, self.first_len, spec.attn_scale)
             _gemm_cols(layer.o, attn, residual=x)
             h = dv2_rms_cols(x, layer.norm2, spec.rms_eps)
-            act = dv2_swiglu_elems(_gemm_cols(layer.gate, h), _gemm_cols(layer.up, h))
+            if n >= 2 and layer.gate.bias is None and layer.up.bias is None:
+                act = dv2_gemm_swiglu((layer.gate.packed, layer.gate.scale, layer.gate.M),
+                                      (layer.up.packed, layer.up.scale, layer.up.M), h)
+            else:
+                act = dv2_swiglu_elems(_gemm_cols(layer.gate, h), _gemm_cols(layer.up, h))
             _gemm_cols(layer.down, act, residual=x)
         self.last_hidden.copy_(x[:, n - 1])
 

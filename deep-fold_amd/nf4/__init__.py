@@ -53,6 +53,7 @@ __all__ = [
     "dv2_swiglu_elems",
     "dv2_add_cols",
     "dv2_gemm_qkv",
+    "dv2_gemm_swiglu",
     "library_path",
 ]
 
@@ -132,6 +133,8 @@ EXPORTS = (
     ("chr_dv2_gemm_add", ctypes.c_int, [_DP, _P, _P, _I, _P, ctypes.c_int64, _P, _P, _P]),
     ("chr_dv2_gemm_qkv_ws", ctypes.c_int64, [_DP, _DP, _DP, _I]),
     ("chr_dv2_gemm_qkv", ctypes.c_int, [_DP, _DP, _DP, _P, _P, _I, _P, ctypes.c_int64, _P, _P]),
+    ("chr_dv2_gemm_swiglu_ws", ctypes.c_int64, [_DP, _DP, _I]),
+    ("chr_dv2_gemm_swiglu", ctypes.c_int, [_DP, _DP, _P, _P, _I, _P, ctypes.c_int64, _P]),
     ("chr_dv2_mark_written", ctypes.c_int, [_P, _P, _P]),
     ("chr_dv2_argmax_commit", ctypes.c_int, [_P, _I, _P, _P, _P, _P, _P, _I, _P]),
     ("chr_nf4_abi_version", ctypes.c_int, []),
@@ -866,4 +869,28 @@ def dv2_gemm_qkv(q, k, v, x: torch.Tensor, bias: torch.Tensor | None = None) -> 
                               x.data_ptr(), y.data_ptr(), n, ws.data_ptr() if need else None, need,
                               None if bias is None else bias.data_ptr(), _stream())
     _check_rc("chr_dv2_gemm_qkv", rc)
+    return y
+
+
+def dv2_gemm_swiglu(gate, up, x: torch.Tensor) -> torch.Tensor:
+    """``silu(gate @ x) * (up @ x)`` in one GEMM launch and its reduce; ``gate`` and ``up`` are
+    ``(packed, scale, M)`` triples of one shape; ``x`` is bf16 ``[K, N]``, N = 2..64."""
+    _bf16_cuda(x, "x")
+    _need(x.dim() == 2 and 2 <= x.size(1) <= PLAN_MAX_N, f"x must be [K, N] with N in 2..{PLAN_MAX_N}")
+    K, n = int(x.size(0)), int(x.size(1))
+    kp = _k_pad(K)
+    devs = []
+    for name, (packed, scale, M) in (("gate", gate), ("up", up)):
+        _check_packed(packed, scale, int(M), K, kp, name)
+        _need(packed.is_contiguous() and scale.is_contiguous(), f"{name} blobs must be contiguous")
+        devs.append(_dev(packed, scale, int(M), K, kp))
+    _need(devs[0].M == devs[1].M, "gate and up must have the same number of rows")
+    lib = _load_ext()
+    need = int(lib.chr_dv2_gemm_swiglu_ws(ctypes.byref(devs[0]), ctypes.byref(devs[1]), n))
+    _need(need > 0, "chr_dv2_gemm_swiglu_ws refused the shapes")
+    ws = torch.empty(need, dtype=torch.float32, device=x.device)
+    y = torch.empty((devs[0].M, n), dtype=torch.bfloat16, device=x.device)
+    rc = lib.chr_dv2_gemm_swiglu(ctypes.byref(devs[0]), ctypes.byref(devs[1]), x.data_ptr(), y.data_ptr(),
+                                 n, ws.data_ptr(), need, _stream())
+    _check_rc("chr_dv2_gemm_swiglu", rc)
     return y

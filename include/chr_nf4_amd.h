@@ -270,6 +270,16 @@ int chr_dv2_gemm_qkv(const chr_nf4_dev_t *q, const chr_nf4_dev_t *k, const chr_n
                      const void *x, void *y, int32_t N, float *ws, int64_t ws_floats,
                      const void *bias, void *stream);
 
+/* Gate and up of a layer in one launch with the SwiGLU in the split-K reduce (the prefill twin
+ * of chr_nf4_gemv_swiglu; gpu/decodev2/prefill.py:133 runs two GEMMs, F.silu and a product):
+ * y [M, N] = silu(gate x) * (up x), gate and up rounded to bf16 first and the activation
+ * rounded to bf16 before the product, as those separate bf16 ops round.  Both matrices are
+ * M x K.  N = 2..64.  The launch always goes through fp32 partials: chr_dv2_gemm_swiglu_ws
+ * gives the workspace elements it needs (-1: bad arguments).  No reference counterpart. */
+int64_t chr_dv2_gemm_swiglu_ws(const chr_nf4_dev_t *gate, const chr_nf4_dev_t *up, int32_t N);
+int chr_dv2_gemm_swiglu(const chr_nf4_dev_t *gate, const chr_nf4_dev_t *up, const void *x,
+                        void *y, int32_t N, float *ws, int64_t ws_floats, void *stream);
+
 /* Library version, for the loader's sanity check. */
 int chr_nf4_abi_version(void);
 

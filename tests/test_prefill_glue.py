@@ -258,6 +258,29 @@ def test_stacked_qkv_equals_three_gemms(mq, mk, k, n, bias):
         nf4.dv2_gemm_qkv(mats[0], mats[1], (mats[2][0], mats[2][1], mk + 1), x)
 
 
+@pytest.mark.parametrize("m,k,n", [(256, 512, 8), (13824, 5120, 64), (130, 1088, 5), (384, 256, 2)])
+def test_stacked_gate_up_with_swiglu_in_the_reduce(m, k, n):
+    say("gemm_swiglu", m, k, n)
+    rng = np.random.default_rng(m + n)
+    mats = []
+    for _ in range(2):
+        p, s_ = oc.c_encode((rng.standard_normal((m, k)) * 0.05).astype(np.float32))
+        mats.append((up(p), up_scale(s_), m))
+    kp = mats[0][0].shape[1] * 2
+    x = bf16_tensor(rnd((k, n), 1))
+    got = nf4.dv2_gemm_swiglu(mats[0], mats[1], x)
+    g = nf4.nf4_gemm(mats[0][0], mats[0][1], x, m, k, kp, max_n=64)
+    u = nf4.nf4_gemm(mats[1][0], mats[1][1], x, m, k, kp, max_n=64)
+    want = F.silu(g) * u
+    # the stack has its own split-K, so gate and up may differ from the single GEMMs in the
+    # last bf16 digit before the activation
+    d = (got.float() - want.float()).abs()
+    tol = 2 ** -6 * torch.maximum(want.float().abs(), torch.full_like(d, 2 ** -10))
+    assert tuple(got.shape) == (m, n) and bool((d <= tol).all())
+    with pytest.raises(RuntimeError):
+        nf4.dv2_gemm_swiglu(mats[0], (mats[1][0], mats[1][1], m - 1), x)
+
+
 # ---- the chunked prefill built from them ------------------------------------------------
 
 LONG = [4, 5, 6, 7, 1, 2, 3, 4]
