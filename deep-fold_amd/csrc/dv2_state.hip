@@ -116,16 +116,30 @@ __global__ __launch_bounds__(kArgmaxBlock) void argmax_commit(
   // a thread, so "strictly better" keeps the lowest index of equal values.
   const bool vec = (reinterpret_cast<uintptr_t>(logits) & 15u) == 0;
   const int n8 = vec ? n >> 3 : 0;
-  for (int c = threadIdx.x; c < n8; c += kArgmaxBlock) {
-    const uint4 raw = reinterpret_cast<const uint4 *>(logits)[c];
-    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+  // kBatch loads are in flight together: one workgroup walks the whole vocabulary, so the
+  // loop is a chain of memory round trips and their number is what it costs
+  constexpr int kBatch = 8;
+  for (int c0 = threadIdx.x; c0 < n8; c0 += kArgmaxBlock * kBatch) {
+    uint4 raw[kBatch];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const float v = (j & 1) ? bf16_hi(w[j >> 1]) : bf16_lo(w[j >> 1]);
-      const int i = (c << 3) + j;
-      if (better(v, i, bv, bi)) {
-        bv = v;
-        bi = i;
+    for (int b = 0; b < kBatch; ++b) {
+      const int c = c0 + b * kArgmaxBlock;
+      raw[b] = reinterpret_cast<const uint4 *>(logits)[c < n8 ? c : c0];
+    }
+#pragma unroll
+    for (int b = 0; b < kBatch; ++b) {
+      const int c = c0 + b * kArgmaxBlock;
+      if (c < n8) {
+        const uint32_t w[4] = {raw[b].x, raw[b].y, raw[b].z, raw[b].w};
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float v = (j & 1) ? bf16_hi(w[j >> 1]) : bf16_lo(w[j >> 1]);
+          const int i = (c << 3) + j;
+          if (better(v, i, bv, bi)) {
+            bv = v;
+            bi = i;
+          }
+        }
       }
     }
   }
