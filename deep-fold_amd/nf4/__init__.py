@@ -41,6 +41,7 @@ __all__ = [
     "dv2_argmax_commit",
     "dv2_begin_step",
     "ATTN_WG_WAVES",
+    "ATTN_CHUNK_WAVES",
     "ATTN_PARTS",
     "ATTN_PART_WAVES",
     "dv2_attn_state_floats",
@@ -787,7 +788,13 @@ def dv2_rope_kv_cols(q, k, v, q_out, k_cache, v_cache, cos, sin, start) -> None:
     _check_rc("chr_dv2_rope_kv_cols", rc)
 
 
-def dv2_attn_chunk(q, k, v, out, first_len, scale: float, n_waves: int = ATTN_WG_WAVES,
+#: wavefronts per (head, token) workgroup of the chunk attention: a chunk launches n_q * N
+#: workgroups, so small ones fill the card better than the decode step's 16 (measured at 40
+#: heads x 64 tokens: 30 vs 56 us at 256 cached rows, 172 vs 215 us at 2048)
+ATTN_CHUNK_WAVES = 4
+
+
+def dv2_attn_chunk(q, k, v, out, first_len, scale: float, n_waves: int = ATTN_CHUNK_WAVES,
                    feature_major: bool = True) -> None:
     """Causal attention of a chunk: token ``t`` of ``q [N, n_q*hd]`` sees cache rows
     ``0 .. first_len + t - 1``.  ``out`` is ``[n_q*hd, N]`` when ``feature_major`` else
