@@ -351,6 +351,162 @@ __global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flas
   }
 }
 
+// Chunk attention that shares the cache between the query heads of a KV head: one workgroup
+// per (KV head, token), REP = n_q / n_kv query heads each.  A cache row is loaded once and
+// dotted with all REP queries, so L2 traffic (what bounds a chunk: n_q * N workgroups re-read
+// the prefix) drops by REP.  Rows, update order, lane-group fold and LDS merge are those of
+// attn_flash<LPT, true> for each head, so a head's output is bit for bit the same.
+constexpr int kMaxGqaWaves = 8;
+
+template <int LPT, int REP>
+__global__ __launch_bounds__(kWave * kMaxGqaWaves) void attn_chunk_gqa(const AttnArgs a) {
+  constexpr int TPW = kWave / LPT;
+  constexpr int UNR = 4;
+  constexpr int HD = 8 * LPT;
+  const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
+  const int wg_waves = static_cast<int>(blockDim.x >> 6);
+  const int kv_head = static_cast<int>(blockIdx.x);
+  const int tok = static_cast<int>(blockIdx.y);
+  const int lane = threadIdx.x & (kWave - 1);
+  const int li = lane % LPT;
+  const int grp = lane / LPT;
+  const int d0 = li * 8;
+  const int vl = min(*a.valid_len + tok, a.max_seq);
+  const int stride = wg_waves * TPW;
+  const size_t row_stride = static_cast<size_t>(a.n_kv) * HD;
+
+  uint32_t kraw[UNR][4], vraw[UNR][4];
+  auto load_block = [&](int t0) {
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      const int t = t0 + grp * wg_waves + u * stride;
+      uint4 kv = make_uint4(0, 0, 0, 0), vv = make_uint4(0, 0, 0, 0);
+      if (t < vl) {
+        const size_t off =
+            static_cast<size_t>(t) * row_stride + static_cast<size_t>(kv_head) * HD + d0;
+        kv = *reinterpret_cast<const uint4 *>(a.k_cache + off);
+        vv = *reinterpret_cast<const uint4 *>(a.v_cache + off);
+      }
+      kraw[u][0] = kv.x;
+      kraw[u][1] = kv.y;
+      kraw[u][2] = kv.z;
+      kraw[u][3] = kv.w;
+      vraw[u][0] = vv.x;
+      vraw[u][1] = vv.y;
+      vraw[u][2] = vv.z;
+      vraw[u][3] = vv.w;
+    }
+  };
+  load_block(wave);
+
+  float qf[REP][8];
+  const uint16_t *qh = a.q + static_cast<size_t>(tok) * a.q_tok_stride +
+                       static_cast<size_t>(kv_head) * REP * HD + d0;
+#pragma unroll
+  for (int r = 0; r < REP; ++r) {
+    widen8(*reinterpret_cast<const uint4 *>(qh + r * HD), qf[r]);
+  }
+  float m[REP], l[REP], acc[REP][8];
+#pragma unroll
+  for (int r = 0; r < REP; ++r) {
+    m[r] = kNegBig;
+    l[r] = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      acc[r][i] = 0.f;
+    }
+  }
+  for (int t0 = wave; t0 < vl; t0 += UNR * stride) {
+    if (t0 != wave) {
+      load_block(t0);
+    }
+#pragma unroll
+    for (int u = 0; u < UNR; ++u) {
+      const bool live = t0 + grp * wg_waves + u * stride < vl;
+      float kf[8], vf[8];
+      widen8(make_uint4(kraw[u][0], kraw[u][1], kraw[u][2], kraw[u][3]), kf);
+      widen8(make_uint4(vraw[u][0], vraw[u][1], vraw[u][2], vraw[u][3]), vf);
+#pragma unroll
+      for (int r = 0; r < REP; ++r) {
+        float dot = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          dot = fmaf(qf[r][i], kf[i], dot);
+        }
+        dot = group_sum<LPT>(dot) * a.scale;
+        if (live) {
+          const float m2 = fmaxf(m[r], dot);
+          const float alpha = __expf(m[r] - m2);
+          const float e = __expf(dot - m2);
+          l[r] = l[r] * alpha + e;
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            acc[r][i] = acc[r][i] * alpha + e * vf[i];
+          }
+          m[r] = m2;
+        }
+      }
+    }
+  }
+
+  __shared__ float sm[REP][kMaxGqaWaves], sl[REP][kMaxGqaWaves];
+  __shared__ __align__(16) float so[REP][kMaxGqaWaves * HD];
+#pragma unroll
+  for (int r = 0; r < REP; ++r) {
+    if constexpr (TPW > 1) {  // fold the lane groups (different time steps, same dims)
+      float mg = m[r];
+#pragma unroll
+      for (int off = LPT; off < kWave; off <<= 1) {
+        mg = fmaxf(mg, __shfl_xor(mg, off, kWave));
+      }
+      const float w = __expf(m[r] - mg);
+      l[r] *= w;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        acc[r][i] *= w;
+      }
+#pragma unroll
+      for (int off = LPT; off < kWave; off <<= 1) {
+        l[r] += __shfl_xor(l[r], off, kWave);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          acc[r][i] += __shfl_xor(acc[r][i], off, kWave);
+        }
+      }
+      m[r] = mg;
+    }
+    if (lane == 0) {
+      sm[r][wave] = m[r];
+      sl[r][wave] = l[r];
+    }
+    if (grp == 0) {
+      float *oh = so[r] + wave * HD + d0;
+      *reinterpret_cast<float4 *>(oh) = make_float4(acc[r][0], acc[r][1], acc[r][2], acc[r][3]);
+      *reinterpret_cast<float4 *>(oh + 4) = make_float4(acc[r][4], acc[r][5], acc[r][6], acc[r][7]);
+    }
+  }
+  __syncthreads();
+  for (int r = wave; r < REP; r += wg_waves) {
+    uint16_t *dst = a.out + static_cast<size_t>(tok) * a.out_tok_stride +
+                    static_cast<size_t>(kv_head * REP + r) * HD * a.out_dim_stride;
+    merge_head(sm[r], sl[r], so[r], dst, 0, HD, wg_waves, lane, nullptr, a.out_dim_stride);
+  }
+}
+
+template <int LPT>
+bool launch_chunk_gqa(const AttnArgs &a, int n_rep, int n_waves, int n_tok, hipStream_t st) {
+  const dim3 grid(static_cast<unsigned>(a.n_kv), static_cast<unsigned>(n_tok));
+  const dim3 block(static_cast<unsigned>(kWave * n_waves));
+  switch (n_rep) {
+    case 2: attn_chunk_gqa<LPT, 2><<<grid, block, 0, st>>>(a); return true;
+    case 4: attn_chunk_gqa<LPT, 4><<<grid, block, 0, st>>>(a); return true;
+    case 5: attn_chunk_gqa<LPT, 5><<<grid, block, 0, st>>>(a); return true;
+    case 6: attn_chunk_gqa<LPT, 6><<<grid, block, 0, st>>>(a); return true;
+    case 8: attn_chunk_gqa<LPT, 8><<<grid, block, 0, st>>>(a); return true;
+    default: return false;
+  }
+}
+
 // Any hd <= 256: lane l owns dims l, l+64, l+128, l+192; one time step per
 // iteration.  Slow path for head sizes that are not 8 * 2^n.
 template <bool INWG>
@@ -660,7 +816,20 @@ int attn_common(const void *q, const void *k, const void *v, void *out, const vo
                       (v_act == nullptr || aligned16(v_act)) &&
                       (cos == nullptr || aligned16(cos)) && (sin == nullptr || aligned16(sin)) &&
                       (mode != 0 || aligned16(a.o_s));
-  if (mode != 0) {
+  // a chunk (several tokens) of a grouped-query model: share each cache row between the
+  // query heads of its KV head when a kernel for the head size and group size exists
+  bool shared = false;
+  if (mode == 1 && n_tok > 1 && !rope && vec_ok && n_split <= kMaxGqaWaves) {
+    const int n_rep = n_q / n_kv;
+    if (hd == 128) {
+      shared = launch_chunk_gqa<16>(a, n_rep, n_split, n_tok, st);
+    } else if (hd == 64) {
+      shared = launch_chunk_gqa<8>(a, n_rep, n_split, n_tok, st);
+    }
+  }
+  if (shared) {
+    // launched above
+  } else if (mode != 0) {
     launch_flash<true>(a, vec_ok, st, n_tok);
   } else {
     launch_flash<false>(a, vec_ok, st);

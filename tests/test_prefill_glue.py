@@ -107,7 +107,10 @@ def test_rope_kv_cols_skips_rows_past_the_cache():
 
 @pytest.mark.parametrize("n_q,n_kv,hd,max_seq,first,n,waves", [
     (4, 2, 16, 64, 1, 8, 16), (16, 2, 128, 256, 100, 32, 16), (40, 8, 128, 600, 481, 32, 16),
-    (6, 3, 256, 80, 40, 5, 4), (4, 2, 48, 64, 1, 32, 1), (8, 8, 64, 40, 9, 32, 16)])
+    (6, 3, 256, 80, 40, 5, 4), (4, 2, 48, 64, 1, 32, 1), (8, 8, 64, 40, 9, 32, 16),
+    # grouped-query models with at most 8 wavefronts: cache rows shared by the heads of a KV head
+    (40, 8, 128, 600, 481, 32, 4), (16, 2, 128, 256, 100, 64, 8), (4, 2, 64, 96, 30, 17, 4),
+    (12, 2, 64, 128, 1, 64, 2), (8, 2, 128, 200, 130, 9, 1), (10, 2, 128, 64, 3, 5, 3)])
 def test_attn_chunk(n_q, n_kv, hd, max_seq, first, n, waves):
     say("attn_chunk", n_q, n_kv, hd, max_seq, first, n, waves)
     q = rnd((n, n_q * hd), 11)
