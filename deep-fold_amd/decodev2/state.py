@@ -72,4 +72,4 @@ class DecodeState:
         """``next_token = argmax(logits)``; with ``commit`` feed it back without a
         host round trip: ``token = next``, ``position += 1``, ``finished |= eos``."""
         dv2_argmax_commit(self.arena.logits.view(-1), self.next_token, self.token, self.position,
-                          self.finished, self.eos_id, commit=commit)
+                          self.finished, self.eos_id, commit=commit, ws=self.arena.argmax_ws)

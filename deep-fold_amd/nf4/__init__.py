@@ -39,6 +39,7 @@ __all__ = [
     "nf4_quantize",
     "dv2_mark_written",
     "dv2_argmax_commit",
+    "dv2_argmax_ws_bytes",
     "dv2_begin_step",
     "ATTN_WG_WAVES",
     "ATTN_CHUNK_WAVES",
@@ -138,6 +139,8 @@ EXPORTS = (
     ("chr_dv2_gemm_swiglu", ctypes.c_int, [_DP, _DP, _P, _P, _I, _P, ctypes.c_int64, _P]),
     ("chr_dv2_mark_written", ctypes.c_int, [_P, _P, _P]),
     ("chr_dv2_argmax_commit", ctypes.c_int, [_P, _I, _P, _P, _P, _P, _P, _I, _P]),
+    ("chr_dv2_argmax_ws_bytes", ctypes.c_int64, []),
+    ("chr_dv2_argmax_commit_ws", ctypes.c_int, [_P, _I, _P, _P, _P, _P, _P, _I, _P, ctypes.c_int64, _P]),
     ("chr_nf4_abi_version", ctypes.c_int, []),
 )
 
@@ -604,10 +607,13 @@ def dv2_mark_written(position: torch.Tensor, valid_len: torch.Tensor) -> None:
 
 def dv2_argmax_commit(logits: torch.Tensor, next_token: torch.Tensor, token: torch.Tensor | None = None,
                       position: torch.Tensor | None = None, finished: torch.Tensor | None = None,
-                      eos_id: torch.Tensor | None = None, commit: bool = False) -> None:
+                      eos_id: torch.Tensor | None = None, commit: bool = False,
+                      ws: torch.Tensor | None = None) -> None:
     """``next_token = argmax(logits)`` (first maximum wins); with ``commit`` also
     ``token = next``, ``position += 1``, ``finished |= next == eos``
-    (``gpu/decodev2/step.py:182``, ``gpu/decodev2/state.py:98-103``)."""
+    (``gpu/decodev2/step.py:182``, ``gpu/decodev2/state.py:98-103``).  With ``ws``
+    (``dv2_argmax_ws_bytes()`` bytes on the GPU) a large vocabulary is searched by 128
+    workgroups and a small second launch instead of one workgroup."""
     _need(logits.is_cuda and logits.dtype == torch.bfloat16 and logits.is_contiguous(),
           "logits must be contiguous CUDA bf16")
     _need(next_token.is_cuda and next_token.dtype == torch.int64 and next_token.numel() == 1,
@@ -622,10 +628,21 @@ def dv2_argmax_commit(logits: torch.Tensor, next_token: torch.Tensor, token: tor
         _need(eos_id is not None and eos_id.is_cuda and eos_id.dtype == torch.int64,
               "eos_id must be CUDA int64")
         ptrs = [token.data_ptr(), position.data_ptr(), finished.data_ptr(), eos_id.data_ptr()]
+    if ws is not None:
+        _need(ws.is_cuda and ws.is_contiguous(), "ws must be a contiguous CUDA tensor")
+        rc = _load_ext().chr_dv2_argmax_commit_ws(
+            logits.data_ptr(), int(logits.numel()), next_token.data_ptr(), ptrs[0], ptrs[1], ptrs[2],
+            ptrs[3], 1 if commit else 0, ws.data_ptr(), int(ws.numel() * ws.element_size()), _stream())
+        _check_rc("chr_dv2_argmax_commit_ws", rc)
+        return
     rc = _load_ext().chr_dv2_argmax_commit(logits.data_ptr(), int(logits.numel()), next_token.data_ptr(),
                                            ptrs[0], ptrs[1], ptrs[2], ptrs[3], 1 if commit else 0,
                                            _stream())
     _check_rc("chr_dv2_argmax_commit", rc)
+
+
+def dv2_argmax_ws_bytes() -> int:
+    return int(_load_ext().chr_dv2_argmax_ws_bytes())
 
 
 def dv2_begin_step(packed: torch.Tensor, scale: torch.Tensor, K: int, token: torch.Tensor,  # noqa: N803

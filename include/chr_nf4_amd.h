@@ -280,6 +280,16 @@ int64_t chr_dv2_gemm_swiglu_ws(const chr_nf4_dev_t *gate, const chr_nf4_dev_t *u
 int chr_dv2_gemm_swiglu(const chr_nf4_dev_t *gate, const chr_nf4_dev_t *up, const void *x,
                         void *y, int32_t N, float *ws, int64_t ws_floats, void *stream);
 
+/* chr_dv2_argmax_commit as two launches for a large vocabulary: 128 workgroups leave the best
+ * (value, index) of a slice each in ws, a small launch picks among them and commits; same
+ * tie and NaN rules.  ws: chr_dv2_argmax_ws_bytes() bytes of device memory, 8-byte aligned;
+ * with ws NULL or too small, or n < 16384, this is chr_dv2_argmax_commit.
+ * No reference counterpart. */
+int64_t chr_dv2_argmax_ws_bytes(void);
+int chr_dv2_argmax_commit_ws(const void *logits, int32_t n, void *next_token, void *token,
+                             void *position, void *finished, const void *eos_id, int32_t commit,
+                             void *ws, int64_t ws_bytes, void *stream);
+
 /* Library version, for the loader's sanity check. */
 int chr_nf4_abi_version(void);
 

@@ -660,3 +660,43 @@ def test_gemv_attn_rejects_bad_arguments():
         nf4.dv2_gemv_attn(dp, ds, state[:10], 2, 64, 64, 128, 128, y, None, 4)  # state too small
     nf4.dv2_gemv_attn(dp, ds, state, 2, 64, 64, 128, 128, y, None, 4)           # zero states -> zeros
     assert float(y.float().abs().max()) == 0.0
+
+
+# ---- argmax + commit ----------------------------------------------------------------------
+
+@pytest.mark.parametrize("n", [5, 1000, 16384, 50001, 152064])
+@pytest.mark.parametrize("two_launch", [False, True])
+def test_argmax_commit(n, two_launch):
+    say("argmax", n, two_launch)
+    rng = np.random.default_rng(n)
+    ws = torch.zeros(nf4.dv2_argmax_ws_bytes() // 8, dtype=torch.int64, device=DEV) if two_launch else None
+
+    def run(logits, commit=False, eos=7):
+        nt = torch.full((), -1, dtype=torch.int64, device=DEV)
+        tok = torch.full((), -1, dtype=torch.int64, device=DEV)
+        pos = torch.full((), 10, dtype=torch.int64, device=DEV)
+        fin = torch.zeros((), dtype=torch.uint8, device=DEV)
+        nf4.dv2_argmax_commit(logits, nt, tok, pos, fin, torch.tensor(eos, dtype=torch.int64, device=DEV),
+                              commit=commit, ws=ws)
+        return int(nt.item()), int(tok.item()), int(pos.item()), int(fin.item())
+
+    vals = oc.bf16_round(rng.standard_normal(n).astype(np.float32))
+    assert run(bf16_tensor(vals))[0] == int(np.argmax(vals))        # numpy: first maximum
+    # ties: the lowest index wins, wherever the equal values sit
+    for where in ([0, n - 1], [n // 2, n // 2 + 1], [n - 1]):
+        t = vals.copy()
+        t[where] = 9.0
+        assert run(bf16_tensor(t))[0] == min(where)
+    flat = np.zeros(n, dtype=np.float32)
+    assert run(bf16_tensor(flat))[0] == 0
+    t = vals.copy()
+    t[n // 3] = np.nan                                               # a NaN logit is surfaced
+    t[n - 1] = np.inf
+    assert run(bf16_tensor(t))[0] == n // 3
+    # commit feeds the pick back and flags eos
+    t = vals.copy()
+    t[min(7, n - 1)] = 50.0
+    pick = min(7, n - 1)
+    assert run(bf16_tensor(t), commit=True, eos=pick) == (pick, pick, 11, 1)
+    assert run(bf16_tensor(t), commit=True, eos=pick + 1) == (pick, pick, 11, 0)
+    assert run(bf16_tensor(t), commit=False) == (pick, -1, 10, 0)
