@@ -4,6 +4,7 @@
 from __future__ import annotations
 
 import json
+import os
 import struct
 
 import numpy as np
@@ -13,14 +14,9 @@ import torch
 from deepfold_amd import chr0
 
 # docs/spec/chr0.md section 2.4: the header of the three-tensor toy model, byte for byte
-GOLDEN_JSON = (
-    '{"magic":"CHR0","version":1,"arch":"toy","hidden_size":64,"intermediate_size":128,'
-    '"num_layers":1,"vocab_size":0,"tile":{"row":64,"col_group":8},"tensors":{'
-    '"model.layers.0.mlp.down_proj":{"layer":0,"kind":"down","codec":"nf4","shape":[32,128],'
-    '"group_size":64,"data":[2752,4800],"scale":[4800,4928]},'
-    '"model.layers.0.self_attn.q_proj":{"layer":0,"kind":"q","codec":"nf4","shape":[64,64],'
-    '"group_size":64,"data":[576,2624],"scale":[2624,2752]},'
-    '"model.norm":{"kind":"norm","codec":"bf16","shape":[64],"data":[4928,5056]}}}')
+# (tests/golden/chr0_toy_header.json, no trailing newline)
+GOLDEN_JSON = open(os.path.join(os.path.dirname(__file__), "golden", "chr0_toy_header.json"),
+                   encoding="utf-8").read()
 
 
 def toy_entries(seed=0):

@@ -9,32 +9,24 @@ grid).  Both restatements (C and numpy) must pass each check.
 
 from __future__ import annotations
 
+import json
+import os
+
 import numpy as np
 import pytest
 
 from oracle import nf4_oracle as oc
 
-GOLDEN64_HEX = "778788889999A9AAAABABBBBCBCCCCCCDDDDDDDDEDEEEEEEEEEEEEFEFFFFFFFF"
-GOLDEN2X64_ROW1_HEX = "00001011111121222233434454556676878899AABABBCCCCDDDDEEEEEEFEFFFF"
-PAD01_HEX = "F7" + "77" * 31
-GOLDEN64_IDX = [
-    7, 7, 7, 8, 8, 8, 8, 8, 9, 9, 9, 9, 9, 10, 10, 10,
-    10, 10, 10, 11, 11, 11, 11, 11, 11, 12, 12, 12, 12, 12, 12, 12,
-    13, 13, 13, 13, 13, 13, 13, 13, 13, 14, 14, 14, 14, 14, 14, 14,
-    14, 14, 14, 14, 14, 14, 14, 15, 15, 15, 15, 15, 15, 15, 15, 15,
-]
-LEVEL_LITERALS = [
-    -1.0, -0.6961928009986877, -0.5250730514526367, -0.39491748809814453,
-    -0.28444138169288635, -0.18477343022823334, -0.09105003625154495, 0.0,
-    0.07958029955625534, 0.16093020141124725, 0.24611230194568634, 0.33791524171829224,
-    0.44070982933044434, 0.5626170039176941, 0.7229568362236023, 1.0,
-]
-# docs/spec/nf4.md section 2.3: float32 midpoints of neighbouring levels.
-MIDPOINT_BITS = [
-    0xBF591CD8, 0xBF1C5270, 0xBEEB8480, 0xBEADEA76, 0xBE703CEC, 0xBE0D38BC, 0xBD3A7871,
-    0x3D22FAFF, 0x3DF64862, 0x3E5067E0, 0x3E9582D4, 0x3EC753F9, 0x3F006D04, 0x3F248DAF,
-    0x3F5C89DA,
-]
+# tests/golden/nf4_golden.json holds the vectors, each with the reference line it comes from
+_G = {k: v["value"] for k, v in json.load(open(os.path.join(os.path.dirname(__file__), "golden",
+                                                             "nf4_golden.json"))).items()
+      if isinstance(v, dict)}
+GOLDEN64_HEX = _G["golden64_hex"]
+GOLDEN2X64_ROW1_HEX = _G["golden2x64_row1_hex"]
+PAD01_HEX = _G["pad01_hex"]
+GOLDEN64_IDX = _G["golden64_idx"]
+LEVEL_LITERALS = _G["level_literals"]
+MIDPOINT_BITS = [int(b, 16) for b in _G["midpoint_bits"]]
 
 ENCODERS = [pytest.param(oc.c_encode, id="c"), pytest.param(oc.np_encode, id="numpy")]
 DECODERS = [pytest.param(oc.c_decode, id="c"), pytest.param(oc.np_decode, id="numpy")]
