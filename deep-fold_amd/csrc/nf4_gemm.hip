@@ -220,23 +220,51 @@ struct XRegs {
   uint32_t d[16 * NB];  // up to 4 NB 16-byte vectors (N = 32 NB), as plain dwords
 };
 
+// Vector staging of the activation tile (N in {8, 16, 32, 64}).  An item is a pair of rows
+// (k, k+1) and one 8-column vector q: two 16-byte loads, which are interleaved into eight
+// dwords {x[k][n], x[k+1][n]} and stored at xs[n][k/2], one 32-bit store each.  Items are dealt
+// to lanes so that the 64 stores of a wavefront instruction fall into 64 different LDS banks
+// (a column row is 132 dwords = 4 mod 64: bank = 4n + k/2 mod 64).
+//   N >= 16: lane -> k pair 32a + (lane & 31), vector 2b + (lane >> 5), a = I % 4, b = I / 4
+//   N == 8 : lane -> k pair 64I + lane, vector 0
+// with I = wavefront + 4 rep numbering the wavefront instructions of the tile.
+__device__ __forceinline__ bool x_item(int N, int I, int lane, int &kp, int &q) {
+  if (N == 8) {
+    kp = 64 * I + lane;
+    q = 0;
+    return I < 2;
+  }
+  kp = 32 * (I & 3) + (lane & 31);
+  q = 2 * (I >> 2) + (lane >> 5);
+  return I < N / 4;  // 128 k pairs x N/8 vectors = 16 N items = N/4 instructions
+}
+
 template <bool VEC, int NB>
 __device__ __forceinline__ void fetch_x(XRegs<NB> &r, const uint16_t *__restrict__ x, int k0, int K,
                                         int N, int tid) {
-  const int n_elem = min(kBK, K - k0) * N;  // valid elements of the tile (rows >= K are zero)
-  const uint16_t *base = x + static_cast<size_t>(k0) * N;
   if constexpr (VEC) {
+    const int wave = tid >> 6, lane = tid & 63;
 #pragma unroll
-    for (int j = 0; j < 4 * NB; ++j) {
-      const int v = tid + j * kGroupThreads;
-      uint4 t = make_uint4(0, 0, 0, 0);
-      if (v * 8 < n_elem) {  // N % 8 == 0 here, so a vector never straddles the end
-        t = *reinterpret_cast<const uint4 *>(base + v * 8);
+    for (int rep = 0; rep < 2 * NB; ++rep) {
+      int kp, q;
+      uint4 a = make_uint4(0, 0, 0, 0), b = make_uint4(0, 0, 0, 0);
+      if (x_item(N, wave + 4 * rep, lane, kp, q)) {
+        const int k = k0 + 2 * kp;  // rows >= K are zero
+        if (k < K) {
+          a = *reinterpret_cast<const uint4 *>(x + static_cast<size_t>(k) * N + 8 * q);
+        }
+        if (k + 1 < K) {
+          b = *reinterpret_cast<const uint4 *>(x + static_cast<size_t>(k + 1) * N + 8 * q);
+        }
       }
-      r.d[4 * j + 0] = t.x;
-      r.d[4 * j + 1] = t.y;
-      r.d[4 * j + 2] = t.z;
-      r.d[4 * j + 3] = t.w;
+      r.d[8 * rep + 0] = a.x;
+      r.d[8 * rep + 1] = a.y;
+      r.d[8 * rep + 2] = a.z;
+      r.d[8 * rep + 3] = a.w;
+      r.d[8 * rep + 4] = b.x;
+      r.d[8 * rep + 5] = b.y;
+      r.d[8 * rep + 6] = b.z;
+      r.d[8 * rep + 7] = b.w;
     }
   } else {
     (void)r;
@@ -247,19 +275,18 @@ template <bool VEC, int NB>
 __device__ __forceinline__ void scatter_x(const XRegs<NB> &r, const uint16_t *__restrict__ x,
                                           uint16_t *xs, int k0, int K, int N, int tid) {
   if constexpr (VEC) {
-    const int shift = N == 64 ? 6 : (N == 32 ? 5 : (N == 16 ? 4 : 3));  // VEC: N in {8, 16, 32, 64}
+    const int wave = tid >> 6, lane = tid & 63;
+    uint32_t *xd = reinterpret_cast<uint32_t *>(xs);
 #pragma unroll
-    for (int j = 0; j < 4 * NB; ++j) {
-      const int v = tid + j * kGroupThreads;
-      if (v * 8 < kBK * N) {
-        const int f = v * 8;
-        const int kk = f >> shift;
-        const int n0 = f & (N - 1);
+    for (int rep = 0; rep < 2 * NB; ++rep) {
+      int kp, q;
+      if (x_item(N, wave + 4 * rep, lane, kp, q)) {
+        uint32_t *dst = xd + (8 * q) * (kXStride / 2) + kp;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          const uint32_t w = r.d[4 * j + e];
-          xs[(n0 + 2 * e) * kXStride + kk] = static_cast<uint16_t>(w & 0xFFFFu);
-          xs[(n0 + 2 * e + 1) * kXStride + kk] = static_cast<uint16_t>(w >> 16);
+          const uint32_t a = r.d[8 * rep + e], b = r.d[8 * rep + 4 + e];
+          dst[(2 * e) * (kXStride / 2)] = (a & 0xFFFFu) | (b << 16);
+          dst[(2 * e + 1) * (kXStride / 2)] = (a >> 16) | (b & 0xFFFF0000u);
         }
       }
     }
