@@ -115,21 +115,25 @@ int resolved_one_wave() {
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
 // Split-K.  A workgroup is quickest with about three K tiles (measured at every 14B linear
-// shape, N = 8 and 32: fewer tiles leave the fetch latency uncovered, more leave compute units
-// idle), so split = ceil(n_ktiles / 3), as long as the grid stays within the four workgroups
-// a compute unit holds at once; split is recomputed from tiles_per_split so the pair always
-// agrees with what the kernel indexes (gpu/nf4/nf4_gemm.cu:1526-1543).
+// shape: fewer tiles leave the fetch latency uncovered, more leave compute units idle), so
+// split = ceil(n_ktiles / 3) -- but no more splits than it takes to reach a target number of
+// workgroups, because every split writes and re-reads M*N fp32 partials: three workgroups per
+// compute unit for chunks of up to 32 columns, 1.6 for wider ones (whose partials are twice
+// as large; a 27648-row gate+up stack at N=64 takes 65 us with 2 splits, 74 with 4, 87 with
+// 10).  split is recomputed from tiles_per_split so the pair always agrees with what the
+// kernel indexes (gpu/nf4/nf4_gemm.cu:1526-1543).
 constexpr int kTilesPerSplit = 3;
-constexpr int kResidentPerCu = 4;
 constexpr int kMaxAutoSplit = 32;
 
-void pick_split(int grid_x, int n_ktiles, int have_ws, int *split, int *tiles_per_split) {
+void pick_split(int grid_x, int n_ktiles, int N, int have_ws, int *split, int *tiles_per_split) {
   const Tuning &t = tuning();
   int want = 1;
   if (have_ws) {
-    const int room = (resolved_one_wave() * kResidentPerCu) / grid_x;
+    const int cus = resolved_one_wave();
+    const int target = N > kBN ? cus * 8 / 5 : cus * 3;
+    const int by_grid = std::max(1, ceil_div(target, grid_x));
     const int by_tiles = ceil_div(n_ktiles, kTilesPerSplit);
-    want = t.split_k > 0 ? t.split_k : std::min(kMaxAutoSplit, std::min(by_tiles, room));
+    want = t.split_k > 0 ? t.split_k : std::min(kMaxAutoSplit, std::min(by_tiles, by_grid));
   }
   want = std::max(1, std::min(want, n_ktiles));
   const int tps = ceil_div(n_ktiles, want);
@@ -158,7 +162,7 @@ int plan_impl(const chr_nf4_dev_t &h, int32_t N, int32_t have_ws, chr_nf4_plan_t
     p.block = kGemmBlock;
     p.grid_x = ceil_div(h.M, kBM);
     p.n_ktiles = ceil_div(h.K_pad, kBK);
-    pick_split(p.grid_x, p.n_ktiles, have_ws, &p.grid_y, &p.tiles_per_split);
+    pick_split(p.grid_x, p.n_ktiles, N, have_ws, &p.grid_y, &p.tiles_per_split);
     p.smem_bytes = gemm_lds_bytes(N <= 32 ? 1 : 2);
     if (p.grid_y > 1) {
       p.ws_floats = static_cast<int64_t>(p.grid_y) * h.M * N;
@@ -611,7 +615,7 @@ StackPlan plan_stack(const chr_nf4_dev_t *h, int nseg, int N, int have_ws) {
     sp.grid_x += sp.segs.blocks[i];
   }
   sp.n_ktiles = ceil_div(h[0].K_pad, kBK);
-  pick_split(sp.grid_x, sp.n_ktiles, have_ws, &sp.grid_y, &sp.tiles_per_split);
+  pick_split(sp.grid_x, sp.n_ktiles, N, have_ws, &sp.grid_y, &sp.tiles_per_split);
   sp.ws_floats = sp.grid_y > 1 ? static_cast<int64_t>(sp.grid_y) * sp.M_all * N : 0;
   return sp;
 }

@@ -11,8 +11,8 @@ are ``M``, in features ``K``):
 
 * ``N == 1``  row-streaming GEMV, no split-K (path ``GEMV``).
 * ``N = 2..16`` / ``17..32``  MFMA tile, 128 rows x 32 columns per workgroup,
-  split-K over ``grid_y`` at about three K tiles per workgroup while the grid fits
-  the four workgroups a compute unit holds (paths ``PREFILL`` / ``PREFILL_N32``).
+  split-K over ``grid_y`` at about three K tiles per workgroup, up to three workgroups
+  per compute unit (paths ``PREFILL`` / ``PREFILL_N32``).
 * ``N = 33..64``  the same tile with two 32-column blocks per weight fragment
   (``PREFILL_N64``); launched only through ``chr_nf4_gemm_ws_max`` with ``max_n`` > 32,
   the plain entries keep the reference's ceiling of 32.
@@ -58,7 +58,6 @@ _BK = 256
 _BLOCK = 256
 _MAX_AUTO_SPLIT = 32
 _TILES_PER_SPLIT = 3
-_RESIDENT_PER_CU = 4
 
 
 def _gemm_lds(col_blocks: int) -> int:
@@ -114,13 +113,15 @@ class Plan:
         return self.path != PREFILL_N64
 
 
-def _pick_split(grid_x: int, n_ktiles: int, have_ws: bool, force_split: int,
+def _pick_split(grid_x: int, n_ktiles: int, N: int, have_ws: bool, force_split: int,  # noqa: N803
                 one_wave: int) -> tuple[int, int]:
     want = 1
     if have_ws:
-        room = (int(one_wave) * _RESIDENT_PER_CU) // grid_x
+        # workgroups worth splitting for: 3 per compute unit, 1.6 for chunks wider than 32
+        target = int(one_wave) * 8 // 5 if N > 32 else int(one_wave) * 3
+        by_grid = max(1, _ceil_div(target, grid_x))
         by_tiles = _ceil_div(n_ktiles, _TILES_PER_SPLIT)
-        want = force_split if force_split > 0 else min(_MAX_AUTO_SPLIT, by_tiles, room)
+        want = force_split if force_split > 0 else min(_MAX_AUTO_SPLIT, by_tiles, by_grid)
     want = max(1, min(want, n_ktiles))
     tiles_per_split = _ceil_div(n_ktiles, want)
     return _ceil_div(n_ktiles, tiles_per_split), tiles_per_split
@@ -145,7 +146,7 @@ def plan(M: int, K: int, N: int = 1, *, K_pad: int | None = None, have_ws: bool 
     path = PREFILL if N <= 16 else (PREFILL_N32 if N <= 32 else PREFILL_N64)
     grid_x = _ceil_div(M, _BM)
     n_ktiles = _ceil_div(kp, _BK)
-    split, tps = _pick_split(grid_x, n_ktiles, have_ws, force_split, one_wave)
+    split, tps = _pick_split(grid_x, n_ktiles, N, have_ws, force_split, one_wave)
     ws = split * M * N if split > 1 else 0
     smem = _gemm_lds(1 if N <= 32 else 2)
     return Plan(path, grid_x, split, _BLOCK, _BM, _BK, n_ktiles, tps, grid_x * split, smem, ws)

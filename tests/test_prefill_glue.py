@@ -223,8 +223,14 @@ def test_wide_chunk_equals_two_narrow_ones(m, k, n):
     first = min(32, n - 2)  # at least two columns: one alone would go to the GEMV
     hi = nf4.nf4_gemm(dp, ds, x[:, first:].contiguous(), m, k, kp)
     assert tuple(wide.shape) == (m, n)
-    assert (bf16_bits(wide[:, :32].contiguous()) == bf16_bits(lo)).all()
-    assert (bf16_bits(wide[:, first:].contiguous()) == bf16_bits(hi.view(m, n - first))).all()
+    same_split = (nf4.nf4_plan(m, k, n)["grid_y"] == nf4.nf4_plan(m, k, 32)["grid_y"]
+                  == nf4.nf4_plan(m, k, n - first)["grid_y"])
+    for got, want_ in ((wide[:, :32].contiguous(), lo), (wide[:, first:].contiguous(), hi.view(m, n - first))):
+        if same_split:  # same K order, same partial sums: the same bits
+            assert (bf16_bits(got) == bf16_bits(want_)).all()
+        else:           # wider chunks split K less: equal up to the fp32 summation order
+            d = (got.float() - want_.float()).abs().max().item()
+            assert d <= 2 ** -7 * max(1.0, want_.float().abs().max().item())
     bias, res = bf16_tensor(rnd((m,), 2)), bf16_tensor(rnd((m, n), 3))
     want = res + (wide + bias[:, None])
     got = nf4.nf4_gemm(dp, ds, x, m, k, kp, max_n=64, bias=bias, residual=res)
@@ -275,10 +281,11 @@ def test_stacked_gate_up_with_swiglu_in_the_reduce(m, k, n):
     g = nf4.nf4_gemm(mats[0][0], mats[0][1], x, m, k, kp, max_n=64)
     u = nf4.nf4_gemm(mats[1][0], mats[1][1], x, m, k, kp, max_n=64)
     want = F.silu(g) * u
-    # the stack has its own split-K, so gate and up may differ from the single GEMMs in the
-    # last bf16 digit before the activation
+    # the stack has its own split-K, so gate and up may each differ from the single GEMMs in
+    # the last bf16 digit before the activation: 2^-7 (gate through silu) + 2^-8 (up) + two
+    # roundings of 2^-9 is just over 2^-6 of the product
     d = (got.float() - want.float()).abs()
-    tol = 2 ** -6 * torch.maximum(want.float().abs(), torch.full_like(d, 2 ** -10))
+    tol = 2 ** -5 * torch.maximum(want.float().abs(), torch.full_like(d, 2 ** -10))
     assert tuple(got.shape) == (m, n) and bool((d <= tol).all())
     with pytest.raises(RuntimeError):
         nf4.dv2_gemm_swiglu(mats[0], (mats[1][0], mats[1][1], m - 1), x)
