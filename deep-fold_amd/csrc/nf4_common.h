@@ -15,11 +15,13 @@ constexpr int kWave = 64;   // lanes per wavefront on gfx950
 
 // binary32 bit patterns of the QLoRA NF4 levels (internal/nf4/nf4.go:18-35,
 // bits as listed in internal/nf4/nf4_test.go:12-29).
-__device__ __constant__ const uint32_t kLutBits[16] = {
-    0xBF800000u, 0xBF3239B1u, 0xBF066B30u, 0xBECA32A0u, 0xBE91A24Du, 0xBE3D353Fu,
-    0xBDBA7871u, 0x00000000u, 0x3DA2FAFFu, 0x3E24CAE3u, 0x3E7C04DDu, 0x3EAD033Au,
-    0x3EE1A4B8u, 0x3F1007ABu, 0x3F3913B3u, 0x3F800000u,
-};
+#define CHR_NF4_LEVEL_BITS                                                                   \
+  0xBF800000u, 0xBF3239B1u, 0xBF066B30u, 0xBECA32A0u, 0xBE91A24Du, 0xBE3D353Fu, 0xBDBA7871u, \
+      0x00000000u, 0x3DA2FAFFu, 0x3E24CAE3u, 0x3E7C04DDu, 0x3EAD033Au, 0x3EE1A4B8u,          \
+      0x3F1007ABu, 0x3F3913B3u, 0x3F800000u
+__device__ __constant__ const uint32_t kLutBits[16] = {CHR_NF4_LEVEL_BITS};
+// the same sixteen words for code that wants them as compile-time constants
+constexpr uint32_t kLevelBits[16] = {CHR_NF4_LEVEL_BITS};
 
 __device__ __forceinline__ float bits_to_f32(uint32_t u) { return __uint_as_float(u); }
 __device__ __forceinline__ uint32_t f32_to_bits(float f) { return __float_as_uint(f); }

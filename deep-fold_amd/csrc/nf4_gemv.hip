@@ -33,6 +33,7 @@ namespace chr {
 namespace {
 
 constexpr int kMaxWaves = 16;  // wavefronts per workgroup, upper bound
+constexpr int kStagedThreads = 1024;  // workgroup of the kernel that stages x in LDS, fixed
 
 // Static LDS of the GEMV kernels.  The codebook comes first so that its LDS
 // address is 0 and a lookup address is just 4*code.
@@ -79,10 +80,10 @@ struct StreamArgs {
   float rms_eps;
 };
 
-// Sum of a value over the whole workgroup, the same in every thread.
+// Sum of a value over a workgroup of kStagedThreads threads, the same in every thread.
 __device__ __forceinline__ float block_sum(float v, float *part) {
   v = wave_sum(v);
-  const int waves = blockDim.x >> 6;
+  const int waves = kStagedThreads >> 6;
   if ((threadIdx.x & (kWave - 1)) == 0) {
     part[threadIdx.x >> 6] = v;
   }
@@ -96,27 +97,29 @@ __device__ __forceinline__ float block_sum(float v, float *part) {
 }
 
 // ---- activations staged in LDS ------------------------------------------------------
-// A "piece" is 8 consecutive activations (16 bytes of bf16).  In the steps where every
-// lane holds a 16-byte chunk of weights, lane l of step j needs pieces 4c..4c+3 of chunk
-// c = 64j + l; they are stored as [j][q][l] so that one ds_read_b128 of the wavefront
-// covers 64 consecutive pieces (no bank conflicts).  The 8-byte tail chunks need two
-// pieces each and are stored as [step][q][l] the same way after the full steps.
-__host__ __device__ inline int x_pieces(int K_pad) {
-  const int chunks = K_pad >> 5;
-  const int nfull = chunks >> 6;
-  const int tail_half = (chunks & 63) * 2;
-  return nfull * 256 + ((tail_half + 63) >> 6) * 128;
+// A "piece" is 8 consecutive activations (16 bytes of bf16).  The staged kernel walks a
+// row in steps of 64 lanes x 8 packed bytes: lane l of step t holds the 16 codes of half
+// chunk h = 64t + l and needs pieces 2h and 2h+1.  They are stored as [t][q][l], so one
+// ds_read_b128 of the wavefront covers 64 consecutive pieces (no bank conflicts).
+__host__ __device__ inline int x_half_steps(int K_pad) { return ((K_pad >> 4) + kWave - 1) >> 6; }
+
+__host__ __device__ inline int x_pieces(int K_pad) { return x_half_steps(K_pad) * 128; }
+
+__device__ __forceinline__ int x_slot(int piece) {
+  const int h = piece >> 1, q = piece & 1;
+  return ((h >> 6) << 7) + (q << 6) + (h & 63);
 }
 
-__device__ __forceinline__ int x_slot(int piece, int nfull) {
-  const int full = nfull << 8;
-  if (piece < full) {
-    const int c = piece >> 2, q = piece & 3;
-    return ((c >> 6) << 8) + (q << 6) + (c & 63);
+// Zero the slots of the last step that no piece of the row maps to.
+__device__ __forceinline__ void zero_unused_slots(uint4 *xs, int K_pad) {
+  const int n_half = K_pad >> 4;
+  const int last = (x_half_steps(K_pad) - 1) << 7;
+  for (int i = last + threadIdx.x; i < last + 128; i += kStagedThreads) {
+    const int h = ((last >> 7) << 6) + (i & 63);
+    if (h >= n_half) {
+      xs[i] = make_uint4(0, 0, 0, 0);
+    }
   }
-  const int t = piece - full;
-  const int h = t >> 1, q = t & 1;
-  return full + ((h >> 6) << 7) + (q << 6) + (h & 63);
 }
 
 // Fill the LDS copy: zero for k in [K, K_pad) and for unused slots.  With rms_w the
@@ -187,96 +190,101 @@ __device__ __forceinline__ uint4 merged_attn_piece(const StreamArgs &a, int i) {
   return make_uint4(r[0], r[1], r[2], r[3]);
 }
 
-__device__ __forceinline__ void stage_x(const StreamArgs &a, uint4 *xs, float *part) {
-  if (a.attn_state != nullptr) {
-    const int nfull_a = (a.K_pad >> 5) >> 6;
-    for (int i = threadIdx.x; i < (a.K_pad >> 3); i += blockDim.x) {
-      xs[x_slot(i, nfull_a)] = merged_attn_piece(a, i);
-    }
-    const int full = nfull_a << 8;
-    const int tail_half = ((a.K_pad >> 5) & 63) * 2;
-    for (int i = full + threadIdx.x; i < x_pieces(a.K_pad); i += blockDim.x) {
-      const int h = (((i - full) >> 7) << 6) + (i & 63);
-      if (h >= tail_half) {
-        xs[i] = make_uint4(0, 0, 0, 0);
+constexpr int kXKeep = 4;  // 16-byte vectors of x a thread keeps between request and use
+
+// The common case of staging: K a multiple of 8, aligned pointers, x short enough to sit in
+// registers between its request and its use, no attention merge.
+__device__ __forceinline__ bool stage_fast_ok(const StreamArgs &a) {
+  return a.attn_state == nullptr && (a.K & 7) == 0 && aligned16(a.x) &&
+         (a.rms_w == nullptr || aligned16(a.rms_w)) &&
+         (a.K_pad >> 3) <= kXKeep * kStagedThreads;
+}
+
+// Fast staging, first half: request x (and the norm weights with it: one memory round
+// trip, not two).  Every request is unconditional per lane (an index past the end reads
+// the last vector and is dropped at the use), so later code can wait for these loads by
+// count while younger loads are still in flight.
+__device__ __forceinline__ void x_request(const StreamArgs &a, uint4 (&v)[kXKeep],
+                                          uint4 (&g)[kXKeep]) {
+  const int nk = a.K >> 3;
+#pragma unroll
+  for (int j = 0; j < kXKeep; ++j) {
+    v[j] = make_uint4(0, 0, 0, 0);
+    g[j] = make_uint4(0, 0, 0, 0);
+    if (j * kStagedThreads < nk) {
+      const int i = min(static_cast<int>(threadIdx.x) + j * kStagedThreads, nk - 1);
+      v[j] = reinterpret_cast<const uint4 *>(a.x)[i];
+      if (a.rms_w != nullptr) {
+        g[j] = reinterpret_cast<const uint4 *>(a.rms_w)[i];
       }
+    }
+  }
+}
+
+// Fast staging, second half: normalise if asked, store the pieces, barrier.  With rms_w
+// the value stored is bf16( (w*x) * rsqrt(mean(x^2)+eps) ), i.e. what a separate RMSNorm
+// launch would have handed over (gpu/nf4/nf4_gemv.cu:264-289).
+__device__ __forceinline__ void x_store(const StreamArgs &a, uint4 *xs, float *part,
+                                        const uint4 (&v)[kXKeep], const uint4 (&g)[kXKeep]) {
+  const int nk = a.K >> 3;
+  const int nvec = a.K_pad >> 3;
+  zero_unused_slots(xs, a.K_pad);
+  float inv = 1.f;
+  if (a.rms_w != nullptr) {
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < kXKeep; ++j) {
+      const int i = threadIdx.x + j * kStagedThreads;
+      const uint32_t u[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+      float s4 = 0.f;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        s4 = fmaf(bf16_lo(u[q]), bf16_lo(u[q]), s4);
+        s4 = fmaf(bf16_hi(u[q]), bf16_hi(u[q]), s4);
+      }
+      ss += i < nk ? s4 : 0.f;
+    }
+    ss = block_sum(ss, part);
+    inv = rsqrtf(ss / static_cast<float>(a.K) + a.rms_eps);
+  }
+#pragma unroll
+  for (int j = 0; j < kXKeep; ++j) {
+    const int i = threadIdx.x + j * kStagedThreads;
+    if (i < nvec) {
+      uint4 o = i < nk ? v[j] : make_uint4(0, 0, 0, 0);
+      if (a.rms_w != nullptr && i < nk) {
+        const uint32_t u[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+        const uint32_t gw[4] = {g[j].x, g[j].y, g[j].z, g[j].w};
+        uint32_t r[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const uint32_t lo = f32_to_bf16((bf16_lo(gw[q]) * bf16_lo(u[q])) * inv);
+          const uint32_t hi = f32_to_bf16((bf16_hi(gw[q]) * bf16_hi(u[q])) * inv);
+          r[q] = lo | (hi << 16);
+        }
+        o = make_uint4(r[0], r[1], r[2], r[3]);
+      }
+      xs[x_slot(i)] = o;
+    }
+  }
+  __syncthreads();
+}
+
+// Staging for the other cases: the attention merge, a ragged K, unaligned pointers.
+__device__ __forceinline__ void stage_x(const StreamArgs &a, uint4 *xs, float *part) {
+  zero_unused_slots(xs, a.K_pad);
+  if (a.attn_state != nullptr) {
+    for (int i = threadIdx.x; i < (a.K_pad >> 3); i += kStagedThreads) {
+      xs[x_slot(i)] = merged_attn_piece(a, i);
     }
     __syncthreads();
     return;
   }
-  constexpr int kKeep = 4;  // 16-byte vectors of x a thread keeps between the two passes
-  const int nfull = (a.K_pad >> 5) >> 6;
-  const int slots = x_pieces(a.K_pad);
-  const int nvec = a.K_pad >> 3;
-  const bool vec_ok = (a.K & 7) == 0 && aligned16(a.x) &&
-                      (a.rms_w == nullptr || aligned16(a.rms_w)) &&
-                      nvec <= kKeep * static_cast<int>(blockDim.x);
-  // Slots of the last tail step that no piece maps to (lanes past the end of the row).
   {
-    const int full = nfull << 8;
-    const int tail_half = ((a.K_pad >> 5) & 63) * 2;
-    for (int i = full + threadIdx.x; i < slots; i += blockDim.x) {
-      const int h = (((i - full) >> 7) << 6) + (i & 63);
-      if (h >= tail_half) {
-        xs[i] = make_uint4(0, 0, 0, 0);
-      }
-    }
-  }
-  if (vec_ok) {
-    // x and the norm weights are requested together: one memory round trip, not two.
-    uint4 v[kKeep], g[kKeep];
-    float ss = 0.f;
-#pragma unroll
-    for (int j = 0; j < kKeep; ++j) {
-      const int i = threadIdx.x + j * blockDim.x;
-      v[j] = make_uint4(0, 0, 0, 0);
-      g[j] = make_uint4(0, 0, 0, 0);
-      if (i * 8 < a.K) {
-        v[j] = reinterpret_cast<const uint4 *>(a.x)[i];
-        if (a.rms_w != nullptr) {
-          g[j] = reinterpret_cast<const uint4 *>(a.rms_w)[i];
-        }
-      }
-    }
-    float inv = 1.f;
-    if (a.rms_w != nullptr) {
-#pragma unroll
-      for (int j = 0; j < kKeep; ++j) {
-        const uint32_t u[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          ss = fmaf(bf16_lo(u[q]), bf16_lo(u[q]), ss);
-          ss = fmaf(bf16_hi(u[q]), bf16_hi(u[q]), ss);
-        }
-      }
-      ss = block_sum(ss, part);
-      inv = rsqrtf(ss / static_cast<float>(a.K) + a.rms_eps);
-    }
-#pragma unroll
-    for (int j = 0; j < kKeep; ++j) {
-      const int i = threadIdx.x + j * blockDim.x;
-      if (i < nvec) {
-        uint4 o = v[j];
-        if (a.rms_w != nullptr && i * 8 < a.K) {
-          const uint32_t u[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
-          const uint32_t gw[4] = {g[j].x, g[j].y, g[j].z, g[j].w};
-          uint32_t r[4];
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const uint32_t lo = f32_to_bf16((bf16_lo(gw[q]) * bf16_lo(u[q])) * inv);
-            const uint32_t hi = f32_to_bf16((bf16_hi(gw[q]) * bf16_hi(u[q])) * inv);
-            r[q] = lo | (hi << 16);
-          }
-          o = make_uint4(r[0], r[1], r[2], r[3]);
-        }
-        xs[x_slot(i, nfull)] = o;
-      }
-    }
-  } else {
     float inv = 1.f;
     if (a.rms_w != nullptr) {
       float ss = 0.f;
-      for (int i = threadIdx.x; i < a.K; i += blockDim.x) {
+      for (int i = threadIdx.x; i < a.K; i += kStagedThreads) {
         const float v = bf16_to_f32(a.x[i]);
         ss = fmaf(v, v, ss);
       }
@@ -284,7 +292,7 @@ __device__ __forceinline__ void stage_x(const StreamArgs &a, uint4 *xs, float *p
       inv = rsqrtf(ss / static_cast<float>(a.K) + a.rms_eps);
     }
     uint16_t *xh = reinterpret_cast<uint16_t *>(xs);
-    for (int i = threadIdx.x; i < a.K_pad; i += blockDim.x) {
+    for (int i = threadIdx.x; i < a.K_pad; i += kStagedThreads) {
       uint16_t v = 0;
       if (i < a.K) {
         v = a.x[i];
@@ -292,7 +300,7 @@ __device__ __forceinline__ void stage_x(const StreamArgs &a, uint4 *xs, float *p
           v = f32_to_bf16((bf16_to_f32(a.rms_w[i]) * bf16_to_f32(v)) * inv);
         }
       }
-      xh[(x_slot(i >> 3, nfull) << 3) + (i & 7)] = v;
+      xh[(x_slot(i >> 3) << 3) + (i & 7)] = v;
     }
   }
   __syncthreads();
@@ -334,10 +342,55 @@ __device__ __forceinline__ void rows_step(const uint32_t (&w)[R][NW], const floa
   }
 }
 
-// One wavefront, R weight rows sharing x.  x4 points at the activations as 16-byte
-// pieces: K_pad/8 of them in global memory (XL == false), or the LDS copy made by
-// stage_x in its [step][q][lane] order (XL == true).
-template <int R, bool XL>
+// ---- pair table (kernels that stage x in LDS) ---------------------------------------
+// One packed byte holds two codes; the table maps a byte to the two levels as a bf16
+// pair, and every lane owns a copy: entry (byte, lane) is the dword at byte address
+// byte*256 + lane*4, so the 64 lookups of a wavefront always fall in 64 different banks
+// whatever the codes are.  The table starts at LDS address 0 (these kernels have no
+// static LDS), which makes a lookup address one v_perm_b32: byte 1 = the packed byte,
+// byte 0 = 4*lane.  A pair meets two activations, kept as the bf16 pair they arrive as,
+// in one v_dot2c_f32_bf16: per two weights one address op, one LDS read and one
+// multiply-add, against two of each with the 16-entry table.
+constexpr int kPairTableBytes = 256 * 64 * 4;
+constexpr int kStagedSmallBytes = 512;  // GemvLds of a staged kernel, after the table
+static_assert(sizeof(GemvLds) <= kStagedSmallBytes, "GemvLds must fit its slot");
+
+typedef __attribute__((ext_vector_type(2))) __bf16 Bf16x2;
+
+__device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float acc) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(Bf16x2, a),
+                                         __builtin_bit_cast(Bf16x2, b), acc, false);
+}
+
+__device__ __forceinline__ uint32_t lds0_u32(uint32_t addr) {
+  return *reinterpret_cast<const __attribute__((address_space(3))) uint32_t *>(addr);
+}
+
+template <int J>
+__device__ __forceinline__ uint32_t pair_at(uint32_t w, uint32_t lane4) {
+  // selector: result byte 0 <- lane4 byte 0, byte 1 <- w byte J, bytes 2..3 <- 0x00
+  constexpr uint32_t sel = 0x0C0C0400u + (static_cast<uint32_t>(J) << 8);
+  return lds0_u32(__builtin_amdgcn_perm(w, lane4, sel));
+}
+
+// bf16 bits (round to nearest even) of a finite binary32 pattern, usable at compile time.
+constexpr uint32_t bf16_bits_rne(uint32_t b) { return (b + 0x7FFFu + ((b >> 16) & 1u)) >> 16; }
+
+// Fill the table from a workgroup of exactly 16 wavefronts; the caller's next barrier
+// publishes it.  Wavefront v writes the bytes whose low code is v: byte = v + 16*j has
+// high code j, a compile-time constant, so an entry costs one OR and one LDS store.
+__device__ __forceinline__ void fill_pair_table(uint32_t *table, int wave, int lane) {
+  const uint32_t lo = bf16_bits_rne(kLutBits[wave]);
+#pragma unroll
+  for (int j = 0; j < 16; ++j) {
+    const uint32_t hi = bf16_bits_rne(kLevelBits[j]) << 16;
+    table[((wave + 16 * j) << 6) + lane] = lo | hi;
+  }
+}
+
+// One wavefront, R weight rows sharing x, which is read from global memory (K_pad/8
+// 16-byte pieces at x4).
+template <int R>
 __device__ __forceinline__ void rows_dot(const uint8_t *const (&prow)[R],
                                          const uint16_t *const (&srow)[R], const uint4 *x4,
                                          int K_pad, const float *lut, int lane,
@@ -364,9 +417,8 @@ __device__ __forceinline__ void rows_dot(const uint8_t *const (&prow)[R],
         w[r][3] = v.w;
         sc[r] = srow[r][c >> 1];
       }
-      const uint4 *xp = XL ? x4 + (t << 8) + lane : x4 + (c << 2);
-      constexpr int xq = XL ? 64 : 1;
-      const uint4 x0 = xp[0], x1 = xp[xq], x2 = xp[2 * xq], x3 = xp[3 * xq];
+      const uint4 *xp = x4 + (c << 2);
+      const uint4 x0 = xp[0], x1 = xp[1], x2 = xp[2], x3 = xp[3];
       float xf[32];
       widen8(x0, xf);
       widen8(x1, xf + 8);
@@ -374,8 +426,7 @@ __device__ __forceinline__ void rows_dot(const uint8_t *const (&prow)[R],
       widen8(x3, xf + 24);
       rows_step<R, 4>(w, xf, sc, lut, acc);
     } else {
-      const int h0 = (t - nfull) << 6;
-      const int h = h0 + lane;
+      const int h = ((t - nfull) << 6) + lane;
       if (h < tail_half) {
         const int hc = base_half + h;  // half-chunk index in the row: 16 weights
         uint32_t w[R][2];
@@ -387,8 +438,8 @@ __device__ __forceinline__ void rows_dot(const uint8_t *const (&prow)[R],
           w[r][1] = v.y;
           sc[r] = srow[r][hc >> 2];
         }
-        const uint4 *xp = XL ? x4 + (nfull << 8) + ((h0 >> 6) << 7) + lane : x4 + (hc << 1);
-        const uint4 x0 = xp[0], x1 = xp[XL ? 64 : 1];
+        const uint4 *xp = x4 + (hc << 1);
+        const uint4 x0 = xp[0], x1 = xp[1];
         float xf[16];
         widen8(x0, xf);
         widen8(x1, xf + 8);
@@ -400,13 +451,53 @@ __device__ __forceinline__ void rows_dot(const uint8_t *const (&prow)[R],
 
 __device__ __forceinline__ float silu(float v) { return v / (1.f + expf(-v)); }
 
+// Segment, first row and row count of a row group numbered through the segments.
+template <bool SWIGLU>
+__device__ __forceinline__ void group_rows(const StreamArgs &a, int grp, int U, int &seg,
+                                           int &row0, int &M) {
+  int g = grp;
+  seg = 0;
+  if (!SWIGLU) {
+    if (g >= a.groups[0]) {
+      g -= a.groups[0];
+      seg = 1;
+      if (g >= a.groups[1]) {
+        g -= a.groups[1];
+        seg = 2;
+      }
+    }
+  }
+  M = a.M[seg];
+  row0 = g * U;
+}
+
+template <int R, bool SWIGLU>
+__device__ __forceinline__ void group_pointers(const StreamArgs &a, int grp,
+                                               const uint8_t *(&prow)[R],
+                                               const uint16_t *(&srow)[R]) {
+  constexpr int U = SWIGLU ? R / 2 : R;
+  int seg, row0, M;
+  group_rows<SWIGLU>(a, grp, U, seg, row0, M);
+  const size_t pstride = static_cast<size_t>(a.K_pad >> 1);
+  const size_t sstride = static_cast<size_t>(a.K_pad >> 6);
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int r = min(row0 + u, M - 1);  // rows past M are computed, never stored
+    prow[u] = a.packed[seg] + r * pstride;
+    srow[u] = a.scale[seg] + r * sstride;
+    if constexpr (SWIGLU) {
+      prow[U + u] = a.packed2 + r * pstride;
+      srow[U + u] = a.scale2 + r * sstride;
+    }
+  }
+}
+
+// Plain kernel: four wavefronts per workgroup, x read from global memory.
 // SWIGLU == false: R rows of one segment per wavefront, epilogue y = acc (+ add).
 // SWIGLU == true : R/2 gate rows and the matching R/2 up rows per wavefront,
 //                  epilogue y = silu(gate) * up from the unrounded fp32 sums.
-// XLDS: x is first copied (and optionally RMS-normalised) into LDS.
-template <int R, bool SWIGLU, bool XLDS>
-__global__ __launch_bounds__(XLDS ? 1024 : 256) void gemv_stream(const StreamArgs a) {
-  extern __shared__ uint4 xs[];
+template <int R, bool SWIGLU>
+__global__ __launch_bounds__(256) void gemv_stream(const StreamArgs a) {
   __shared__ GemvLds lds;
   constexpr int U = SWIGLU ? R / 2 : R;  // output rows per wavefront
   const int lane = threadIdx.x & (kWave - 1);
@@ -418,61 +509,218 @@ __global__ __launch_bounds__(XLDS ? 1024 : 256) void gemv_stream(const StreamArg
   if (threadIdx.x < 16) {
     lds.lut[threadIdx.x] = bits_to_f32(kLutBits[threadIdx.x]);
   }
-  // Row groups (U rows each) are numbered through the segments.  Without the LDS
-  // copy a wavefront takes exactly one group; with it the grid is one workgroup per
-  // compute unit and a wavefront walks groups wave*grid + block, + grid*waves, ..,
-  // so the copy is made once per compute unit and units stay balanced to one group.
+  // Row groups (U rows each) are numbered through the segments; a wavefront takes exactly
+  // one group, or, with ksplit, the wavefronts of a workgroup share one along K.
   const int total = a.groups[0] + a.groups[1] + a.groups[2];
-  const bool ksplit = !XLDS && !SWIGLU && a.ksplit > 1;
-  const int first = XLDS     ? wave * static_cast<int>(gridDim.x) + static_cast<int>(blockIdx.x)
-                    : ksplit ? static_cast<int>(blockIdx.x)
-                             : static_cast<int>(blockIdx.x) * waves + wave;
-  const int stride = static_cast<int>(gridDim.x) * waves;
-  const size_t pstride = static_cast<size_t>(a.K_pad >> 1);
-  const size_t sstride = static_cast<size_t>(a.K_pad >> 6);
-
-  if constexpr (XLDS) {
-    stage_x(a, xs, lds.part);
-  } else {
-    __syncthreads();
+  const bool ksplit = !SWIGLU && a.ksplit > 1;
+  const int grp = ksplit ? static_cast<int>(blockIdx.x)
+                         : static_cast<int>(blockIdx.x) * waves + wave;
+  __syncthreads();
+  if (grp >= total) {
+    return;
   }
+  int seg, row0, M;
+  group_rows<SWIGLU>(a, grp, U, seg, row0, M);
+  const uint8_t *prow[R];
+  const uint16_t *srow[R];
+  group_pointers<R, SWIGLU>(a, grp, prow, srow);
 
-  auto run_group = [&](int grp) {
-    int g = grp;
-    int seg = 0;
-    if (!SWIGLU) {
-      if (g >= a.groups[0]) {
-        g -= a.groups[0];
-        seg = 1;
-        if (g >= a.groups[1]) {
-          g -= a.groups[1];
-          seg = 2;
-        }
-      }
-    }
-    const int M = a.M[seg];
-    const int row0 = g * U;
-    const uint8_t *prow[R];
-    const uint16_t *srow[R];
+  float acc[R] = {};
+  rows_dot<R>(prow, srow, reinterpret_cast<const uint4 *>(a.x), a.K_pad, lds.lut, lane, acc,
+              ksplit ? wave : 0, ksplit ? waves : 1);
+
+  if constexpr (SWIGLU) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int r = min(row0 + u, M - 1);  // rows past M are computed, never stored
-      prow[u] = a.packed[seg] + r * pstride;
-      srow[u] = a.scale[seg] + r * sstride;
-      if constexpr (SWIGLU) {
-        prow[U + u] = a.packed2 + r * pstride;
-        srow[U + u] = a.scale2 + r * sstride;
+      const float gsum = wave_sum(acc[u]);
+      const float usum = wave_sum(acc[U + u]);
+      const int r = row0 + u;
+      if (lane == u && r < M) {
+        a.y[0][r] = f32_to_bf16(silu(gsum) * usum);
       }
     }
-
-    float acc[R] = {};
-    if constexpr (XLDS) {
-      rows_dot<R, true>(prow, srow, static_cast<const uint4 *>(xs), a.K_pad, lds.lut, lane, acc);
-    } else {
-      rows_dot<R, false>(prow, srow, reinterpret_cast<const uint4 *>(a.x), a.K_pad, lds.lut, lane,
-                         acc, ksplit ? wave : 0, ksplit ? waves : 1);
+  } else {
+    const uint16_t *add = a.add[seg];
+    uint16_t *y = a.y[seg];
+    float sums[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      sums[u] = wave_sum(acc[u]);
     }
+    bool writer = true;
+    if (ksplit) {
+      // every wavefront of the workgroup holds a partial of the same rows: add them in
+      // wavefront order, wavefront 0 finishes
+      if (lane == 0) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          lds.ksum[wave][u] = sums[u];
+        }
+      }
+      __syncthreads();
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        float t = 0.f;
+        for (int w = 0; w < waves; ++w) {
+          t += lds.ksum[w][u];
+        }
+        sums[u] = t;
+      }
+      writer = wave == 0;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const float sv = sums[u];
+      const int r = row0 + u;
+      if (writer && lane == u && r < M) {
+        float v = sv;
+        if (add != nullptr) {
+          v += bf16_to_f32(add[r]);
+        }
+        y[r] = f32_to_bf16(v);
+      }
+    }
+  }
+}
 
+// ---- staged kernel: x in LDS, pair table, weight prefetch two steps ahead ----------
+// Request half step t of R rows: 8 packed bytes per lane.  Lanes past the end of the row
+// read the row's last half chunk instead (in bounds, one instruction form for every
+// step) and are switched off where the scale is applied.
+template <int R>
+__device__ __forceinline__ void load_step(const uint8_t *const (&prow)[R],
+                                          const uint16_t *const (&srow)[R], int n_half, int t,
+                                          int lane, uint2 (&w)[R], uint16_t (&sc)[R]) {
+  const int h = min((t << 6) + lane, n_half - 1);
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    w[r] = *(reinterpret_cast<const uint2 *>(prow[r]) + h);
+    sc[r] = srow[r][h >> 2];
+  }
+}
+
+template <int R>
+__device__ __forceinline__ void dot_step(const uint2 (&w)[R], const uint16_t (&sc)[R],
+                                         const uint4 *xs, int n_half, int t, int lane,
+                                         float (&acc)[R]) {
+  const uint32_t lane4 = static_cast<uint32_t>(lane) << 2;
+  const bool on = (t << 6) + lane < n_half;
+  const uint4 *xp = xs + (t << 7) + lane;
+  const uint4 x0 = xp[0], x1 = xp[64];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    float pa = 0.f, pb = 0.f;
+    pa = dot2_bf16(pair_at<0>(w[r].x, lane4), x0.x, pa);
+    pb = dot2_bf16(pair_at<1>(w[r].x, lane4), x0.y, pb);
+    pa = dot2_bf16(pair_at<2>(w[r].x, lane4), x0.z, pa);
+    pb = dot2_bf16(pair_at<3>(w[r].x, lane4), x0.w, pb);
+    pa = dot2_bf16(pair_at<0>(w[r].y, lane4), x1.x, pa);
+    pb = dot2_bf16(pair_at<1>(w[r].y, lane4), x1.y, pb);
+    pa = dot2_bf16(pair_at<2>(w[r].y, lane4), x1.z, pa);
+    pb = dot2_bf16(pair_at<3>(w[r].y, lane4), x1.w, pb);
+    const float scale = on ? f16_to_f32(sc[r]) : 0.f;
+    acc[r] = fmaf(scale, pa + pb, acc[r]);
+  }
+}
+
+// bf16 at a wavefront-uniform address, read on the scalar unit as the aligned dword that
+// holds it: the read then does not join the in-order queue of vector loads, so taking it
+// does not wait for weights requested ahead.
+__device__ __forceinline__ float uniform_bf16(const uint16_t *p) {
+  typedef const __attribute__((address_space(4))) uint32_t *ScalarWord;
+  const uintptr_t u = reinterpret_cast<uintptr_t>(p);
+  const uint32_t word = *reinterpret_cast<ScalarWord>(u & ~static_cast<uintptr_t>(3));
+  return (u & 2) != 0 ? bf16_hi(word) : bf16_lo(word);
+}
+
+// One workgroup of 16 wavefronts per compute unit; a wavefront walks the row groups
+// wave*grid + block, + 16*grid, ..  The half steps of those groups, in order, are the
+// wavefront's work list; an item is S consecutive ones (it may span two groups).  The S
+// requests of an item are issued back to back into one of two register buffers; while item i is
+// computed from one buffer, item i+1 is already in flight into the other, across group
+// borders too, so a wavefront always has S*R*8 bytes per lane on the way.  Between a
+// request and its use the code is straight-line (the loop is written out for both buffer
+// parities and the last item has its own copy without a request), so the wait counts the
+// compiler derives are exact: step j waits for its own data while steps j+1.. and the
+// whole next item are still arriving.  The first item is requested before x is staged:
+// the weight stream starts with the kernel.
+//   SWIGLU == false: R rows of one segment per group, epilogue y = acc (+ add).
+//   SWIGLU == true : R/2 gate rows and the matching R/2 up rows, y = silu(gate) * up
+//                    from the unrounded fp32 sums.
+template <int R, int S, bool SWIGLU>
+__global__ __launch_bounds__(1024) void gemv_staged(const StreamArgs a) {
+  extern __shared__ uint4 dyn_lds[];  // [pair table][GemvLds][x pieces], table at address 0
+  char *base = reinterpret_cast<char *>(dyn_lds);
+  GemvLds &lds = *reinterpret_cast<GemvLds *>(base + kPairTableBytes);
+  uint4 *xs = reinterpret_cast<uint4 *>(base + kPairTableBytes + kStagedSmallBytes);
+  constexpr int U = SWIGLU ? R / 2 : R;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
+  constexpr int waves = kStagedThreads >> 6;
+  const int total = a.groups[0] + a.groups[1] + a.groups[2];
+  const int first = wave * static_cast<int>(gridDim.x) + static_cast<int>(blockIdx.x);
+  const int stride = static_cast<int>(gridDim.x) * waves;
+  const int n_half = a.K_pad >> 4;
+  const int nsteps = x_half_steps(a.K_pad);
+  const int my_groups = first < total ? (total - first + stride - 1) / stride : 0;
+  const int n_steps_all = my_groups * nsteps;      // half steps of this wavefront, in order
+  const int n_items = (n_steps_all + S - 1) / S;   // S of them per item, across group borders
+
+  // request cursor: half step pi of the list = step pt of group pg
+  int pi = 0, pg = first, pt = 0;
+  const uint8_t *prow[R];
+  const uint16_t *srow[R];
+  uint2 wa[S][R], wb[S][R];
+  uint16_t sa[S][R], sb[S][R];
+
+  // Past the end of the list the cursor stays on the last half step: the repeat is
+  // served by the cache and keeps the number of loads per item fixed.
+#define CHR_REQUEST(W, SC)                                              \
+  _Pragma("unroll") for (int j = 0; j < S; ++j) {                       \
+    load_step<R>(prow, srow, n_half, pt, lane, W[j], SC[j]);            \
+    if (pi + 1 < n_steps_all) {                                         \
+      ++pi;                                                             \
+      if (++pt == nsteps) {                                             \
+        pt = 0;                                                         \
+        pg += stride;                                                   \
+        group_pointers<R, SWIGLU>(a, pg, prow, srow);                   \
+      }                                                                 \
+    }                                                                   \
+  }
+
+  // Order of the first requests: x, then the first item of weights, and only then the
+  // wait for x.  Vector loads return in order, so x must be the older request or its wait
+  // would be a wait for the weights too.  Each case below is its own straight-line path
+  // (the two copies of the stores and barriers are the price): a path that merged
+  // "weights requested" with "nothing requested" would make the wait a wait for all.
+  if (stage_fast_ok(a)) {
+    uint4 xv[kXKeep], xg[kXKeep];
+    x_request(a, xv, xg);
+    if (n_items > 0) {
+      group_pointers<R, SWIGLU>(a, first, prow, srow);
+      CHR_REQUEST(wa, sa)
+      fill_pair_table(reinterpret_cast<uint32_t *>(dyn_lds), wave, lane);
+      x_store(a, xs, lds.part, xv, xg);
+    } else {
+      fill_pair_table(reinterpret_cast<uint32_t *>(dyn_lds), wave, lane);
+      x_store(a, xs, lds.part, xv, xg);
+    }
+  } else {
+    fill_pair_table(reinterpret_cast<uint32_t *>(dyn_lds), wave, lane);
+    stage_x(a, xs, lds.part);
+    if (n_items > 0) {
+      group_pointers<R, SWIGLU>(a, first, prow, srow);
+      CHR_REQUEST(wa, sa)
+    }
+  }
+
+  // compute cursor: half step ci of the list = step ct of group cg
+  int ci = 0, cg = first, ct = 0;
+  float acc[R] = {};
+
+  auto finish_group = [&](int grp) {
+    int seg, row0, M;
+    group_rows<SWIGLU>(a, grp, U, seg, row0, M);
     if constexpr (SWIGLU) {
 #pragma unroll
       for (int u = 0; u < U; ++u) {
@@ -486,55 +734,60 @@ __global__ __launch_bounds__(XLDS ? 1024 : 256) void gemv_stream(const StreamArg
     } else {
       const uint16_t *add = a.add[seg];
       uint16_t *y = a.y[seg];
-      float sums[U];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        sums[u] = wave_sum(acc[u]);
-      }
-      bool writer = true;
-      if (ksplit) {
-        // every wavefront of the workgroup holds a partial of the same rows: add them in
-        // wavefront order, wavefront 0 finishes
-        if (lane == 0) {
-#pragma unroll
-          for (int u = 0; u < U; ++u) {
-            lds.ksum[wave][u] = sums[u];
-          }
-        }
-        __syncthreads();
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-          float t = 0.f;
-          for (int w = 0; w < waves; ++w) {
-            t += lds.ksum[w][u];
-          }
-          sums[u] = t;
-        }
-        writer = wave == 0;
-      }
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const float s = sums[u];
+        float v = wave_sum(acc[u]);
         const int r = row0 + u;
-        if (writer && lane == u && r < M) {
-          float v = s;
-          if (add != nullptr) {
-            v += bf16_to_f32(add[r]);
-          }
+        if (add != nullptr) {
+          v += uniform_bf16(add + min(r, M - 1));
+        }
+        if (lane == u && r < M) {
           y[r] = f32_to_bf16(v);
         }
       }
     }
-  };
-  if constexpr (XLDS) {
-    for (int grp = first; grp < total; grp += stride) {
-      run_group(grp);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      acc[r] = 0.f;
     }
-  } else {
-    if (first < total) {
-      run_group(first);  // exactly one group per wavefront
+  };
+
+#define CHR_COMPUTE(W, SC)                                              \
+  _Pragma("unroll") for (int j = 0; j < S; ++j) {                       \
+    if (ci < n_steps_all) {                                             \
+      dot_step<R>(W[j], SC[j], xs, n_half, ct, lane, acc);              \
+      ++ci;                                                             \
+      if (++ct == nsteps) {                                             \
+        finish_group(cg);                                               \
+        ct = 0;                                                         \
+        cg += stride;                                                   \
+      }                                                                 \
+    }                                                                   \
+  }
+
+  if (n_items > 0) {
+    int i = 0;
+    while (true) {
+      // item i is in (wa, sa)
+      if (i + 1 >= n_items) {
+        CHR_COMPUTE(wa, sa)
+        break;
+      }
+      CHR_REQUEST(wb, sb)
+      CHR_COMPUTE(wa, sa)
+      ++i;
+      // item i is in (wb, sb)
+      if (i + 1 >= n_items) {
+        CHR_COMPUTE(wb, sb)
+        break;
+      }
+      CHR_REQUEST(wa, sa)
+      CHR_COMPUTE(wb, sb)
+      ++i;
     }
   }
+#undef CHR_COMPUTE
+#undef CHR_REQUEST
 }
 
 // ---- RMSNorm -----------------------------------------------------------------
@@ -624,7 +877,6 @@ int forced_staged() {
 }
 
 constexpr int kThreads = 256;
-constexpr int kStagedThreads = 1024;  // workgroup of the kernels that stage x in LDS
 constexpr size_t kMaxDynLds = 150 * 1024;
 
 template <typename Kern>
@@ -643,25 +895,61 @@ int prep_lds(Kern kern, size_t dyn) {
   return 0;
 }
 
+// Half steps per item of the staged kernel.  Measured on the 14B shapes: one step leaves
+// too little in flight (13824x5120: 12.9 us), two are best (10.3 us), three and five cost
+// more again (10.4, 11.0 us) -- deeper request queues do not pay on this memory system.
+constexpr int kItemSteps = 2;
+
+inline size_t staged_lds_bytes(int K_pad) {
+  return kPairTableBytes + kStagedSmallBytes + static_cast<size_t>(x_pieces(K_pad)) * 16;
+}
+
+// Kernel family for a launch of m_total weight rows: 1 staged, 0 plain, -1 staging is
+// required but x does not fit the LDS.  Staging is required by the fused RMSNorm, a
+// ragged K and the attention merge; otherwise the staged kernel is taken from 16M codes
+// up (below that its set-up costs more than its cheaper inner loop returns: 2048x2048
+// measures 4.2 us staged, 3.9 us plain; 11008x2048 6.0 against 6.2 us).
+int pick_family(const StreamArgs &a, int m_total) {
+  const bool fits = staged_lds_bytes(a.K_pad) <= kMaxDynLds;
+  if (a.rms_w != nullptr || a.K != a.K_pad || a.attn_state != nullptr) {
+    return fits ? 1 : -1;
+  }
+  const int forced = forced_staged();
+  if (forced >= 0) {
+    return forced == 1 && fits ? 1 : 0;
+  }
+  const long long codes = static_cast<long long>(m_total) * a.K_pad;
+  return fits && codes >= (16ll << 20) ? 1 : 0;
+}
+
+// Rows per wavefront of the staged kernel: one, so that even 5120 rows give every
+// wavefront of 256 compute units work, and two from 32768 rows up (lm_head 152064x5120:
+// 75 us against 81 us).
+int staged_rows_for_m(int M) {
+  const int f = forced_rows();
+  if (f > 0) {
+    return f;
+  }
+  return M >= 32768 ? 2 : 1;
+}
+
 template <int R, bool SWIGLU>
-int launch_stream(StreamArgs &a, int n_seg, hipStream_t st) {
+int launch_stream(StreamArgs &a, int n_seg, bool staged, hipStream_t st) {
   constexpr int U = SWIGLU ? R / 2 : R;
   int total = 0;
   for (int i = 0; i < 3; ++i) {
     a.groups[i] = i < n_seg ? (a.M[i] + U - 1) / U : 0;
     total += a.groups[i];
   }
-  const size_t dyn = static_cast<size_t>(x_pieces(a.K_pad)) * 16;
-  const bool must_stage = a.rms_w != nullptr || a.K != a.K_pad || a.attn_state != nullptr;
-  const int forced = forced_staged();
-  const bool staged = must_stage || (forced == 1 && dyn <= kMaxDynLds);
   if (staged) {
-    if (prep_lds(gemv_stream<R, SWIGLU, true>, dyn) != 0) {
-      return -6;
-    }
+    const size_t dyn = staged_lds_bytes(a.K_pad);
     const int waves = kStagedThreads / kWave;
     const int grid = std::min(device_cu_count(), (total + waves - 1) / waves);
-    gemv_stream<R, SWIGLU, true><<<dim3(grid), dim3(kStagedThreads), dyn, st>>>(a);
+    constexpr auto kern = gemv_staged<R, kItemSteps, SWIGLU>;
+    if (prep_lds(kern, dyn) != 0) {
+      return -6;
+    }
+    kern<<<dim3(grid), dim3(kStagedThreads), dyn, st>>>(a);
   } else {
     const int waves = kThreads / kWave;
     // Long rows and few of them (a down projection): a wavefront walking a whole row pays
@@ -671,20 +959,40 @@ int launch_stream(StreamArgs &a, int n_seg, hipStream_t st) {
     const bool split = !SWIGLU && nsteps >= 4 && total * 4 <= 16 * device_cu_count() * 4;
     a.ksplit = split ? waves : 1;
     const int grid = split ? total : (total + waves - 1) / waves;
-    gemv_stream<R, SWIGLU, false><<<dim3(grid), dim3(kThreads), 0, st>>>(a);
+    gemv_stream<R, SWIGLU><<<dim3(grid), dim3(kThreads), 0, st>>>(a);
   }
   return launch_rc();
 }
 
 int launch_rows(StreamArgs &a, int n_seg, int m_for_policy, hipStream_t st) {
-  switch (rows_for_m(m_for_policy)) {
-    case 4:
-      return launch_stream<4, false>(a, n_seg, st);
-    case 2:
-      return launch_stream<2, false>(a, n_seg, st);
-    default:
-      return launch_stream<1, false>(a, n_seg, st);
+  const int family = pick_family(a, m_for_policy);
+  if (family < 0) {
+    return -6;
   }
+  const bool staged = family == 1;
+  switch (staged ? staged_rows_for_m(m_for_policy) : rows_for_m(m_for_policy)) {
+    case 4:
+      return launch_stream<4, false>(a, n_seg, staged, st);
+    case 2:
+      return launch_stream<2, false>(a, n_seg, staged, st);
+    default:
+      return launch_stream<1, false>(a, n_seg, staged, st);
+  }
+}
+
+// A gate/up pair is two weight streams per output row: the staged kernel takes one pair
+// per wavefront (two from 32768 pairs up), the plain one two pairs when there are enough.
+int launch_pairs(StreamArgs &a, int m_pairs, hipStream_t st) {
+  const int family = pick_family(a, 2 * m_pairs);
+  if (family < 0) {
+    return -6;
+  }
+  const bool staged = family == 1;
+  const int rows = staged ? 2 * staged_rows_for_m(m_pairs) : (rows_for_m(2 * m_pairs) >= 2 ? 4 : 2);
+  if (rows >= 4) {
+    return launch_stream<4, true>(a, 1, staged, st);
+  }
+  return launch_stream<2, true>(a, 1, staged, st);
 }
 
 }  // namespace
@@ -844,12 +1152,7 @@ extern "C" int chr_nf4_gemv_swiglu(const chr_nf4_dev_t *gate, const chr_nf4_dev_
   a.K = gate->K;
   a.K_pad = gate->K_pad;
   a.rms_eps = rms_eps;
-  hipStream_t st = static_cast<hipStream_t>(stream);
-  // A gate/up pair is two weight streams per output row.
-  if (rows_for_m(2 * gate->M) >= 2) {
-    return launch_stream<4, true>(a, 1, st);
-  }
-  return launch_stream<2, true>(a, 1, st);
+  return launch_pairs(a, gate->M, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int chr_nf4_rms(const void *x, const void *w, void *y, int32_t n, float eps,

@@ -51,12 +51,47 @@ def ulp_bf16(v: np.ndarray) -> np.ndarray:
     return 2.0 ** (e - 7)
 
 
-def check_linear(y: torch.Tensor, y_ref: np.ndarray, *, what: str = "", ulps: float = 1.0) -> dict:
+#: The staged GEMV (x in LDS: fused RMSNorm, ragged K, attention merge, and every matrix
+#: from 16M codes up) multiplies bf16-rounded levels, as the reference's tensor-core path
+#: does with the whole dequantised weight (gpu/nf4/nf4_gemm.cu:322).
+STAGED_MIN_CODES = 16 << 20
+
+
+def takes_staged_gemv(m: int, k: int, *, fused: bool = False) -> bool:
+    """Whether a GEMV launch of m rows takes the staged kernel (the library's policy)."""
+    return fused or k != oc.k_pad(k) or m * oc.k_pad(k) >= STAGED_MIN_CODES
+
+
+def staged_gemv_model(packed: np.ndarray, scale: np.ndarray, m: int, k: int,
+                      x: np.ndarray) -> np.ndarray:
+    """The staged GEMV's arithmetic in float64: levels rounded to bf16, products exact,
+    the fp16 scale applied to each group's sum.  x is [k] or [k, n]."""
+    kp = oc.k_pad(k)
+    g = kp // oc.GROUP
+    packed = np.asarray(packed).reshape(m, kp // 2)
+    sc = np.ascontiguousarray(scale).view(np.float16).reshape(m, g).astype(np.float64)
+    lut = oc.bf16_round(oc.LUT.astype(np.float32)).astype(np.float64)
+    xs = np.zeros((kp,) + tuple(np.shape(x)[1:]), dtype=np.float64)
+    xs[:k] = np.asarray(x, dtype=np.float64)
+    xg = xs.reshape((g, oc.GROUP) + xs.shape[1:])
+    out = np.empty((m,) + xs.shape[1:], dtype=np.float64)
+    for r0 in range(0, m, 512):  # row blocks keep the float64 level array small
+        r1 = min(m, r0 + 512)
+        lv = lut[oc.np_unpack(packed[r0:r1])].reshape(r1 - r0, g, oc.GROUP)
+        part = np.einsum("mgk,gk...->mg...", lv, xg)
+        out[r0:r1] = np.einsum("mg...,mg->m...", part, sc[r0:r1])
+    return out
+
+
+def check_linear(y: torch.Tensor, y_ref: np.ndarray, *, what: str = "", ulps: float = 1.0,
+                 model: np.ndarray | None = None) -> dict:
     """y (bf16 on GPU) against a float32/float64 oracle result of the same shape.
 
     Three bounds: the reference's floor-1 bound max(0.05, ULP/2); max-rel 1e-2;
-    and a tighter one of this build: within ``ulps`` bf16 ULP of the oracle value
-    (plus 1e-3 of the output's rms for cancellation-heavy rows)."""
+    and a tighter one of this build: within ``ulps`` bf16 ULP of the expected value
+    (plus 1e-3 of the output's rms for cancellation-heavy rows).  The expected value of
+    the tight bound is ``model`` when given (the kernel's own arithmetic written out on
+    the CPU, e.g. ``staged_gemv_model``), else the oracle value."""
     got = to_f32(y).reshape(-1).astype(np.float64)
     ref = np.asarray(y_ref, dtype=np.float64).reshape(-1)
     assert got.shape == ref.shape, (got.shape, ref.shape)
@@ -68,6 +103,10 @@ def check_linear(y: torch.Tensor, y_ref: np.ndarray, *, what: str = "", ulps: fl
     denom = np.abs(ref).max()
     if denom > 0:
         assert err.max() / denom <= MAX_REL, f"{what}: max-rel {err.max() / denom:.3e}"
-    assert (err <= ulps * u + 1e-3 * rms + 1e-30).all(), (
-        f"{what}: worst {np.max(err / (u + 1e-30)):.2f} bf16 ULP")
+    tight = ref if model is None else np.asarray(model, dtype=np.float64).reshape(-1)
+    assert tight.shape == ref.shape, (tight.shape, ref.shape)
+    terr = np.abs(got - tight)
+    tu = ulp_bf16(tight)
+    assert (terr <= ulps * tu + 1e-3 * rms + 1e-30).all(), (
+        f"{what}: worst {np.max(terr / (tu + 1e-30)):.2f} bf16 ULP")
     return {"maxabs": float(err.max()), "rms": rms}

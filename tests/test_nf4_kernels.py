@@ -11,7 +11,7 @@ from deepfold_amd import nf4
 from oracle import nf4_oracle as oc
 
 from helpers import (DEV, bf16_bits, bf16_tensor, check_linear, rand_x, to_f32, ulp_bf16, up,
-                     up_scale)
+                     up_scale, staged_gemv_model, takes_staged_gemv)
 
 pytestmark = pytest.mark.gpu
 
@@ -132,7 +132,8 @@ def test_gemv_toy_blobs(m, k):
     y = nf4.nf4_gemv(dp, ds, bf16_tensor(x), m, k, oc.k_pad(k))
     assert tuple(y.shape) == (m, 1)
     ref = oc.c_matmul_f64(oc.c_decode(p, s, m, k), x[:, None])
-    check_linear(y, ref, what=f"gemv {m}x{k}")
+    model = staged_gemv_model(p, s, m, k, x) if takes_staged_gemv(m, k) else None
+    check_linear(y, ref, what=f"gemv {m}x{k}", model=model)
     # same inputs, same bits
     y2 = nf4.nf4_gemv(dp, ds, bf16_tensor(x), m, k, oc.k_pad(k))
     assert (bf16_bits(y) == bf16_bits(y2)).all()
@@ -161,26 +162,51 @@ def test_gemv_zero_level_matrix():
     assert (to_f32(y) == 0).all()
 
 
-def test_gemv_config1_shape_quantized_weights():
+def test_gemv_config1_shape_quantized_weights(monkeypatch):
     m, k = 13824, 5120
     say("gemv config 1", m, k)
     w, p, s, dp, ds = quantized(m, k, 1)
     x = rand_x(k, None, 2)
     y = nf4.nf4_gemv(dp, ds, bf16_tensor(x), m, k, k)
     ref = oc.c_matmul_f64(oc.c_decode(p, s, m, k), x[:, None])
-    check_linear(y, ref, what="config 1")
-    # the float32 two-pass CPU linear of the reference agrees to the same bound
-    check_linear(y, oc.c_linear(p, s, m, k, x[:, None]), what="config 1 vs f32 oracle", ulps=1.5)
+    assert takes_staged_gemv(m, k)
+    model = staged_gemv_model(p, s, m, k, x)
+    check_linear(y, ref, what="config 1", model=model)
+    # the float32 two-pass CPU linear of the reference agrees to the same bounds
+    check_linear(y, oc.c_linear(p, s, m, k, x[:, None]), what="config 1 vs f32 oracle", ulps=1.5,
+                 model=model)
+    # the plain kernel (fp32 levels) on the same inputs: the tight bound against the oracle itself
+    monkeypatch.setenv("CHR_NF4_GEMV_STAGED", "0")
+    y0 = nf4.nf4_gemv(dp, ds, bf16_tensor(x), m, k, k)
+    check_linear(y0, ref, what="config 1, plain kernel")
 
 
+@pytest.mark.parametrize("staged", [0, 1])
 @pytest.mark.parametrize("rows", [1, 2, 4])
-def test_gemv_rows_per_wavefront_agree(rows, monkeypatch):
+def test_gemv_rows_per_wavefront_agree(rows, staged, monkeypatch):
     m, k = 1030, 5120
     p, s, dp, ds = blobs(m, k, 31)
     x = rand_x(k, None, 4)
     monkeypatch.setenv("CHR_NF4_GEMV_NR", str(rows))
+    monkeypatch.setenv("CHR_NF4_GEMV_STAGED", str(staged))
     y = nf4.nf4_gemv(dp, ds, bf16_tensor(x), m, k, k)
-    check_linear(y, oc.c_matmul_f64(oc.c_decode(p, s, m, k), x[:, None]), what=f"NR={rows}")
+    model = staged_gemv_model(p, s, m, k, x) if staged else None
+    check_linear(y, oc.c_matmul_f64(oc.c_decode(p, s, m, k), x[:, None]),
+                 what=f"NR={rows} staged={staged}", model=model)
+
+
+@pytest.mark.parametrize("m,k", [(4100, 5120), (700, 13824), (2100, 6208), (9000, 2048)])
+def test_gemv_staged_walks_many_groups_per_wavefront(m, k, monkeypatch):
+    """More row groups than the 4096 wavefronts of a launch on some shapes, fewer on others, a
+    K whose last half step is partly filled (6208), items that span two row groups."""
+    p, s, dp, ds = blobs(m, k, 33)
+    x = rand_x(k, None, 6)
+    monkeypatch.setenv("CHR_NF4_GEMV_STAGED", "1")
+    for rows in (1, 2):
+        monkeypatch.setenv("CHR_NF4_GEMV_NR", str(rows))
+        y = nf4.nf4_gemv(dp, ds, bf16_tensor(x), m, k, oc.k_pad(k))
+        check_linear(y, oc.c_matmul_f64(oc.c_decode(p, s, m, k), x[:, None]),
+                     what=f"staged {m}x{k} NR={rows}", model=staged_gemv_model(p, s, m, k, x))
 
 
 def test_gemv_residual_add_may_alias_out():
@@ -200,7 +226,7 @@ def test_gemv_residual_add_may_alias_out():
 
 
 @pytest.mark.parametrize("m,k", [(256, 2048), (130, 65)])
-def test_gemv_fused_rms(m, k):
+def test_gemv_fused_rms(m, k, monkeypatch):
     p, s, dp, ds = blobs(m, k, 51)
     rng = np.random.default_rng(7)
     x = oc.bf16_round(rng.standard_normal(k).astype(np.float32) * 3)
@@ -211,16 +237,17 @@ def test_gemv_fused_rms(m, k):
     xh = oc.bf16_round(((g.astype(np.float64) * x) * inv).astype(np.float32))
     # normalised x is rounded to bf16 before the dots; allow one bf16 step of x
     ref = oc.c_matmul_f64(oc.c_decode(p, s, m, k), xh[:, None])
-    check_linear(y, ref, what="fused rms", ulps=4)
-    # equals the two-launch form bit for bit when the RMS rounding agrees
+    check_linear(y, ref, what="fused rms", ulps=4, model=staged_gemv_model(p, s, m, k, xh))
+    # equals the two-launch form (same kernel family) bit for bit when the RMS rounding agrees
     h = torch.empty(k, dtype=torch.bfloat16, device=DEV)
     nf4.nf4_rms(bf16_tensor(x), bf16_tensor(g), h, eps)
+    monkeypatch.setenv("CHR_NF4_GEMV_STAGED", "1")
     y2 = nf4.nf4_gemv(dp, ds, h, m, k, oc.k_pad(k))
     check_linear(y, to_f32(y2), what="fused rms vs rms+gemv", ulps=1)
 
 
 @pytest.mark.parametrize("m,k", [(64, 512), (96, 1088), (40, 5120), (8, 13824)])
-def test_gemv_fused_rms_is_deterministic_with_a_partial_tail_step(m, k):
+def test_gemv_fused_rms_is_deterministic_with_a_partial_tail_step(m, k, monkeypatch):
     """K whose last step is only partly filled: the staged copy of x zero-fills the unused
     slots and must never touch the used ones, whatever order the lanes run in."""
     p, s, dp, ds = blobs(m, k, 77)
@@ -229,6 +256,7 @@ def test_gemv_fused_rms_is_deterministic_with_a_partial_tail_step(m, k):
     g = bf16_tensor(oc.bf16_round(1 + 0.1 * rng.standard_normal(k).astype(np.float32)))
     h = torch.empty(k, dtype=torch.bfloat16, device=DEV)
     nf4.nf4_rms(x, g, h, 1e-6)
+    monkeypatch.setenv("CHR_NF4_GEMV_STAGED", "1")  # the two-launch form in the same kernel family
     want = nf4.nf4_gemv(dp, ds, h, m, k, oc.k_pad(k))
     first = None
     for rep in range(25):
@@ -296,7 +324,10 @@ def test_qkv_equals_three_gemvs(mq, mk, k, bias):
         ref = oc.c_matmul_f64(oc.c_decode(p, s, m, k), x[:, None]).reshape(-1)
         if b is not None:
             ref = ref + b
-        check_linear(o, ref, what="qkv")
+        model = None
+        if takes_staged_gemv(mq + 2 * mk, k):
+            model = staged_gemv_model(p, s, m, k, x) + (0 if b is None else b)
+        check_linear(o, ref, what="qkv", model=model)
         single = torch.empty(m, dtype=torch.bfloat16, device=DEV)
         nf4.nf4_gemv(dp, ds, dx, m, k, kp, single, None if b is None else bf16_tensor(b))
         assert np.abs(to_f32(single) - to_f32(o)).max() <= 1e-3 + np.abs(to_f32(o)).max() * 2 ** -7
@@ -314,7 +345,11 @@ def test_swiglu_equals_pair(m, k):
     g = oc.c_matmul_f64(oc.c_decode(pg, sg, m, k), x[:, None]).reshape(-1)
     u = oc.c_matmul_f64(oc.c_decode(pu, su, m, k), x[:, None]).reshape(-1)
     ref = g / (1 + np.exp(-g)) * u
-    check_linear(out, ref, what="swiglu", ulps=1.5)
+    model = None
+    if takes_staged_gemv(2 * m, k):
+        gm = staged_gemv_model(pg, sg, m, k, x)
+        model = gm / (1 + np.exp(-gm)) * staged_gemv_model(pu, su, m, k, x)
+    check_linear(out, ref, what="swiglu", ulps=1.5, model=model)
 
 
 # ------------------------------------------------------------------------ RMS
