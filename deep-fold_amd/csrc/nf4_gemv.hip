@@ -706,12 +706,15 @@ __global__ __launch_bounds__(1024) void gemv_staged(const StreamArgs a) {
       x_store(a, xs, lds.part, xv, xg);
     }
   } else {
-    fill_pair_table(reinterpret_cast<uint32_t *>(dyn_lds), wave, lane);
-    stage_x(a, xs, lds.part);
+    // The other staging forms read what they need in loops of their own; the first item
+    // is requested ahead of them all the same: its trip to memory (the long one) then
+    // overlaps the staging, at the price of the staging's first loads returning behind it.
     if (n_items > 0) {
       group_pointers<R, SWIGLU>(a, first, prow, srow);
       CHR_REQUEST(wa, sa)
     }
+    fill_pair_table(reinterpret_cast<uint32_t *>(dyn_lds), wave, lane);
+    stage_x(a, xs, lds.part);
   }
 
   // compute cursor: half step ci of the list = step ct of group cg
