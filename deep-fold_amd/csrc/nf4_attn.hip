@@ -187,12 +187,12 @@ __global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flas
   const size_t row_stride = static_cast<size_t>(a.n_kv) * hd;
   // plain dwords: arrays of vector structs would not stay in registers
   uint32_t kraw[UNR][4], vraw[UNR][4];
-  auto load_block = [&](int t0) {
+  auto load_block = [&](int t0, int limit) {
 #pragma unroll
     for (int u = 0; u < UNR; ++u) {
       const int t = t0 + grp * a.n_split + u * stride;
       uint4 kv = make_uint4(0, 0, 0, 0), vv = make_uint4(0, 0, 0, 0);
-      if (t < vl) {  // the row at *position may be mid-write: it is replaced below
+      if (t < limit) {  // the row at *position may be mid-write: it is replaced below
         const size_t off =
             static_cast<size_t>(t) * row_stride + static_cast<size_t>(kv_head) * hd + d0;
         kv = *reinterpret_cast<const uint4 *>(a.k_cache + off);
@@ -208,7 +208,11 @@ __global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flas
       vraw[u][3] = vv.w;
     }
   };
-  load_block(split);
+  // The first block is bounded by the cache size, a launch argument, not by the valid
+  // length, a device scalar: its requests leave with the first instructions of the kernel
+  // instead of after a round trip for that scalar.  Rows past the valid length are
+  // allocated memory with arbitrary contents; they are dropped below (live[]) unused.
+  load_block(split, a.max_seq);
 
   float qf[8];
   float kcur[8];
@@ -250,7 +254,7 @@ __global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flas
   float acc[8] = {};
   for (int t0 = split; t0 < vl; t0 += UNR * stride) {
     if (t0 != split) {
-      load_block(t0);
+      load_block(t0, vl);
     }
     bool live[UNR], cur[UNR];
 #pragma unroll
