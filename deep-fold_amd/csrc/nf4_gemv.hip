@@ -2,27 +2,29 @@
 // fused SwiGLU, and RMSNorm.  Replaces the entry points of
 // gpu/nf4/nf4_gemv.cu:790-924, 996-1011.
 //
-// Row streaming.  A workgroup is four wavefronts of 64 lanes; every wavefront
-// owns R weight rows and walks the whole K axis of each.  Lane l reads the
-// 16-byte chunk l + 64*j of a row (32 codes, half a scale group), so one
-// wavefront load instruction covers 1 KiB of contiguous packed bytes.  The K
-// remainder that does not fill 64 such chunks is read as 8-byte half chunks, so
-// K = 5120 (160 chunks) costs 2 + 1 steps, not 3.  The R rows of a wavefront
-// share the activation registers: x is read and widened to fp32 once per step.
+// Two kernels, chosen per launch (pick_family).
 //
-// The 16 codebook levels sit at LDS address 0 as 16 consecutive dwords: 16
-// distinct addresses in 16 distinct banks, so 64 lanes with arbitrary codes
-// never conflict.  A lookup address is one VALU op per code (a byte-select AND);
-// lookups of the next packed dword are issued before the FMAs of the current
-// one.  The per-group scale multiplies each 32-term partial once.
+// Staged (gemv_staged): one workgroup of 16 wavefronts per compute unit.  x is copied to
+// LDS once per workgroup (RMS-normalised, zero-padded or merged from attention states on
+// the way if asked).  Packed bytes are looked up two codes at a time in a 256-entry table
+// of bf16 level pairs of which every lane owns a copy (conflict-free for any codes), and
+// meet the matching bf16 pair of x in one v_dot2c_f32_bf16.  Lane l of half step t reads
+// the 8 packed bytes 8*(64t + l) of a row; requests run one two-step item ahead of the
+// arithmetic through two register buffers.  Taken for a fused RMSNorm, a ragged K, the
+// attention merge, and every launch of 16M codes or more.
 //
-// x is read straight from global memory (it is small and L2-resident).  Only a
-// ragged K or the fused RMSNorm make the workgroup stage a bf16 copy in LDS
-// first (zero past K, normalised and rounded as a separate RMSNorm launch would).
+// Plain (gemv_stream): four wavefronts per workgroup; every wavefront owns R weight rows
+// and walks the whole K axis of each.  Lane l reads the 16-byte chunk l + 64*j of a row
+// (the K remainder as 8-byte half chunks, so K = 5120 costs 2 + 1 steps), x comes straight
+// from global memory, and the 16 fp32 levels sit at LDS address 0: 16 distinct addresses
+// in 16 distinct banks, a lookup address is one byte-select AND.  Taken for small launches,
+// where the staged kernel's set-up costs more than its inner loop returns.
 //
-// Numerics: weight = fp32 LUT * fp32(scale) never rounded below fp32, x widened
-// bf16->fp32, fp32 accumulation, residual / bias added in fp32, one bf16
-// rounding at the store (gpu/nf4/nf4_gemv.cu:70-101, 217-245).
+// Numerics.  Plain: weight = fp32 LUT * fp32(scale) never rounded below fp32, x widened
+// bf16->fp32 (gpu/nf4/nf4_gemv.cu:70-101, 217-245).  Staged: levels rounded to bf16,
+// exact products, the fp16 scale applied in fp32 to each 16-weight partial: the
+// precision class of the reference's tensor-core path (gpu/nf4/nf4_gemm.cu:322).  Both:
+// fp32 accumulation, residual / bias added in fp32, one bf16 rounding at the store.
 
 #include "nf4_common.h"
 
