@@ -43,9 +43,11 @@ namespace chr {
 
 int gemv_entry(const chr_nf4_dev_t *w, const void *x, void *y, void *stream, const void *add,
                const void *rms_w, float rms_eps);
-int gemv_rows_per_wg(int M, int K_pad);
-int gemv_threads_per_wg(int M, int K_pad);
-int gemv_lds_bytes(int K_pad);
+int gemv_rows_per_wg(int M, int K, int K_pad);
+int gemv_threads_per_wg(int M, int K, int K_pad);
+int gemv_grid_x(int M, int K, int K_pad);
+int gemv_step_codes(int M, int K, int K_pad);
+int gemv_lds_bytes(int M, int K, int K_pad);
 
 namespace {
 
@@ -144,16 +146,18 @@ void pick_split(int grid_x, int n_ktiles, int N, int have_ws, int *split, int *t
 int plan_impl(const chr_nf4_dev_t &h, int32_t N, int32_t have_ws, chr_nf4_plan_t *out) {
   chr_nf4_plan_t p{};
   if (N == 1) {
-    // Row-streaming GEMV: every wavefront walks whole rows, no split-K.
+    // Row-streaming GEMV: every wavefront walks whole rows, no split-K.  bm is the rows a
+    // workgroup covers per pass (the staged kernel, one workgroup per compute unit, makes
+    // ceil(M / bm / grid_x) passes).
     p.path = 1;
-    p.bm = gemv_rows_per_wg(h.M, h.K_pad);
-    p.bk = 2048;  // codes one wavefront load step covers
-    p.block = gemv_threads_per_wg(h.M, h.K_pad);
-    p.grid_x = ceil_div(h.M, p.bm);
+    p.bm = gemv_rows_per_wg(h.M, h.K, h.K_pad);
+    p.bk = gemv_step_codes(h.M, h.K, h.K_pad);
+    p.block = gemv_threads_per_wg(h.M, h.K, h.K_pad);
+    p.grid_x = gemv_grid_x(h.M, h.K, h.K_pad);
     p.grid_y = 1;
     p.n_ktiles = ceil_div(h.K_pad, p.bk);
     p.tiles_per_split = p.n_ktiles;
-    p.smem_bytes = gemv_lds_bytes(h.K_pad);
+    p.smem_bytes = gemv_lds_bytes(h.M, h.K, h.K_pad);
     p.ws_floats = 0;
   } else {
     p.path = N <= 16 ? 2 : (N <= 32 ? 3 : 4);

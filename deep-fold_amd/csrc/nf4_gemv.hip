@@ -1061,21 +1061,36 @@ int gemv_attn_entry(const chr_nf4_dev_t *w, const float *state, int n_q, int hd,
   return launch_rows(a, 1, w->M, static_cast<hipStream_t>(stream));
 }
 
-// Launch geometry of the N=1 path, reported by the planner.
-int gemv_rows_per_wg(int M, int K_pad) {
-  (void)K_pad;
-  return (kThreads / kWave) * rows_for_m(M);
+// Launch geometry of the N=1 path, reported by the planner: what chr_nf4_gemv launches for
+// this matrix without fused extras.
+bool gemv_plan_staged(int M, int K, int K_pad) {
+  StreamArgs a{};
+  a.K = K;
+  a.K_pad = K_pad;
+  return pick_family(a, M) == 1;
 }
 
-int gemv_threads_per_wg(int M, int K_pad) {
-  (void)M;
-  (void)K_pad;
-  return kThreads;
+int gemv_rows_per_wg(int M, int K, int K_pad) {
+  return gemv_plan_staged(M, K, K_pad) ? (kStagedThreads / kWave) * staged_rows_for_m(M)
+                                       : (kThreads / kWave) * rows_for_m(M);
 }
 
-int gemv_lds_bytes(int K_pad) {
-  (void)K_pad;
-  return static_cast<int>(sizeof(GemvLds));
+int gemv_threads_per_wg(int M, int K, int K_pad) {
+  return gemv_plan_staged(M, K, K_pad) ? kStagedThreads : kThreads;
+}
+
+int gemv_grid_x(int M, int K, int K_pad) {
+  const int bm = gemv_rows_per_wg(M, K, K_pad);
+  const int blocks = (M + bm - 1) / bm;
+  return gemv_plan_staged(M, K, K_pad) ? std::min(device_cu_count(), blocks) : blocks;
+}
+
+// codes of a row one wavefront request covers
+int gemv_step_codes(int M, int K, int K_pad) { return gemv_plan_staged(M, K, K_pad) ? 1024 : 2048; }
+
+int gemv_lds_bytes(int M, int K, int K_pad) {
+  return gemv_plan_staged(M, K, K_pad) ? static_cast<int>(staged_lds_bytes(K_pad))
+                                       : static_cast<int>(sizeof(GemvLds));
 }
 
 }  // namespace chr

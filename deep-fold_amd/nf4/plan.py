@@ -34,6 +34,9 @@ __all__ = [
     "Plan",
     "k_pad",
     "gemv_rows_per_wavefront",
+    "gemv_is_staged",
+    "staged_lds_bytes",
+    "STAGED_MIN_CODES",
     "plan",
 ]
 
@@ -80,10 +83,35 @@ def _ceil_div(a: int, b: int) -> int:
     return -(-int(a) // int(b))
 
 
-def gemv_rows_per_wavefront(m: int, forced: int = 0) -> int:
+#: The staged GEMV kernel (x and a 64 KB level-pair table in LDS, 1024-thread workgroups, one
+#: per compute unit) is taken from this many codes up, and whenever K is ragged.
+STAGED_MIN_CODES = 16 << 20
+_STAGED_TABLE_BYTES = 256 * 64 * 4
+_STAGED_SMALL_BYTES = 512
+_MAX_DYN_LDS = 150 * 1024
+
+
+def staged_lds_bytes(k_pad_: int) -> int:
+    """LDS of a staged GEMV launch: table, reduction scratch, x in 512-code half steps."""
+    half_steps = _ceil_div(int(k_pad_) // 16, 64)
+    return _STAGED_TABLE_BYTES + _STAGED_SMALL_BYTES + half_steps * 128 * 16
+
+
+def gemv_is_staged(m: int, k: int, k_pad_: int | None = None) -> bool:
+    """Kernel family ``chr_nf4_gemv`` takes for a plain launch (no fused norm)."""
+    kp = k_pad(k) if k_pad_ is None else int(k_pad_)
+    fits = staged_lds_bytes(kp) <= _MAX_DYN_LDS
+    if int(k) != kp:
+        return fits
+    return fits and int(m) * kp >= STAGED_MIN_CODES
+
+
+def gemv_rows_per_wavefront(m: int, forced: int = 0, staged: bool = False) -> int:
     """Rows one wavefront of the GEMV walks together (they share x)."""
     if forced in (1, 2, 4):
         return forced
+    if staged:
+        return 2 if m >= 32768 else 1
     if m >= 32768:
         return 4
     return 2 if m >= 4096 else 1
@@ -138,6 +166,13 @@ def plan(M: int, K: int, N: int = 1, *, K_pad: int | None = None, have_ws: bool 
     if kp != k_pad(K):
         raise ValueError(f"K_pad={kp} != 64*ceil(K/64) = {k_pad(K)}")
     if N == 1:
+        if gemv_is_staged(M, K, kp):
+            # one workgroup of 16 wavefronts per compute unit; bm = rows it covers per pass
+            bm = 16 * gemv_rows_per_wavefront(M, gemv_rows, staged=True)
+            n_ktiles = _ceil_div(kp, 1024)
+            grid_x = min(int(one_wave), _ceil_div(M, bm))
+            return Plan(GEMV, grid_x, 1, 1024, bm, 1024, n_ktiles, n_ktiles, grid_x,
+                        staged_lds_bytes(kp), 0)
         bm = 4 * gemv_rows_per_wavefront(M, gemv_rows)
         n_ktiles = _ceil_div(kp, 2048)
         grid_x = _ceil_div(M, bm)

@@ -5,6 +5,7 @@ from __future__ import annotations
 import numpy as np
 import torch
 
+from deepfold_amd.nf4 import plan as pyplan
 from oracle import nf4_oracle as oc
 
 DEV = "cuda"
@@ -51,15 +52,12 @@ def ulp_bf16(v: np.ndarray) -> np.ndarray:
     return 2.0 ** (e - 7)
 
 
-#: The staged GEMV (x in LDS: fused RMSNorm, ragged K, attention merge, and every matrix
-#: from 16M codes up) multiplies bf16-rounded levels, as the reference's tensor-core path
-#: does with the whole dequantised weight (gpu/nf4/nf4_gemm.cu:322).
-STAGED_MIN_CODES = 16 << 20
-
-
 def takes_staged_gemv(m: int, k: int, *, fused: bool = False) -> bool:
-    """Whether a GEMV launch of m rows takes the staged kernel (the library's policy)."""
-    return fused or k != oc.k_pad(k) or m * oc.k_pad(k) >= STAGED_MIN_CODES
+    """Whether a GEMV launch of m rows takes the staged kernel (x in LDS: fused RMSNorm,
+    ragged K, attention merge, and every matrix from 16M codes up).  That kernel multiplies
+    bf16-rounded levels, as the reference's tensor-core path does with the whole dequantised
+    weight (gpu/nf4/nf4_gemm.cu:322)."""
+    return fused or pyplan.gemv_is_staged(m, k)
 
 
 def staged_gemv_model(packed: np.ndarray, scale: np.ndarray, m: int, k: int,
