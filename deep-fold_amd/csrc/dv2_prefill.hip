@@ -77,7 +77,7 @@ __global__ __launch_bounds__(kColsBlock) void rms_cols(const uint16_t *__restric
     }
   }
   __syncthreads();
-  if (threadIdx.x < N) {
+  if (static_cast<int>(threadIdx.x) < N) {
     float t = 0.f;
     for (int i = 0; i < kColsWaves; ++i) {
       t += part[i][threadIdx.x];

@@ -75,7 +75,6 @@ constexpr int gemm_lds_bytes(int nb) {
   return 64 + kKHalves * nb * kBN * kXStride * 2 + kGemmWaves * kWStage +
          kGemmWaves * 32 * kGroupsPerTile * 2;
 }
-constexpr int kGemmLds = gemm_lds_bytes(1);
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -350,16 +349,6 @@ __device__ __forceinline__ void stash_w(const WRegs &r, uint8_t *wst, uint16_t *
         make_uint4(r.d[4 * j + 0], r.d[4 * j + 1], r.d[4 * j + 2], r.d[4 * j + 3]);
   }
   *reinterpret_cast<uint32_t *>(sst + (lane >> 1) * kGroupsPerTile + ((lane & 1) << 1)) = r.sc;
-}
-
-__device__ __forceinline__ bf16x8 dequant8(uint32_t w, float s, const float *lut) {
-  const Levels8 v = lookup8(w, lut);
-  bf16x8 a;
-#pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    a[j] = static_cast<__bf16>(v.l[j] * s);
-  }
-  return a;
 }
 
 // NB: 32-column blocks of the activation tile (1 for N <= 32, 2 for N <= 64); one

@@ -53,13 +53,6 @@ __device__ __forceinline__ float fma8(const Levels8 &v, const float *xf, float a
   return acc;
 }
 
-__device__ __forceinline__ float dot8(uint32_t w, const float4 xa, const float4 xb,
-                                      const float *lut, float acc) {
-  const Levels8 v = lookup8(w, lut);
-  const float xf[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
-  return fma8(v, xf, acc);
-}
-
 struct StreamArgs {
   // up to three row segments sharing x (one for a plain GEMV, three for q/k/v)
   const uint8_t *packed[3];
