@@ -10,7 +10,7 @@ import torch.nn.functional as F
 from deepfold_amd import nf4
 from oracle import nf4_oracle as oc
 
-from helpers import (DEV, bf16_bits, bf16_tensor, check_linear, rand_x, to_f32, ulp_bf16, up,
+from helpers import (DEV, MAX_REL, bf16_bits, bf16_tensor, check_linear, rand_x, to_f32, ulp_bf16, up,
                      up_scale, staged_gemv_model, takes_staged_gemv)
 
 pytestmark = pytest.mark.gpu
@@ -137,6 +137,37 @@ def test_gemv_toy_blobs(m, k):
     # same inputs, same bits
     y2 = nf4.nf4_gemv(dp, ds, bf16_tensor(x), m, k, oc.k_pad(k))
     assert (bf16_bits(y) == bf16_bits(y2)).all()
+
+
+@pytest.mark.parametrize("m,k", [(152064, 5120), (151936, 2048), (92544, 6144), (27648, 5120),
+                                 (5120, 13824), (5120, 27648)])
+def test_gemv_full_size_sampled_rows(m, k, monkeypatch):
+    """The vocabulary and FFN shapes of the benchmark architectures at full size: every
+    wavefront of the staged launch walks several row groups.  2048 sampled rows are held to
+    the full bounds (oracle, and the staged kernel's arithmetic written out on the CPU); all
+    rows must agree with the plain kernel on the same inputs."""
+    say("gemv full size", m, k)
+    gen = torch.Generator(device=DEV)
+    gen.manual_seed(m + k)
+    w = torch.randn((m, k), generator=gen, device=DEV, dtype=torch.float32) * 0.02
+    dp, ds = nf4.nf4_quantize(w)
+    del w
+    x = rand_x(k, None, 21)
+    dx = bf16_tensor(x)
+    assert takes_staged_gemv(m, k)
+    y = nf4.nf4_gemv(dp, ds, dx, m, k, k)
+    monkeypatch.setenv("CHR_NF4_GEMV_STAGED", "0")
+    y0 = nf4.nf4_gemv(dp, ds, dx, m, k, k)
+    a, b = to_f32(y).reshape(-1), to_f32(y0).reshape(-1)
+    assert np.abs(a - b).max() <= MAX_REL * np.abs(b).max()
+    rows = np.sort(np.random.default_rng(5).choice(m, 2048, replace=False))
+    idx = torch.from_numpy(rows).to(DEV)
+    p = dp.view(m, -1)[idx].cpu().numpy()
+    sc = ds.view(m, -1)[idx].cpu().numpy()
+    ref = oc.c_matmul_f64(oc.c_decode(p, sc, len(rows), k), x[:, None])
+    check_linear(y.view(-1)[idx], ref, what=f"staged {m}x{k}, sampled rows",
+                 model=staged_gemv_model(p, sc, len(rows), k, x))
+    check_linear(y0.view(-1)[idx], ref, what=f"plain {m}x{k}, sampled rows")
 
 
 def test_gemv_pad_codes_do_not_matter():
