@@ -13,10 +13,13 @@ constexpr int kColsBlock = 1024;
 constexpr int kColsWaves = kColsBlock / kWave;
 constexpr int kMaxCols = 64;
 
-// y[k][n] = bf16( (w[k] * x[k][n]) * rsqrt(mean_k x[k][n]^2 + eps) ).  Every workgroup sums the
-// squares of the whole tile itself (it is a few hundred KB and sits in L2; all workgroups add in
-// one order, so all hold the same bits) and then normalises its own slice of rows: one launch,
-// no cross-workgroup hand-over.
+// y[k][n] = bf16( (w[k] * x[k][n]) * rsqrt(mean_k x[k][n]^2 + eps) ).  Every workgroup needs the
+// column sums of squares of the whole tile and then normalises its own slice of rows: one
+// launch, no cross-workgroup hand-over.  The sums come from one of two places:
+//   sq == nullptr: the workgroup reads the whole tile itself (a few hundred KB, in L2; all
+//                  workgroups add in one order, so all hold the same bits);
+//   sq != nullptr: the launch that stored x left sums per block of rows, sq[sq_blocks][N]
+//                  (chr_dv2_gemm_add_sq), and only those are added.  N divides 1024 then.
 //
 // Thread t owns column t % CP of rows t / CP, t / CP + 1024 / CP, ..; CP is N rounded up to a
 // power of two, threads whose column is >= N idle.  VEC: N is 8, 16, 32 or 64 and rows are 16-byte
@@ -25,7 +28,9 @@ template <bool VEC>
 __global__ __launch_bounds__(kColsBlock) void rms_cols(const uint16_t *__restrict__ x,
                                                        const uint16_t *__restrict__ w,
                                                        uint16_t *__restrict__ y, int rows, int N,
-                                                       int cp, float eps, int rows_per_wg) {
+                                                       int cp, float eps, int rows_per_wg,
+                                                       const float *__restrict__ sq,
+                                                       int sq_blocks) {
   __shared__ float part[kColsWaves][kMaxCols];
   __shared__ float inv[kMaxCols];
   const int lane = threadIdx.x & (kWave - 1);
@@ -36,47 +41,68 @@ __global__ __launch_bounds__(kColsBlock) void rms_cols(const uint16_t *__restric
   const int r0 = threadIdx.x / tpr;
   const int rstep = kColsBlock / tpr;
   const bool live = col < N;
-  float ss[W];
-#pragma unroll
-  for (int i = 0; i < W; ++i) {
-    ss[i] = 0.f;
-  }
-  if (live) {
-#pragma unroll 4
-    for (int k = r0; k < rows; k += rstep) {
-      const uint16_t *p = x + static_cast<size_t>(k) * N + col;
-      if (VEC) {
-        const uint4 v = *reinterpret_cast<const uint4 *>(p);
-        const uint32_t d[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float lo = bf16_lo(d[i]);
-          const float hi = bf16_hi(d[i]);
-          ss[2 * i] = fmaf(lo, lo, ss[2 * i]);
-          ss[2 * i + 1] = fmaf(hi, hi, ss[2 * i + 1]);
-        }
-      } else {
-        const float v = bf16_to_f32(*p);
-        ss[0] = fmaf(v, v, ss[0]);
+  if (sq != nullptr) {
+    // thread t adds the blocks t / N, t / N + 1024 / N, .. of column t % N; the 1024 / N
+    // partial sums of a column meet in the 16 rows of part[], folded in a fixed order
+    const int scol = threadIdx.x % N;
+    const int sub = threadIdx.x / N;
+    const int nsub = kColsBlock / N;         // 16 .. 128
+    const int fold = nsub / kColsWaves;      // partial sums per row of part[]
+    float t = 0.f;
+#pragma unroll 8
+    for (int b = sub; b < sq_blocks; b += nsub) {
+      t += sq[static_cast<size_t>(b) * N + scol];
+    }
+    for (int f = 0; f < fold; ++f) {
+      if (sub % fold == f) {
+        float *slot = &part[sub / fold][scol];
+        *slot = f == 0 ? t : *slot + t;
       }
+      __syncthreads();
     }
-  }
-  // lanes that share a column sit tpr apart: fold the wavefront down to its first tpr lanes
-#pragma unroll
-  for (int i = 0; i < W; ++i) {
-    for (int off = kWave / 2; off >= tpr; off >>= 1) {
-      ss[i] += __shfl_down(ss[i], off, kWave);
-    }
-  }
-  if (lane < tpr) {
+  } else {
+    float ss[W];
 #pragma unroll
     for (int i = 0; i < W; ++i) {
-      if (lane * W + i < kMaxCols) {
-        part[wave][lane * W + i] = ss[i];
+      ss[i] = 0.f;
+    }
+    if (live) {
+#pragma unroll 4
+      for (int k = r0; k < rows; k += rstep) {
+        const uint16_t *p = x + static_cast<size_t>(k) * N + col;
+        if (VEC) {
+          const uint4 v = *reinterpret_cast<const uint4 *>(p);
+          const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float lo = bf16_lo(d[i]);
+            const float hi = bf16_hi(d[i]);
+            ss[2 * i] = fmaf(lo, lo, ss[2 * i]);
+            ss[2 * i + 1] = fmaf(hi, hi, ss[2 * i + 1]);
+          }
+        } else {
+          const float v = bf16_to_f32(*p);
+          ss[0] = fmaf(v, v, ss[0]);
+        }
       }
     }
+    // lanes that share a column sit tpr apart: fold the wavefront down to its first tpr lanes
+#pragma unroll
+    for (int i = 0; i < W; ++i) {
+      for (int off = kWave / 2; off >= tpr; off >>= 1) {
+        ss[i] += __shfl_down(ss[i], off, kWave);
+      }
+    }
+    if (lane < tpr) {
+#pragma unroll
+      for (int i = 0; i < W; ++i) {
+        if (lane * W + i < kMaxCols) {
+          part[wave][lane * W + i] = ss[i];
+        }
+      }
+    }
+    __syncthreads();
   }
-  __syncthreads();
   if (static_cast<int>(threadIdx.x) < N) {
     float t = 0.f;
     for (int i = 0; i < kColsWaves; ++i) {
@@ -222,8 +248,11 @@ __global__ __launch_bounds__(256) void add_cols(uint16_t *__restrict__ y,
 
 using namespace chr;
 
-extern "C" int chr_dv2_rms_cols(const void *x, const void *w, void *y, int32_t rows, int32_t N,
-                                float eps, void *stream) {
+namespace chr {
+namespace {
+
+int rms_cols_launch(const void *x, const void *w, void *y, int32_t rows, int32_t N, float eps,
+                    const float *sq, int32_t sq_blocks, void *stream) {
   if (x == nullptr || w == nullptr || y == nullptr) {
     return -1;
   }
@@ -231,6 +260,9 @@ extern "C" int chr_dv2_rms_cols(const void *x, const void *w, void *y, int32_t r
     return -3;
   }
   if (N < 1 || N > kMaxCols) {
+    return -2;
+  }
+  if (sq != nullptr && (kColsBlock % N != 0 || kColsBlock / N < kColsWaves || sq_blocks < 1)) {
     return -2;
   }
   const bool vec = (N == 8 || N == 16 || N == 32 || N == 64) && aligned16(x) && aligned16(y);
@@ -246,13 +278,29 @@ extern "C" int chr_dv2_rms_cols(const void *x, const void *w, void *y, int32_t r
   if (vec) {
     rms_cols<true><<<grid, dim3(kColsBlock), 0, st>>>(
         static_cast<const uint16_t *>(x), static_cast<const uint16_t *>(w),
-        static_cast<uint16_t *>(y), rows, N, cp, eps, rows_per_wg);
+        static_cast<uint16_t *>(y), rows, N, cp, eps, rows_per_wg, sq, sq_blocks);
   } else {
     rms_cols<false><<<grid, dim3(kColsBlock), 0, st>>>(
         static_cast<const uint16_t *>(x), static_cast<const uint16_t *>(w),
-        static_cast<uint16_t *>(y), rows, N, cp, eps, rows_per_wg);
+        static_cast<uint16_t *>(y), rows, N, cp, eps, rows_per_wg, sq, sq_blocks);
   }
   return launch_rc();
+}
+
+}  // namespace
+}  // namespace chr
+
+extern "C" int chr_dv2_rms_cols(const void *x, const void *w, void *y, int32_t rows, int32_t N,
+                                float eps, void *stream) {
+  return rms_cols_launch(x, w, y, rows, N, eps, nullptr, 0, stream);
+}
+
+extern "C" int chr_dv2_rms_cols_sq(const void *x, const void *w, void *y, int32_t rows, int32_t N,
+                                   float eps, const float *sq, int32_t sq_blocks, void *stream) {
+  if (sq == nullptr) {
+    return -1;
+  }
+  return rms_cols_launch(x, w, y, rows, N, eps, sq, sq_blocks, stream);
 }
 
 extern "C" int chr_dv2_rope_kv_cols(const void *q, const void *k, const void *v, void *q_out,

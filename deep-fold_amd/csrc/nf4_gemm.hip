@@ -519,6 +519,50 @@ __global__ __launch_bounds__(256) void reduce_splitk(const float *__restrict__ p
   y[i] = v;
 }
 
+// reduce_splitk that also leaves, for the RMSNorm that reads y next, the column sums of
+// squares of what it stored: sq[b][n] = sum over the rows of block b of y[row][n]^2, taken
+// from the bf16 values as stored.  A block is 1024 elements (1024 / N rows), one per thread as
+// in reduce_splitk (fewer threads with more elements each were three times slower: the sums
+// over the splits are chains of dependent loads).  N divides 256, so the threads of a column
+// sit N apart; they are added in thread order (deterministic).
+constexpr int kSqElems = 1024;  // elements of y per block of the sums = threads of a block
+
+__global__ __launch_bounds__(kSqElems) void reduce_splitk_sq(const float *__restrict__ partial,
+                                                             uint16_t *__restrict__ y, int rows,
+                                                             int split, int N,
+                                                             const uint16_t *__restrict__ bias,
+                                                             const uint16_t *res,
+                                                             float *__restrict__ sq) {
+  __shared__ float part[kSqElems];
+  const int i = blockIdx.x * kSqElems + threadIdx.x;
+  float sqv = 0.f;
+  if (i < rows) {
+    float s = 0.f;
+    for (int j = 0; j < split; ++j) {
+      s += partial[static_cast<size_t>(j) * rows + i];
+    }
+    uint16_t v = f32_to_bf16(s);
+    if (bias != nullptr) {
+      v = f32_to_bf16(bf16_to_f32(v) + bf16_to_f32(bias[i / N]));
+    }
+    if (res != nullptr) {
+      v = f32_to_bf16(bf16_to_f32(res[i]) + bf16_to_f32(v));
+    }
+    y[i] = v;
+    const float f = bf16_to_f32(v);
+    sqv = f * f;
+  }
+  part[threadIdx.x] = sqv;
+  __syncthreads();
+  if (static_cast<int>(threadIdx.x) < N) {
+    float t = 0.f;
+    for (int k = threadIdx.x; k < kSqElems; k += N) {
+      t += part[k];
+    }
+    sq[static_cast<size_t>(blockIdx.x) * N + threadIdx.x] = t;
+  }
+}
+
 // Gate rows stacked over up rows: y[i] = silu(bf16 gate) * bf16 up with the roundings of the
 // reference's separate ops (F.silu on bf16, then a bf16 product; gpu/decodev2/ops.py:23-24).
 __global__ __launch_bounds__(256) void reduce_swiglu(const float *__restrict__ partial,
@@ -618,7 +662,8 @@ StackPlan plan_stack(const chr_nf4_dev_t *h, int nseg, int N, int have_ws) {
 // w[0..nseg) share K and x; y, bias and res cover the stacked rows.
 int gemm_launch(const chr_nf4_dev_t *const *w, int nseg, const void *x, void *y, int32_t N,
                 float *ws, int64_t ws_floats, void *stream, int32_t max_n, const void *bias,
-                const void *res, int32_t live_max = kLiveMaxN, bool swiglu = false) {
+                const void *res, int32_t live_max = kLiveMaxN, bool swiglu = false,
+                float *colsq = nullptr) {
   if (x == nullptr || y == nullptr) {
     return -1;
   }
@@ -701,10 +746,17 @@ int gemm_launch(const chr_nf4_dev_t *const *w, int nseg, const void *x, void *y,
         partial, yp, half_rows, sp.grid_y);
   } else if (partial != nullptr) {
     const int rows = sp.M_all * N;
+    if (colsq != nullptr && 256 % N == 0) {
+      reduce_splitk_sq<<<dim3(static_cast<unsigned>(ceil_div(rows, kSqElems))), dim3(kSqElems),
+                         0, st>>>(partial, yp, rows, sp.grid_y, N, bp, rp, colsq);
+      return launch_rc();
+    }
     reduce_splitk<<<dim3(static_cast<unsigned>(ceil_div(rows, 256))), dim3(256), 0, st>>>(
         partial, yp, rows, sp.grid_y, N, bp, rp);
   }
-  return launch_rc();
+  const int rc = launch_rc();
+  // a caller that asked for the column sums learns that this launch did not write them
+  return rc == 0 && colsq != nullptr ? 1 : rc;
 }
 
 }  // namespace
@@ -719,6 +771,20 @@ extern "C" int chr_dv2_gemm_add(const chr_nf4_dev_t *w, const void *x, void *y, 
                                 float *ws, int64_t ws_floats, const void *bias,
                                 const void *residual, void *stream) {
   return gemm_launch(&w, 1, x, y, N, ws, ws_floats, stream, kPlanMaxN, bias, residual, kPlanMaxN);
+}
+
+extern "C" int chr_dv2_gemm_add_sq(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N,
+                                   float *ws, int64_t ws_floats, const void *bias,
+                                   const void *residual, float *colsq, void *stream) {
+  if (colsq == nullptr) {
+    return -1;
+  }
+  return gemm_launch(&w, 1, x, y, N, ws, ws_floats, stream, kPlanMaxN, bias, residual, kPlanMaxN,
+                     false, colsq);
+}
+
+extern "C" int32_t chr_dv2_sq_rows(int32_t N) {
+  return N >= 1 && N <= kSqElems && kSqElems % N == 0 ? kSqElems / N : 0;
 }
 
 extern "C" int64_t chr_dv2_gemm_qkv_ws(const chr_nf4_dev_t *q, const chr_nf4_dev_t *k,

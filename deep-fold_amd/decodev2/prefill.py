@@ -13,7 +13,7 @@ from __future__ import annotations
 import torch
 
 from ..nf4 import (LIVE_MAX_N, PLAN_MAX_N, dv2_add_cols, dv2_attn_chunk, dv2_gemm_qkv, dv2_gemm_swiglu,
-                   dv2_rms_cols, dv2_rope_kv_cols, dv2_swiglu_elems, nf4_gemm)
+                   dv2_rms_cols, dv2_rope_kv_cols, dv2_sq_blocks, dv2_swiglu_elems, nf4_gemm)
 from .embed import gather_embed
 from .linear import DeviceLinear, DeviceWeights, nf4_linear
 from .ops import causal_attend, rms, split_qkv, swiglu
@@ -63,11 +63,16 @@ def forward_prefill(state: DecodeState, weights: DeviceWeights, token_ids: torch
     state.pick_next(commit=False)
 
 
-def _gemm_cols(mat: DeviceLinear, x: torch.Tensor, residual: torch.Tensor | None = None) -> torch.Tensor:
+def _gemm_cols(mat: DeviceLinear, x: torch.Tensor, residual: torch.Tensor | None = None,
+               colsq: torch.Tensor | None = None):
     """``[K, N] -> [M, N]`` with the bias, if any, added per row; with ``residual`` the
     result is added to it in place.  One column (a one-token chunk) goes to the GEMV and
-    takes its bias and residual from separate launches."""
+    takes its bias and residual from separate launches.  With ``colsq`` the return value is
+    whether the launch left the result's column sums of squares there."""
     if x.size(1) >= 2:
+        if colsq is not None:
+            return nf4_gemm(mat.packed, mat.scale, x, mat.M, mat.K, mat.K_pad, int(PLAN_MAX_N),
+                            bias=mat.bias, residual=residual, colsq=colsq)[1]
         return nf4_gemm(mat.packed, mat.scale, x, mat.M, mat.K, mat.K_pad, int(PLAN_MAX_N),
                         bias=mat.bias, residual=residual)
     y = nf4_gemm(mat.packed, mat.scale, x, mat.M, mat.K, mat.K_pad)
@@ -75,8 +80,8 @@ def _gemm_cols(mat: DeviceLinear, x: torch.Tensor, residual: torch.Tensor | None
         dv2_add_cols(y, bias=mat.bias)
     if residual is not None:
         dv2_add_cols(residual, y)
-        return residual
-    return y
+        return False if colsq is not None else residual
+    return False if colsq is not None else y
 
 
 class ChunkPrefill:
@@ -106,6 +111,9 @@ class ChunkPrefill:
         self.start = torch.zeros((), dtype=torch.int64, device=dev)
         self.first_len = torch.zeros((), dtype=torch.int32, device=dev)
         self.last_hidden = torch.zeros(spec.hidden, dtype=torch.bfloat16, device=dev)
+        # column sums of squares of the residual stream, left by the launch that last wrote it
+        self._colsq = torch.zeros(dv2_sq_blocks(spec.hidden, self.MAX_WIDTH) * self.MAX_WIDTH,
+                                  dtype=torch.float32, device=dev)
         self._graphs: dict[int, torch.cuda.CUDAGraph] = {}
         # stacked q/k/v biases for the one-launch q/k/v GEMM (zeros where a matrix has none)
         self._qkv_bias: list[torch.Tensor | None] = []
@@ -123,8 +131,9 @@ class ChunkPrefill:
         x = gather_embed(weights.embed, self.ids[:n]).t().contiguous()  # [hidden, n]
         q_rows = torch.empty((n, spec.q_dim), dtype=torch.bfloat16, device=x.device)
         attn = torch.empty((spec.q_dim, n), dtype=torch.bfloat16, device=x.device)
+        sq = None  # self._colsq while it holds x's sums (the embedding gather leaves none)
         for li, layer in enumerate(weights.layers):
-            h = dv2_rms_cols(x, layer.norm1, spec.rms_eps)
+            h = dv2_rms_cols(x, layer.norm1, spec.rms_eps, colsq=sq)
             if layer.wqkv is not None:
                 y = _gemm_cols(layer.wqkv, h)  # rows are [Q | K | V]
                 q, k, v = y[:spec.q_dim], y[spec.q_dim:spec.q_dim + spec.kv_dim], y[spec.q_dim + spec.kv_dim:]
@@ -137,14 +146,14 @@ class ChunkPrefill:
             k_cache, v_cache = state.kv.layer(li)
             dv2_rope_kv_cols(q, k, v, q_rows, k_cache, v_cache, state.cos, state.sin, self.start)
             dv2_attn_chunk(q_rows, k_cache, v_cache, attn, self.first_len, spec.attn_scale)
-            _gemm_cols(layer.o, attn, residual=x)
-            h = dv2_rms_cols(x, layer.norm2, spec.rms_eps)
+            sq = self._colsq if _gemm_cols(layer.o, attn, residual=x, colsq=self._colsq) else None
+            h = dv2_rms_cols(x, layer.norm2, spec.rms_eps, colsq=sq)
             if n >= 2 and layer.gate.bias is None and layer.up.bias is None:
                 act = dv2_gemm_swiglu((layer.gate.packed, layer.gate.scale, layer.gate.M),
                                       (layer.up.packed, layer.up.scale, layer.up.M), h)
             else:
                 act = dv2_swiglu_elems(_gemm_cols(layer.gate, h), _gemm_cols(layer.up, h))
-            _gemm_cols(layer.down, act, residual=x)
+            sq = self._colsq if _gemm_cols(layer.down, act, residual=x, colsq=self._colsq) else None
         self.last_hidden.copy_(x[:, n - 1])
 
     def _replay(self, n: int) -> None:

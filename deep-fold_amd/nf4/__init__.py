@@ -50,6 +50,7 @@ __all__ = [
     "dv2_gemv_attn",
     "dv2_attn",
     "dv2_rms_cols",
+    "dv2_sq_blocks",
     "dv2_rope_kv_cols",
     "dv2_attn_chunk",
     "dv2_swiglu_elems",
@@ -133,6 +134,9 @@ EXPORTS = (
     ("chr_dv2_swiglu_elems", ctypes.c_int, [_P, _P, _P, ctypes.c_int64, _P]),
     ("chr_dv2_add_cols", ctypes.c_int, [_P, _P, _P, _I, _I, _P]),
     ("chr_dv2_gemm_add", ctypes.c_int, [_DP, _P, _P, _I, _P, ctypes.c_int64, _P, _P, _P]),
+    ("chr_dv2_gemm_add_sq", ctypes.c_int, [_DP, _P, _P, _I, _P, ctypes.c_int64, _P, _P, _P, _P]),
+    ("chr_dv2_sq_rows", ctypes.c_int32, [_I]),
+    ("chr_dv2_rms_cols_sq", ctypes.c_int, [_P, _P, _P, _I, _I, ctypes.c_float, _P, _I, _P]),
     ("chr_dv2_gemm_qkv_ws", ctypes.c_int64, [_DP, _DP, _DP, _I]),
     ("chr_dv2_gemm_qkv", ctypes.c_int, [_DP, _DP, _DP, _P, _P, _I, _P, ctypes.c_int64, _P, _P]),
     ("chr_dv2_gemm_swiglu_ws", ctypes.c_int64, [_DP, _DP, _I]),
@@ -273,12 +277,17 @@ def nf4_set_tuning(path: int = 0, split_k: int = 0, one_wave: int = 0) -> None:
 
 def nf4_gemm(packed: torch.Tensor, scale: torch.Tensor, x: torch.Tensor, M: int, K: int,  # noqa: N803
              K_pad: int, max_n: int = LIVE_MAX_N, *, bias: torch.Tensor | None = None,  # noqa: N803
-             residual: torch.Tensor | None = None) -> torch.Tensor:
+             residual: torch.Tensor | None = None, colsq: torch.Tensor | None = None):
     """Fused NF4 dequant-MFMA GEMM.  ``x`` is bf16 ``[K, N]`` or ``[K]``; returns
     ``y [M, N]`` (``gpu/nf4/__init__.py:151-176``, ``bindings.cpp:35-97``).  With
     ``bias`` (bf16 ``[M]``) and/or ``residual`` (bf16 ``[M, N]``, N >= 2) the result is
     ``residual + (y + bias)``, written over ``residual``, in the same launches.  With
-    ``max_n=64`` chunks of 33..64 columns run too (one pass over the weights)."""
+    ``max_n=64`` chunks of 33..64 columns run too (one pass over the weights).
+
+    With ``colsq`` (fp32, at least ``dv2_sq_blocks(M, N) * N`` elements, N >= 2) the return
+    value is ``(y, written)``: ``written`` says whether the launch left the column sums of
+    squares of ``y`` there for ``dv2_rms_cols(..., colsq=)`` (it does when it has a split-K
+    reduction and N divides 256)."""
     n = 1 if x.dim() == 1 else int(x.size(-1))
     cap = int(max_n)
     if cap < 1 or cap > PLAN_MAX_N:
@@ -307,7 +316,7 @@ def nf4_gemm(packed: torch.Tensor, scale: torch.Tensor, x: torch.Tensor, M: int,
     if p.ws_floats > 0:
         ws = torch.empty(int(p.ws_floats), dtype=torch.float32, device=x.device)
         ws_ptr = ws.data_ptr()
-    if bias is None and residual is None and not wide:
+    if bias is None and residual is None and not wide and colsq is None:
         rc = lib.chr_nf4_gemm_ws_max(ctypes.byref(w), x.data_ptr(), y.data_ptr(), n, ws_ptr,
                                      int(p.ws_floats), _stream(), cap)
         _check_rc("chr_nf4_gemm", rc)
@@ -318,11 +327,30 @@ def nf4_gemm(packed: torch.Tensor, scale: torch.Tensor, x: torch.Tensor, M: int,
                             and t.numel() == numel), f"{name} must be contiguous CUDA bf16 of {numel} elements")
     if residual is not None:
         y = residual.view(M, n)
+    if colsq is not None:
+        _need(colsq.is_cuda and colsq.dtype == torch.float32 and colsq.is_contiguous()
+              and colsq.numel() >= dv2_sq_blocks(M, n) * n, "colsq must be contiguous CUDA fp32 of "
+              f"{dv2_sq_blocks(M, n) * n} elements")
+        rc = lib.chr_dv2_gemm_add_sq(ctypes.byref(w), x.data_ptr(), y.data_ptr(), n, ws_ptr,
+                                     int(p.ws_floats), None if bias is None else bias.data_ptr(),
+                                     None if residual is None else residual.data_ptr(),
+                                     colsq.data_ptr(), _stream())
+        if rc not in (0, 1):
+            _check_rc("chr_dv2_gemm_add_sq", rc)
+        return y, rc == 0
     rc = lib.chr_dv2_gemm_add(ctypes.byref(w), x.data_ptr(), y.data_ptr(), n, ws_ptr, int(p.ws_floats),
                               None if bias is None else bias.data_ptr(),
                               None if residual is None else residual.data_ptr(), _stream())
     _check_rc("chr_dv2_gemm_add", rc)
     return y
+
+
+def dv2_sq_blocks(rows: int, n: int) -> int:
+    """Row blocks whose column sums of squares ``nf4_gemm(..., colsq=)`` leaves for an
+    ``[rows, n]`` result: ``rows`` over 1024 / n rows per block, so ``blocks * n`` is at most
+    ``rows * n * n / 1024 + n`` elements; 0 when ``n`` does not divide 1024."""
+    per = int(_load_ext().chr_dv2_sq_rows(int(n)))
+    return -(-int(rows) // per) if per > 0 else 0
 
 
 def nf4_gemv(packed: torch.Tensor, scale: torch.Tensor, x: torch.Tensor, M: int, K: int,  # noqa: N803
@@ -764,8 +792,11 @@ def _bf16_cuda(t: torch.Tensor, what: str) -> None:
           f"{what} must be a contiguous CUDA bfloat16 tensor")
 
 
-def dv2_rms_cols(x: torch.Tensor, w: torch.Tensor, eps: float, out: torch.Tensor | None = None) -> torch.Tensor:
-    """RMSNorm of every column of feature-major ``x [rows, N]`` (N <= 64)."""
+def dv2_rms_cols(x: torch.Tensor, w: torch.Tensor, eps: float, out: torch.Tensor | None = None,
+                 colsq: torch.Tensor | None = None) -> torch.Tensor:
+    """RMSNorm of every column of feature-major ``x [rows, N]`` (N <= 64).  ``colsq``: the
+    column sums of squares the launch that produced ``x`` left (``nf4_gemm(..., colsq=)``
+    returned ``written``); the tile is then not read a second time for them."""
     _bf16_cuda(x, "x")
     _bf16_cuda(w, "w")
     _need(x.dim() == 2 and w.numel() == x.size(0), "x must be [rows, N] and w hold rows elements")
@@ -773,6 +804,14 @@ def dv2_rms_cols(x: torch.Tensor, w: torch.Tensor, eps: float, out: torch.Tensor
         out = torch.empty_like(x)
     _bf16_cuda(out, "out")
     _need(out.shape == x.shape, "out must have x's shape")
+    if colsq is not None:
+        blocks = dv2_sq_blocks(x.size(0), x.size(1))
+        _need(blocks > 0 and colsq.is_cuda and colsq.dtype == torch.float32 and colsq.is_contiguous()
+              and colsq.numel() >= blocks * x.size(1), "colsq does not cover x")
+        rc = _load_ext().chr_dv2_rms_cols_sq(x.data_ptr(), w.data_ptr(), out.data_ptr(), int(x.size(0)),
+                                             int(x.size(1)), float(eps), colsq.data_ptr(), blocks, _stream())
+        _check_rc("chr_dv2_rms_cols_sq", rc)
+        return out
     rc = _load_ext().chr_dv2_rms_cols(x.data_ptr(), w.data_ptr(), out.data_ptr(), int(x.size(0)),
                                       int(x.size(1)), float(eps), _stream())
     _check_rc("chr_dv2_rms_cols", rc)

@@ -219,6 +219,12 @@ int chr_dv2_gemv_attn(const chr_nf4_dev_t *w, const float *state, int32_t n_q, i
 int chr_dv2_rms_cols(const void *x, const void *w, void *y, int32_t rows, int32_t N, float eps,
                      void *stream);
 
+/* chr_dv2_rms_cols with the column sums of squares supplied (what chr_dv2_gemm_add_sq left for
+ * this x: sq[sq_blocks * N]) instead of read from the tile.  N must divide 1024.
+ * No reference counterpart. */
+int chr_dv2_rms_cols_sq(const void *x, const void *w, void *y, int32_t rows, int32_t N, float eps,
+                        const float *sq, int32_t sq_blocks, void *stream);
+
 /* Rotate-half RoPE of q [n_q*hd, N] and k [n_kv*hd, N] at positions *start + n
  * (start: device int64), writing rotated q token-major to q_out [N, n_q*hd] and rotated k
  * and v to cache rows *start + n of [max_seq, n_kv, hd] (gpu/decodev2/prefill.py:100-108).
@@ -258,6 +264,20 @@ int chr_dv2_add_cols(void *y, const void *a, const void *bias, int32_t rows, int
  * No reference counterpart. */
 int chr_dv2_gemm_add(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N, float *ws,
                      int64_t ws_floats, const void *bias, const void *residual, void *stream);
+
+/* chr_dv2_gemm_add that also leaves, for the RMSNorm that reads y next, the column sums of
+ * squares of the values it stored: with R = chr_dv2_sq_rows(N) = 1024 / N rows per block,
+ * colsq[b * N + n] = sum over rows R b .. R b + R - 1 of y[row][n]^2 (fp32,
+ * ceil(M / R) * N elements, no NULL).  The sums are taken in the split-K reduction, so they
+ * exist only when the launch has one and N divides 256: returns 0 when colsq was written, 1
+ * when the product was computed but colsq was not (the caller then normalises with
+ * chr_dv2_rms_cols), a negative code as chr_dv2_gemm_add.  chr_dv2_sq_rows gives 0 for an N
+ * that does not divide 1024.  No reference counterpart (the reference's prefill normalises
+ * with a torch op, gpu/decodev2/prefill.py:58-133). */
+int chr_dv2_gemm_add_sq(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N, float *ws,
+                        int64_t ws_floats, const void *bias, const void *residual, float *colsq,
+                        void *stream);
+int32_t chr_dv2_sq_rows(int32_t N);
 
 /* q, k and v of one layer in one launch (the prefill twin of chr_nf4_gemv_qkv,
  * gpu/decodev2/ops.py:27-35 calls three GEMMs): the three matrices share x [K, N] and K; y is

@@ -207,6 +207,44 @@ def test_gemm_with_bias_and_residual_in_its_reduction(m, k, n):
         nf4.nf4_gemm(dp, ds, x[:, :1].contiguous(), m, k, kp, bias=bias)
 
 
+@pytest.mark.parametrize("m,k,n", [(5120, 5120, 64), (5120, 13824, 32), (2050, 1088, 16), (130, 5120, 8),
+                                   (5120, 5120, 40), (256, 128, 64)])
+def test_gemm_leaves_column_sums_for_the_norm(m, k, n):
+    """The split-K reduce that stores y also leaves y's column sums of squares per block of
+    rows; the RMSNorm that takes them gives what the one that reads the tile gives."""
+    say("gemm_add_sq", m, k, n)
+    rng = np.random.default_rng(m + k + n)
+    p, s_ = oc.c_encode((rng.standard_normal((m, k)) * 0.05).astype(np.float32))
+    dp, ds = up(p), up_scale(s_)
+    kp = p.shape[1] * 2
+    x = bf16_tensor(rnd((k, n), 1))
+    res = rnd((m, n), 3, 2.0)
+    blocks = nf4.dv2_sq_blocks(m, n)
+    per = 1024 // n if 1024 % n == 0 else 0
+    colsq = torch.full((max(1, blocks) * n,), float("nan"), dtype=torch.float32, device=DEV)
+    r0 = bf16_tensor(res)
+    want = nf4.nf4_gemm(dp, ds, x, m, k, kp, 64, residual=r0)
+    r1 = bf16_tensor(res)
+    got, written = nf4.nf4_gemm(dp, ds, x, m, k, kp, 64, residual=r1, colsq=colsq)
+    assert (bf16_bits(got) == bf16_bits(want)).all()  # same product, same roundings
+    split = nf4.nf4_plan(m, k, n)["grid_y"]
+    assert written == (split > 1 and 256 % n == 0), (written, split)
+    if not written:
+        return
+    y = to_f32(got).astype(np.float64)
+    sq = colsq[: blocks * n].view(blocks, n).double().cpu().numpy()
+    for b in (0, blocks // 2, blocks - 1):
+        ref = (y[per * b: per * b + per] ** 2).sum(axis=0)
+        assert np.abs(sq[b] - ref).max() <= 1e-5 * max(1.0, ref.max()), b
+    w = bf16_tensor(rnd((m,), 4))
+    a = nf4.dv2_rms_cols(got, w, 1e-6)
+    b_ = nf4.dv2_rms_cols(got, w, 1e-6, colsq=colsq)
+    # the two sums differ in order only: at most one bf16 step where a value sits on a tie
+    da = np.abs(to_f32(a) - to_f32(b_))
+    assert (da <= 2 ** -7 * np.maximum(np.abs(to_f32(a)), 2.0 ** -20)).all()
+    assert (da > 0).mean() < 0.01
+
+
 @pytest.mark.parametrize("m,k,n", [(256, 512, 64), (130, 1088, 33), (5120, 5120, 64), (384, 256, 40),
                                    (13824, 5120, 48)])
 def test_wide_chunk_equals_two_narrow_ones(m, k, n):
