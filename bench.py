@@ -145,7 +145,8 @@ def bench_prefill(torch, nf4):
     return rows
 
 
-def bench_decode(torch, spec_name: str, prompt_len: int, new_tokens: int, schedule: str | None = None):
+def bench_decode(torch, spec_name: str, prompt_len: int, new_tokens: int, schedule: str | None = None,
+                 prefill_width: int | None = None):
     """Resident greedy decode on random-init weights: chunked prefill of a random
     prompt, then ``new_tokens`` graph replays with no host read in between."""
     from deepfold_amd import decodev2 as dv2
@@ -169,7 +170,8 @@ def bench_decode(torch, spec_name: str, prompt_len: int, new_tokens: int, schedu
     dv2.consume_prompt(state, weights, prompt)
     torch.cuda.synchronize()
     prefill_glue_ms = (time.perf_counter() - t0) * 1e3
-    pre = dv2.ChunkPrefill(state, weights)
+    pre = dv2.ChunkPrefill(state, weights, width=prefill_width)
+    width = pre.width
     state.reset()
     dv2.consume_prompt(state, weights, prompt, prefill=pre)
     state.reset()
@@ -213,7 +215,7 @@ def bench_decode(torch, spec_name: str, prompt_len: int, new_tokens: int, schedu
         "new_tokens": new_tokens, "context_start": start_pos, "context_end": end_pos,
         "tok_s": 1e3 / ms_tok, "ms_per_token": ms_tok, "tok_s_host_clock": new_tokens / wall,
         "eager_ms_per_token": eager_ms, "prefill_ms": prefill_ms,
-        "prefill_torch_glue_ms": prefill_glue_ms,
+        "prefill_torch_glue_ms": prefill_glue_ms, "prefill_chunk_tokens": width,
         "prefill_tok_s": prompt_len / (prefill_ms * 1e-3),
         "weight_gb_per_token": spec.weight_bytes_per_token() / 1e9,
         "kv_mb_per_token_mean": spec.kv_bytes(mean_ctx) / 1e6,
@@ -335,6 +337,9 @@ def main() -> int:
                          "traffic to scale hardware counters by)")
     ap.add_argument("--prompt", type=int, default=512)
     ap.add_argument("--new-tokens", type=int, default=256)
+    ap.add_argument("--prefill-width", type=int, default=None,
+                    help="tokens per prefill chunk of the feature-major prefill (default 64; the "
+                         "reference's chunks are 32)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build drives one GPU; --gpus N with N > 1 is not supported "
@@ -391,7 +396,8 @@ def main() -> int:
         },
     }
     if not args.no_decode:
-        out["decode"] = [bench_decode(torch, name.strip(), args.prompt, args.new_tokens, args.schedule)
+        out["decode"] = [bench_decode(torch, name.strip(), args.prompt, args.new_tokens, args.schedule,
+                                      args.prefill_width)
                          for name in args.decode_models.split(",") if name.strip()]
     if not args.no_prefill:
         out["prefill"] = bench_prefill(torch, nf4)
