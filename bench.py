@@ -199,6 +199,15 @@ def bench_decode(torch, spec_name: str, prompt_len: int, new_tokens: int, schedu
     dev_ms = e0.elapsed_time(e1)
     end_pos = int(state.position.item())
     assert end_pos == start_pos + new_tokens
+    # the same replays with the host reading every token id before it launches the next
+    # step (gpu/decodev2/profile_step.py:409-483 reports both)
+    n_read = min(32, new_tokens)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(n_read):
+        graph.replay()
+        int(state.next_token.item())
+    host_read_ms = (time.perf_counter() - t0) * 1e3 / n_read
     # eager step for comparison (a few tokens)
     t0 = time.perf_counter()
     for _ in range(8):
@@ -214,7 +223,7 @@ def bench_decode(torch, spec_name: str, prompt_len: int, new_tokens: int, schedu
         "vocab": spec.vocab, "max_seq": spec.max_seq, "prompt_tokens": prompt_len,
         "new_tokens": new_tokens, "context_start": start_pos, "context_end": end_pos,
         "tok_s": 1e3 / ms_tok, "ms_per_token": ms_tok, "tok_s_host_clock": new_tokens / wall,
-        "eager_ms_per_token": eager_ms, "prefill_ms": prefill_ms,
+        "tok_s_host_read": 1e3 / host_read_ms, "eager_ms_per_token": eager_ms, "prefill_ms": prefill_ms,
         "prefill_torch_glue_ms": prefill_glue_ms, "prefill_chunk_tokens": width,
         "prefill_tok_s": prompt_len / (prefill_ms * 1e-3),
         "weight_gb_per_token": spec.weight_bytes_per_token() / 1e9,
@@ -259,9 +268,24 @@ def cpu_baseline(m: int, k: int, budget_s: float = 12.0) -> dict:
             if dt >= budget:
                 return dt / n, n
 
+    def fused_for(threads: int, budget: float):
+        """decode + dot in one pass over the packed bytes (no fp32 copy of W)"""
+        L.or_set_threads(threads)
+        xf = np.ascontiguousarray(x.reshape(-1))
+        L.or_gemv_fused(packed.ctypes.data, s16.ctypes.data, m, k, xf.ctypes.data, y.ctypes.data)
+        n = 0
+        t0 = time.perf_counter()
+        while True:
+            L.or_gemv_fused(packed.ctypes.data, s16.ctypes.data, m, k, xf.ctypes.data, y.ctypes.data)
+            n += 1
+            dt = time.perf_counter() - t0
+            if dt >= budget:
+                return dt / n
+
     cores = min(int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or (os.cpu_count() or 1), 64)
-    t_all, n_all = run_for(cores, budget_s * 0.6)
-    t_one, n_one = run_for(1, budget_s * 0.4)
+    t_all, n_all = run_for(cores, budget_s * 0.5)
+    t_one, n_one = run_for(1, budget_s * 0.35)
+    t_fused = fused_for(cores, budget_s * 0.15)
     by = algorithmic_bytes(m, k)
     return {
         "value": by / t_all / 1e9,
@@ -273,6 +297,8 @@ def cpu_baseline(m: int, k: int, budget_s: float = 12.0) -> dict:
         "us_per_gemv": t_all * 1e6,
         "single_thread_gbps": by / t_one / 1e9,
         "single_thread_us_per_gemv": t_one * 1e6,
+        "fused_decode_dot_gbps": by / t_fused / 1e9,
+        "fused_decode_dot_us_per_gemv": t_fused * 1e6,
     }
 
 
