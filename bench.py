@@ -62,7 +62,7 @@ def make_weights(torch, nf4, m: int, k: int, copies: int, seed: int):
 
 def graph_time(torch, launch, n_launches: int, reps: int = 5) -> float:
     """Capture ``n_launches`` calls of ``launch(i)`` into one HIP graph and return
-    the best average milliseconds per launch over ``reps`` replays (events on the
+    the median over ``reps`` replays of the average milliseconds per launch (events on the
     capture stream bracket each replay)."""
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
@@ -79,16 +79,16 @@ def graph_time(torch, launch, n_launches: int, reps: int = 5) -> float:
         side.synchronize()
         e0 = torch.cuda.Event(enable_timing=True)
         e1 = torch.cuda.Event(enable_timing=True)
-        best = None
+        windows = []
         for _ in range(reps):
             e0.record(side)
             graph.replay()
             e1.record(side)
             side.synchronize()
-            ms = e0.elapsed_time(e1)
-            best = ms if best is None else min(best, ms)
+            windows.append(e0.elapsed_time(e1))
     torch.cuda.current_stream().wait_stream(side)
-    return best / n_launches
+    windows.sort()
+    return windows[len(windows) // 2] / n_launches
 
 
 def bench_gemv(torch, nf4, steps: int, warmup: int, copies: int):
