@@ -578,7 +578,7 @@ __global__ __launch_bounds__(256) void gemv_stream(const StreamArgs a) {
   }
 }
 
-// ---- staged kernel: x in LDS, pair table, weight prefetch two steps ahead ----------
+// ---- staged kernel: x in LDS, pair table, weight requests one item ahead -----------
 // Request half step t of R rows: 8 packed bytes per lane.  Lanes past the end of the row
 // read the row's last half chunk instead (in bounds, one instruction form for every
 // step) and are switched off where the scale is applied.
