@@ -88,6 +88,12 @@ void chr_nf4_set_tuning(int32_t path, int32_t split_k, int32_t one_wave);
 /* N=1 GEMV.  x bf16 [K], y bf16 [M].  add: optional bf16 [M] residual, may
  * alias y.  rms_w: optional bf16 [K]; when set, RMSNorm(x, rms_w, rms_eps),
  * rounded to bf16, is what the dots consume.
+ * Arithmetic: fp32 accumulation, one bf16 rounding of y.  Launches of fewer than 16M codes
+ * multiply fp32 levels (as nf4_gemv.cu:70-101); launches from 16M codes up, and every
+ * launch with rms_w or K != K_pad, multiply levels rounded to bf16 (the precision of the
+ * reference's tensor-core path, nf4_gemm.cu:322) and need K_pad * 2 <= 85 KB of LDS for x
+ * (-6 when rms_w or a ragged K require it and it does not fit).  CHR_NF4_GEMV_STAGED=0|1
+ * in the environment forces either form where both are possible.
  * Replaces chr_nf4_gemv (chr_gpu.h:92-93; nf4_gemv.cu:790-834). */
 int chr_nf4_gemv(const chr_nf4_dev_t *w, const void *x, void *y, void *stream,
                  const void *add, const void *rms_w, float rms_eps);
