@@ -119,6 +119,33 @@ def bench_gemv(torch, nf4, steps: int, warmup: int, copies: int):
     return ms, eager_ms, copies, by
 
 
+def bench_gemv_shapes(torch, nf4):
+    """The GEMV at the other 14B layer shapes and at the vocabulary projection: the fixed
+    cost of a launch weighs less the longer the weight stream is.  Same method as the
+    primary workload (graph replay, rotating copies beyond the 256 MB Infinity Cache)."""
+    rows = []
+    for name, m, k in (("qkv", 7168, 5120), ("o", 5120, 5120), ("down", 5120, 13824),
+                       ("gate+up rows", 27648, 5120), ("lm_head", 152064, 5120)):
+        by = algorithmic_bytes(m, k)
+        copies = max(2, -(-600 * 1024 * 1024 // by) + 1)
+        weights = make_weights(torch, nf4, m, k, copies, seed=4321)
+        g = torch.Generator(device="cuda")
+        g.manual_seed(98)
+        x = torch.randn(k, generator=g, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+        y = torch.empty(m, dtype=torch.bfloat16, device="cuda")
+
+        def launch(i, weights=weights, copies=copies, x=x, y=y, m=m, k=k):
+            p, s = weights[i % copies]
+            nf4.nf4_gemv(p, s, x, m, k, k, y)
+
+        ms = graph_time(torch, launch, 120)
+        rows.append({"layer": name, "M": m, "K": k, "us": ms * 1e3, "gbps": by / ms / 1e6,
+                     "hbm_frac": by / ms / 1e6 / HBM_PEAK_GBPS})
+        del weights
+        torch.cuda.empty_cache()
+    return rows
+
+
 def bench_prefill(torch, nf4):
     """MFMA GEMM chunks at the 14B linear shapes; weights rotate through > 512 MB."""
     shapes = {"qkv": (7168, 5120), "o": (5120, 5120), "gate_up": (13824, 5120), "down": (5120, 13824)}
@@ -357,6 +384,7 @@ def main() -> int:
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill GEMM sweep")
     ap.add_argument("--no-ring", action="store_true", help="skip the host-streaming ring leg")
     ap.add_argument("--decode-models", default="14b", help="comma list of 3b,14b,20b,32b")
+    ap.add_argument("--no-shapes", action="store_true", help="skip the GEMV sweep over other shapes")
     ap.add_argument("--schedule", default=None, help="decode launch schedule: plain or fold_rms")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
                     help="first run four plain device copies of this size (a kernel of known "
@@ -421,6 +449,8 @@ def main() -> int:
             "algorithmic_bytes_per_launch": by,
         },
     }
+    if not args.no_shapes:
+        out["gemv_shapes"] = bench_gemv_shapes(torch, nf4)
     if not args.no_decode:
         out["decode"] = [bench_decode(torch, name.strip(), args.prompt, args.new_tokens, args.schedule,
                                       args.prefill_width)
