@@ -148,6 +148,27 @@ __device__ __forceinline__ float wave_sum(float v) {
   return (r0 + r1) + (r2 + r3);
 }
 
+// ---- streaming loads -------------------------------------------------------------
+// Packed weights and their scales are read once per launch: the non-temporal hint (the nt bit
+// of the load) keeps them from displacing what is reused (x, tables, the KV cache) on their
+// way through the caches.  Measured on the N=1 kernel: 11.1 -> 10.1 us at 13824x5120.
+typedef uint32_t U32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t U32x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint4 stream_load16(const void *p) {
+  const U32x4 v = __builtin_nontemporal_load(static_cast<const U32x4 *>(p));
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+
+__device__ __forceinline__ uint2 stream_load8(const void *p) {
+  const U32x2 v = __builtin_nontemporal_load(static_cast<const U32x2 *>(p));
+  return make_uint2(v.x, v.y);
+}
+
+__device__ __forceinline__ uint16_t stream_load2(const uint16_t *p) {
+  return __builtin_nontemporal_load(p);
+}
+
 // ---- host-side argument checks shared by the entry points -------------------
 inline bool k_pad_ok(int K, int K_pad) {
   if (K < 1 || K_pad < K) {

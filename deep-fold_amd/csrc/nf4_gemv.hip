@@ -405,12 +405,12 @@ __device__ __forceinline__ void rows_dot(const uint8_t *const (&prow)[R],
       uint16_t sc[R];
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        const uint4 v = *(reinterpret_cast<const uint4 *>(prow[r]) + c);
+        const uint4 v = stream_load16(reinterpret_cast<const uint4 *>(prow[r]) + c);
         w[r][0] = v.x;
         w[r][1] = v.y;
         w[r][2] = v.z;
         w[r][3] = v.w;
-        sc[r] = srow[r][c >> 1];
+        sc[r] = stream_load2(srow[r] + (c >> 1));
       }
       const uint4 *xp = x4 + (c << 2);
       const uint4 x0 = xp[0], x1 = xp[1], x2 = xp[2], x3 = xp[3];
@@ -428,10 +428,10 @@ __device__ __forceinline__ void rows_dot(const uint8_t *const (&prow)[R],
         uint16_t sc[R];
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-          const uint2 v = *(reinterpret_cast<const uint2 *>(prow[r]) + hc);
+          const uint2 v = stream_load8(reinterpret_cast<const uint2 *>(prow[r]) + hc);
           w[r][0] = v.x;
           w[r][1] = v.y;
-          sc[r] = srow[r][hc >> 2];
+          sc[r] = stream_load2(srow[r] + (hc >> 2));
         }
         const uint4 *xp = x4 + (hc << 1);
         const uint4 x0 = xp[0], x1 = xp[1];
@@ -589,8 +589,8 @@ __device__ __forceinline__ void load_step(const uint8_t *const (&prow)[R],
   const int h = min((t << 6) + lane, n_half - 1);
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    w[r] = *(reinterpret_cast<const uint2 *>(prow[r]) + h);
-    sc[r] = srow[r][h >> 2];
+    w[r] = stream_load8(reinterpret_cast<const uint2 *>(prow[r]) + h);
+    sc[r] = stream_load2(srow[r] + (h >> 2));
   }
 }
 
