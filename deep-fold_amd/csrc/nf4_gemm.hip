@@ -486,7 +486,13 @@ __global__ __launch_bounds__(kGemmBlock) void gemm_mfma(const GemmSegs segs,
         for (int i = 0; i < 16; ++i) {
           const int r = rbase + 8 * (i >> 2) + (i & 3);
           if (r < M) {
-            p[static_cast<size_t>(out0 + r) * N + n] = acc[nb][i];
+            float *dst = p + static_cast<size_t>(out0 + r) * N + n;
+            if constexpr (NB == 2) {
+              // wide chunks: full 128-byte runs per row, read once by the reduce
+              __builtin_nontemporal_store(acc[nb][i], dst);
+            } else {
+              *dst = acc[nb][i];
+            }
           }
         }
       }
@@ -507,7 +513,7 @@ __global__ __launch_bounds__(256) void reduce_splitk(const float *__restrict__ p
   }
   float s = 0.f;
   for (int j = 0; j < split; ++j) {
-    s += partial[static_cast<size_t>(j) * rows + i];
+    s += __builtin_nontemporal_load(partial + static_cast<size_t>(j) * rows + i);
   }
   uint16_t v = f32_to_bf16(s);
   if (bias != nullptr) {
@@ -539,7 +545,7 @@ __global__ __launch_bounds__(kSqElems) void reduce_splitk_sq(const float *__rest
   if (i < rows) {
     float s = 0.f;
     for (int j = 0; j < split; ++j) {
-      s += partial[static_cast<size_t>(j) * rows + i];
+      s += __builtin_nontemporal_load(partial + static_cast<size_t>(j) * rows + i);
     }
     uint16_t v = f32_to_bf16(s);
     if (bias != nullptr) {
@@ -575,8 +581,8 @@ __global__ __launch_bounds__(256) void reduce_swiglu(const float *__restrict__ p
   float g = 0.f, u = 0.f;
   for (int j = 0; j < split; ++j) {
     const float *p = partial + static_cast<size_t>(j) * 2 * half_rows;
-    g += p[i];
-    u += p[half_rows + i];
+    g += __builtin_nontemporal_load(p + i);
+    u += __builtin_nontemporal_load(p + half_rows + i);
   }
   const float a = bf16_to_f32(f32_to_bf16(g));
   const float act = bf16_to_f32(f32_to_bf16(a / (1.f + expf(-a))));
