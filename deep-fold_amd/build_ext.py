@@ -59,7 +59,27 @@ def build(force: bool = True, verbose: bool = False) -> str:
         raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{err}")
     if verbose and err.strip():
         print(err, file=sys.stderr)
+    build_host_check()
     return LIB
+
+
+#: A caller of the C-ABI written in C++ with no Python in the process; the tests run it.
+HOST_CHECK_SRC = os.path.join(CSRC, "..", "..", "tests", "cabi", "host_check.cpp")
+HOST_CHECK = os.path.splitext(HOST_CHECK_SRC)[0]
+
+
+def build_host_check() -> str | None:
+    """Link ``tests/cabi/host_check`` against the library just built (skipped when the
+    package is used without its test tree)."""
+    if not os.path.exists(HOST_CHECK_SRC):
+        return None
+    include = os.path.join(CSRC, "..", "..", "include")
+    cmd = [hipcc(), "-O2", "-std=c++17", "-I", include, "-o", HOST_CHECK, HOST_CHECK_SRC,
+           "-L", CSRC, "-lchr_nf4_amd", "-Wl,-rpath,$ORIGIN/../../deep-fold_amd/csrc"]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed on host_check.cpp ({proc.returncode}):\n{proc.stderr}")
+    return HOST_CHECK
 
 
 if __name__ == "__main__":
