@@ -4,6 +4,11 @@
 // Replaces gpu/nf4/nf4_gemm.cu:665-678 (reduce), 933-1450 (prefill tiles),
 // 1497-1785 (tuning, planner, entry points).
 //
+// Two tile kernels share the planner, the row blocks (128 rows), the split-K partials and the
+// reduces.  gemm_rows (described where it is defined) serves every launch whose K slice is at
+// most four K tiles long, which is what the planner's split-K produces; gemm_mfma, described
+// here, serves the longer slices of launches without a workspace.
+//
 // Tile.  A workgroup is four wavefronts and owns 128 output rows; each
 // wavefront owns 32 of them and all N columns, accumulating one 32x32 fp32
 // tile with v_mfma_f32_32x32x16_bf16.  For that instruction lane l supplies
@@ -76,6 +81,26 @@ constexpr int gemm_lds_bytes(int nb) {
          kGemmWaves * 32 * kGroupsPerTile * 2;
 }
 
+// The row-streaming tile (gemm_rows): eight wavefronts x 16 rows, one K slice of up to
+// four K tiles per workgroup.
+constexpr int kRowsWaves = 8;
+constexpr int kRowsBlock = kRowsWaves * 64;
+constexpr int kRowsStepK = 128;  // k per wavefront step: 16 rows x 64 bytes
+constexpr int kRowsMaxTiles = 4;
+static_assert(kRowsWaves * 16 == kBM, "both tiles number their row blocks the same way");
+// bf16 elements of one token's row of the transposed slice: 4 dwords more than a multiple
+// of 64, so the sixteen 16-byte B reads of a quarter wavefront fall in 64 different banks
+constexpr int rows_x_stride(int tps) { return tps * kBK + kXPad; }
+// the sixteen levels at LDS address 0 (lookup8_lds0), then nc blocks of sixteen token rows
+constexpr int rows_lds_bytes(int nc, int tps) { return 64 + nc * 16 * rows_x_stride(tps) * 2; }
+// pairs of 16-byte activation vectors a thread stages (N = 16 nc at most)
+constexpr int rows_x_items(int nc, int tps) {
+  return (tps * (kBK / 2) * 2 * nc + kRowsBlock - 1) / kRowsBlock;
+}
+// 64 token rows of four tiles would not leave room for two workgroups per compute unit
+constexpr int rows_max_tiles(int nc) { return nc == 4 ? 2 : kRowsMaxTiles; }
+constexpr int rows_col_blocks(int N) { return N <= 16 ? 1 : (N <= 32 ? 2 : 4); }
+
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
@@ -91,6 +116,13 @@ int env_int(const char *name, int dflt) {
     return dflt;
   }
   return std::atoi(e);
+}
+
+// Which tile a launch runs: the row-streaming one whenever its K slice is short enough to be
+// requested whole.  CHR_NF4_GEMM_ROWS=0 keeps every launch on the K-tiled kernel.
+bool rows_kernel_serves(int N, int tiles_per_split) {
+  static const bool on = env_int("CHR_NF4_GEMM_ROWS", 1) != 0;
+  return on && tiles_per_split <= rows_max_tiles(rows_col_blocks(N));
 }
 
 Tuning &tuning() {
@@ -167,6 +199,10 @@ int plan_impl(const chr_nf4_dev_t &h, int32_t N, int32_t have_ws, chr_nf4_plan_t
     p.n_ktiles = ceil_div(h.K_pad, kBK);
     pick_split(p.grid_x, p.n_ktiles, N, have_ws, &p.grid_y, &p.tiles_per_split);
     p.smem_bytes = gemm_lds_bytes(N <= 32 ? 1 : 2);
+    if (rows_kernel_serves(N, p.tiles_per_split)) {
+      p.block = kRowsBlock;
+      p.smem_bytes = rows_lds_bytes(rows_col_blocks(N), p.tiles_per_split);
+    }
     if (p.grid_y > 1) {
       p.ws_floats = static_cast<int64_t>(p.grid_y) * h.M * N;
     }
@@ -500,6 +536,276 @@ __global__ __launch_bounds__(kGemmBlock) void gemm_mfma(const GemmSegs segs,
   }
 }
 
+// ---------------------------------------------------------------------------------------
+// Row-streaming tile: every weight byte goes from global memory straight into the register
+// that feeds the matrix core; only the activations pass through LDS.
+//
+// A workgroup is eight wavefronts and owns kBM = 128 rows x one K slice of TPS * kBK
+// columns (grid.y numbers the slices, so the partials are laid out as for gemm_mfma).  A
+// wavefront owns 16 rows and multiplies with v_mfma_f32_16x16x32_bf16, whose A operand is
+// 16 rows x 32 k: lane l supplies eight k of row l % 16, the k slots being numbered by
+// l / 16.  Which k sits in which slot is free as long as A and B agree, so a step of the
+// wavefront is 128 k wide, lane l loads the 16 bytes (32 codes) of row l % 16 at byte
+// 16 * (l / 16) of the step -- sixteen rows x 64 contiguous bytes per load instruction --
+// and MFMA j of the step takes dword j of every lane: k = 32 * (l / 16) + 8 j .. + 8.  The B
+// operand is read from the transposed activation slice at the same k.  All 32 k of a lane
+// lie in one 64-wide group, so one scale per lane and step is enough.
+//
+// Nothing is pipelined: a slice is at most four K tiles, so a lane requests its whole share
+// (at most eight 16-byte loads of codes) at the top of the kernel, behind the activation
+// requests, and the memory system sees the full grid's weights at once.
+//
+// Requests past the end of a row or of x are clamped to valid addresses and the activation
+// slice holds zeros from k = K on, so they contribute nothing; rows >= M are computed from
+// row M - 1 and dropped in the epilogue.
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+template <bool VEC, int NC, int TPS>
+__global__ __launch_bounds__(kRowsBlock) void gemm_rows(const GemmSegs segs,
+                                                        const uint16_t *__restrict__ x,
+                                                        uint16_t *__restrict__ y,
+                                                        float *__restrict__ partial, int M_all,
+                                                        int K, int K_pad, int N,
+                                                        const uint16_t *__restrict__ bias,
+                                                        const uint16_t *res) {
+  constexpr int SK = TPS * kBK;
+  constexpr int XS = rows_x_stride(TPS);
+  constexpr int STEPS = SK / kRowsStepK;
+  constexpr int XI = rows_x_items(NC, TPS);
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  float *lut = reinterpret_cast<float *>(lds_raw);
+  uint16_t *xs = reinterpret_cast<uint16_t *>(lds_raw + 64);
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  if (tid < 16) {
+    lut[tid] = bits_to_f32(kLutBits[tid]);
+  }
+  int bx = static_cast<int>(blockIdx.x);
+  int seg = 0;
+  if (bx >= segs.blocks[0]) {
+    bx -= segs.blocks[0];
+    seg = 1;
+    if (bx >= segs.blocks[1]) {
+      bx -= segs.blocks[1];
+      seg = 2;
+    }
+  }
+  const uint8_t *__restrict__ packed = segs.packed[seg];
+  const uint16_t *__restrict__ scale = segs.scale[seg];
+  const int M = segs.M[seg];
+  const int out0 = segs.row0[seg];
+  const int row_base = bx * kBM + wave * 16;
+  const int k0 = static_cast<int>(blockIdx.y) * SK;
+  const int r = lane & 15;  // row of the A operand, token of the B operand
+  const int g = lane >> 4;  // which quarter of a step's k
+
+  // 1. activation requests: item (k pair kp, vector q) is rows k0 + 2 kp, + 1 of x, columns
+  //    8 q .. + 8; q runs fastest over the threads so a row's vectors are fetched together
+  const int nv = N >> 3;
+  const int n_items = (SK / 2) * nv;
+  uint4 xa[XI], xb[XI];
+  int xkp[XI], xq[XI];
+  if constexpr (VEC) {
+#pragma unroll
+    for (int it = 0; it < XI; ++it) {
+      const int idx = min(tid + it * kRowsBlock, n_items - 1);
+      const int kp = idx / nv;
+      const int q = idx - kp * nv;
+      xkp[it] = kp;
+      xq[it] = q;
+      const int k = k0 + 2 * kp;
+      xa[it] = *reinterpret_cast<const uint4 *>(x + static_cast<size_t>(min(k, K - 1)) * N + 8 * q);
+      xb[it] =
+          *reinterpret_cast<const uint4 *>(x + static_cast<size_t>(min(k + 1, K - 1)) * N + 8 * q);
+    }
+  }
+
+  // 2. weight and scale requests, the whole slice of this lane's row
+  const int row_bytes = K_pad >> 1;
+  const int groups = K_pad >> 6;
+  const int row = min(row_base + r, M - 1);
+  const uint8_t *prow = packed + static_cast<size_t>(row) * row_bytes;
+  const uint16_t *srow = scale + static_cast<size_t>(row) * groups;
+  uint4 wq[STEPS];
+  uint16_t sc[STEPS];
+#pragma unroll
+  for (int s = 0; s < STEPS; ++s) {
+    const int off = min((k0 >> 1) + 64 * s + 16 * g, row_bytes - 16);
+    wq[s] = *reinterpret_cast<const uint4 *>(prow + off);
+    sc[s] = srow[min((k0 >> 6) + 2 * s + (g >> 1), groups - 1)];
+  }
+
+  // 3. token rows N .. 16 NC of the slice are never staged: zero them
+  {
+    uint32_t *z = reinterpret_cast<uint32_t *>(xs + N * XS);
+    const int nz = (16 * NC - N) * (XS / 2);
+    for (int i = tid; i < nz; i += kRowsBlock) {
+      z[i] = 0u;
+    }
+  }
+
+  // 4. transpose the activations into LDS: rows k, k + 1 are interleaved into dwords
+  //    {x[k][n], x[k + 1][n]} and stored at xs[n][k / 2]
+  if constexpr (VEC) {
+    uint32_t *xd = reinterpret_cast<uint32_t *>(xs);
+#pragma unroll
+    for (int it = 0; it < XI; ++it) {
+      if (tid + it * kRowsBlock < n_items) {
+        const int k = k0 + 2 * xkp[it];
+        const bool ka = k < K, kb = k + 1 < K;
+        const uint32_t a[4] = {ka ? xa[it].x : 0u, ka ? xa[it].y : 0u, ka ? xa[it].z : 0u,
+                               ka ? xa[it].w : 0u};
+        const uint32_t b[4] = {kb ? xb[it].x : 0u, kb ? xb[it].y : 0u, kb ? xb[it].z : 0u,
+                               kb ? xb[it].w : 0u};
+        uint32_t *dst = xd + (8 * xq[it]) * (XS / 2) + xkp[it];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          dst[(2 * e) * (XS / 2)] = (a[e] & 0xFFFFu) | (b[e] << 16);
+          dst[(2 * e + 1) * (XS / 2)] = (a[e] >> 16) | (b[e] & 0xFFFF0000u);
+        }
+      }
+    }
+  } else {
+    // any N, any alignment: element by element
+    for (int i = tid; i < SK * N; i += kRowsBlock) {
+      const int kk = i / N;
+      const int n = i - kk * N;
+      const int k = k0 + kk;
+      xs[n * XS + kk] = k < K ? x[static_cast<size_t>(k) * N + n] : static_cast<uint16_t>(0);
+    }
+  }
+  __syncthreads();
+
+  // 5. multiply
+  f32x4 acc[NC];
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  const uint16_t *xl = xs + r * XS + 32 * g;
+#pragma unroll
+  for (int s = 0; s < STEPS; ++s) {
+    const float sf = f16_to_f32(sc[s]);
+    const uint32_t w[4] = {wq[s].x, wq[s].y, wq[s].z, wq[s].w};
+#pragma unroll
+    for (int jh = 0; jh < 4; jh += 2) {
+      // the sixteen lookups and the B reads of two MFMA k blocks are issued before the
+      // first conversion, so their LDS latency is paid once per pair
+      Levels8 lv[2];
+      bf16x8 b[2][NC];
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        lv[t] = lookup8_lds0(w[jh + t]);
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+          b[t][c] = *reinterpret_cast<const bf16x8 *>(xl + c * 16 * XS + kRowsStepK * s +
+                                                      8 * (jh + t));
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        bf16x8 a;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          a[e] = static_cast<__bf16>(lv[t].l[e] * sf);
+        }
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+          acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[t][c], acc[c], 0, 0, 0);
+        }
+      }
+    }
+  }
+
+  // acc[c][i] is C[row 4 * (lane / 16) + i][col 16 c + lane % 16] of the 16-row tile
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const int n = 16 * c + r;
+    if (n < N) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int rr = row_base + 4 * g + i;
+        if (rr < M) {
+          const size_t at = static_cast<size_t>(out0 + rr) * N + n;
+          if (partial == nullptr) {
+            // unsplit: the epilogue of reduce_splitk, here (res may alias y: same thread,
+            // same element)
+            uint16_t v = f32_to_bf16(acc[c][i]);
+            if (bias != nullptr) {
+              v = f32_to_bf16(bf16_to_f32(v) + bf16_to_f32(bias[out0 + rr]));
+            }
+            if (res != nullptr) {
+              v = f32_to_bf16(bf16_to_f32(res[at]) + bf16_to_f32(v));
+            }
+            y[at] = v;
+          } else {
+            partial[static_cast<size_t>(blockIdx.y) * M_all * N + at] = acc[c][i];
+          }
+        }
+      }
+    }
+  }
+}
+
+struct RowsArgs {
+  GemmSegs segs;
+  const uint16_t *x;
+  uint16_t *y;
+  float *partial;
+  int M_all, K, K_pad, N;
+  const uint16_t *bias, *res;
+};
+
+template <bool VEC, int NC, int TPS>
+int rows_one(const RowsArgs &a, dim3 grid, hipStream_t st, bool attr_only) {
+  if (attr_only) {
+    return hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_rows<VEC, NC, TPS>),
+                               hipFuncAttributeMaxDynamicSharedMemorySize,
+                               rows_lds_bytes(NC, TPS)) == hipSuccess
+               ? 0
+               : -6;
+  }
+  gemm_rows<VEC, NC, TPS><<<grid, dim3(kRowsBlock), rows_lds_bytes(NC, TPS), st>>>(
+      a.segs, a.x, a.y, a.partial, a.M_all, a.K, a.K_pad, a.N, a.bias, a.res);
+  return 0;
+}
+
+template <bool VEC, int NC>
+int rows_by_tiles(int tps, const RowsArgs &a, dim3 grid, hipStream_t st, bool attr_only) {
+  switch (tps) {
+    case 1:
+      return rows_one<VEC, NC, 1>(a, grid, st, attr_only);
+    case 2:
+      return rows_one<VEC, NC, 2>(a, grid, st, attr_only);
+    case 3:
+      if constexpr (NC < 4) return rows_one<VEC, NC, 3>(a, grid, st, attr_only);
+      return -6;
+    case 4:
+      if constexpr (NC < 4) return rows_one<VEC, NC, 4>(a, grid, st, attr_only);
+      return -6;
+    default:
+      return -6;
+  }
+}
+
+// nc: 16-column blocks (1, 2 or 4).  attr_only raises the kernel's LDS limit instead of
+// launching it.
+int rows_dispatch(bool vec, int nc, int tps, const RowsArgs &a, dim3 grid, hipStream_t st,
+                  bool attr_only) {
+  if (vec) {
+    return nc == 1   ? rows_by_tiles<true, 1>(tps, a, grid, st, attr_only)
+           : nc == 2 ? rows_by_tiles<true, 2>(tps, a, grid, st, attr_only)
+                     : rows_by_tiles<true, 4>(tps, a, grid, st, attr_only);
+  }
+  return nc == 1   ? rows_by_tiles<false, 1>(tps, a, grid, st, attr_only)
+         : nc == 2 ? rows_by_tiles<false, 2>(tps, a, grid, st, attr_only)
+                   : rows_by_tiles<false, 4>(tps, a, grid, st, attr_only);
+}
+
+
 // y[i] = bf16( sum over splits, in split order, of partial[s][i] ), then optionally
 // bf16(y + bias[row]) and bf16(res[i] + y): the roundings of separate bias and residual adds.
 __global__ __launch_bounds__(256) void reduce_splitk(const float *__restrict__ partial,
@@ -603,6 +909,17 @@ int gemm_lds_ready() {
           hipSuccess) {
         (void)hipGetLastError();
         return -6;
+      }
+    }
+    const RowsArgs none{};
+    for (int vec = 0; vec < 2; ++vec) {
+      for (int nc = 1; nc <= 4; nc *= 2) {
+        for (int tps = 1; tps <= rows_max_tiles(nc); ++tps) {
+          if (rows_dispatch(vec != 0, nc, tps, none, dim3(1), nullptr, true) != 0) {
+            (void)hipGetLastError();
+            return -6;
+          }
+        }
       }
     }
     return 0;
@@ -729,7 +1046,14 @@ int gemm_launch(const chr_nf4_dev_t *const *w, int nseg, const void *x, void *y,
   const auto *rp = static_cast<const uint16_t *>(res);
   const dim3 block(kGemmBlock);
   const int K = h[0].K, K_pad = h[0].K_pad;
-  if (N <= kBN) {
+  const int nc = rows_col_blocks(N);
+  if (rows_kernel_serves(N, sp.tiles_per_split)) {
+    const RowsArgs ra{sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp};
+    // the vector staging needs whole 16-byte vectors per row of x
+    if (rows_dispatch((N & 7) == 0, nc, sp.tiles_per_split, ra, grid, st, false) != 0) {
+      return -6;
+    }
+  } else if (N <= kBN) {
     if (vec) {
       gemm_mfma<true, 1><<<grid, block, gemm_lds_bytes(1), st>>>(
           sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, sp.n_ktiles, sp.tiles_per_split, bp, rp);

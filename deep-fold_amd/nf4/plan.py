@@ -10,12 +10,17 @@ Kernel families by token count ``N`` (the reference's name for it; out features
 are ``M``, in features ``K``):
 
 * ``N == 1``  row-streaming GEMV, no split-K (path ``GEMV``).
-* ``N = 2..16`` / ``17..32``  MFMA tile, 128 rows x 32 columns per workgroup,
+* ``N = 2..16`` / ``17..32``  MFMA tile, 128 rows per workgroup,
   split-K over ``grid_y`` at about three K tiles per workgroup, up to three workgroups
   per compute unit (paths ``PREFILL`` / ``PREFILL_N32``).
-* ``N = 33..64``  the same tile with two 32-column blocks per weight fragment
+* ``N = 33..64``  the same with twice the token columns
   (``PREFILL_N64``); launched only through ``chr_nf4_gemm_ws_max`` with ``max_n`` > 32,
   the plain entries keep the reference's ceiling of 32.
+
+Two kernels serve the MFMA paths.  Slices of at most four K tiles (two above 32 columns) run
+the row-streaming tile: 512 threads, every weight byte loaded straight into the register
+that feeds the matrix core.  Longer slices (unsplit launches of a long K) run the K-tiled
+one: 256 threads, weights staged through LDS one tile ahead.
 """
 
 from __future__ import annotations
@@ -36,6 +41,7 @@ __all__ = [
     "gemv_rows_per_wavefront",
     "gemv_is_staged",
     "staged_lds_bytes",
+    "gemm_streams_rows",
     "STAGED_MIN_CODES",
     "plan",
 ]
@@ -141,6 +147,14 @@ class Plan:
         return self.path != PREFILL_N64
 
 
+def gemm_streams_rows(N: int, tiles_per_split: int) -> bool:  # noqa: N803
+    """Whether a launch runs the row-streaming tile (weights straight from global memory into
+    the MFMA operand, the whole K slice requested at once) instead of the K-tiled one: slices
+    of at most four K tiles, two for chunks wider than 32 columns.  ``CHR_NF4_GEMM_ROWS=0`` in
+    the environment keeps the library on the K-tiled kernel; this mirror ignores it."""
+    return tiles_per_split <= (2 if N > 32 else 4)
+
+
 def _pick_split(grid_x: int, n_ktiles: int, N: int, have_ws: bool, force_split: int,  # noqa: N803
                 one_wave: int) -> tuple[int, int]:
     want = 1
@@ -183,5 +197,9 @@ def plan(M: int, K: int, N: int = 1, *, K_pad: int | None = None, have_ws: bool 
     n_ktiles = _ceil_div(kp, _BK)
     split, tps = _pick_split(grid_x, n_ktiles, N, have_ws, force_split, one_wave)
     ws = split * M * N if split > 1 else 0
+    if gemm_streams_rows(N, tps):
+        nc = 1 if N <= 16 else (2 if N <= 32 else 4)
+        smem = 64 + nc * 16 * (tps * _BK + 8) * 2   # codebook + transposed activation slice
+        return Plan(path, grid_x, split, 512, _BM, _BK, n_ktiles, tps, grid_x * split, smem, ws)
     smem = _gemm_lds(1 if N <= 32 else 2)
     return Plan(path, grid_x, split, _BLOCK, _BM, _BK, n_ktiles, tps, grid_x * split, smem, ws)

@@ -450,6 +450,30 @@ def test_gemm_every_split_agrees(n):
         assert (d <= 2.0 ** (np.floor(np.log2(np.maximum(np.abs(outs[0]), 2.0 ** -120))) - 7) + 1e-30).all()
 
 
+@pytest.mark.parametrize("n", [5, 8, 16, 24, 32, 40, 64])
+@pytest.mark.parametrize("k,split,tiles", [(1024, 1, 4), (1000, 2, 2), (1024, 4, 1), (768, 1, 3),
+                                           (2048, 1, 8), (2048, 8, 1)])
+def test_gemm_every_tile_variant(n, k, split, tiles):
+    """Slice lengths of one to four K tiles (the row-streaming tile, one build per length and
+    per 16-column block count; two tiles at most above 32 columns) and an eight-tile slice
+    (the K-tiled kernel), with whole-vector and ragged column counts and a ragged row block."""
+    m = 200
+    say("gemm variant", m, k, n, split)
+    p, s, dp, ds = blobs(m, k, 310 + k)
+    x = rand_x(k, n, 17)
+    try:
+        nf4.nf4_set_tuning(split_k=split)
+        plan = nf4.nf4_plan(m, k, n)
+        assert (plan["grid_y"], plan["tiles_per_split"]) == (split, tiles)
+        streams = tiles <= (2 if n > 32 else 4)
+        assert plan["block"] == (512 if streams else 256)
+        y = nf4.nf4_gemm(dp, ds, bf16_tensor(x), m, k, oc.k_pad(k), max_n=64)
+    finally:
+        nf4.nf4_set_tuning()
+    ref = oc.c_matmul_f64(oc.bf16_round(oc.c_decode(p, s, m, k)), x)
+    check_linear(y, ref, what=f"gemm {m}x{k} n{n} split {split}")
+
+
 def test_gemm_n1_routes_to_gemv():
     m, k = 384, 2048
     p, s, dp, ds = blobs(m, k, 303)

@@ -261,8 +261,9 @@ def test_wide_chunk_equals_two_narrow_ones(m, k, n):
     first = min(32, n - 2)  # at least two columns: one alone would go to the GEMV
     hi = nf4.nf4_gemm(dp, ds, x[:, first:].contiguous(), m, k, kp)
     assert tuple(wide.shape) == (m, n)
-    same_split = (nf4.nf4_plan(m, k, n)["grid_y"] == nf4.nf4_plan(m, k, 32)["grid_y"]
-                  == nf4.nf4_plan(m, k, n - first)["grid_y"])
+    # the same split by the same kernel (the plan's block size tells the two tiles apart)
+    plans = [nf4.nf4_plan(m, k, c) for c in (n, 32, n - first)]
+    same_split = len({(q["grid_y"], q["block"]) for q in plans}) == 1
     for got, want_ in ((wide[:, :32].contiguous(), lo), (wide[:, first:].contiguous(), hi.view(m, n - first))):
         if same_split:  # same K order, same partial sums: the same bits
             assert (bf16_bits(got) == bf16_bits(want_)).all()
