@@ -806,6 +806,60 @@ int rows_dispatch(bool vec, int nc, int tps, const RowsArgs &a, dim3 grid, hipSt
 }
 
 
+// Sums of P elements over the splits, each in split order.  The loads of eight splits are
+// issued before the first add: written as a plain loop a sum is a chain of dependent trips to
+// memory (load, wait, add), seven of them for a 5120-wide K.  Every load is unconditional --
+// a load under a branch is waited for where the branch ends -- and slots past the last split
+// read split 0 again (the line is already on its way), their values unused.  The first eight
+// splits stand outside the loop, whose head waits for every load issued before it.
+template <int P>
+__device__ __forceinline__ void sum_splits(const float *const (&p)[P], size_t stride, int split,
+                                           float (&s)[P]) {
+  float v[P][8];
+#pragma unroll
+  for (int u = 0; u < 8; ++u) {
+#pragma unroll
+    for (int e = 0; e < P; ++e) {
+      v[e][u] = __builtin_nontemporal_load(p[e] + (u < split ? u : 0) * stride);
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < P; ++e) {
+    s[e] = 0.f;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      if (u < split) {
+        s[e] += v[e][u];
+      }
+    }
+  }
+  for (int j0 = 8; j0 < split; j0 += 8) {
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+#pragma unroll
+      for (int e = 0; e < P; ++e) {
+        v[e][u] = __builtin_nontemporal_load(p[e] + (j0 + u < split ? j0 + u : 0) * stride);
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < P; ++e) {
+#pragma unroll
+      for (int u = 0; u < 8; ++u) {
+        if (j0 + u < split) {
+          s[e] += v[e][u];
+        }
+      }
+    }
+  }
+}
+
+__device__ __forceinline__ float sum_splits(const float *p, size_t stride, int split) {
+  const float *const ps[1] = {p};
+  float s[1];
+  sum_splits<1>(ps, stride, split, s);
+  return s[0];
+}
+
 // y[i] = bf16( sum over splits, in split order, of partial[s][i] ), then optionally
 // bf16(y + bias[row]) and bf16(res[i] + y): the roundings of separate bias and residual adds.
 __global__ __launch_bounds__(256) void reduce_splitk(const float *__restrict__ partial,
@@ -817,16 +871,18 @@ __global__ __launch_bounds__(256) void reduce_splitk(const float *__restrict__ p
   if (i >= rows) {
     return;
   }
-  float s = 0.f;
-  for (int j = 0; j < split; ++j) {
-    s += __builtin_nontemporal_load(partial + static_cast<size_t>(j) * rows + i);
-  }
+  // Bias and residual are requested before the partials are waited for.  The loads are
+  // unconditional (an absent operand reads y instead, a valid address whose value is not
+  // used): a load under a branch is waited for where the branch ends.
+  const uint16_t b = (bias != nullptr ? bias : y)[i / N];
+  const uint16_t r = (res != nullptr ? res : y)[i];
+  const float s = sum_splits(partial + i, static_cast<size_t>(rows), split);
   uint16_t v = f32_to_bf16(s);
   if (bias != nullptr) {
-    v = f32_to_bf16(bf16_to_f32(v) + bf16_to_f32(bias[i / N]));
+    v = f32_to_bf16(bf16_to_f32(v) + bf16_to_f32(b));
   }
   if (res != nullptr) {
-    v = f32_to_bf16(bf16_to_f32(res[i]) + bf16_to_f32(v));
+    v = f32_to_bf16(bf16_to_f32(r) + bf16_to_f32(v));
   }
   y[i] = v;
 }
@@ -849,16 +905,15 @@ __global__ __launch_bounds__(kSqElems) void reduce_splitk_sq(const float *__rest
   const int i = blockIdx.x * kSqElems + threadIdx.x;
   float sqv = 0.f;
   if (i < rows) {
-    float s = 0.f;
-    for (int j = 0; j < split; ++j) {
-      s += __builtin_nontemporal_load(partial + static_cast<size_t>(j) * rows + i);
-    }
+    const uint16_t b = (bias != nullptr ? bias : y)[i / N];  // unconditional, as in reduce_splitk
+    const uint16_t r = (res != nullptr ? res : y)[i];
+    const float s = sum_splits(partial + i, static_cast<size_t>(rows), split);
     uint16_t v = f32_to_bf16(s);
     if (bias != nullptr) {
-      v = f32_to_bf16(bf16_to_f32(v) + bf16_to_f32(bias[i / N]));
+      v = f32_to_bf16(bf16_to_f32(v) + bf16_to_f32(b));
     }
     if (res != nullptr) {
-      v = f32_to_bf16(bf16_to_f32(res[i]) + bf16_to_f32(v));
+      v = f32_to_bf16(bf16_to_f32(r) + bf16_to_f32(v));
     }
     y[i] = v;
     const float f = bf16_to_f32(v);
@@ -884,12 +939,11 @@ __global__ __launch_bounds__(256) void reduce_swiglu(const float *__restrict__ p
   if (i >= half_rows) {
     return;
   }
-  float g = 0.f, u = 0.f;
-  for (int j = 0; j < split; ++j) {
-    const float *p = partial + static_cast<size_t>(j) * 2 * half_rows;
-    g += __builtin_nontemporal_load(p + i);
-    u += __builtin_nontemporal_load(p + half_rows + i);
-  }
+  const size_t stride = static_cast<size_t>(2) * half_rows;
+  const float *const ps[2] = {partial + i, partial + half_rows + i};
+  float gu[2];
+  sum_splits<2>(ps, stride, split, gu);
+  const float g = gu[0], u = gu[1];
   const float a = bf16_to_f32(f32_to_bf16(g));
   const float act = bf16_to_f32(f32_to_bf16(a / (1.f + expf(-a))));
   y[i] = f32_to_bf16(act * bf16_to_f32(f32_to_bf16(u)));
