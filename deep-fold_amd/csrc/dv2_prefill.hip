@@ -41,6 +41,19 @@ __global__ __launch_bounds__(kColsBlock) void rms_cols(const uint16_t *__restric
   const int r0 = threadIdx.x / tpr;
   const int rstep = kColsBlock / tpr;
   const bool live = col < N;
+  // The first row this thread writes out (its only one at 5120 rows) is requested before the
+  // sums, which do not depend on it; rows and columns out of range read element 0 and drop it.
+  const int k_lo = blockIdx.x * rows_per_wg;
+  const int k_hi = min(rows, k_lo + rows_per_wg);
+  const bool first = live && k_lo + r0 < k_hi;
+  const size_t at0 = first ? static_cast<size_t>(k_lo + r0) * N + col : 0;
+  const uint16_t w0 = w[first ? k_lo + r0 : 0];
+  uint4 x0 = make_uint4(0, 0, 0, 0);
+  if constexpr (VEC) {
+    x0 = *reinterpret_cast<const uint4 *>(x + at0);
+  } else {
+    x0.x = x[at0];
+  }
   if (sq != nullptr) {
     // thread t adds the blocks t / N, t / N + 1024 / N, .. of column t % N; the 1024 / N
     // partial sums of a column meet in the 16 rows of part[], folded in a fixed order
@@ -48,10 +61,24 @@ __global__ __launch_bounds__(kColsBlock) void rms_cols(const uint16_t *__restric
     const int sub = threadIdx.x / N;
     const int nsub = kColsBlock / N;         // 16 .. 128
     const int fold = nsub / kColsWaves;      // partial sums per row of part[]
+    // The loads of 24 blocks (all of a thread's share at 5120 rows) are issued before the
+    // first add, every one unconditional: slots past the last block read the thread's first
+    // block again and are not added.  As a plain loop the sum was a chain of trips to memory.
     float t = 0.f;
-#pragma unroll 8
-    for (int b = sub; b < sq_blocks; b += nsub) {
-      t += sq[static_cast<size_t>(b) * N + scol];
+    constexpr int kBatch = 24;
+    for (int b0 = sub; b0 < sq_blocks; b0 += kBatch * nsub) {
+      float v[kBatch];
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) {
+        const int b = b0 + u * nsub;
+        v[u] = sq[static_cast<size_t>(b < sq_blocks ? b : sub) * N + scol];
+      }
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) {
+        if (b0 + u * nsub < sq_blocks) {
+          t += v[u];
+        }
+      }
     }
     for (int f = 0; f < fold; ++f) {
       if (sub % fold == f) {
@@ -114,13 +141,12 @@ __global__ __launch_bounds__(kColsBlock) void rms_cols(const uint16_t *__restric
   if (!live) {
     return;
   }
-  const int k_lo = blockIdx.x * rows_per_wg;
-  const int k_hi = min(rows, k_lo + rows_per_wg);
   for (int k = k_lo + r0; k < k_hi; k += rstep) {
     const size_t at = static_cast<size_t>(k) * N + col;
-    const float wk = bf16_to_f32(w[k]);
+    const bool pre = k == k_lo + r0;  // the row requested at the top
+    const float wk = bf16_to_f32(pre ? w0 : w[k]);
     if (VEC) {
-      const uint4 v = *reinterpret_cast<const uint4 *>(x + at);
+      const uint4 v = pre ? x0 : *reinterpret_cast<const uint4 *>(x + at);
       const uint32_t d[4] = {v.x, v.y, v.z, v.w};
       uint32_t o[4];
 #pragma unroll
@@ -131,7 +157,8 @@ __global__ __launch_bounds__(kColsBlock) void rms_cols(const uint16_t *__restric
       }
       *reinterpret_cast<uint4 *>(y + at) = make_uint4(o[0], o[1], o[2], o[3]);
     } else {
-      y[at] = f32_to_bf16((wk * bf16_to_f32(x[at])) * inv[col]);
+      const uint16_t xv = pre ? static_cast<uint16_t>(x0.x) : x[at];
+      y[at] = f32_to_bf16((wk * bf16_to_f32(xv)) * inv[col]);
     }
   }
 }
@@ -142,7 +169,7 @@ __global__ __launch_bounds__(kColsBlock) void rms_cols(const uint16_t *__restric
 // kv heads); a thread takes one token and eight consecutive dims d0 .. d0+7 of the lower
 // half plus their partners d0+half ..: lanes run along the tokens, so the reads of a row are
 // contiguous, and every store is a 16-byte vector of one token's row.  VEC needs hd % 16 == 0
-// and 16-byte aligned outputs; otherwise one pair of dims per thread.
+// and 16-byte aligned outputs and tables; otherwise one pair of dims per thread.
 template <bool VEC>
 __global__ __launch_bounds__(256) void rope_kv_cols(const uint16_t *__restrict__ q,
                                                     const uint16_t *__restrict__ k,
@@ -159,7 +186,7 @@ __global__ __launch_bounds__(256) void rope_kv_cols(const uint16_t *__restrict__
   const bool is_q = hid < n_q;
   const int head = is_q ? hid : hid - n_q;
   const uint16_t *src = (is_q ? q : k) + static_cast<size_t>(head) * hd * N;
-  const uint16_t *vsrc = v + static_cast<size_t>(head) * hd * N;
+  const uint16_t *vsrc = v + static_cast<size_t>(is_q ? 0 : head) * hd * N;
   const int half = hd / 2;
   constexpr int W = VEC ? 8 : 1;  // dims of each half a thread rotates
   const int items = (half / W) * N;
@@ -172,18 +199,46 @@ __global__ __launch_bounds__(256) void rope_kv_cols(const uint16_t *__restrict__
     }
     const uint16_t *c = cos + static_cast<size_t>(p) * hd;
     const uint16_t *sn = sin + static_cast<size_t>(p) * hd;
-    uint16_t lo[W], hi[W], vlo[W], vhi[W];
+    // Every load of the item is issued before the first rotation, and none sits under a
+    // branch (q heads read v's head 0, a valid address, and drop it): a load inside a
+    // conditional is waited for where the conditional ends, which made an item a chain of
+    // two dozen trips to memory.
+    uint16_t t0[W], t1[W], c0[W], c1[W], s0v[W], s1v[W], vlo[W], vhi[W];
+    if constexpr (VEC) {
+      // eight consecutive dims of a table row are one 16-byte vector
+      auto get8 = [](const uint16_t *src8, uint16_t (&dst)[W]) {
+        const uint4 t = *reinterpret_cast<const uint4 *>(src8);
+        const uint32_t d4[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+        for (int e = 0; e < W; ++e) {
+          dst[e] = static_cast<uint16_t>(d4[e >> 1] >> (16 * (e & 1)));
+        }
+      };
+      get8(c + d0, c0);
+      get8(c + d0 + half, c1);
+      get8(sn + d0, s0v);
+      get8(sn + d0 + half, s1v);
+    } else {
+      c0[0] = c[d0];
+      c1[0] = c[d0 + half];
+      s0v[0] = sn[d0];
+      s1v[0] = sn[d0 + half];
+    }
 #pragma unroll
     for (int e = 0; e < W; ++e) {
       const int d = d0 + e;
-      const float t0 = bf16_to_f32(src[static_cast<size_t>(d) * N + n]);
-      const float t1 = bf16_to_f32(src[static_cast<size_t>(d + half) * N + n]);
-      lo[e] = f32_to_bf16(t0 * bf16_to_f32(c[d]) + (-t1) * bf16_to_f32(sn[d]));
-      hi[e] = f32_to_bf16(t1 * bf16_to_f32(c[d + half]) + t0 * bf16_to_f32(sn[d + half]));
-      if (!is_q) {
-        vlo[e] = vsrc[static_cast<size_t>(d) * N + n];
-        vhi[e] = vsrc[static_cast<size_t>(d + half) * N + n];
-      }
+      t0[e] = src[static_cast<size_t>(d) * N + n];
+      t1[e] = src[static_cast<size_t>(d + half) * N + n];
+      vlo[e] = vsrc[static_cast<size_t>(d) * N + n];
+      vhi[e] = vsrc[static_cast<size_t>(d + half) * N + n];
+    }
+    uint16_t lo[W], hi[W];
+#pragma unroll
+    for (int e = 0; e < W; ++e) {
+      const float a0 = bf16_to_f32(t0[e]);
+      const float a1 = bf16_to_f32(t1[e]);
+      lo[e] = f32_to_bf16(a0 * bf16_to_f32(c0[e]) + (-a1) * bf16_to_f32(s0v[e]));
+      hi[e] = f32_to_bf16(a1 * bf16_to_f32(c1[e]) + a0 * bf16_to_f32(s1v[e]));
     }
     auto put = [](uint16_t *dst, const uint16_t (&val)[W]) {
       if constexpr (VEC) {
@@ -317,7 +372,8 @@ extern "C" int chr_dv2_rope_kv_cols(const void *q, const void *k, const void *v,
   if (N < 1 || N > kMaxCols) {
     return -2;
   }
-  const bool vec = (hd % 16) == 0 && aligned16(q_out) && aligned16(k_cache) && aligned16(v_cache);
+  const bool vec = (hd % 16) == 0 && aligned16(q_out) && aligned16(k_cache) && aligned16(v_cache) &&
+                   aligned16(cos) && aligned16(sin);
   const int items = (hd / 2 / (vec ? 8 : 1)) * N;
   const dim3 grid(static_cast<unsigned>(n_q + n_kv), static_cast<unsigned>((items + 255) / 256));
   hipStream_t st = static_cast<hipStream_t>(stream);

@@ -379,29 +379,32 @@ __global__ __launch_bounds__(kWave * kMaxGqaWaves) void attn_chunk_gqa(const Att
   const int stride = wg_waves * TPW;
   const size_t row_stride = static_cast<size_t>(a.n_kv) * HD;
 
-  uint32_t kraw[UNR][4], vraw[UNR][4];
-  auto load_block = [&](int t0) {
+  // Two register sets: the block after the one being multiplied is already on its way.  The
+  // requests are unconditional (rows past the prefix are clamped to its last row and masked
+  // by `live` below), so the wait before the arithmetic counts exactly the newer block.
+  struct Block {
+    uint32_t k[UNR][4], v[UNR][4];
+  };
+  auto load_block = [&](Block &b, int t0) {
 #pragma unroll
     for (int u = 0; u < UNR; ++u) {
-      const int t = t0 + grp * wg_waves + u * stride;
-      uint4 kv = make_uint4(0, 0, 0, 0), vv = make_uint4(0, 0, 0, 0);
-      if (t < vl) {
-        const size_t off =
-            static_cast<size_t>(t) * row_stride + static_cast<size_t>(kv_head) * HD + d0;
-        kv = *reinterpret_cast<const uint4 *>(a.k_cache + off);
-        vv = *reinterpret_cast<const uint4 *>(a.v_cache + off);
-      }
-      kraw[u][0] = kv.x;
-      kraw[u][1] = kv.y;
-      kraw[u][2] = kv.z;
-      kraw[u][3] = kv.w;
-      vraw[u][0] = vv.x;
-      vraw[u][1] = vv.y;
-      vraw[u][2] = vv.z;
-      vraw[u][3] = vv.w;
+      const int t = max(min(t0 + grp * wg_waves + u * stride, vl - 1), 0);  // vl may be 0
+      const size_t off =
+          static_cast<size_t>(t) * row_stride + static_cast<size_t>(kv_head) * HD + d0;
+      const uint4 kv = *reinterpret_cast<const uint4 *>(a.k_cache + off);
+      const uint4 vv = *reinterpret_cast<const uint4 *>(a.v_cache + off);
+      b.k[u][0] = kv.x;
+      b.k[u][1] = kv.y;
+      b.k[u][2] = kv.z;
+      b.k[u][3] = kv.w;
+      b.v[u][0] = vv.x;
+      b.v[u][1] = vv.y;
+      b.v[u][2] = vv.z;
+      b.v[u][3] = vv.w;
     }
   };
-  load_block(wave);
+  Block cur, nxt;
+  load_block(cur, wave);
 
   float qf[REP][8];
   const uint16_t *qh = a.q + static_cast<size_t>(tok) * a.q_tok_stride +
@@ -421,15 +424,13 @@ __global__ __launch_bounds__(kWave * kMaxGqaWaves) void attn_chunk_gqa(const Att
     }
   }
   for (int t0 = wave; t0 < vl; t0 += UNR * stride) {
-    if (t0 != wave) {
-      load_block(t0);
-    }
+    load_block(nxt, t0 + UNR * stride);
 #pragma unroll
     for (int u = 0; u < UNR; ++u) {
       const bool live = t0 + grp * wg_waves + u * stride < vl;
       float kf[8], vf[8];
-      widen8(make_uint4(kraw[u][0], kraw[u][1], kraw[u][2], kraw[u][3]), kf);
-      widen8(make_uint4(vraw[u][0], vraw[u][1], vraw[u][2], vraw[u][3]), vf);
+      widen8(make_uint4(cur.k[u][0], cur.k[u][1], cur.k[u][2], cur.k[u][3]), kf);
+      widen8(make_uint4(cur.v[u][0], cur.v[u][1], cur.v[u][2], cur.v[u][3]), vf);
 #pragma unroll
       for (int r = 0; r < REP; ++r) {
         float dot = 0.f;
@@ -451,6 +452,7 @@ __global__ __launch_bounds__(kWave * kMaxGqaWaves) void attn_chunk_gqa(const Att
         }
       }
     }
+    cur = nxt;
   }
 
   __shared__ float sm[REP][kMaxGqaWaves], sl[REP][kMaxGqaWaves];
