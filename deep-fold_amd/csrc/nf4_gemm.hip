@@ -806,18 +806,20 @@ int rows_dispatch(bool vec, int nc, int tps, const RowsArgs &a, dim3 grid, hipSt
 }
 
 
-// Sums of P elements over the splits, each in split order.  The loads of eight splits are
-// issued before the first add: written as a plain loop a sum is a chain of dependent trips to
-// memory (load, wait, add), seven of them for a 5120-wide K.  Every load is unconditional --
-// a load under a branch is waited for where the branch ends -- and slots past the last split
-// read split 0 again (the line is already on its way), their values unused.  The first eight
-// splits stand outside the loop, whose head waits for every load issued before it.
-template <int P>
-__device__ __forceinline__ void sum_splits(const float *const (&p)[P], size_t stride, int split,
-                                           float (&s)[P]) {
-  float v[P][8];
+// Sums of P elements over the splits, each in split order.  The loads of a batch of B splits
+// are issued before the first add: written as a plain loop a sum is a chain of dependent trips
+// to memory (load, wait, add), seven of them for a 5120-wide K.  Every load of a batch is
+// unconditional -- a load under a branch is waited for where the branch ends -- and slots
+// past the last split read split 0 again, their values unused; B is picked so that at most
+// half the slots are such repeats (the partials are read with the streaming hint, a repeat
+// is a second trip).  The first batch stands outside the loop, whose head waits for every
+// load issued before it.
+template <int P, int B>
+__device__ __forceinline__ void sum_splits_by(const float *const (&p)[P], size_t stride,
+                                              int split, float (&s)[P]) {
+  float v[P][B];
 #pragma unroll
-  for (int u = 0; u < 8; ++u) {
+  for (int u = 0; u < B; ++u) {
 #pragma unroll
     for (int e = 0; e < P; ++e) {
       v[e][u] = __builtin_nontemporal_load(p[e] + (u < split ? u : 0) * stride);
@@ -827,15 +829,15 @@ __device__ __forceinline__ void sum_splits(const float *const (&p)[P], size_t st
   for (int e = 0; e < P; ++e) {
     s[e] = 0.f;
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
+    for (int u = 0; u < B; ++u) {
       if (u < split) {
         s[e] += v[e][u];
       }
     }
   }
-  for (int j0 = 8; j0 < split; j0 += 8) {
+  for (int j0 = B; j0 < split; j0 += B) {
 #pragma unroll
-    for (int u = 0; u < 8; ++u) {
+    for (int u = 0; u < B; ++u) {
 #pragma unroll
       for (int e = 0; e < P; ++e) {
         v[e][u] = __builtin_nontemporal_load(p[e] + (j0 + u < split ? j0 + u : 0) * stride);
@@ -844,12 +846,24 @@ __device__ __forceinline__ void sum_splits(const float *const (&p)[P], size_t st
 #pragma unroll
     for (int e = 0; e < P; ++e) {
 #pragma unroll
-      for (int u = 0; u < 8; ++u) {
+      for (int u = 0; u < B; ++u) {
         if (j0 + u < split) {
           s[e] += v[e][u];
         }
       }
     }
+  }
+}
+
+template <int P>
+__device__ __forceinline__ void sum_splits(const float *const (&p)[P], size_t stride, int split,
+                                           float (&s)[P]) {
+  if (split <= 2) {
+    sum_splits_by<P, 2>(p, stride, split, s);
+  } else if (split <= 4) {
+    sum_splits_by<P, 4>(p, stride, split, s);
+  } else {
+    sum_splits_by<P, 8>(p, stride, split, s);
   }
 }
 
