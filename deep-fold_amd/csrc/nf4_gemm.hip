@@ -289,17 +289,22 @@ __device__ __forceinline__ void fetch_x(XRegs<NB> &r, const uint16_t *__restrict
     const int wave = tid >> 6, lane = tid & 63;
 #pragma unroll
     for (int rep = 0; rep < 2 * NB; ++rep) {
+      // Every load is issued whatever the item: a load under a branch is waited for where
+      // the branch ends, which would put the whole fetch in front of the arithmetic it is
+      // meant to overlap.  Items past the tile read vector 0 of a valid row, rows >= K read
+      // row K - 1; both are replaced by zeros afterwards.
       int kp, q;
-      uint4 a = make_uint4(0, 0, 0, 0), b = make_uint4(0, 0, 0, 0);
-      if (x_item(N, wave + 4 * rep, lane, kp, q)) {
-        const int k = k0 + 2 * kp;  // rows >= K are zero
-        if (k < K) {
-          a = *reinterpret_cast<const uint4 *>(x + static_cast<size_t>(k) * N + 8 * q);
-        }
-        if (k + 1 < K) {
-          b = *reinterpret_cast<const uint4 *>(x + static_cast<size_t>(k + 1) * N + 8 * q);
-        }
-      }
+      const bool item = x_item(N, wave + 4 * rep, lane, kp, q);
+      const int k = k0 + 2 * kp;
+      const int qv = item ? q : 0;
+      uint4 a = *reinterpret_cast<const uint4 *>(x + static_cast<size_t>(min(k, K - 1)) * N + 8 * qv);
+      uint4 b =
+          *reinterpret_cast<const uint4 *>(x + static_cast<size_t>(min(k + 1, K - 1)) * N + 8 * qv);
+      // masks, not branches: a conditional assignment compiles to a branch behind the load
+      const uint32_t ka = item && k < K ? ~0u : 0u;
+      const uint32_t kb = item && k + 1 < K ? ~0u : 0u;
+      a = make_uint4(a.x & ka, a.y & ka, a.z & ka, a.w & ka);
+      b = make_uint4(b.x & kb, b.y & kb, b.z & kb, b.w & kb);
       r.d[8 * rep + 0] = a.x;
       r.d[8 * rep + 1] = a.y;
       r.d[8 * rep + 2] = a.z;
@@ -359,10 +364,14 @@ __device__ __forceinline__ void fetch_w(WRegs &r, const uint8_t *__restrict__ pa
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int row = min(row_base + 8 * j + (lane >> 3), M - 1);
-    uint4 t = make_uint4(0x77777777u, 0x77777777u, 0x77777777u, 0x77777777u);
-    if (col < row_bytes) {
-      t = *reinterpret_cast<const uint4 *>(packed + static_cast<size_t>(row) * row_bytes + col);
-    }
+    // unconditional (see fetch_x): past the end of the row its last 16 bytes are read and
+    // replaced by the code of 0.0
+    uint4 t = *reinterpret_cast<const uint4 *>(packed + static_cast<size_t>(row) * row_bytes +
+                                               min(col, row_bytes - 16));
+    const uint32_t pad = col >= row_bytes ? ~0u : 0u;  // a mask, not a branch
+    const uint32_t fill = 0x77777777u & pad;
+    t = make_uint4((t.x & ~pad) | fill, (t.y & ~pad) | fill, (t.z & ~pad) | fill,
+                   (t.w & ~pad) | fill);
     r.d[4 * j + 0] = t.x;
     r.d[4 * j + 1] = t.y;
     r.d[4 * j + 2] = t.z;
@@ -372,8 +381,9 @@ __device__ __forceinline__ void fetch_w(WRegs &r, const uint8_t *__restrict__ pa
   const int g = (k0 >> 6) + ((lane & 1) << 1);
   const int groups = K_pad >> 6;
   const uint16_t *sp = scale + static_cast<size_t>(srow) * groups;
-  const uint32_t s0 = g < groups ? sp[g] : 0u;
-  const uint32_t s1 = g + 1 < groups ? sp[g + 1] : 0u;
+  const uint32_t l0 = sp[min(g, groups - 1)], l1 = sp[min(g + 1, groups - 1)];
+  const uint32_t s0 = g < groups ? l0 : 0u;
+  const uint32_t s1 = g + 1 < groups ? l1 : 0u;
   r.sc = s0 | (s1 << 16);
 }
 
@@ -455,9 +465,13 @@ __global__ __launch_bounds__(kGemmBlock) void gemm_mfma(const GemmSegs segs,
     scatter_x<VEC, NB>(xr, x, xs, k0, K, N, tid);
     stash_w(wr, wst, sst, lane);
     __syncthreads();
-    if (tile + 1 < tile1) {  // next tile's trip to memory overlaps this tile's arithmetic
-      fetch_w(wr, packed, scale, row_base, M, K_pad, k0 + kBK, lane);
-      fetch_x<VEC, NB>(xr, x, k0 + kBK, K, N, tid);
+    {
+      // The next tile's trip to memory overlaps this tile's arithmetic.  Unconditional, so
+      // that the wait for it lands where the data is used (the last tile fetches itself
+      // again and the result is dropped).
+      const int kn = min(k0 + kBK, (tile1 - 1) * kBK);
+      fetch_w(wr, packed, scale, row_base, M, K_pad, kn, lane);
+      fetch_x<VEC, NB>(xr, x, kn, K, N, tid);
     }
     const int kend = min(kBK, K_pad - k0);
     for (int kk = 0; kk < kend; kk += 64) {
