@@ -29,7 +29,9 @@ def rnd(shape, seed, scale=1.0):
     return oc.bf16_round((rng.standard_normal(shape) * scale).astype(np.float32))
 
 
-@pytest.mark.parametrize("rows,n", [(64, 1), (256, 7), (5120, 32), (1000, 16), (2050, 31), (5120, 64), (300, 40)])
+# (13824, 64): more rows per workgroup than one pass of its threads writes out
+@pytest.mark.parametrize("rows,n", [(64, 1), (256, 7), (5120, 32), (1000, 16), (2050, 31), (5120, 64), (300, 40),
+                                    (13824, 64)])
 def test_rms_cols(rows, n):
     say("rms_cols", rows, n)
     x = rnd((rows, n), rows + n, 1.5)
@@ -207,8 +209,9 @@ def test_gemm_with_bias_and_residual_in_its_reduction(m, k, n):
         nf4.nf4_gemm(dp, ds, x[:, :1].contiguous(), m, k, kp, bias=bias)
 
 
+# (13824, 1088, 64): 54 blocks of column sums per thread of the norm, more than one batch of loads
 @pytest.mark.parametrize("m,k,n", [(5120, 5120, 64), (5120, 13824, 32), (2050, 1088, 16), (130, 5120, 8),
-                                   (5120, 5120, 40), (256, 128, 64)])
+                                   (5120, 5120, 40), (256, 128, 64), (13824, 1088, 64)])
 def test_gemm_leaves_column_sums_for_the_norm(m, k, n):
     """The split-K reduce that stores y also leaves y's column sums of squares per block of
     rows; the RMSNorm that takes them gives what the one that reads the tile gives."""
