@@ -158,6 +158,32 @@ inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 constexpr int kTilesPerSplit = 3;
 constexpr int kMaxAutoSplit = 32;
 
+// Chunks of up to 32 columns run the row-streaming tile, whose workgroups (one slice of 1..4
+// K tiles each) all start at once: what a launch costs is the work of the busiest compute
+// unit, ceil(workgroups / compute units) slices, plus what every split adds to the partials
+// and their reduce.  Measured per K tile of a slice ~2 us, per split ~0.2 us, and a launch
+// that leaves one workgroup per compute unit (nothing to overlap its fetch with) ~1.4 times
+// its tiles: 5120x5120 takes 10 splits (15.3 us at N=32) where "three tiles per workgroup"
+// gave 7 (280 workgroups on 256 units: 16.9 us); 7168x5120 keeps 7, 5120x13824 keeps 18.
+// Ties go to the longer slice (fewer partials).  fallback: the split for slices this tile
+// cannot take (more than 4 x 32 K tiles).
+int pick_split_rows(int grid_x, int n_ktiles, int cus, int fallback) {
+  int best = 0, best_cost = 0;
+  for (int tps = 1; tps <= kRowsMaxTiles; ++tps) {
+    const int split = ceil_div(n_ktiles, tps);
+    if (split > kMaxAutoSplit || ceil_div(n_ktiles, split) != tps) {
+      continue;  // too many splits, or the same split as a shorter slice already gave
+    }
+    const int rounds = ceil_div(grid_x * split, cus);
+    const int cost = rounds * tps * (rounds == 1 ? 28 : 20) + split * 2;  // tenths of a us
+    if (best == 0 || cost <= best_cost) {
+      best = split;
+      best_cost = cost;
+    }
+  }
+  return best > 0 ? best : fallback;
+}
+
 void pick_split(int grid_x, int n_ktiles, int N, int have_ws, int *split, int *tiles_per_split) {
   const Tuning &t = tuning();
   int want = 1;
@@ -167,6 +193,9 @@ void pick_split(int grid_x, int n_ktiles, int N, int have_ws, int *split, int *t
     const int by_grid = std::max(1, ceil_div(target, grid_x));
     const int by_tiles = ceil_div(n_ktiles, kTilesPerSplit);
     want = t.split_k > 0 ? t.split_k : std::min(kMaxAutoSplit, std::min(by_tiles, by_grid));
+    if (t.split_k == 0 && N <= kBN) {
+      want = pick_split_rows(grid_x, n_ktiles, cus, want);
+    }
   }
   want = std::max(1, std::min(want, n_ktiles));
   const int tps = ceil_div(n_ktiles, want);

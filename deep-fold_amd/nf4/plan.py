@@ -155,6 +155,22 @@ def gemm_streams_rows(N: int, tiles_per_split: int) -> bool:  # noqa: N803
     return tiles_per_split <= (2 if N > 32 else 4)
 
 
+def _pick_split_rows(grid_x: int, n_ktiles: int, cus: int, fallback: int) -> int:
+    """Split for the row-streaming tile (chunks of up to 32 columns): slices of 1..4 K tiles,
+    cost = slices of the busiest compute unit x tiles (2 us each; 2.8 when a launch leaves one
+    workgroup per unit) + 0.2 us per split, ties to the longer slice."""
+    best, best_cost = 0, 0
+    for tps in range(1, 5):
+        split = _ceil_div(n_ktiles, tps)
+        if split > _MAX_AUTO_SPLIT or _ceil_div(n_ktiles, split) != tps:
+            continue
+        rounds = _ceil_div(grid_x * split, cus)
+        cost = rounds * tps * (28 if rounds == 1 else 20) + split * 2
+        if best == 0 or cost <= best_cost:
+            best, best_cost = split, cost
+    return best if best > 0 else fallback
+
+
 def _pick_split(grid_x: int, n_ktiles: int, N: int, have_ws: bool, force_split: int,  # noqa: N803
                 one_wave: int) -> tuple[int, int]:
     want = 1
@@ -164,6 +180,8 @@ def _pick_split(grid_x: int, n_ktiles: int, N: int, have_ws: bool, force_split: 
         by_grid = max(1, _ceil_div(target, grid_x))
         by_tiles = _ceil_div(n_ktiles, _TILES_PER_SPLIT)
         want = force_split if force_split > 0 else min(_MAX_AUTO_SPLIT, by_tiles, by_grid)
+        if force_split <= 0 and N <= 32:
+            want = _pick_split_rows(grid_x, n_ktiles, int(one_wave), want)
     want = max(1, min(want, n_ktiles))
     tiles_per_split = _ceil_div(n_ktiles, want)
     return _ceil_div(n_ktiles, tiles_per_split), tiles_per_split
