@@ -10,10 +10,11 @@ Kernel families by token count ``N`` (the reference's name for it; out features
 are ``M``, in features ``K``):
 
 * ``N == 1``  row-streaming GEMV, no split-K (path ``GEMV``).
-* ``N = 2..16`` / ``17..32``  MFMA tile, 128 rows per workgroup,
-  split-K over ``grid_y`` at about three K tiles per workgroup, up to three workgroups
-  per compute unit (paths ``PREFILL`` / ``PREFILL_N32``).
-* ``N = 33..64``  the same with twice the token columns
+* ``N = 2..16`` / ``17..32``  MFMA tile, 128 rows per workgroup, split-K over ``grid_y``
+  in slices of one to four K tiles, the length that costs the busiest compute unit least
+  (``_pick_split_rows``; paths ``PREFILL`` / ``PREFILL_N32``).
+* ``N = 33..64``  the same with twice the token columns, about three K tiles per workgroup
+  and no more splits than reach 1.6 workgroups per compute unit
   (``PREFILL_N64``); launched only through ``chr_nf4_gemm_ws_max`` with ``max_n`` > 32,
   the plain entries keep the reference's ceiling of 32.
 
