@@ -154,12 +154,12 @@ def bench_prefill(torch, nf4):
         by1 = algorithmic_bytes(m, k, 1)
         copies = -(-512 * 1024 * 1024 // by1) + 1
         weights = make_weights(torch, nf4, m, k, copies, seed=4321)
-        for n in (8, 16, 32):
+        for n in (8, 16, 32, 64):  # 64: the chunk width of the feature-major prefill
             x = (torch.randn((k, n), device="cuda") ).to(torch.bfloat16)
 
             def launch(i):
                 p, s = weights[i % copies]
-                nf4.nf4_gemm(p, s, x, m, k, k)
+                nf4.nf4_gemm(p, s, x, m, k, k, max_n=64)
 
             ms = graph_time(torch, launch, 3 * copies, reps=3)
             by = algorithmic_bytes(m, k, n)
