@@ -383,6 +383,48 @@ __device__ __forceinline__ void fill_pair_table(uint32_t *table, int wave, int l
   }
 }
 
+// ---- two-term pair table ----------------------------------------------------------------
+// A level is kept as the sum of two bf16 values: head = bf16(level) and tail =
+// bf16(level - head), 16 to 17 significant bits together, so the products with bf16
+// activations are exact and the weight error falls from 2^-9 to below 2^-17 relative: under
+// the rounding of an fp32 accumulation over a row.  An entry is 8 bytes {head pair, tail
+// pair}; 32 copies (lane & 31) make the 64-bit reads conflict-free (the LDS serves a
+// ds_read_b64 half a wavefront at a time), so the table is still 64 KB and a lookup is
+// still one v_perm_b32 (byte 1 = the packed byte, byte 0 = 8 * (lane & 31)) and one LDS
+// read; the second term costs one more v_dot2c_f32_bf16 per pair.
+constexpr uint32_t level_tail_bf16(uint32_t level_bits) {
+  const float level = __builtin_bit_cast(float, level_bits);
+  const float head = __builtin_bit_cast(float, bf16_bits_rne(level_bits) << 16);
+  return bf16_bits_rne(__builtin_bit_cast(uint32_t, level - head));
+}
+
+// Filled by a workgroup of exactly 16 wavefronts.  Wavefront v owns the bytes whose low
+// code is v; lanes 0..31 write the copies of high code 2jj, lanes 32..63 those of 2jj+1.
+__device__ __forceinline__ void fill_pair2_table(uint2 *table, int wave, int lane) {
+  const uint32_t lo_h = bf16_bits_rne(kLutBits[wave]);
+  const uint32_t lo_t = level_tail_bf16(kLutBits[wave]);
+  const int copy = lane & 31;
+  const bool odd = lane >= 32;
+#pragma unroll
+  for (int jj = 0; jj < 8; ++jj) {
+    const int j = 2 * jj + (odd ? 1 : 0);
+    const uint32_t hi_h = odd ? bf16_bits_rne(kLevelBits[2 * jj + 1]) : bf16_bits_rne(kLevelBits[2 * jj]);
+    const uint32_t hi_t = odd ? level_tail_bf16(kLevelBits[2 * jj + 1]) : level_tail_bf16(kLevelBits[2 * jj]);
+    table[((wave + 16 * j) << 5) + copy] = make_uint2(lo_h | (hi_h << 16), lo_t | (hi_t << 16));
+  }
+}
+
+__device__ __forceinline__ uint2 lds0_u64(uint32_t addr) {
+  const U32x2 v = *reinterpret_cast<const __attribute__((address_space(3))) U32x2 *>(addr);
+  return make_uint2(v.x, v.y);
+}
+
+template <int J>
+__device__ __forceinline__ uint2 pair2_at(uint32_t w, uint32_t lane8) {
+  constexpr uint32_t sel = 0x0C0C0400u + (static_cast<uint32_t>(J) << 8);
+  return lds0_u64(__builtin_amdgcn_perm(w, lane8, sel));
+}
+
 // One wavefront, R weight rows sharing x, which is read from global memory (K_pad/8
 // 16-byte pieces at x4).
 template <int R>
@@ -594,27 +636,53 @@ __device__ __forceinline__ void load_step(const uint8_t *const (&prow)[R],
   }
 }
 
-template <int R>
+// TERMS == 1: levels as one bf16 (pair table of dwords, 64 copies).  TERMS == 2: levels as
+// head + tail (two-term table, 32 copies of 8-byte entries).
+template <int R, int TERMS>
 __device__ __forceinline__ void dot_step(const uint2 (&w)[R], const uint16_t (&sc)[R],
                                          const uint4 *xs, int n_half, int t, int lane,
                                          float (&acc)[R]) {
-  const uint32_t lane4 = static_cast<uint32_t>(lane) << 2;
   const bool on = (t << 6) + lane < n_half;
   const uint4 *xp = xs + (t << 7) + lane;
   const uint4 x0 = xp[0], x1 = xp[64];
+  if constexpr (TERMS == 1) {
+    const uint32_t lane4 = static_cast<uint32_t>(lane) << 2;
 #pragma unroll
-  for (int r = 0; r < R; ++r) {
-    float pa = 0.f, pb = 0.f;
-    pa = dot2_bf16(pair_at<0>(w[r].x, lane4), x0.x, pa);
-    pb = dot2_bf16(pair_at<1>(w[r].x, lane4), x0.y, pb);
-    pa = dot2_bf16(pair_at<2>(w[r].x, lane4), x0.z, pa);
-    pb = dot2_bf16(pair_at<3>(w[r].x, lane4), x0.w, pb);
-    pa = dot2_bf16(pair_at<0>(w[r].y, lane4), x1.x, pa);
-    pb = dot2_bf16(pair_at<1>(w[r].y, lane4), x1.y, pb);
-    pa = dot2_bf16(pair_at<2>(w[r].y, lane4), x1.z, pa);
-    pb = dot2_bf16(pair_at<3>(w[r].y, lane4), x1.w, pb);
-    const float scale = on ? f16_to_f32(sc[r]) : 0.f;
-    acc[r] = fmaf(scale, pa + pb, acc[r]);
+    for (int r = 0; r < R; ++r) {
+      float pa = 0.f, pb = 0.f;
+      pa = dot2_bf16(pair_at<0>(w[r].x, lane4), x0.x, pa);
+      pb = dot2_bf16(pair_at<1>(w[r].x, lane4), x0.y, pb);
+      pa = dot2_bf16(pair_at<2>(w[r].x, lane4), x0.z, pa);
+      pb = dot2_bf16(pair_at<3>(w[r].x, lane4), x0.w, pb);
+      pa = dot2_bf16(pair_at<0>(w[r].y, lane4), x1.x, pa);
+      pb = dot2_bf16(pair_at<1>(w[r].y, lane4), x1.y, pb);
+      pa = dot2_bf16(pair_at<2>(w[r].y, lane4), x1.z, pa);
+      pb = dot2_bf16(pair_at<3>(w[r].y, lane4), x1.w, pb);
+      const float scale = on ? f16_to_f32(sc[r]) : 0.f;
+      acc[r] = fmaf(scale, pa + pb, acc[r]);
+    }
+  } else {
+    const uint32_t lane8 = static_cast<uint32_t>(lane & 31) << 3;
+    const uint32_t xw[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const uint2 e[8] = {pair2_at<0>(w[r].x, lane8), pair2_at<1>(w[r].x, lane8),
+                          pair2_at<2>(w[r].x, lane8), pair2_at<3>(w[r].x, lane8),
+                          pair2_at<0>(w[r].y, lane8), pair2_at<1>(w[r].y, lane8),
+                          pair2_at<2>(w[r].y, lane8), pair2_at<3>(w[r].y, lane8)};
+      // heads and tails in separate sums: the tails are 2^-9 of the heads and would lose
+      // their low bits if they were added into the large sum one by one
+      float ha = 0.f, hb = 0.f, ta = 0.f, tb = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; j += 2) {
+        ha = dot2_bf16(e[j].x, xw[j], ha);
+        ta = dot2_bf16(e[j].y, xw[j], ta);
+        hb = dot2_bf16(e[j + 1].x, xw[j + 1], hb);
+        tb = dot2_bf16(e[j + 1].y, xw[j + 1], tb);
+      }
+      const float scale = on ? f16_to_f32(sc[r]) : 0.f;
+      acc[r] = fmaf(scale, (ha + hb) + (ta + tb), acc[r]);
+    }
   }
 }
 
@@ -642,7 +710,7 @@ __device__ __forceinline__ float uniform_bf16(const uint16_t *p) {
 //   SWIGLU == false: R rows of one segment per group, epilogue y = acc (+ add).
 //   SWIGLU == true : R/2 gate rows and the matching R/2 up rows, y = silu(gate) * up
 //                    from the unrounded fp32 sums.
-template <int R, int S, bool SWIGLU>
+template <int R, int S, bool SWIGLU, int TERMS>
 __global__ __launch_bounds__(1024) void gemv_staged(const StreamArgs a) {
   extern __shared__ uint4 dyn_lds[];  // [pair table][GemvLds][x pieces], table at address 0
   char *base = reinterpret_cast<char *>(dyn_lds);
@@ -683,6 +751,14 @@ __global__ __launch_bounds__(1024) void gemv_staged(const StreamArgs a) {
     }                                                                   \
   }
 
+  auto fill_table = [&]() {
+    if constexpr (TERMS == 1) {
+      fill_pair_table(reinterpret_cast<uint32_t *>(dyn_lds), wave, lane);
+    } else {
+      fill_pair2_table(reinterpret_cast<uint2 *>(dyn_lds), wave, lane);
+    }
+  };
+
   // Order of the first requests: x, then the first item of weights, and only then the
   // wait for x.  Vector loads return in order, so x must be the older request or its wait
   // would be a wait for the weights too.  Each case below is its own straight-line path
@@ -694,10 +770,10 @@ __global__ __launch_bounds__(1024) void gemv_staged(const StreamArgs a) {
     if (n_items > 0) {
       group_pointers<R, SWIGLU>(a, first, prow, srow);
       CHR_REQUEST(wa, sa)
-      fill_pair_table(reinterpret_cast<uint32_t *>(dyn_lds), wave, lane);
+      fill_table();
       x_store(a, xs, lds.part, xv, xg);
     } else {
-      fill_pair_table(reinterpret_cast<uint32_t *>(dyn_lds), wave, lane);
+      fill_table();
       x_store(a, xs, lds.part, xv, xg);
     }
   } else {
@@ -708,7 +784,7 @@ __global__ __launch_bounds__(1024) void gemv_staged(const StreamArgs a) {
       group_pointers<R, SWIGLU>(a, first, prow, srow);
       CHR_REQUEST(wa, sa)
     }
-    fill_pair_table(reinterpret_cast<uint32_t *>(dyn_lds), wave, lane);
+    fill_table();
     stage_x(a, xs, lds.part);
   }
 
@@ -753,7 +829,7 @@ __global__ __launch_bounds__(1024) void gemv_staged(const StreamArgs a) {
 #define CHR_COMPUTE(W, SC)                                              \
   _Pragma("unroll") for (int j = 0; j < S; ++j) {                       \
     if (ci < n_steps_all) {                                             \
-      dot_step<R>(W[j], SC[j], xs, n_half, ct, lane, acc);              \
+      dot_step<R, TERMS>(W[j], SC[j], xs, n_half, ct, lane, acc);              \
       ++ci;                                                             \
       if (++ct == nsteps) {                                             \
         finish_group(cg);                                               \
@@ -874,6 +950,13 @@ int forced_staged() {
   return -1;
 }
 
+// Terms a level is kept as in the staged kernel: 2 (head + tail bf16, the default) or 1
+// (one bf16, 2^-9 relative weight error; CHR_NF4_GEMV_TERMS=1, read on every launch).
+int level_terms() {
+  const char *e = std::getenv("CHR_NF4_GEMV_TERMS");
+  return e != nullptr && e[0] == '1' && e[1] == '\0' ? 1 : 2;
+}
+
 constexpr int kThreads = 256;
 constexpr size_t kMaxDynLds = 150 * 1024;
 
@@ -943,11 +1026,19 @@ int launch_stream(StreamArgs &a, int n_seg, bool staged, hipStream_t st) {
     const size_t dyn = staged_lds_bytes(a.K_pad);
     const int waves = kStagedThreads / kWave;
     const int grid = std::min(device_cu_count(), (total + waves - 1) / waves);
-    constexpr auto kern = gemv_staged<R, kItemSteps, SWIGLU>;
-    if (prep_lds(kern, dyn) != 0) {
-      return -6;
+    if (level_terms() == 1) {
+      constexpr auto kern = gemv_staged<R, kItemSteps, SWIGLU, 1>;
+      if (prep_lds(kern, dyn) != 0) {
+        return -6;
+      }
+      kern<<<dim3(grid), dim3(kStagedThreads), dyn, st>>>(a);
+    } else {
+      constexpr auto kern = gemv_staged<R, kItemSteps, SWIGLU, 2>;
+      if (prep_lds(kern, dyn) != 0) {
+        return -6;
+      }
+      kern<<<dim3(grid), dim3(kStagedThreads), dyn, st>>>(a);
     }
-    kern<<<dim3(grid), dim3(kStagedThreads), dyn, st>>>(a);
   } else {
     const int waves = kThreads / kWave;
     // Long rows and few of them (a down projection): a wavefront walking a whole row pays

@@ -2,6 +2,8 @@
 
 from __future__ import annotations
 
+import os
+
 import numpy as np
 import torch
 
@@ -60,15 +62,29 @@ def takes_staged_gemv(m: int, k: int, *, fused: bool = False) -> bool:
     return fused or pyplan.gemv_is_staged(m, k)
 
 
+def staged_levels(terms: int | None = None) -> np.ndarray:
+    """The 16 levels as the staged GEMV multiplies them, in float64: head = bf16(level) plus
+    tail = bf16(level - head) (two terms, the default), or the head alone
+    (CHR_NF4_GEMV_TERMS=1)."""
+    if terms is None:
+        terms = 1 if os.environ.get("CHR_NF4_GEMV_TERMS") == "1" else 2
+    lut32 = oc.LUT.astype(np.float32)
+    head = oc.bf16_round(lut32)
+    if terms == 1:
+        return head.astype(np.float64)
+    tail = oc.bf16_round((lut32 - head).astype(np.float32))
+    return head.astype(np.float64) + tail.astype(np.float64)
+
+
 def staged_gemv_model(packed: np.ndarray, scale: np.ndarray, m: int, k: int,
-                      x: np.ndarray) -> np.ndarray:
-    """The staged GEMV's arithmetic in float64: levels rounded to bf16, products exact,
-    the fp16 scale applied to each group's sum.  x is [k] or [k, n]."""
+                      x: np.ndarray, terms: int | None = None) -> np.ndarray:
+    """The staged GEMV's arithmetic in float64: levels as ``staged_levels`` gives them,
+    products exact, the fp16 scale applied to each group's sum.  x is [k] or [k, n]."""
     kp = oc.k_pad(k)
     g = kp // oc.GROUP
     packed = np.asarray(packed).reshape(m, kp // 2)
     sc = np.ascontiguousarray(scale).view(np.float16).reshape(m, g).astype(np.float64)
-    lut = oc.bf16_round(oc.LUT.astype(np.float32)).astype(np.float64)
+    lut = staged_levels(terms)
     xs = np.zeros((kp,) + tuple(np.shape(x)[1:]), dtype=np.float64)
     xs[:k] = np.asarray(x, dtype=np.float64)
     xg = xs.reshape((g, oc.GROUP) + xs.shape[1:])
