@@ -9,9 +9,13 @@ lm_head, layers[*].{norm1,norm2,q,k,v,wqkv,o,gate,up,down}).
 
 Pinned by: each piece against the textbook routine it reduces to (torch
 ``rms_norm``, ``silu``, ``scaled_dot_product_attention``, rotate-half RoPE) in
-``tests/test_step_oracle.py``; the composite has no stored answer in the
-reference (its tests compute the ids at run time), so the whole-step comparison
-is GPU path vs this oracle on the same seeded models.
+``tests/test_step_oracle.py``; the composition (norm placement, residuals, RoPE on
+q and k only, GQA head map, bias placement, InternLM's wqkv row order) against
+``transformers``' ``LlamaForCausalLM`` / ``Qwen2ForCausalLM`` in float32 on the
+dequantised weights of the same seeded models, teacher-forced logits to 2e-5 of
+the logit scale and the greedy chain token by token
+(``tests/test_step_oracle_hf.py``).  The reference itself stores no expected ids
+(its tests compute them at run time).
 """
 
 from __future__ import annotations
