@@ -61,26 +61,33 @@ def make_weights(torch, nf4, m: int, k: int, copies: int, seed: int):
 
 
 def graph_time(torch, launch, n_launches: int, reps: int = 5) -> float:
-    """Capture ``n_launches`` calls of ``launch(i)`` into one HIP graph and return
-    the median over ``reps`` replays of the average milliseconds per launch (events on the
-    capture stream bracket each replay)."""
+    """Capture ``n_launches`` calls of ``launch(i)`` into a HIP graph, once per timed window
+    with ``i`` running on from where the window before stopped (so a window never starts on
+    the copies the one before it has just left in the caches), and return the median over
+    the ``reps`` windows of the average milliseconds per launch.  Events on the capture
+    stream bracket each replay."""
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
         for i in range(min(n_launches, 32)):
             launch(i)
         side.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        graph.capture_begin()
-        for i in range(n_launches):
-            launch(i)
-        graph.capture_end()
-        graph.replay()
+        graphs = []
+        for r in range(reps + 1):
+            graph = torch.cuda.CUDAGraph()
+            graph.capture_begin()
+            for i in range(n_launches):
+                launch(r * n_launches + i)
+            graph.capture_end()
+            graphs.append(graph)
+        graphs[0].replay()   # untimed: first replay of a graph pays its upload
+        for graph in graphs[1:]:
+            graph.replay()
         side.synchronize()
         e0 = torch.cuda.Event(enable_timing=True)
         e1 = torch.cuda.Event(enable_timing=True)
         windows = []
-        for _ in range(reps):
+        for graph in graphs[1:]:
             e0.record(side)
             graph.replay()
             e1.record(side)
@@ -89,6 +96,42 @@ def graph_time(torch, launch, n_launches: int, reps: int = 5) -> float:
     torch.cuda.current_stream().wait_stream(side)
     windows.sort()
     return windows[len(windows) // 2] / n_launches
+
+
+#: kernel forms of the N=1 path, by the environment switches the library reads per launch
+GEMV_FORMS = {
+    # levels as head + tail bf16 (17 significant bits), exact products, fp32 accumulation
+    "two_term": {"CHR_NF4_GEMV_STAGED": None, "CHR_NF4_GEMV_TERMS": None},
+    # levels rounded to one bf16
+    "one_term": {"CHR_NF4_GEMV_STAGED": None, "CHR_NF4_GEMV_TERMS": "1"},
+    # 16 fp32 levels, x widened to fp32, 128-bit loads (the plain kernel)
+    "fp32_levels": {"CHR_NF4_GEMV_STAGED": "0", "CHR_NF4_GEMV_TERMS": None},
+}
+
+
+class gemv_form:
+    """Select a kernel form for the launches (and captures) inside the block."""
+
+    def __init__(self, name: str) -> None:
+        self.env = GEMV_FORMS[name]
+        self.saved: dict[str, str | None] = {}
+
+    def __enter__(self):
+        for k, v in self.env.items():
+            self.saved[k] = os.environ.get(k)
+            if v is None:
+                os.environ.pop(k, None)
+            else:
+                os.environ[k] = v
+        return self
+
+    def __exit__(self, *exc):
+        for k, v in self.saved.items():
+            if v is None:
+                os.environ.pop(k, None)
+            else:
+                os.environ[k] = v
+        return False
 
 
 def bench_gemv(torch, nf4, steps: int, warmup: int, copies: int):
@@ -114,9 +157,13 @@ def bench_gemv(torch, nf4, steps: int, warmup: int, copies: int):
     torch.cuda.synchronize()
     eager_ms = (time.perf_counter() - t0) * 1e3 / steps
     ms = graph_time(torch, launch, steps)
+    forms = {}
+    for name in ("one_term", "fp32_levels"):
+        with gemv_form(name):
+            forms[name] = graph_time(torch, launch, steps)
     del weights
     torch.cuda.empty_cache()
-    return ms, eager_ms, copies, by
+    return ms, eager_ms, copies, by, forms
 
 
 def bench_gemv_shapes(torch, nf4):
@@ -172,8 +219,20 @@ def bench_prefill(torch, nf4):
     return rows
 
 
+#: the decode configurations the metric names, per architecture: (prompt tokens, prefill chunk
+#: width or None for the launches' own 64, new tokens).  3B: 512-token prompt, 256 tokens.
+#: 20B: 1024-token prompt prefilled in 32-position chunks, 256 tokens.  32B: the step at a
+#: 2048-token context (the last 256 positions of the cache).
+DECODE_CONFIGS = {
+    "3b": (512, None, 256),
+    "14b": (512, None, 256),
+    "20b": (1024, 32, 256),
+    "32b": (2048 - 256 - 1, None, 256),
+}
+
+
 def bench_decode(torch, spec_name: str, prompt_len: int, new_tokens: int, schedule: str | None = None,
-                 prefill_width: int | None = None):
+                 prefill_width: int | None = None, torch_glue: bool = True):
     """Resident greedy decode on random-init weights: chunked prefill of a random
     prompt, then ``new_tokens`` graph replays with no host read in between."""
     from deepfold_amd import decodev2 as dv2
@@ -188,15 +247,17 @@ def bench_decode(torch, spec_name: str, prompt_len: int, new_tokens: int, schedu
     g = torch.Generator(device="cpu")
     g.manual_seed(7)
     prompt = torch.randint(0, spec.vocab, (prompt_len,), generator=g).tolist()
-    # prefill in 32-position chunks: the token-major torch glue of the reference's sequence,
-    # then the feature-major launches (first pass captures one graph per chunk width, the
-    # timed pass replays them)
-    state.reset()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    dv2.consume_prompt(state, weights, prompt)
-    torch.cuda.synchronize()
-    prefill_glue_ms = (time.perf_counter() - t0) * 1e3
+    # prefill: the token-major torch glue of the reference's sequence (32-position chunks;
+    # timed on request only, it is slow), then the feature-major launches (first pass
+    # captures one graph per chunk width, the timed pass replays them)
+    prefill_glue_ms = None
+    if torch_glue:
+        state.reset()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        dv2.consume_prompt(state, weights, prompt)
+        torch.cuda.synchronize()
+        prefill_glue_ms = (time.perf_counter() - t0) * 1e3
     pre = dv2.ChunkPrefill(state, weights, width=prefill_width)
     width = pre.width
     state.reset()
@@ -209,7 +270,6 @@ def bench_decode(torch, spec_name: str, prompt_len: int, new_tokens: int, schedu
     prefill_ms = (time.perf_counter() - t0) * 1e3
     del pre
     state.token.copy_(state.next_token)
-    # graph capture advances the state by warmup+1 tokens; that is part of the run
     graph = dv2.capture_greedy(state, weights, warmup=2, schedule=schedule)
     torch.cuda.synchronize()
     start_pos = int(state.position.item())
@@ -258,6 +318,7 @@ def bench_decode(torch, spec_name: str, prompt_len: int, new_tokens: int, schedu
         "roofline_ms_per_token": roof_ms, "roofline_tok_s": 1e3 / roof_ms,
         "roofline_frac": roof_ms / ms_tok, "achieved_gbps": bytes_tok / (ms_tok * 1e-3) / 1e9,
         "weights_load_s": load_s,
+        "gemv_levels": "two bf16 terms (default)",
     }
     del graph, state, weights
     torch.cuda.empty_cache()
@@ -329,22 +390,26 @@ def cpu_baseline(m: int, k: int, budget_s: float = 12.0) -> dict:
     }
 
 
-def bench_ring(torch, nf4, n_matrices: int = 6, forwards: int = 10):
-    """Streaming variant (weights in pinned host memory, two device slots): a tape of
-    32B-architecture FFN matrices (27648x5120) through the ring, one GEMV each."""
+def bench_ring(torch, nf4, n_matrices: int = 192, distinct: int = 48, forwards: int = 3):
+    """Streaming variant at model scale: the FFN matrices of the 32B architecture (64 layers
+    x gate, up, down = 192 matrices of 27648x5120 codes, 75.2 MB each, 14.4 GB per token)
+    live in pinned host memory and pass through two device slots, one GEMV each.  The tape
+    has 192 entries over ``distinct`` different host images (the bytes that cross the bus per
+    token are the same; holding 192 distinct images would only pin more host memory)."""
     from deepfold_amd import ring as rg
 
     m, k = 27648, 5120
     g = torch.Generator(device="cuda")
     g.manual_seed(5)
-    tape = []
-    for i in range(n_matrices):
+    images = []
+    for i in range(distinct):
         w = torch.randn((m, k), generator=g, device="cuda", dtype=torch.float32) * 0.02
         packed, scale = nf4.nf4_quantize(w)
         del w
-        tape.append(rg.StreamedMatrix.on_host(f"ffn{i}", rg.HostImage.from_blobs(packed.cpu(), scale.cpu(), k)))
+        images.append(rg.HostImage.from_blobs(packed, scale, k))
         del packed, scale
-    ring = rg.CopyRing(rg.SlotPair(tape[0].host_image.nbytes, "cuda"))
+    tape = [rg.StreamedMatrix.on_host(f"ffn{i}", images[i % distinct]) for i in range(n_matrices)]
+    ring = rg.CopyRing(rg.SlotPair(images[0].nbytes, "cuda"))
     x = torch.randn(k, generator=g, device="cuda").to(torch.bfloat16)
 
     def forward():
@@ -361,14 +426,16 @@ def bench_ring(torch, nf4, n_matrices: int = 6, forwards: int = 10):
         forward()
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / forwards
-    nbytes = n_matrices * tape[0].host_image.nbytes
+    nbytes = n_matrices * images[0].nbytes
     return {
-        "workload": f"{n_matrices} x NF4 [{m},{k}] streamed from pinned host memory through 2 slots, "
-                    "one GEMV each",
-        "slot_bytes": tape[0].host_image.nbytes,
+        "workload": f"{n_matrices} x NF4 [{m},{k}] (the 32B architecture's FFN matrices of one token, "
+                    f"{distinct} distinct host images) streamed from pinned host memory through 2 "
+                    "slots, one GEMV each",
+        "slot_bytes": images[0].nbytes,
+        "bytes_per_forward": nbytes,
         "ms_per_forward": dt * 1e3,
         "h2d_gbps": nbytes / dt / 1e9,
-        "pinned": rg.is_pinned(tape[0].host_image.arena),
+        "pinned": rg.is_pinned(images[0].arena),
         "copies_per_forward": n_matrices,
     }
 
@@ -383,14 +450,16 @@ def main() -> int:
     ap.add_argument("--no-decode", action="store_true", help="skip the model decode leg")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill GEMM sweep")
     ap.add_argument("--no-ring", action="store_true", help="skip the host-streaming ring leg")
-    ap.add_argument("--decode-models", default="14b", help="comma list of 3b,14b,20b,32b")
+    ap.add_argument("--decode-models", default="3b,14b,20b,32b", help="comma list of 3b,14b,20b,32b")
     ap.add_argument("--no-shapes", action="store_true", help="skip the GEMV sweep over other shapes")
     ap.add_argument("--schedule", default=None, help="decode launch schedule: plain or fold_rms")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
                     help="first run four plain device copies of this size (a kernel of known "
                          "traffic to scale hardware counters by)")
-    ap.add_argument("--prompt", type=int, default=512)
-    ap.add_argument("--new-tokens", type=int, default=256)
+    ap.add_argument("--prompt", type=int, default=None,
+                    help="prompt tokens of every decode model (default: each model's own "
+                         "configuration, see DECODE_CONFIGS)")
+    ap.add_argument("--new-tokens", type=int, default=None)
     ap.add_argument("--prefill-width", type=int, default=None,
                     help="tokens per prefill chunk of the feature-major prefill (default 64; the "
                          "reference's chunks are 32)")
@@ -417,8 +486,16 @@ def main() -> int:
         torch.cuda.synchronize()
         del src, dst
 
-    ms, eager_ms, copies, by = bench_gemv(torch, nf4, args.steps, args.warmup, args.copies)
+    ms, eager_ms, copies, by, forms = bench_gemv(torch, nf4, args.steps, args.warmup, args.copies)
     achieved = by / (ms * 1e-3) / 1e9
+
+    def roofline_of(ms_launch: float, kernel: str, multiplies: str) -> dict:
+        a = by / (ms_launch * 1e-3) / 1e9
+        return {"bound": "hbm", "achieved": a, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                "frac": a / HBM_PEAK_GBPS, "traffic": None, "kernel": kernel,
+                "multiplies": multiplies, "us_per_launch": ms_launch * 1e3,
+                "algorithmic_bytes_per_launch": by}
+
     out = {
         "metric": "nf4_gemv_hbm_gbps",
         "value": achieved,
@@ -430,7 +507,11 @@ def main() -> int:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32",
+        # what the timed kernel multiplies: NF4 levels kept as two bf16 terms (head + tail,
+        # 17 significant bits) times bf16 activations, exact products, fp32 accumulation
+        "dtype": "bf16",
+        "dtype_note": "levels as head+tail bf16 pairs x bf16 activations (v_dot2c_f32_bf16), "
+                      "fp32 accumulate, one bf16 rounding of y",
         "data": "synthetic",
         "config": {
             "workload": f"decode GEMV x[1,{K}] bf16 @ W[{M},{K}] NF4 group-64, {copies} rotating weight "
@@ -445,16 +526,36 @@ def main() -> int:
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS,
             "traffic": GEMV_TRAFFIC_BYTES if (M, K) == (13824, 5120) else None,
-            "kernel": "gemv_staged",
+            "kernel": "gemv_staged (two-term levels)",
             "algorithmic_bytes_per_launch": by,
         },
+        # the same launches on the same copies through the other two kernel forms
+        "roofline_one_term": roofline_of(forms["one_term"], "gemv_staged (one bf16 level)",
+                                         "bf16 levels x bf16 activations"),
+        "roofline_fp32_levels": roofline_of(forms["fp32_levels"], "gemv_stream (plain)",
+                                            "fp32 levels x fp32-widened activations, 128-bit loads"),
     }
     if not args.no_shapes:
         out["gemv_shapes"] = bench_gemv_shapes(torch, nf4)
     if not args.no_decode:
-        out["decode"] = [bench_decode(torch, name.strip(), args.prompt, args.new_tokens, args.schedule,
-                                      args.prefill_width)
-                         for name in args.decode_models.split(",") if name.strip()]
+        rows = []
+        for name in (n.strip() for n in args.decode_models.split(",")):
+            if not name:
+                continue
+            prompt, width, new = DECODE_CONFIGS[name]
+            prompt = args.prompt if args.prompt is not None else prompt
+            new = args.new_tokens if args.new_tokens is not None else new
+            width = args.prefill_width if args.prefill_width is not None else width
+            rows.append(bench_decode(torch, name, prompt, new, args.schedule, width,
+                                     torch_glue=(name == "14b")))
+            if name == "14b":
+                # the same model with one-term (bf16) levels in the GEMVs: the faster,
+                # less exact form a caller can opt into
+                with gemv_form("one_term"):
+                    fast = bench_decode(torch, name, prompt, new, args.schedule, width, torch_glue=False)
+                fast["gemv_levels"] = "one bf16 term (CHR_NF4_GEMV_TERMS=1)"
+                rows.append(fast)
+        out["decode"] = rows
     if not args.no_prefill:
         out["prefill"] = bench_prefill(torch, nf4)
     if not args.no_ring:

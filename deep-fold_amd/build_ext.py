@@ -36,6 +36,10 @@ def hipcc() -> str:
     return exe
 
 
+def have_hipcc() -> bool:
+    return bool(shutil.which("hipcc")) or os.path.exists("/opt/rocm/bin/hipcc")
+
+
 def stale() -> bool:
     if not os.path.exists(LIB):
         return True

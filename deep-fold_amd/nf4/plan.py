@@ -26,6 +26,8 @@ one: 256 threads, weights staged through LDS one tile ahead.
 
 from __future__ import annotations
 
+import os
+
 from dataclasses import dataclass
 
 __all__ = [
@@ -152,8 +154,23 @@ def gemm_streams_rows(N: int, tiles_per_split: int) -> bool:  # noqa: N803
     """Whether a launch runs the row-streaming tile (weights straight from global memory into
     the MFMA operand, the whole K slice requested at once) instead of the K-tiled one: slices
     of at most four K tiles, two for chunks wider than 32 columns.  ``CHR_NF4_GEMM_ROWS=0`` in
-    the environment keeps the library on the K-tiled kernel; this mirror ignores it."""
-    return tiles_per_split <= (2 if N > 32 else 4)
+    the environment keeps the library on the K-tiled kernel; like the library, this mirror
+    reads the switch once, when it is first needed."""
+    return _rows_kernel_on() and tiles_per_split <= (2 if N > 32 else 4)
+
+
+_ROWS_ON: bool | None = None
+
+
+def _rows_kernel_on() -> bool:
+    global _ROWS_ON
+    if _ROWS_ON is None:
+        raw = os.environ.get("CHR_NF4_GEMM_ROWS", "")
+        try:
+            _ROWS_ON = int(raw) != 0 if raw.strip() else True
+        except ValueError:
+            _ROWS_ON = False     # atoi() of a non-number is 0
+    return _ROWS_ON
 
 
 def _pick_split_rows(grid_x: int, n_ktiles: int, cus: int, fallback: int) -> int:

@@ -1,10 +1,12 @@
-"""Host side of a streamed NF4 matrix: one pinned byte arena holding the packed codes
-followed by the fp16 scales, so the whole matrix is a single host-to-device copy
-(``gpu/host/host_image.py:31-137``).
+"""Host side of a streamed NF4 matrix (operator surface of
+``gpu/host/host_image.py:31-137``): one byte arena holding the packed codes and, right
+behind them, the fp16 scales, so that a matrix moves to the device as a single copy and a
+slot can be viewed as (packed, scale) without touching a byte.
 
-The arena is allocated pinned from the start when a GPU is present (pinning memory
-that already exists is not available on these hosts); without a GPU it is ordinary
-memory, which is what the protocol tests use."""
+With a GPU present the arena is pinned memory from the moment it is allocated (these
+hosts cannot pin memory that already exists); without one it is ordinary memory, which is
+what the protocol tests use.
+"""
 
 from __future__ import annotations
 
@@ -16,84 +18,91 @@ from ..nf4.plan import k_pad
 
 __all__ = ["GROUP", "HostImage", "arena_nbytes", "is_pinned", "pack_arena", "unpack_arena"]
 
-GROUP = 64
+GROUP = 64          # weights per fp16 scale
+_SCALE_BYTES = 2
+
+
+def _layout(m: int, pad: int) -> tuple[int, int, int]:
+    """(bytes of codes, scale groups per row, bytes of scales) of an ``[m, pad]`` matrix."""
+    groups = pad // GROUP
+    return m * (pad // 2), groups, m * groups * _SCALE_BYTES
 
 
 def arena_nbytes(m: int, k: int) -> int:
-    """Bytes of packed‖scale for an ``[M, K]`` matrix."""
-    pad = k_pad(int(k))
-    return int(m) * (pad // 2) + int(m) * (pad // GROUP) * 2
+    """Bytes of codes plus scales for an ``[M, K]`` matrix."""
+    codes, _, scales = _layout(int(m), k_pad(int(k)))
+    return codes + scales
 
 
 def is_pinned(t: torch.Tensor) -> bool:
-    """``Tensor.is_pinned`` is a method; a bare truth test of it is always true."""
-    return bool(t.is_cpu and t.is_pinned())
-
-
-def _new_arena(n: int) -> torch.Tensor:
-    pin = torch.cuda.is_available()
-    return torch.empty(int(n), dtype=torch.uint8, pin_memory=pin)
+    """Whether ``t`` is page-locked host memory (``Tensor.is_pinned`` is a method: testing
+    the attribute itself is always true)."""
+    return t.device.type == "cpu" and bool(t.is_pinned())
 
 
 def pack_arena(packed: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
-    """``packed [M, K_pad/2]`` u8 and ``scale [M, K_pad/64]`` f16 -> one 1-d u8 arena."""
-    if packed.dtype is not torch.uint8:
+    """``packed [M, K_pad/2]`` u8 and ``scale [M, K_pad/64]`` f16 -> a new 1-d u8 arena,
+    codes first."""
+    if packed.dtype != torch.uint8:
         raise TypeError(f"packed must be uint8, got {packed.dtype}")
-    if scale.dtype is not torch.float16:
+    if scale.dtype != torch.float16:
         raise TypeError(f"scale must be float16, got {scale.dtype}")
-    if packed.dim() != 2 or scale.dim() != 2:
+    if packed.ndim != 2 or scale.ndim != 2:
         raise ValueError(f"packed {tuple(packed.shape)} / scale {tuple(scale.shape)}: expected rank 2")
-    m, width = int(packed.shape[0]), int(packed.shape[1])
-    if int(scale.shape[0]) != m:
-        raise ValueError(f"M mismatch: packed {m} vs scale {int(scale.shape[0])}")
-    groups = (width * 2) // GROUP
-    if int(scale.shape[1]) != groups:
-        raise ValueError(f"scale n_groups {int(scale.shape[1])} != K_pad/64 ({groups})")
-    code_bytes = packed.contiguous().reshape(-1).cpu()
-    scale_bytes = scale.contiguous().cpu().view(torch.uint8).reshape(-1)
-    arena = _new_arena(code_bytes.numel() + scale_bytes.numel())
-    arena[: code_bytes.numel()].copy_(code_bytes)
-    arena[code_bytes.numel():].copy_(scale_bytes)
+    m, row_bytes = packed.shape
+    codes, groups, scales = _layout(m, 2 * row_bytes)
+    if scale.shape[0] != m:
+        raise ValueError(f"M mismatch: packed {m} vs scale {scale.shape[0]}")
+    if scale.shape[1] != groups:
+        raise ValueError(f"scale n_groups {scale.shape[1]} != K_pad/64 ({groups})")
+    arena = torch.empty(codes + scales, dtype=torch.uint8, pin_memory=torch.cuda.is_available())
+    # write through the two views the arena will later be read through
+    into_codes, into_scales = unpack_arena(arena, m, 2 * row_bytes, k_pad_=2 * row_bytes)
+    into_codes.copy_(packed)
+    into_scales.copy_(scale)
     return arena
 
 
 def unpack_arena(arena: torch.Tensor, m: int, k: int, *, k_pad_: int | None = None):
-    """packed / scale views of ``arena`` (same storage, no copy)."""
-    if arena.dtype is not torch.uint8 or arena.dim() != 1:
+    """(packed, scale) views of ``arena``: the same storage, no copy."""
+    if arena.dtype != torch.uint8 or arena.ndim != 1:
         raise TypeError(f"arena must be uint8 1d, got {arena.dtype} {tuple(arena.shape)}")
-    m = int(m)
-    pad = int(k_pad_) if k_pad_ is not None else k_pad(int(k))
-    code_n = m * (pad // 2)
-    groups = pad // GROUP
-    if int(arena.numel()) != code_n + m * groups * 2:
-        raise ValueError(f"arena {int(arena.numel())} bytes != packed {code_n} + scale {m * groups * 2}")
-    return arena[:code_n].view(m, pad // 2), arena[code_n:].view(torch.float16).view(m, groups)
+    rows = int(m)
+    pad = k_pad(int(k)) if k_pad_ is None else int(k_pad_)
+    codes, groups, scales = _layout(rows, pad)
+    if arena.numel() != codes + scales:
+        raise ValueError(f"arena {arena.numel()} bytes != packed {codes} + scale {scales}")
+    packed, tail = arena.split([codes, scales])
+    return packed.view(rows, pad // 2), tail.view(torch.float16).view(rows, groups)
 
 
 @dataclass(frozen=True)
 class HostImage:
-    """One NF4 matrix on the host as packed‖scale."""
+    """One NF4 matrix on the host: codes then scales in one arena."""
 
     arena: torch.Tensor
     M: int
     K: int
     K_pad: int
 
+    def _views(self):
+        return unpack_arena(self.arena, self.M, self.K, k_pad_=self.K_pad)
+
     @property
     def packed(self) -> torch.Tensor:
-        return unpack_arena(self.arena, self.M, self.K, k_pad_=self.K_pad)[0]
+        return self._views()[0]
 
     @property
     def scale(self) -> torch.Tensor:
-        return unpack_arena(self.arena, self.M, self.K, k_pad_=self.K_pad)[1]
+        return self._views()[1]
 
     @property
     def nbytes(self) -> int:
-        return int(self.arena.numel())
+        return self.arena.numel()
 
     @classmethod
     def from_blobs(cls, packed: torch.Tensor, scale: torch.Tensor, k: int) -> "HostImage":
-        pad = int(packed.shape[1]) * 2
+        pad = 2 * int(packed.shape[1])
         if pad != k_pad(int(k)):
             raise ValueError(f"packed width {packed.shape[1]} != K_pad/2 ({k_pad(int(k)) // 2})")
         return cls(pack_arena(packed, scale), int(packed.shape[0]), int(k), pad)

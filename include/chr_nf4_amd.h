@@ -73,8 +73,9 @@ int chr_nf4_gemm_plan(const chr_nf4_dev_t *w, int32_t N, int32_t have_ws,
 int chr_nf4_gemm_ws(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N,
                     float *ws, int64_t ws_floats, void *stream);
 
-/* Same launch, N up to max_n (clamped to [1, 64]); N > 32 is refused with -2
- * because no 64-column tile is built, as in the reference's live path.
+/* Same launch with the column ceiling given by the caller: max_n is clamped to
+ * [1, 64] and N > max_n is refused with -2.  Chunks of 33..64 columns run the
+ * 64-column tile (the reference plans that width but never launches it).
  * Replaces chr_nf4_gemm_ws_max (chr_gpu.h:75-76; nf4_gemm.cu:1669-1771). */
 int chr_nf4_gemm_ws_max(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N,
                         float *ws, int64_t ws_floats, void *stream, int32_t max_n);

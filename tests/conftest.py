@@ -18,11 +18,14 @@ def pytest_configure(config):
     from oracle import nf4_oracle
 
     nf4_oracle.build(force=False)
-    # The HIP library is built ahead of time (hipcc cross-compiles); build it
-    # here only when nothing is there.
+    # The HIP library is built ahead of time (hipcc cross-compiles).  Where the toolchain
+    # is at hand, rebuild when a source is newer than the library, so that an edited
+    # kernel is never tested through a stale build; without hipcc use what is there.
     from deepfold_amd import build_ext
 
     if not os.path.exists(build_ext.LIB):
+        build_ext.build(force=True)
+    elif build_ext.stale() and build_ext.have_hipcc():
         build_ext.build(force=True)
 
 

@@ -483,13 +483,20 @@ def test_gemm_n1_routes_to_gemv():
     assert (bf16_bits(y) == bf16_bits(nf4.nf4_gemv(dp, ds, x, m, k, k))).all()
 
 
-def test_gemm_quantized_prefill_shape():
-    m, k, n = 7168, 5120, 32
-    say("gemm qkv shape", m, k, n)
-    w, p, s, dp, ds = quantized(m, k, 21)
-    x = rand_x(k, n, 16)
-    y = nf4.nf4_gemm(dp, ds, bf16_tensor(x), m, k, k)
-    check_linear(y, oc.c_matmul_f64(oc.bf16_round(oc.c_decode(p, s, m, k)), x), what="prefill qkv")
+PREFILL_14B = [("qkv", 7168, 5120), ("o", 5120, 5120), ("gate_up", 13824, 5120), ("down", 5120, 13824)]
+
+
+@pytest.mark.parametrize("name,m,k", PREFILL_14B, ids=[s[0] for s in PREFILL_14B])
+def test_gemm_full_14b_shapes(name, m, k):
+    """Every 14B linear shape at N = 8, 16, 32 through ``nf4_gemm`` at full size, all rows
+    against the oracle product on bf16-rounded weights."""
+    w, p, s, dp, ds = quantized(m, k, 21 + m % 97)
+    ref_w = oc.bf16_round(oc.c_decode(p, s, m, k))
+    for n in (8, 16, 32):
+        say("gemm 14B shape", name, m, k, n)
+        x = rand_x(k, n, 16 + n)
+        y = nf4.nf4_gemm(dp, ds, bf16_tensor(x), m, k, k)
+        check_linear(y, oc.c_matmul_f64(ref_w, x), what=f"prefill {name} n{n}")
 
 
 # ------------------------------------------------------------------ attention
