@@ -40,6 +40,8 @@
 
 #include "nf4_common.h"
 
+#include <atomic>
+
 #include <algorithm>
 #include <cstdlib>
 #include <utility>
@@ -1258,6 +1260,58 @@ extern "C" int chr_nf4_gemm_ws(const chr_nf4_dev_t *w, const void *x, void *y, i
 extern "C" int chr_nf4_gemm(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N,
                             void *stream) {
   return chr_nf4_gemm_ws(w, x, y, N, nullptr, 0, stream);
+}
+
+// ---- a GEMM entry that allocates nothing ----------------------------------------------------
+// The split-K partials of chr_nf4_gemm_ws live in a workspace the caller allocates.  This
+// entry keeps them in a file-scope device array instead, for callers that cannot allocate
+// (code under graph capture, tight serving loops).  Every device the library runs on holds
+// its own copy of the array, at its own address, until the process ends.
+namespace {
+
+constexpr int64_t kScratchFloats = int64_t{4} << 20;  // 16 MiB of fp32 partials
+static __device__ __align__(256) float scratch[kScratchFloats];
+
+constexpr int kMaxDevices = 64;
+
+// Device address of this device's copy of the array; null if the runtime refuses.  The
+// array's name is only a handle in host code: the address a kernel can use comes from
+// hipGetSymbolAddress, once per device, with that device current.
+float *scratch_on_current_device() {
+  static std::atomic<float *> known[kMaxDevices];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  float *p = known[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    void *addr = nullptr;
+    if (hipGetSymbolAddress(&addr, HIP_SYMBOL(scratch)) != hipSuccess || addr == nullptr) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    p = static_cast<float *>(addr);
+    known[dev].store(p, std::memory_order_release);  // racing first calls store the same value
+  }
+  return p;
+}
+
+}  // namespace
+
+extern "C" int64_t chr_nf4_gemm_noalloc_max_floats(void) { return kScratchFloats; }
+
+extern "C" int chr_nf4_gemm_noalloc(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N,
+                                    void *stream) {
+  float *ws = scratch_on_current_device();
+  if (ws == nullptr) {
+    return -6;
+  }
+  // Same planner, same kernels and the same order of sums as chr_nf4_gemm_ws with a workspace
+  // of kScratchFloats floats: a launch whose partials do not fit comes back as -7 from the
+  // size check below, before anything is launched.  The partials need no clearing: every
+  // split writes its whole [M, N] slab before the reduce reads it.
+  return chr_nf4_gemm_ws(w, x, y, N, ws, kScratchFloats, stream);
 }
 
 extern "C" int64_t chr_dv2_gemm_swiglu_ws(const chr_nf4_dev_t *gate, const chr_nf4_dev_t *up,

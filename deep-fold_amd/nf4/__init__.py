@@ -110,6 +110,8 @@ EXPORTS = (
     ("chr_nf4_gemm_plan", ctypes.c_int, [_DP, _I, _I, ctypes.POINTER(_Plan)]),
     ("chr_nf4_gemm_ws", ctypes.c_int, [_DP, _P, _P, _I, _P, ctypes.c_int64, _P]),
     ("chr_nf4_gemm_ws_max", ctypes.c_int, [_DP, _P, _P, _I, _P, ctypes.c_int64, _P, _I]),
+    ("chr_nf4_gemm_noalloc", ctypes.c_int, [_DP, _P, _P, _I, _P]),
+    ("chr_nf4_gemm_noalloc_max_floats", ctypes.c_int64, []),
     ("chr_nf4_set_tuning", None, [_I, _I, _I]),
     ("chr_nf4_gemv", ctypes.c_int, [_DP, _P, _P, _P, _P, _P, _F]),
     ("chr_nf4_gemv_qkv", ctypes.c_int, [_DP, _DP, _DP, _P, _P, _P, _P, _P, _P, _P, _P, _P, _F]),

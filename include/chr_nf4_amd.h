@@ -80,6 +80,21 @@ int chr_nf4_gemm_ws(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N,
 int chr_nf4_gemm_ws_max(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N,
                         float *ws, int64_t ws_floats, void *stream, int32_t max_n);
 
+/* chr_nf4_gemm_ws without a workspace argument and without any allocation: the
+ * split-K partials go to a device array owned by the library (16 MiB of fp32 on
+ * every GPU it runs on, held until the process ends).  N in [1, 32].  Returns
+ * what chr_nf4_gemm_ws returns for a workspace of
+ * chr_nf4_gemm_noalloc_max_floats() floats, bit for bit; a launch whose
+ * partials need more comes back as -7 and nothing runs.  All calls on one GPU
+ * share the array: calls that overlap on that GPU (two streams, two threads)
+ * race.  The first call on a device looks the array's address up and must not
+ * be made under graph capture; later ones can.
+ * No counterpart in the reference: for callers that cannot allocate (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc). */
+int chr_nf4_gemm_noalloc(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N,
+                         void *stream);
+int64_t chr_nf4_gemm_noalloc_max_floats(void);
+
 /* Process-wide planner override: path 0 auto; split_k 0 auto, >0 forced;
  * one_wave = compute units the split-K target is expressed in, 0 = this GPU's.
  * Initial values come from CHR_NF4_PATH / CHR_NF4_SPLIT_K / CHR_NF4_ONE_WAVE.
