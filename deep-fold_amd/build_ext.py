@@ -15,7 +15,7 @@ CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 LIB = os.path.join(CSRC, "libchr_nf4_amd.so")
 SOURCES = ("nf4_gemv.hip", "nf4_codec.hip", "nf4_attn.hip", "nf4_gemm.hip", "dv2_state.hip",
            "dv2_prefill.hip")
-HEADERS = ("nf4_common.h", os.path.join("..", "..", "include", "chr_nf4_amd.h"))
+HEADERS = ("nf4_common.h", "nf4_gemv_ring_regs.h", os.path.join("..", "..", "include", "chr_nf4_amd.h"))
 
 #: -packed-fp32-ops is switched off on purpose: the kernels are written for
 #: scalar fp32 VALU ops only.
@@ -26,6 +26,9 @@ HIPCC_FLAGS = (
     "-fPIC",
     "-shared",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # the ring GEMV's asm names registers that its kernels keep away from the compiler;
+    # clang remarks on every such clobber list
+    "-Wno-inline-asm",
 )
 
 

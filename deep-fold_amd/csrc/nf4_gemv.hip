@@ -27,6 +27,7 @@
 // fp32 accumulation, residual / bias added in fp32, one bf16 rounding at the store.
 
 #include "nf4_common.h"
+#include "nf4_gemv_ring_regs.h"
 
 #include <algorithm>
 #include <cstdlib>
@@ -73,6 +74,9 @@ struct StreamArgs {
   const uint16_t *rms_w;  // optional, bf16 [K]
   int K, K_pad;
   float rms_eps;
+  // ring kernels (one segment): grid size, full passes of 16 * grid groups, and the groups
+  // left after them as left_div * grid + left_mod
+  int ring_grid, ring_passes, ring_left_div, ring_left_mod;
 };
 
 // Sum of a value over a workgroup of kStagedThreads threads, the same in every thread.
@@ -412,6 +416,11 @@ __device__ __forceinline__ void fill_pair2_table(uint2 *table, int wave, int lan
     const uint32_t hi_t = odd ? level_tail_bf16(kLevelBits[2 * jj + 1]) : level_tail_bf16(kLevelBits[2 * jj]);
     table[((wave + 16 * j) << 5) + copy] = make_uint2(lo_h | (hi_h << 16), lo_t | (hi_t << 16));
   }
+}
+
+__device__ __forceinline__ uint4 lds0_u128(uint32_t addr) {
+  const U32x4 v = *reinterpret_cast<const __attribute__((address_space(3))) U32x4 *>(addr);
+  return make_uint4(v.x, v.y, v.z, v.w);
 }
 
 __device__ __forceinline__ uint2 lds0_u64(uint32_t addr) {
@@ -864,6 +873,641 @@ __global__ __launch_bounds__(1024) void gemv_staged(const StreamArgs a) {
 #undef CHR_REQUEST
 }
 
+// ---- ring kernel: weight requests and their waits written by hand ----------------------
+// The staged kernel above leaves the software pipeline to the compiler, whose wait counts
+// turn conservative wherever paths with different loads in flight meet (a loop head, the
+// join after a branch): how deep a pipeline it keeps then depends on register allocation.
+// Here the weight requests, the waits for them and the first instructions that read them
+// are asm, and the registers they go through are fixed ones above the compiler's VGPR
+// budget (nf4_gemv_ring_regs.h), which it therefore never touches.  Vector memory
+// operations complete in order, so "at most N outstanding" means everything but the N
+// youngest has arrived: every wait below is exact by construction.
+//
+// D slots of one item (2 half steps) each form a ring: while the oldest item is computed,
+// D-1 younger ones are in flight, and its slot is requested again as soon as it is done.
+// Work is dealt as in the staged kernel's comment, and the groups left after the last full
+// pass are shared out by half steps (one list per wavefront: own groups, then its run of
+// shared half steps, whose sums meet in LDS).
+struct XRegs {
+  U32x4 v[kXKeep];  // x, 16-byte vectors i = thread + j * 1024
+  U32x4 g[kXKeep];  // the RMSNorm weights at the same places (fused norm only)
+};
+
+// A request whose destination keeps its value where the request is skipped: in/out operand,
+// so both paths hold it in the same registers and nothing is copied while it is in flight.
+__device__ __forceinline__ void request16(U32x4 &d, const void *p, uint32_t &tok) {
+  asm("global_load_dwordx4 %0, %2, off" : "+v"(d), "+s"(tok) : "v"(p));
+}
+
+__device__ __forceinline__ void ring_x_request(const StreamArgs &a, XRegs &x, uint32_t &tok) {
+  const int nk = a.K >> 3;
+#pragma unroll
+  for (int j = 0; j < kXKeep; ++j) {
+    x.v[j] = U32x4{0u, 0u, 0u, 0u};
+    x.g[j] = U32x4{0u, 0u, 0u, 0u};
+    if (j * kStagedThreads < nk) {
+      const int i = min(static_cast<int>(threadIdx.x) + j * kStagedThreads, nk - 1);
+      request16(x.v[j], reinterpret_cast<const uint4 *>(a.x) + i, tok);
+      if (a.rms_w != nullptr) {
+        request16(x.g[j], reinterpret_cast<const uint4 *>(a.rms_w) + i, tok);
+      }
+    }
+  }
+}
+
+// x has arrived once at most YOUNGER vector memory operations are outstanding.
+template <int YOUNGER>
+__device__ __forceinline__ void ring_x_wait(XRegs &x, uint32_t &tok) {
+  static_assert(kXKeep == 4, "operand list below");
+  asm("s_waitcnt vmcnt(%9) ; covers %0 %1 %2 %3 %4 %5 %6 %7"
+      : "+v"(x.v[0]), "+v"(x.v[1]), "+v"(x.v[2]), "+v"(x.v[3]), "+v"(x.g[0]), "+v"(x.g[1]),
+        "+v"(x.g[2]), "+v"(x.g[3]), "+s"(tok)
+      : "n"(YOUNGER));
+}
+
+// The eight lookup addresses of one half step of one row (v_perm_b32: byte 1 = a packed
+// byte, byte 0 = the lane's offset into its table copy) and the row's scale as fp32, read
+// from the fixed registers X, Y (packed dwords) and S (fp16 scale, zero-extended).
+//
+// None of the ring's asm statements is volatile: a volatile asm orders every LDS and global
+// access of the compiler's around it, which serialises a half step (x reads, lookups and
+// products of neighbouring steps could no longer overlap: measured 15 against 10 us).
+// Instead every statement reads and writes one scalar token, TOK, which chains them in
+// program order among themselves and keeps them out of common-subexpression and
+// loop-invariant motion, while the compiler's own memory operations move freely.
+#define CHR_RING_ADDRESSES(X, Y, S, A, SC, LANE_OFF, TOK)                                 \
+  asm("v_perm_b32 %0, " X ", %10, %11\n\t"                                                \
+      "v_perm_b32 %1, " X ", %10, %12\n\t"                                                \
+      "v_perm_b32 %2, " X ", %10, %13\n\t"                                                \
+      "v_perm_b32 %3, " X ", %10, %14\n\t"                                                \
+      "v_perm_b32 %4, " Y ", %10, %11\n\t"                                                \
+      "v_perm_b32 %5, " Y ", %10, %12\n\t"                                                \
+      "v_perm_b32 %6, " Y ", %10, %13\n\t"                                                \
+      "v_perm_b32 %7, " Y ", %10, %14\n\t"                                                \
+      "v_cvt_f32_f16 %8, " S                                                              \
+      : "=&v"(A[0]), "=&v"(A[1]), "=&v"(A[2]), "=&v"(A[3]), "=&v"(A[4]), "=&v"(A[5]),     \
+        "=&v"(A[6]), "=&v"(A[7]), "=&v"(SC), "+s"(TOK)                                    \
+      : "v"(LANE_OFF), "s"(0x0C0C0400u), "s"(0x0C0C0500u), "s"(0x0C0C0600u),              \
+        "s"(0x0C0C0700u))
+
+// One row's half step from its eight lookup addresses: products of level pairs with the
+// bf16 pairs of x (xw), the scale applied to the 16-weight partial.
+template <int TERMS>
+__device__ __forceinline__ float ring_row_dot(const uint32_t (&adr)[8], const uint32_t (&xw)[8]) {
+  if constexpr (TERMS == 1) {
+    float pa = 0.f, pb = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; j += 2) {
+      pa = dot2_bf16(lds0_u32(adr[j]), xw[j], pa);
+      pb = dot2_bf16(lds0_u32(adr[j + 1]), xw[j + 1], pb);
+    }
+    return pa + pb;
+  } else {
+    uint2 e[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      e[j] = lds0_u64(adr[j]);
+    }
+    // heads and tails in separate sums: the tails are 2^-9 of the heads and would lose
+    // their low bits if they were added into the large sum one by one
+    float ha = 0.f, hb = 0.f, ta = 0.f, tb = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; j += 2) {
+      ha = dot2_bf16(e[j].x, xw[j], ha);
+      ta = dot2_bf16(e[j].y, xw[j], ta);
+      hb = dot2_bf16(e[j + 1].x, xw[j + 1], hb);
+      tb = dot2_bf16(e[j + 1].y, xw[j + 1], tb);
+    }
+    return (ha + hb) + (ta + tb);
+  }
+}
+
+// The loop is written for instruction count as much as for memory: at four wavefronts per
+// SIMD a half step of ~70 instructions (what the compiler-pipelined kernel executes, half of
+// it address arithmetic and cursor bookkeeping) makes the launch issue-bound, not HBM-bound.
+// Here a row is walked in pieces of NS half steps with NS a compile-time constant, one ring
+// slot per half step of a piece: a request is two instructions whose row and piece live in a
+// scalar base pointer and whose half step is an immediate offset, the x pieces are read at
+// immediate offsets from one address per piece, and cursors only move where a piece ends.
+// The left-over groups (shared out by half steps) and the requests past the end of the list
+// go through a second, general cursor that the steady loop never touches.
+template <int NS, bool SWIGLU, int TERMS, bool XREG>
+__device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
+  static_assert(NS >= 2 && NS <= (SWIGLU ? 6 : 8), "slots of the ring that have registers");
+  static_assert(!XREG || NS <= 5, "x of a whole row in 8 * NS registers");
+  constexpr int R = SWIGLU ? 2 : 1;
+  constexpr int U = 1;                 // output rows per group
+  constexpr int D = NS;                // slots of the ring
+  constexpr int kStepLoads = 2 * R;    // vector memory operations of one half step
+  // LDS byte address of the x pieces (the pair table starts at LDS address 0)
+  constexpr uint32_t kXsAddr = kPairTableBytes + kStagedSmallBytes;
+  extern __shared__ uint4 dyn_lds[];  // [pair table][GemvLds][x pieces][shared-part sums]
+  char *base = reinterpret_cast<char *>(dyn_lds);
+  GemvLds &lds = *reinterpret_cast<GemvLds *>(base + kPairTableBytes);
+  uint4 *xs = reinterpret_cast<uint4 *>(base + kXsAddr);
+  float *shared_sums = reinterpret_cast<float *>(xs + x_pieces(a.K_pad));
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
+  uint32_t tok = 0;  // orders the asm statements among themselves, see CHR_RING_ADDRESSES
+
+  // One segment only (the host sends launches of several segments to the other kernel):
+  // group g is row g, or gate row g and up row g.  How the rows split into full passes and
+  // left-over groups is the same for every wavefront and comes from the host.
+  constexpr int waves = kStagedThreads >> 6;
+  const int grid = a.ring_grid;
+  const int block = static_cast<int>(blockIdx.x);
+  const int first = wave * grid + block;
+  const int stride = grid * waves;
+  const int n_half = a.K_pad >> 4;
+  const int nsteps = x_half_steps(a.K_pad);   // a multiple of NS (the host's choice of NS)
+  const int pieces = nsteps / NS;             // pieces of a row
+  const int last_t = nsteps - 1;
+  const int rem = n_half - last_t * kWave;  // lanes of a row's last half step that hold a chunk
+  const bool ragged = rem < kWave;
+  const uint64_t row_bytes = static_cast<uint64_t>(a.K_pad >> 1);
+  const uint64_t row_scale_bytes = static_cast<uint64_t>(a.K_pad >> 6) << 1;
+  const uint64_t w_base[2] = {reinterpret_cast<uint64_t>(a.packed[0]),
+                              reinterpret_cast<uint64_t>(a.packed2)};
+  const uint64_t s_base[2] = {reinterpret_cast<uint64_t>(a.scale[0]),
+                              reinterpret_cast<uint64_t>(a.scale2)};
+
+  // per-lane loop constants: byte offsets into a half step of packed bytes / of scales (and
+  // their clamped forms for a ragged last step), the x pieces' LDS address, the lane's copy
+  // of the level table
+  const uint32_t v_w = static_cast<uint32_t>(lane) << 3;
+  const uint32_t v_s = static_cast<uint32_t>(lane >> 2) << 1;
+  const uint32_t v_wl = static_cast<uint32_t>(min(lane, rem - 1)) << 3;
+  const uint32_t v_sl = static_cast<uint32_t>(min(lane, rem - 1) >> 2) << 1;
+  const uint32_t x_lane = kXsAddr + (static_cast<uint32_t>(lane) << 4);
+  const uint32_t lane_off = TERMS == 1 ? static_cast<uint32_t>(lane) << 2
+                                       : static_cast<uint32_t>(lane & 31) << 3;
+  const uint64_t all_lanes = ~uint64_t{0};
+  const uint64_t last_lanes = ragged ? ((uint64_t{1} << rem) - 1) : all_lanes;
+
+  // Set-up is written for the number of scalar instructions ahead of the first requests:
+  // the 16 wavefronts of a workgroup start together and share four scalar units, so every
+  // instruction here costs four cycles of every wavefront's start.  Only what the own
+  // groups' first requests need comes first; the shared part's cursor is set up behind them.
+  const int passes = a.ring_passes;       // full passes: a whole group per wavefront
+  const int left_base = passes * stride;  // first left-over group; fewer than stride follow
+
+  // ---- request cursor over the own groups: piece q_part of group q_group at wq / sq ------
+  uint64_t wq[R], sq[R];
+  int q_left = passes * pieces, q_part = 0, q_group = first;
+  auto q_locate = [&]() {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      wq[r] = w_base[r] + static_cast<uint32_t>(q_group) * row_bytes;
+      sq[r] = s_base[r] + static_cast<uint32_t>(q_group) * row_scale_bytes;
+    }
+  };
+  // after the last request of a piece
+  auto q_advance = [&]() {
+    if (--q_left == 0) {
+      return;
+    }
+    if (++q_part < pieces) {
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        wq[r] += NS * 512;
+        sq[r] += NS * 32;
+      }
+      return;
+    }
+    q_part = 0;
+    q_group += stride;
+    q_locate();
+  };
+
+  // ---- request cursor over the shared half steps [gt, g_end) of group g_group ------------
+  // Once its list is requested it is dead and requests nothing more; the steps from then on
+  // wait for everything in flight instead of for all but the D-1 youngest requests.
+  uint64_t wg[R] = {}, sg[R] = {};
+  int gt = 0, g_end = nsteps, g_group = 0, g_rest = 0;
+  bool g_dead = true;
+  // left-over groups of this workgroup (at most 16) and this wavefront's run of their half
+  // steps: n_shared of them from number sh_k0 on, the first being step sh_t0 of its group
+  int my_left = 0, n_shared = 0, sh_k0 = 0, sh_t0 = 0, sh_end0 = 0;
+  auto g_locate = [&](int grp, int t) {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      wg[r] = w_base[r] + static_cast<uint32_t>(grp) * row_bytes + (static_cast<uint32_t>(t) << 9);
+      sg[r] = s_base[r] + static_cast<uint32_t>(grp) * row_scale_bytes +
+              (static_cast<uint32_t>(t) << 5);
+    }
+    g_group = grp;
+    gt = t;
+  };
+  auto g_setup = [&]() {
+    my_left = a.ring_left_div + (block < a.ring_left_mod ? 1 : 0);
+    const int sh_steps = my_left * nsteps;
+    const int sh_run = (sh_steps + waves - 1) / waves;
+    sh_k0 = wave * sh_run;
+    n_shared = max(0, min(sh_run, sh_steps - sh_k0));
+    if (n_shared > 0) {
+      // sh_k0 / nsteps for small operands: the quotient's distance from the next integer is
+      // at least 0.5 / nsteps, far above the rounding of the product
+      const int sh_j0 = static_cast<int>((static_cast<float>(sh_k0) + 0.5f) *
+                                         __builtin_amdgcn_rcpf(static_cast<float>(nsteps)));
+      sh_t0 = sh_k0 - sh_j0 * nsteps;
+      sh_end0 = min(nsteps, sh_t0 + n_shared);  // end of the run's first row piece
+      g_locate(left_base + block + grid * sh_j0, sh_t0);
+      g_end = sh_end0;
+      g_rest = n_shared - (sh_end0 - sh_t0);
+      g_dead = false;
+    }
+  };
+  auto g_advance = [&]() {
+    if (gt + 1 < g_end) {
+      ++gt;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        wg[r] += 512;
+        sg[r] += 32;
+      }
+      return;
+    }
+    if (g_rest > 0) {
+      g_locate(g_group + grid, 0);
+      g_end = min(nsteps, g_rest);
+      g_rest -= g_end;
+      return;
+    }
+    g_dead = true;
+  };
+  if (q_left > 0) {
+    q_locate();
+  }
+
+  // one half step of one row into its fixed registers: two instructions
+#define CHR_RING_LOAD(W, SREG, CLOB, VW, VS, WP, SP, I)                                   \
+  asm("global_load_dwordx2 " W ", %1, %2 offset:%5 nt\n\t"                                \
+      "global_load_ushort " SREG ", %3, %4 offset:%6 nt"                                  \
+      : "+s"(tok)                                                                         \
+      : "v"(VW), "s"(WP), "v"(VS), "s"(SP), "n"((I) * 512), "n"((I) * 32)                 \
+      : CLOB);
+  // slot I: half step I of the own piece at wq / sq; LASTP = the piece ends its row
+#define CHR_RING_OWN(I, LASTP)                                                            \
+  if constexpr (SWIGLU) {                                                                 \
+    if ((I) == NS - 1 && ragged && (LASTP)) {                                             \
+      CHR_RING_LOAD(RR2_W(I, 0), RR2_S(I, 0), RR2_CLOB(I, 0), v_wl, v_sl, wq[0], sq[0], I) \
+      CHR_RING_LOAD(RR2_W(I, 1), RR2_S(I, 1), RR2_CLOB(I, 1), v_wl, v_sl, wq[R - 1], sq[R - 1], I) \
+    } else {                                                                              \
+      CHR_RING_LOAD(RR2_W(I, 0), RR2_S(I, 0), RR2_CLOB(I, 0), v_w, v_s, wq[0], sq[0], I)  \
+      CHR_RING_LOAD(RR2_W(I, 1), RR2_S(I, 1), RR2_CLOB(I, 1), v_w, v_s, wq[R - 1], sq[R - 1], I) \
+    }                                                                                     \
+  } else {                                                                                \
+    if ((I) == NS - 1 && ragged && (LASTP)) {                                             \
+      CHR_RING_LOAD(RR1_W(I), RR1_S(I), RR1_CLOB(I), v_wl, v_sl, wq[0], sq[0], I)         \
+    } else {                                                                              \
+      CHR_RING_LOAD(RR1_W(I), RR1_S(I), RR1_CLOB(I), v_w, v_s, wq[0], sq[0], I)           \
+    }                                                                                     \
+  }
+  // slot I: the general cursor's half step, if it has one left
+#define CHR_RING_GENERAL(I)                                                               \
+  if (!g_dead) {                                                                          \
+    if constexpr (SWIGLU) {                                                               \
+      if (gt == last_t) {                                                                 \
+        CHR_RING_LOAD(RR2_W(I, 0), RR2_S(I, 0), RR2_CLOB(I, 0), v_wl, v_sl, wg[0], sg[0], 0) \
+        CHR_RING_LOAD(RR2_W(I, 1), RR2_S(I, 1), RR2_CLOB(I, 1), v_wl, v_sl, wg[R - 1], sg[R - 1], 0) \
+      } else {                                                                            \
+        CHR_RING_LOAD(RR2_W(I, 0), RR2_S(I, 0), RR2_CLOB(I, 0), v_w, v_s, wg[0], sg[0], 0) \
+        CHR_RING_LOAD(RR2_W(I, 1), RR2_S(I, 1), RR2_CLOB(I, 1), v_w, v_s, wg[R - 1], sg[R - 1], 0) \
+      }                                                                                   \
+    } else {                                                                              \
+      if (gt == last_t) {                                                                 \
+        CHR_RING_LOAD(RR1_W(I), RR1_S(I), RR1_CLOB(I), v_wl, v_sl, wg[0], sg[0], 0)       \
+      } else {                                                                            \
+        CHR_RING_LOAD(RR1_W(I), RR1_S(I), RR1_CLOB(I), v_w, v_s, wg[0], sg[0], 0)         \
+      }                                                                                   \
+    }                                                                                     \
+    g_advance();                                                                          \
+  }
+  // The first NS requests: the first piece of the first own group where there is one (the
+  // usual case: five request instructions and nothing else), otherwise the first shared
+  // half steps.  all_asked says whether all NS were made.
+  bool all_asked = true;
+#define CHR_RING_FILL_OWN(I) \
+  if constexpr (NS > (I)) { CHR_RING_OWN(I, pieces == 1) }
+#define CHR_RING_FILL_GENERAL(I)                                                          \
+  if constexpr (NS > (I)) {                                                               \
+    all_asked = all_asked && !g_dead;                                                     \
+    CHR_RING_GENERAL(I)                                                                   \
+  }
+#define CHR_RING_FILL                                                                     \
+  if (q_left > 0) {                                                                       \
+    CHR_RING_FILL_OWN(0)                                                                  \
+    CHR_RING_FILL_OWN(1)                                                                  \
+    CHR_RING_FILL_OWN(2)                                                                  \
+    CHR_RING_FILL_OWN(3)                                                                  \
+    CHR_RING_FILL_OWN(4)                                                                  \
+    CHR_RING_FILL_OWN(5)                                                                  \
+    CHR_RING_FILL_OWN(6)                                                                  \
+    CHR_RING_FILL_OWN(7)                                                                  \
+    q_advance();                                                                          \
+    g_setup();                                                                            \
+  } else {                                                                                \
+    g_setup();                                                                            \
+    CHR_RING_FILL_GENERAL(0)                                                              \
+    CHR_RING_FILL_GENERAL(1)                                                              \
+    CHR_RING_FILL_GENERAL(2)                                                              \
+    CHR_RING_FILL_GENERAL(3)                                                              \
+    CHR_RING_FILL_GENERAL(4)                                                              \
+    CHR_RING_FILL_GENERAL(5)                                                              \
+    CHR_RING_FILL_GENERAL(6)                                                              \
+    CHR_RING_FILL_GENERAL(7)                                                              \
+  }
+  // x travels in registers that the compiler allocates: between its request and its wait
+  // there is only this branch's own straight-line code, nothing that could make the compiler
+  // move or spill them (hence the two copies of the ring's fill).
+  if (stage_fast_ok(a)) {
+    XRegs xr;
+    ring_x_request(a, xr, tok);
+    CHR_RING_FILL
+    if constexpr (TERMS == 1) {
+      fill_pair_table(reinterpret_cast<uint32_t *>(dyn_lds), wave, lane);
+    } else {
+      fill_pair2_table(reinterpret_cast<uint2 *>(dyn_lds), wave, lane);
+    }
+    if (!all_asked) {
+      asm("s_waitcnt vmcnt(0)" : "+s"(tok));
+    }
+    ring_x_wait<NS * kStepLoads>(xr, tok);
+    uint4 xv[kXKeep], xg[kXKeep];
+#pragma unroll
+    for (int j = 0; j < kXKeep; ++j) {
+      xv[j] = make_uint4(xr.v[j].x, xr.v[j].y, xr.v[j].z, xr.v[j].w);
+      xg[j] = make_uint4(xr.g[j].x, xr.g[j].y, xr.g[j].z, xr.g[j].w);
+    }
+    x_store(a, xs, lds.part, xv, xg);
+  } else {
+    // The other staging forms read what they need in loops of their own (loads the compiler
+    // counts: its waits then also cover the half steps requested here, which are older).
+    CHR_RING_FILL
+    if constexpr (TERMS == 1) {
+      fill_pair_table(reinterpret_cast<uint32_t *>(dyn_lds), wave, lane);
+    } else {
+      fill_pair2_table(reinterpret_cast<uint2 *>(dyn_lds), wave, lane);
+    }
+    stage_x(a, xs, lds.part);
+  }
+#undef CHR_RING_FILL
+#undef CHR_RING_FILL_GENERAL
+#undef CHR_RING_FILL_OWN
+
+  float acc[R] = {};
+  uint16_t *const y_rows = a.y[0];
+  const uint16_t *const add_rows = a.add[0];
+  auto finish_group = [&](int grp) {
+    if constexpr (SWIGLU) {
+      const float gsum = wave_sum(acc[0]);
+      const float usum = wave_sum(acc[1]);
+      if (lane == 0) {
+        y_rows[grp] = f32_to_bf16(silu(gsum) * usum);
+      }
+    } else {
+      float v = wave_sum(acc[0]);
+      if (add_rows != nullptr) {
+        v += uniform_bf16(add_rows + grp);
+      }
+      if (lane == 0) {
+        y_rows[grp] = f32_to_bf16(v);
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      acc[r] = 0.f;
+    }
+  };
+
+  // 0 in the lanes that MASK (a scalar lane mask) switches off
+#define CHR_RING_MASKED(DST, SRC, MASK) \
+  asm("v_cndmask_b32 %0, 0, %1, %2" : "=v"(DST) : "v"(SRC), "s"(MASK))
+
+  // The sums go through the chain of asm statements once per half step, which keeps a half
+  // step's products ahead of the next half step's wait: left to itself the compiler sinks
+  // all products of a piece to its end and holds every level it has looked up until then.
+#define CHR_RING_PIN                                                                      \
+  if constexpr (SWIGLU) {                                                                 \
+    asm("" : "+v"(acc[0]), "+v"(acc[R - 1]), "+s"(tok));                                  \
+  } else {                                                                                \
+    asm("" : "+v"(acc[0]), "+s"(tok));                                                    \
+  }
+  // The half step in slot I, its x pieces at XA: wait for it (the D-1 younger half steps
+  // stay in flight), turn its packed bytes into lookup addresses, which frees the slot's
+  // registers, request the slot again at once (REQUEST), and only then look the levels up and
+  // multiply: the new request travels while this half step is computed.  MASK_IF says whether
+  // the lanes past the row's end are to be switched off (LANES_ON the lanes that stay).
+#define CHR_RING_STEP(I, X0, X1, WAIT, REQUEST, MASK_IF, LANES_ON)                        \
+  {                                                                                       \
+    const uint4 x0 = X0, x1 = X1;                                                         \
+    const uint32_t xw[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};              \
+    WAIT                                                                                  \
+    if constexpr (SWIGLU) {                                                               \
+      uint32_t ag[8], au[8];                                                              \
+      float sg_, su_;                                                                     \
+      CHR_RING_ADDRESSES(RR2_X(I, 0), RR2_Y(I, 0), RR2_S(I, 0), ag, sg_, lane_off, tok);  \
+      CHR_RING_ADDRESSES(RR2_X(I, 1), RR2_Y(I, 1), RR2_S(I, 1), au, su_, lane_off, tok);  \
+      REQUEST                                                                             \
+      if (MASK_IF) {                                                                      \
+        CHR_RING_MASKED(sg_, sg_, LANES_ON);                                              \
+        CHR_RING_MASKED(su_, su_, LANES_ON);                                              \
+      }                                                                                   \
+      acc[0] = fmaf(sg_, ring_row_dot<TERMS>(ag, xw), acc[0]);                            \
+      acc[1] = fmaf(su_, ring_row_dot<TERMS>(au, xw), acc[1]);                            \
+    } else {                                                                              \
+      uint32_t aw[8];                                                                     \
+      float sw_;                                                                          \
+      CHR_RING_ADDRESSES(RR1_X(I), RR1_Y(I), RR1_S(I), aw, sw_, lane_off, tok);           \
+      REQUEST                                                                             \
+      if (MASK_IF) {                                                                      \
+        CHR_RING_MASKED(sw_, sw_, LANES_ON);                                              \
+      }                                                                                   \
+      acc[0] = fmaf(sw_, ring_row_dot<TERMS>(aw, xw), acc[0]);                            \
+    }                                                                                     \
+    CHR_RING_PIN                                                                          \
+  }
+
+  // every step so far has requested its slot again: D-1 younger half steps are in flight
+#define CHR_RING_WAIT_FULL \
+  asm("s_waitcnt vmcnt(%1)" : "+s"(tok) : "n"((D - 1) * kStepLoads));
+  // the general cursor may have run out: then fewer are, and the wait is for all of them
+#define CHR_RING_WAIT_GENERAL                                                             \
+  if (g_dead) {                                                                           \
+    asm("s_waitcnt vmcnt(0)" : "+s"(tok));                                                \
+  } else {                                                                                \
+    CHR_RING_WAIT_FULL                                                                    \
+  }
+
+  // ---- the own groups, a piece per turn ---------------------------------------------------
+  int c_left = passes * pieces, c_part = 0, c_group = first;
+  // XREG (a row is one piece of at most 5 half steps): the lane's x pieces of the whole row
+  // stay in registers for every own group, which takes two 16-byte LDS reads out of each of
+  // their half steps -- 16 of the ~42 cycles that a half step occupies the LDS for, and the
+  // LDS is what bounds the loop.  The shared half steps still read x from the LDS.
+  uint4 x_row[XREG ? 2 * NS : 1];
+  if constexpr (XREG) {
+    if (c_left > 0) {
+#pragma unroll
+      for (int i = 0; i < NS; ++i) {
+        x_row[2 * i] = lds0_u128(x_lane + i * 2048);
+        x_row[2 * i + 1] = lds0_u128(x_lane + i * 2048 + 1024);
+      }
+    }
+  }
+#define CHR_RING_OWN_STEP(I, WAIT, REQUEST)                                               \
+  if constexpr (NS > (I)) {                                                               \
+    if constexpr (XREG) {                                                                 \
+      CHR_RING_STEP(I, x_row[2 * ((I) % NS)], x_row[2 * ((I) % NS) + 1], WAIT, REQUEST,   \
+                    (I) == NS - 1 && ragged, last_lanes)                                  \
+    } else {                                                                              \
+      CHR_RING_STEP(I, lds0_u128(xa + (I) * 2048), lds0_u128(xa + (I) * 2048 + 1024), WAIT, \
+                    REQUEST, (I) == NS - 1 && ragged && c_last, last_lanes)               \
+    }                                                                                     \
+  }
+#define CHR_RING_PIECE(WAIT, REQUEST_OF, AFTER_REQUESTS)                                  \
+  {                                                                                       \
+    const uint32_t xa = x_lane + static_cast<uint32_t>(c_part) * (NS * 2048);             \
+    const bool c_last = c_part == pieces - 1;                                             \
+    CHR_RING_OWN_STEP(0, WAIT, REQUEST_OF(0))                                             \
+    CHR_RING_OWN_STEP(1, WAIT, REQUEST_OF(1))                                             \
+    CHR_RING_OWN_STEP(2, WAIT, REQUEST_OF(2))                                             \
+    CHR_RING_OWN_STEP(3, WAIT, REQUEST_OF(3))                                             \
+    CHR_RING_OWN_STEP(4, WAIT, REQUEST_OF(4))                                             \
+    CHR_RING_OWN_STEP(5, WAIT, REQUEST_OF(5))                                             \
+    CHR_RING_OWN_STEP(6, WAIT, REQUEST_OF(6))                                             \
+    CHR_RING_OWN_STEP(7, WAIT, REQUEST_OF(7))                                             \
+    AFTER_REQUESTS                                                                        \
+    --c_left;                                                                             \
+    if (c_last) {                                                                         \
+      finish_group(c_group);                                                              \
+      c_group += stride;                                                                  \
+      c_part = 0;                                                                         \
+    } else {                                                                              \
+      ++c_part;                                                                           \
+    }                                                                                     \
+  }
+#define CHR_RING_REQUEST_OWN(I) CHR_RING_OWN(I, q_part == pieces - 1)
+#define CHR_RING_REQUEST_GENERAL(I) CHR_RING_GENERAL(I)
+  // while the piece after this one is an own piece too, every request is an own one
+  while (q_left > 0) {
+    CHR_RING_PIECE(CHR_RING_WAIT_FULL, CHR_RING_REQUEST_OWN, q_advance();)
+  }
+  // the last own piece: its slots go to the shared half steps
+  while (c_left > 0) {
+    CHR_RING_PIECE(CHR_RING_WAIT_GENERAL, CHR_RING_REQUEST_GENERAL, )
+  }
+
+  // ---- the shared half steps: each parks its R sums in LDS --------------------------------
+  {
+    int st = sh_t0, s_end = sh_end0, s_rest = n_shared - (sh_end0 - sh_t0), s_k = sh_k0;
+    int s_todo = n_shared;
+#define CHR_RING_SHARED_STEP(I)                                                           \
+  if constexpr (NS > (I)) {                                                               \
+    if (s_todo > 0) {                                                                     \
+      const uint32_t xa = x_lane + (static_cast<uint32_t>(st) << 11);                     \
+      CHR_RING_STEP(I, lds0_u128(xa), lds0_u128(xa + 1024), CHR_RING_WAIT_GENERAL,        \
+                    CHR_RING_GENERAL(I), ragged && st == last_t, last_lanes)              \
+      _Pragma("unroll") for (int r = 0; r < R; ++r) {                                     \
+        const float v = wave_sum(acc[r]);                                                 \
+        if (lane == 0) {                                                                  \
+          shared_sums[s_k * R + r] = v;                                                   \
+        }                                                                                 \
+        acc[r] = 0.f;                                                                     \
+      }                                                                                   \
+      ++s_k;                                                                              \
+      --s_todo;                                                                           \
+      if (++st == s_end) {                                                                \
+        st = 0;                                                                           \
+        s_end = min(nsteps, s_rest);                                                      \
+        s_rest -= s_end;                                                                  \
+      }                                                                                   \
+    }                                                                                     \
+  }
+    while (s_todo > 0) {
+      CHR_RING_SHARED_STEP(0)
+      CHR_RING_SHARED_STEP(1)
+      CHR_RING_SHARED_STEP(2)
+      CHR_RING_SHARED_STEP(3)
+      CHR_RING_SHARED_STEP(4)
+      CHR_RING_SHARED_STEP(5)
+      CHR_RING_SHARED_STEP(6)
+      CHR_RING_SHARED_STEP(7)
+    }
+#undef CHR_RING_SHARED_STEP
+  }
+  // nothing may still be on its way into the fixed registers when the wavefront ends (this
+  // statement is volatile: it is what keeps the token chain, and with it every request, alive)
+  asm volatile("s_waitcnt vmcnt(0)" : "+s"(tok));
+#undef CHR_RING_REQUEST_GENERAL
+#undef CHR_RING_REQUEST_OWN
+#undef CHR_RING_PIECE
+#undef CHR_RING_OWN_STEP
+#undef CHR_RING_WAIT_GENERAL
+#undef CHR_RING_WAIT_FULL
+#undef CHR_RING_STEP
+#undef CHR_RING_PIN
+#undef CHR_RING_MASKED
+#undef CHR_RING_GENERAL
+#undef CHR_RING_OWN
+#undef CHR_RING_LOAD
+
+  // The shared part: wavefront j finishes the workgroup's j-th left-over group (at most 16).
+  if (my_left > 0) {
+    __syncthreads();
+    if (wave < my_left) {
+      const int row = left_base + block + grid * wave;
+      const float *sums = shared_sums + wave * nsteps * R;
+      float s0 = 0.f, s1 = 0.f;
+      for (int t = 0; t < nsteps; ++t) {
+        s0 += sums[t * R];
+        if constexpr (SWIGLU) {
+          s1 += sums[t * R + 1];
+        }
+      }
+      if (lane == 0) {
+        if constexpr (SWIGLU) {
+          y_rows[row] = f32_to_bf16(silu(s0) * s1);
+        } else {
+          if (add_rows != nullptr) {
+            s0 += bf16_to_f32(add_rows[row]);
+          }
+          y_rows[row] = f32_to_bf16(s0);
+        }
+      }
+    }
+  }
+}
+
+// The compiler's VGPR budget stops where the ring's fixed registers begin.  (On this target
+// the attribute counts vector and accumulation registers together and is ignored when the
+// sum exceeds what the launch bounds allow, so it names half the vector registers meant.)
+template <int NS, int TERMS, bool XREG>
+__global__ __launch_bounds__(1024) __attribute__((amdgpu_num_vgpr(52))) void gemv_ring_rows(
+    const StreamArgs a) {
+  gemv_ring_body<NS, false, TERMS, XREG>(a);
+}
+
+template <int NS, int TERMS, bool XREG>
+__global__ __launch_bounds__(1024) __attribute__((amdgpu_num_vgpr(46))) void gemv_ring_pairs(
+    const StreamArgs a) {
+  gemv_ring_body<NS, true, TERMS, XREG>(a);
+}
+
+// Half steps of a piece (= slots of the ring, 512 bytes per row each) for a row of nsteps
+// half steps: the largest divisor the registers hold, at least 4 so that 1.5 KB per row stay
+// in flight (a pure streaming read of a 35 MB matrix by this grid is fastest with 2 KB per
+// wavefront on the way and loses 15% at 4 KB).  0 = the ring kernel does not take this row
+// length (the compiler-pipelined kernel does).
+int ring_piece_steps(int nsteps, bool pairs) {
+  for (int ns = pairs ? 6 : 8; ns >= 4; --ns) {
+    if (nsteps % ns == 0) {
+      return ns;
+    }
+  }
+  return 0;
+}
+
 // ---- RMSNorm -----------------------------------------------------------------
 constexpr int kRmsBlock = 1024;
 
@@ -981,8 +1625,25 @@ int prep_lds(Kern kern, size_t dyn) {
 // more again (10.4, 11.0 us) -- deeper request queues do not pay on this memory system.
 constexpr int kItemSteps = 2;
 
+// pair table, small statics, x pieces, and (ring kernel) the sums of the shared half steps:
+// up to 16 left-over groups of 2 rows per workgroup
 inline size_t staged_lds_bytes(int K_pad) {
-  return kPairTableBytes + kStagedSmallBytes + static_cast<size_t>(x_pieces(K_pad)) * 16;
+  return kPairTableBytes + kStagedSmallBytes + static_cast<size_t>(x_pieces(K_pad)) * 16 +
+         static_cast<size_t>(x_half_steps(K_pad)) * (kStagedThreads / kWave) * 2 * sizeof(float);
+}
+
+// Whether a staged launch of m groups (rows, or gate/up pairs) goes to the ring kernel where
+// that one takes the row length.  The ring kernel streams faster once it runs (lm_head
+// 152064x5120: 72 against 77 us with one-term levels, 79 against 91 us with two-term ones)
+// but starts about a microsecond later (more scalar set-up ahead of its first requests), so
+// it only pays where a wavefront walks many rows: from 32768 groups up.
+// CHR_NF4_GEMV_RING=0: never; =1: wherever the row length allows (read on every launch).
+bool ring_wanted(int m) {
+  const char *e = std::getenv("CHR_NF4_GEMV_RING");
+  if (e != nullptr && e[1] == '\0' && (e[0] == '0' || e[0] == '1')) {
+    return e[0] == '1';
+  }
+  return m >= 32768;
 }
 
 // Kernel family for a launch of m_total weight rows: 1 staged, 0 plain, -1 staging is
@@ -1003,13 +1664,16 @@ int pick_family(const StreamArgs &a, int m_total) {
   return fits && codes >= (16ll << 20) ? 1 : 0;
 }
 
-// Rows per wavefront of the staged kernel: one, so that even 5120 rows give every
-// wavefront of 256 compute units work, and two from 32768 rows up (lm_head 152064x5120:
-// 75 us against 81 us).
-int staged_rows_for_m(int M) {
+// Rows per wavefront of the staged kernels: one, so that even 5120 rows give every
+// wavefront of 256 compute units work; from 32768 rows up the ring kernel (one row) where
+// it takes the row length, else two rows (lm_head 152064x5120: 75 us against 81 us).
+int staged_rows_for_m(int M, int K_pad, bool pairs) {
   const int f = forced_rows();
   if (f > 0) {
     return f;
+  }
+  if (ring_wanted(M) && ring_piece_steps(x_half_steps(K_pad), pairs) > 0) {
+    return 1;  // the ring kernel walks one row (or one gate/up pair) per group
   }
   return M >= 32768 ? 2 : 1;
 }
@@ -1026,7 +1690,66 @@ int launch_stream(StreamArgs &a, int n_seg, bool staged, hipStream_t st) {
     const size_t dyn = staged_lds_bytes(a.K_pad);
     const int waves = kStagedThreads / kWave;
     const int grid = std::min(device_cu_count(), (total + waves - 1) / waves);
-    if (level_terms() == 1) {
+    const bool one_term = level_terms() == 1;
+    constexpr bool kRingShape = (SWIGLU && R == 2) || (!SWIGLU && R == 1);
+    const int ring_ns = kRingShape && n_seg == 1 && ring_wanted(total)
+                            ? ring_piece_steps(x_half_steps(a.K_pad), SWIGLU) : 0;
+    if (ring_ns > 0) {
+      const int per_pass = grid * waves;
+      a.ring_grid = grid;
+      a.ring_passes = total / per_pass;
+      a.ring_left_div = (total % per_pass) / grid;
+      a.ring_left_mod = (total % per_pass) % grid;
+      if constexpr (kRingShape) {
+        auto go = [&](auto kern) {
+          if (prep_lds(kern, dyn) != 0) {
+            return -6;
+          }
+          kern<<<dim3(grid), dim3(kStagedThreads), dyn, st>>>(a);
+          return 0;
+        };
+        int rc = -6;
+        // a row that is one piece of at most 5 half steps keeps its x in registers (the pair
+        // kernel only with one-term levels: two rows of two-term lookups leave no room)
+        const bool one_piece = x_half_steps(a.K_pad) == ring_ns && ring_ns <= 5;
+        if constexpr (SWIGLU) {
+          switch (ring_ns) {
+            case 4:
+              rc = !one_term ? go(gemv_ring_pairs<4, 2, false>)
+                   : one_piece ? go(gemv_ring_pairs<4, 1, true>) : go(gemv_ring_pairs<4, 1, false>);
+              break;
+            case 5:
+              rc = !one_term ? go(gemv_ring_pairs<5, 2, false>)
+                   : one_piece ? go(gemv_ring_pairs<5, 1, true>) : go(gemv_ring_pairs<5, 1, false>);
+              break;
+            case 6: rc = one_term ? go(gemv_ring_pairs<6, 1, false>) : go(gemv_ring_pairs<6, 2, false>); break;
+          }
+        } else {
+          switch (ring_ns) {
+            case 4:
+              if (one_piece) {
+                rc = one_term ? go(gemv_ring_rows<4, 1, true>) : go(gemv_ring_rows<4, 2, true>);
+              } else {
+                rc = one_term ? go(gemv_ring_rows<4, 1, false>) : go(gemv_ring_rows<4, 2, false>);
+              }
+              break;
+            case 5:
+              if (one_piece) {
+                rc = one_term ? go(gemv_ring_rows<5, 1, true>) : go(gemv_ring_rows<5, 2, true>);
+              } else {
+                rc = one_term ? go(gemv_ring_rows<5, 1, false>) : go(gemv_ring_rows<5, 2, false>);
+              }
+              break;
+            case 6: rc = one_term ? go(gemv_ring_rows<6, 1, false>) : go(gemv_ring_rows<6, 2, false>); break;
+            case 7: rc = one_term ? go(gemv_ring_rows<7, 1, false>) : go(gemv_ring_rows<7, 2, false>); break;
+            case 8: rc = one_term ? go(gemv_ring_rows<8, 1, false>) : go(gemv_ring_rows<8, 2, false>); break;
+          }
+        }
+        if (rc != 0) {
+          return rc;
+        }
+      }
+    } else if (one_term) {
       constexpr auto kern = gemv_staged<R, kItemSteps, SWIGLU, 1>;
       if (prep_lds(kern, dyn) != 0) {
         return -6;
@@ -1059,7 +1782,7 @@ int launch_rows(StreamArgs &a, int n_seg, int m_for_policy, hipStream_t st) {
     return -6;
   }
   const bool staged = family == 1;
-  switch (staged ? staged_rows_for_m(m_for_policy) : rows_for_m(m_for_policy)) {
+  switch (staged ? staged_rows_for_m(m_for_policy, a.K_pad, false) : rows_for_m(m_for_policy)) {
     case 4:
       return launch_stream<4, false>(a, n_seg, staged, st);
     case 2:
@@ -1077,7 +1800,7 @@ int launch_pairs(StreamArgs &a, int m_pairs, hipStream_t st) {
     return -6;
   }
   const bool staged = family == 1;
-  const int rows = staged ? 2 * staged_rows_for_m(m_pairs) : (rows_for_m(2 * m_pairs) >= 2 ? 4 : 2);
+  const int rows = staged ? 2 * staged_rows_for_m(m_pairs, a.K_pad, true) : (rows_for_m(2 * m_pairs) >= 2 ? 4 : 2);
   if (rows >= 4) {
     return launch_stream<4, true>(a, 1, staged, st);
   }
@@ -1155,7 +1878,7 @@ bool gemv_plan_staged(int M, int K, int K_pad) {
 }
 
 int gemv_rows_per_wg(int M, int K, int K_pad) {
-  return gemv_plan_staged(M, K, K_pad) ? (kStagedThreads / kWave) * staged_rows_for_m(M)
+  return gemv_plan_staged(M, K, K_pad) ? (kStagedThreads / kWave) * staged_rows_for_m(M, K_pad, false)
                                        : (kThreads / kWave) * rows_for_m(M);
 }
 

@@ -101,9 +101,30 @@ _MAX_DYN_LDS = 150 * 1024
 
 
 def staged_lds_bytes(k_pad_: int) -> int:
-    """LDS of a staged GEMV launch: table, reduction scratch, x in 512-code half steps."""
+    """LDS of a staged GEMV launch: table, reduction scratch, x in half steps of 1024 codes,
+    and the sums of the half steps that the wavefronts of a workgroup share (up to 16
+    left-over groups of two rows)."""
     half_steps = _ceil_div(int(k_pad_) // 16, 64)
-    return _STAGED_TABLE_BYTES + _STAGED_SMALL_BYTES + half_steps * 128 * 16
+    return (_STAGED_TABLE_BYTES + _STAGED_SMALL_BYTES + half_steps * 128 * 16
+            + half_steps * 16 * 2 * 4)
+
+
+def ring_piece_steps(half_steps: int, pairs: bool = False) -> int:
+    """Half steps per piece of the ring GEMV kernel for a row of ``half_steps``: the largest
+    divisor in 4..8 (4..6 for gate/up pairs), or 0 when that kernel does not take the row."""
+    for ns in range(6 if pairs else 8, 3, -1):
+        if half_steps % ns == 0:
+            return ns
+    return 0
+
+
+def ring_wanted(m: int) -> bool:
+    """Whether a staged launch of ``m`` groups goes to the ring kernel where it takes the row
+    length: from 32768 groups up, or as ``CHR_NF4_GEMV_RING`` (0 / 1) says."""
+    e = os.environ.get("CHR_NF4_GEMV_RING")
+    if e in ("0", "1"):
+        return e == "1"
+    return m >= 32768
 
 
 def gemv_is_staged(m: int, k: int, k_pad_: int | None = None) -> bool:
@@ -115,11 +136,14 @@ def gemv_is_staged(m: int, k: int, k_pad_: int | None = None) -> bool:
     return fits and int(m) * kp >= STAGED_MIN_CODES
 
 
-def gemv_rows_per_wavefront(m: int, forced: int = 0, staged: bool = False) -> int:
+def gemv_rows_per_wavefront(m: int, forced: int = 0, staged: bool = False,
+                            k_pad_: int | None = None) -> int:
     """Rows one wavefront of the GEMV walks together (they share x)."""
     if forced in (1, 2, 4):
         return forced
     if staged:
+        if k_pad_ is not None and ring_wanted(m) and ring_piece_steps(_ceil_div(k_pad_ // 16, 64)):
+            return 1
         return 2 if m >= 32768 else 1
     if m >= 32768:
         return 4
@@ -218,7 +242,7 @@ def plan(M: int, K: int, N: int = 1, *, K_pad: int | None = None, have_ws: bool 
     if N == 1:
         if gemv_is_staged(M, K, kp):
             # one workgroup of 16 wavefronts per compute unit; bm = rows it covers per pass
-            bm = 16 * gemv_rows_per_wavefront(M, gemv_rows, staged=True)
+            bm = 16 * gemv_rows_per_wavefront(M, gemv_rows, staged=True, k_pad_=kp)
             n_ktiles = _ceil_div(kp, 1024)
             grid_x = min(int(one_wave), _ceil_div(M, bm))
             return Plan(GEMV, grid_x, 1, 1024, bm, 1024, n_ktiles, n_ktiles, grid_x,

@@ -383,6 +383,95 @@ def test_swiglu_equals_pair(m, k):
     check_linear(out, ref, what="swiglu", ulps=1.5, model=model)
 
 
+# ----------------------------------------------------------------- ring GEMV kernels
+# The ring kernels take staged launches of one segment whose row length is a multiple of 4..8
+# half steps of 1024 weights (4..6 for gate/up pairs); by default only from 32768 rows up,
+# CHR_NF4_GEMV_RING=1 sends every such launch to them.
+RING_ROWS = [
+    (4100, 4096),   # 4 half steps, x of the row in registers; one full pass and a shared rest
+    (9000, 5120),   # 5 half steps, two passes
+    (3, 5120),      # fewer rows than wavefronts: shared half steps only
+    (4500, 6144), (4200, 7168), (4100, 8192),
+    (700, 13824),   # two pieces of 7 half steps
+    (300, 16384),   # two pieces of 8
+    (4300, 6208),   # last half step partly filled (4 of 64 lanes)
+    (4200, 5056),   # the same with x in registers
+    (4100, 4000),   # K below K_pad
+]
+
+
+@pytest.mark.parametrize("terms", [1, 2])
+@pytest.mark.parametrize("m,k", RING_ROWS)
+def test_ring_gemv(m, k, terms, monkeypatch):
+    say("ring gemv", m, k, terms)
+    monkeypatch.setenv("CHR_NF4_GEMV_STAGED", "1")
+    monkeypatch.setenv("CHR_NF4_GEMV_RING", "1")
+    monkeypatch.setenv("CHR_NF4_GEMV_TERMS", str(terms))
+    p, s, dp, ds = blobs(m, k, 700 + m + k)
+    x = rand_x(k, None, 13)
+    res = oc.bf16_round(np.random.default_rng(m).standard_normal(m).astype(np.float32))
+    y = nf4.nf4_gemv(dp, ds, bf16_tensor(x), m, k, oc.k_pad(k))
+    ref = oc.c_matmul_f64(oc.c_decode(p, s, m, k), x[:, None]).reshape(-1)
+    model = staged_gemv_model(p, s, m, k, x, terms=terms)
+    check_linear(y, ref, what=f"ring {m}x{k}", model=model)
+    # with a residual, and the same bits on a second launch
+    out = torch.empty(m, dtype=torch.bfloat16, device=DEV)
+    nf4.nf4_gemv(dp, ds, bf16_tensor(x), m, k, oc.k_pad(k), out, bf16_tensor(res))
+    check_linear(out, ref + res, what=f"ring {m}x{k} + residual", model=model + res)
+    out2 = torch.empty(m, dtype=torch.bfloat16, device=DEV)
+    nf4.nf4_gemv(dp, ds, bf16_tensor(x), m, k, oc.k_pad(k), out2, bf16_tensor(res))
+    assert (bf16_bits(out) == bf16_bits(out2)).all()
+    # the compiler-pipelined kernel on the same inputs: same arithmetic, another order of sums
+    monkeypatch.setenv("CHR_NF4_GEMV_RING", "0")
+    y0 = nf4.nf4_gemv(dp, ds, bf16_tensor(x), m, k, oc.k_pad(k))
+    check_linear(y, to_f32(y0), what=f"ring {m}x{k} vs pipelined", ulps=1)
+
+
+@pytest.mark.parametrize("terms", [1, 2])
+@pytest.mark.parametrize("m,k", [(4100, 5120), (520, 4096), (2100, 6208)])
+def test_ring_gemv_fused_rms(m, k, terms, monkeypatch):
+    monkeypatch.setenv("CHR_NF4_GEMV_RING", "1")
+    monkeypatch.setenv("CHR_NF4_GEMV_TERMS", str(terms))
+    p, s, dp, ds = blobs(m, k, 53)
+    rng = np.random.default_rng(8)
+    x = oc.bf16_round(rng.standard_normal(k).astype(np.float32) * 3)
+    g = oc.bf16_round(1 + 0.1 * rng.standard_normal(k).astype(np.float32))
+    eps = 1e-6
+    y = nf4.nf4_gemv(dp, ds, bf16_tensor(x), m, k, oc.k_pad(k), rms_w=bf16_tensor(g), rms_eps=eps)
+    h = torch.empty(k, dtype=torch.bfloat16, device=DEV)
+    nf4.nf4_rms(bf16_tensor(x), bf16_tensor(g), h, eps)
+    xh = to_f32(h).reshape(-1)
+    ref = oc.c_matmul_f64(oc.c_decode(p, s, m, k), xh[:, None])
+    check_linear(y, ref, what="ring fused rms", ulps=4, model=staged_gemv_model(p, s, m, k, xh, terms=terms))
+    monkeypatch.setenv("CHR_NF4_GEMV_STAGED", "1")
+    y2 = nf4.nf4_gemv(dp, ds, h, m, k, oc.k_pad(k))
+    check_linear(y, to_f32(y2), what="ring fused rms vs rms+gemv", ulps=1)
+
+
+@pytest.mark.parametrize("terms", [1, 2])
+@pytest.mark.parametrize("m,k", [(4100, 4096), (4400, 5120), (20, 5120), (2300, 6144), (1100, 12288),
+                                 (2100, 5056)])
+def test_ring_swiglu(m, k, terms, monkeypatch):
+    say("ring swiglu", m, k, terms)
+    monkeypatch.setenv("CHR_NF4_GEMV_STAGED", "1")
+    monkeypatch.setenv("CHR_NF4_GEMV_RING", "1")
+    monkeypatch.setenv("CHR_NF4_GEMV_TERMS", str(terms))
+    kp = oc.k_pad(k)
+    pg, sg, dpg, dsg = blobs(m, k, 93)
+    pu, su, dpu, dsu = blobs(m, k, 94)
+    x = rand_x(k, None, 14)
+    out = torch.empty(m, dtype=torch.bfloat16, device=DEV)
+    nf4.nf4_swiglu(dpg, dsg, dpu, dsu, bf16_tensor(x), m, k, kp, out)
+    g = oc.c_matmul_f64(oc.c_decode(pg, sg, m, k), x[:, None]).reshape(-1)
+    u = oc.c_matmul_f64(oc.c_decode(pu, su, m, k), x[:, None]).reshape(-1)
+    gm = staged_gemv_model(pg, sg, m, k, x, terms=terms)
+    model = gm / (1 + np.exp(-gm)) * staged_gemv_model(pu, su, m, k, x, terms=terms)
+    check_linear(out, g / (1 + np.exp(-g)) * u, what="ring swiglu", ulps=1.5, model=model)
+    out2 = torch.empty(m, dtype=torch.bfloat16, device=DEV)
+    nf4.nf4_swiglu(dpg, dsg, dpu, dsu, bf16_tensor(x), m, k, kp, out2)
+    assert (bf16_bits(out) == bf16_bits(out2)).all()
+
+
 # ------------------------------------------------------------------------ RMS
 @pytest.mark.parametrize("n", [64, 2048, 5120, 6144, 100])
 def test_rms(n):
