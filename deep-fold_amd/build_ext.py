@@ -66,6 +66,10 @@ def build(force: bool = True, verbose: bool = False) -> str:
         raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{err}")
     if verbose and err.strip():
         print(err, file=sys.stderr)
+    # the ring GEMV kernels rely on what the compiler did with their asm: read it back
+    from . import ring_asm_check
+
+    ring_asm_check.check_source(hipcc(), HIPCC_FLAGS, os.path.join(CSRC, "nf4_gemv.hip"))
     build_host_check()
     return LIB
 

@@ -1139,9 +1139,15 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
     q_locate();
   }
 
-  // one half step of one row into its fixed registers: two instructions
+  // One half step of one row into its fixed registers: two loads.  The s_nop is for the base
+  // registers: where the compiler parks a scalar in a vector register's lane it brings it
+  // back with v_readlane, and a vector memory instruction may read a scalar register that a
+  // vector instruction wrote only five wait states later.  The compiler inserts those for
+  // its own instructions but does not look inside an asm statement (a build that did spill
+  // scalars this way sent requests to stale addresses).
 #define CHR_RING_LOAD(W, SREG, CLOB, VW, VS, WP, SP, I)                                   \
-  asm("global_load_dwordx2 " W ", %1, %2 offset:%5 nt\n\t"                                \
+  asm("s_nop 4\n\t"                                                                       \
+      "global_load_dwordx2 " W ", %1, %2 offset:%5 nt\n\t"                                \
       "global_load_ushort " SREG ", %3, %4 offset:%6 nt"                                  \
       : "+s"(tok)                                                                         \
       : "v"(VW), "s"(WP), "v"(VS), "s"(SP), "n"((I) * 512), "n"((I) * 32)                 \

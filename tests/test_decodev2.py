@@ -273,11 +273,12 @@ def _two_layers(spec, **over):
 
 @pytest.mark.parametrize("name,spec,seed,bias", [
     ("3b-width", _two_layers(dv2.QWEN25_3B), 11, True),
+    ("14b-width", _two_layers(dv2.QWEN25_14B), 14, True),
     ("20b-width", _two_layers(dv2.INTERNLM25_20B), 12, False),
     ("32b-width", _two_layers(dv2.QWEN25_32B), 13, True),
 ])
 def test_two_layers_at_the_real_widths(name, spec, seed, bias):
-    """Two layers of the 3B / 20B / 32B architectures at their real hidden, FFN and head
+    """Two layers of the 3B / 14B / 20B / 32B architectures at their real hidden, FFN and head
     sizes (a 4096-row vocabulary keeps the oracle's lm_head small): eight greedy ids equal
     the oracle's, eager and from the graph, on both launch schedules."""
     say("real widths", name)
