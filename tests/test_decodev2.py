@@ -70,18 +70,32 @@ def test_eager_greedy_matches_the_oracle(spec, seed, prompt):
     assert int(state.valid_len.item()) == len(prompt) + max(0, len(got) - 1)
 
 
+#: see test_teacher_forced_logits_track_the_oracle
+LOGIT_SLACK = 2.5   # measured: 1.7
+
+
 def test_teacher_forced_logits_track_the_oracle():
     spec = dv2.MEDIUM_LLAMA
     model, state, weights = session(spec, 0)
+    worst = 0.0
     toks = [4, 5, 6, 7, 1, 2, 3, 4, 9, 100]
     want = so.teacher_logits(model, toks)
     state.reset()
     for i, t in enumerate(toks):
         dv2.teacher_force_token(state, weights, t)
         got = state.arena.logits.float().cpu().numpy()[0]
-        # bf16 activations through 4 layers: a loose absolute bound on O(1) logits
-        assert np.abs(got - want[i]).max() <= 0.06 * max(1.0, np.abs(want[i]).max()), i
+        # The residual stream is rounded to bf16 twice per layer (after the o and the down
+        # projection) and the logits once more: independent relative errors of 2^-9 rms each,
+        # which the later layers pass on about unchanged, so the logits are off by about
+        # sqrt(2 L + 1) * 2^-9 of their scale; LOGIT_SLACK covers the roundings inside a layer
+        # (q/k/v, attention output, the SwiGLU product) and the tail of the distribution.
+        scale = max(1.0, float(np.abs(want[i]).max()))
+        bound = LOGIT_SLACK * np.sqrt(2 * spec.n_layers + 1) * 2.0 ** -9 * scale
+        err = float(np.abs(got - want[i]).max())
+        worst = max(worst, err / bound)
+        assert err <= bound, (i, err, bound)
         assert int(state.next_token.item()) == int(got.argmax())
+    say(f"  teacher-forced logits: worst error {worst:.3f} of the bound")
 
 
 def test_dirty_kv_tail_is_ignored():

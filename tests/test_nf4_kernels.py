@@ -615,6 +615,22 @@ def attn_ref(q, kc, vc, valid, scale, n_rep):
     return out
 
 
+#: Attention output against a float64 softmax: the kernel accumulates in fp32 and rounds once
+#: to bf16, so an element is within one bf16 step of the exact value (half a step from the
+#: rounding, the rest from fp32 sums and the fast exponential: measured 0.48 at worst), plus a
+#: floor for elements that cancel to almost nothing.
+ATTN_ULPS = 1.0
+ATTN_FLOOR = 2e-4
+
+
+def check_attn(got: np.ndarray, ref: np.ndarray, what: str) -> None:
+    err = np.abs(got.astype(np.float64) - ref.astype(np.float64))
+    bound = ATTN_ULPS * ulp_bf16(ref.astype(np.float64)) + ATTN_FLOOR
+    worst = float((err / bound).max())
+    say(f"  {what}: worst error {worst:.3f} of the bound, max abs {err.max():.2e}")
+    assert worst <= 1.0, (what, worst)
+
+
 @pytest.mark.parametrize("n_q,n_kv,hd,max_seq,valid", [
     (4, 2, 16, 16, 5), (8, 2, 64, 32, 32), (16, 2, 128, 256, 200), (40, 8, 128, 2048, 2048),
     (4, 4, 32, 64, 1), (6, 3, 256, 40, 33), (4, 2, 48, 64, 50), (16, 2, 128, 300, 37)])
@@ -633,13 +649,13 @@ def test_attn_plain(n_q, n_kv, hd, max_seq, valid):
     ref = attn_ref(q.astype(np.float64), kc.astype(np.float64), vc.astype(np.float64), valid, scale,
                    n_q // n_kv)
     got = to_f32(out).reshape(n_q, hd)
-    assert np.abs(got - ref).max() <= 0.02
+    check_attn(got, ref, "attn vs f64")
     # library cross-check: torch SDPA in float32
     tq = torch.from_numpy(q).reshape(1, n_kv, n_q // n_kv, hd)
     tk = torch.from_numpy(kc[:valid]).permute(1, 0, 2).unsqueeze(0)
     tv = torch.from_numpy(vc[:valid]).permute(1, 0, 2).unsqueeze(0)
     sd = F.scaled_dot_product_attention(tq, tk, tv, scale=scale).reshape(n_q, hd).numpy()
-    assert np.abs(got - sd).max() <= 0.02
+    check_attn(got, sd, "attn vs SDPA")
 
 
 @pytest.mark.parametrize("n_q,n_kv,hd,max_seq,pos", [(4, 2, 16, 16, 0), (4, 2, 16, 16, 7),
@@ -677,7 +693,8 @@ def test_attn_fused_rope_and_cache_write(n_q, n_kv, hd, max_seq, pos):
     vfull = vc.astype(np.float64).copy()
     kfull[pos], vfull[pos] = kr, va
     ref = attn_ref(qr, kfull, vfull, pos + 1, scale, n_q // n_kv)
-    assert np.abs(to_f32(out).reshape(n_q, hd) - ref).max() <= 0.02
+    # q is rotated in fp32 and not rounded again, so the same bound holds with the fusion
+    check_attn(to_f32(out).reshape(n_q, hd), ref, "fused attn vs f64")
 
 
 def test_attn_empty_prefix_gives_zero():
@@ -740,14 +757,15 @@ def test_dv2_attn_equals_the_two_launch_form(n_q, n_kv, hd, max_seq, pos):
         kc_b, vc_b = kc0.clone(), vc0.clone()
         out_b = torch.full((n_q * hd,), 3.0, dtype=torch.bfloat16, device=DEV)
         nf4.dv2_attn(q, kc_b, vc_b, out_b, vl, scale, waves, k_act, v_act, tcos, tsin, position)
-        assert np.abs(to_f32(out_a) - to_f32(out_b)).max() <= 0.01, waves
+        # two orders of merging the same fp32 partial states: one bf16 step apart at most
+        check_attn(to_f32(out_b), to_f32(out_a), f"one launch ({waves} wavefronts) vs two")
         assert (bf16_bits(kc_a) == bf16_bits(kc_b)).all() and (bf16_bits(vc_a) == bf16_bits(vc_b)).all()
     # without RoPE / cache-write fusion, against the float64 reference
     out_d = torch.zeros(n_q * hd, dtype=torch.bfloat16, device=DEV)
     nf4.dv2_attn(q, kc_a, vc_a, out_d, vl, scale)
     ref = attn_ref(to_f32(q).astype(np.float64), to_f32(kc_a).astype(np.float64),
                    to_f32(vc_a).astype(np.float64), pos + 1, scale, n_q // n_kv)
-    assert np.abs(to_f32(out_d).reshape(n_q, hd) - ref).max() <= 0.02
+    check_attn(to_f32(out_d).reshape(n_q, hd), ref, "one-launch attn vs f64")
     with pytest.raises(RuntimeError):
         nf4.dv2_attn(q, kc_a, vc_a, out_d, vl, scale, 17)
 
