@@ -1639,17 +1639,23 @@ inline size_t staged_lds_bytes(int K_pad) {
 }
 
 // Whether a staged launch of m groups (rows, or gate/up pairs) goes to the ring kernel where
-// that one takes the row length.  The ring kernel streams faster once it runs (lm_head
-// 152064x5120: 72 against 77 us with one-term levels, 79 against 91 us with two-term ones)
-// but starts about a microsecond later (more scalar set-up ahead of its first requests), so
-// it only pays where a wavefront walks many rows: from 32768 groups up.
+// that one takes the row length.  The ring kernel streams faster once it runs but starts
+// about a microsecond later (more scalar set-up ahead of its first requests), so it pays
+// where a wavefront walks many rows.  Measured, one-term / two-term levels, ring against
+// pipelined: 13824x5120 11.1 / 12.2 against 10.5 / 12.0 us; 20480x5120 13.2 / 15.4 against
+// 16.0 / 17.3; 27648x5120 18.0 / 21.0 against 19.8 / 21.8; 152064x5120 71 / 78 against
+// 77 / 89.  Rows take it from 20480 up; gate/up pairs (whose kernel has the smaller register
+// budget, and which showed no gain inside a decode step at 13824 pairs) from 32768 up.
 // CHR_NF4_GEMV_RING=0: never; =1: wherever the row length allows (read on every launch).
-bool ring_wanted(int m) {
+constexpr int kRingMinRows = 20480;
+constexpr int kRingMinPairs = 32768;
+
+bool ring_wanted(int m, bool pairs) {
   const char *e = std::getenv("CHR_NF4_GEMV_RING");
   if (e != nullptr && e[1] == '\0' && (e[0] == '0' || e[0] == '1')) {
     return e[0] == '1';
   }
-  return m >= 32768;
+  return m >= (pairs ? kRingMinPairs : kRingMinRows);
 }
 
 // Kernel family for a launch of m_total weight rows: 1 staged, 0 plain, -1 staging is
@@ -1671,14 +1677,15 @@ int pick_family(const StreamArgs &a, int m_total) {
 }
 
 // Rows per wavefront of the staged kernels: one, so that even 5120 rows give every
-// wavefront of 256 compute units work; from 32768 rows up the ring kernel (one row) where
-// it takes the row length, else two rows (lm_head 152064x5120: 75 us against 81 us).
+// wavefront of 256 compute units work; the ring kernel (one row) where ring_wanted says so
+// and it takes the row length; else two rows from 32768 up (lm_head 152064x5120: 75 us
+// against 81 us).
 int staged_rows_for_m(int M, int K_pad, bool pairs) {
   const int f = forced_rows();
   if (f > 0) {
     return f;
   }
-  if (ring_wanted(M) && ring_piece_steps(x_half_steps(K_pad), pairs) > 0) {
+  if (ring_wanted(M, pairs) && ring_piece_steps(x_half_steps(K_pad), pairs) > 0) {
     return 1;  // the ring kernel walks one row (or one gate/up pair) per group
   }
   return M >= 32768 ? 2 : 1;
@@ -1698,7 +1705,7 @@ int launch_stream(StreamArgs &a, int n_seg, bool staged, hipStream_t st) {
     const int grid = std::min(device_cu_count(), (total + waves - 1) / waves);
     const bool one_term = level_terms() == 1;
     constexpr bool kRingShape = (SWIGLU && R == 2) || (!SWIGLU && R == 1);
-    const int ring_ns = kRingShape && n_seg == 1 && ring_wanted(total)
+    const int ring_ns = kRingShape && n_seg == 1 && ring_wanted(total, SWIGLU)
                             ? ring_piece_steps(x_half_steps(a.K_pad), SWIGLU) : 0;
     if (ring_ns > 0) {
       const int per_pass = grid * waves;

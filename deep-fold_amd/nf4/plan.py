@@ -118,13 +118,18 @@ def ring_piece_steps(half_steps: int, pairs: bool = False) -> int:
     return 0
 
 
-def ring_wanted(m: int) -> bool:
+RING_MIN_ROWS = 20480
+RING_MIN_PAIRS = 32768
+
+
+def ring_wanted(m: int, pairs: bool = False) -> bool:
     """Whether a staged launch of ``m`` groups goes to the ring kernel where it takes the row
-    length: from 32768 groups up, or as ``CHR_NF4_GEMV_RING`` (0 / 1) says."""
+    length: rows from 20480 up, gate/up pairs from 32768 up, or as ``CHR_NF4_GEMV_RING``
+    (0 / 1) says."""
     e = os.environ.get("CHR_NF4_GEMV_RING")
     if e in ("0", "1"):
         return e == "1"
-    return m >= 32768
+    return m >= (RING_MIN_PAIRS if pairs else RING_MIN_ROWS)
 
 
 def gemv_is_staged(m: int, k: int, k_pad_: int | None = None) -> bool:
