@@ -74,9 +74,8 @@ struct StreamArgs {
   const uint16_t *rms_w;  // optional, bf16 [K]
   int K, K_pad;
   float rms_eps;
-  // ring kernels (one segment): grid size, full passes of 16 * grid groups, and the groups
-  // left after them as left_div * grid + left_mod
-  int ring_grid, ring_passes, ring_left_div, ring_left_mod;
+  // ring kernels: grid size, full passes of 16 * grid groups, and the groups left after them
+  int ring_grid, ring_passes, ring_left;
 };
 
 // Sum of a value over a workgroup of kStagedThreads threads, the same in every thread.
@@ -883,11 +882,9 @@ __global__ __launch_bounds__(1024) void gemv_staged(const StreamArgs a) {
 // operations complete in order, so "at most N outstanding" means everything but the N
 // youngest has arrived: every wait below is exact by construction.
 //
-// D slots of one item (2 half steps) each form a ring: while the oldest item is computed,
-// D-1 younger ones are in flight, and its slot is requested again as soon as it is done.
-// Work is dealt as in the staged kernel's comment, and the groups left after the last full
-// pass are shared out by half steps (one list per wavefront: own groups, then its run of
-// shared half steps, whose sums meet in LDS).
+// NS slots of one half step each form a ring: while the oldest is computed, NS-1 younger
+// ones are in flight, and its slot is requested again as soon as its bytes have been turned
+// into lookup addresses.  Work is dealt as in the staged kernel's comment.
 struct XRegs {
   U32x4 v[kXKeep];  // x, 16-byte vectors i = thread + j * 1024
   U32x4 g[kXKeep];  // the RMSNorm weights at the same places (fused norm only)
@@ -988,31 +985,33 @@ __device__ __forceinline__ float ring_row_dot(const uint32_t (&adr)[8], const ui
 // Here a row is walked in pieces of NS half steps with NS a compile-time constant, one ring
 // slot per half step of a piece: a request is two instructions whose row and piece live in a
 // scalar base pointer and whose half step is an immediate offset, the x pieces are read at
-// immediate offsets from one address per piece, and cursors only move where a piece ends.
-// The left-over groups (shared out by half steps) and the requests past the end of the list
-// go through a second, general cursor that the steady loop never touches.
+// immediate offsets from one address per piece, and the cursors only move where a piece ends.
+//
+// Work is dealt by whole groups: wavefront w of workgroup b walks groups w*grid + b,
+// + 16*grid, ..; after the last full pass the first wavefronts take one more.  (Dealing the
+// left-over groups out by half steps, sums meeting in LDS, made all wavefronts finish
+// together and the launch slower: 10.8 against 10.3 us at 13824x5120 -- while the last
+// groups run, the fewer wavefronts still at work are served faster.)
 template <int NS, bool SWIGLU, int TERMS, bool XREG>
 __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
   static_assert(NS >= 2 && NS <= (SWIGLU ? 6 : 8), "slots of the ring that have registers");
   static_assert(!XREG || NS <= 5, "x of a whole row in 8 * NS registers");
   constexpr int R = SWIGLU ? 2 : 1;
-  constexpr int U = 1;                 // output rows per group
   constexpr int D = NS;                // slots of the ring
   constexpr int kStepLoads = 2 * R;    // vector memory operations of one half step
   // LDS byte address of the x pieces (the pair table starts at LDS address 0)
   constexpr uint32_t kXsAddr = kPairTableBytes + kStagedSmallBytes;
-  extern __shared__ uint4 dyn_lds[];  // [pair table][GemvLds][x pieces][shared-part sums]
+  extern __shared__ uint4 dyn_lds[];  // [pair table][GemvLds][x pieces]
   char *base = reinterpret_cast<char *>(dyn_lds);
   GemvLds &lds = *reinterpret_cast<GemvLds *>(base + kPairTableBytes);
   uint4 *xs = reinterpret_cast<uint4 *>(base + kXsAddr);
-  float *shared_sums = reinterpret_cast<float *>(xs + x_pieces(a.K_pad));
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
   uint32_t tok = 0;  // orders the asm statements among themselves, see CHR_RING_ADDRESSES
 
-  // One segment only (the host sends launches of several segments to the other kernel):
-  // group g is row g, or gate row g and up row g.  How the rows split into full passes and
-  // left-over groups is the same for every wavefront and comes from the host.
+  // Group g is row g of the segments laid end to end (one segment for a plain GEMV, three
+  // for q/k/v), or gate row g and up row g.  How the groups split into full passes and
+  // left-over ones is the same for every wavefront and comes from the host.
   constexpr int waves = kStagedThreads >> 6;
   const int grid = a.ring_grid;
   const int block = static_cast<int>(blockIdx.x);
@@ -1026,10 +1025,9 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
   const bool ragged = rem < kWave;
   const uint64_t row_bytes = static_cast<uint64_t>(a.K_pad >> 1);
   const uint64_t row_scale_bytes = static_cast<uint64_t>(a.K_pad >> 6) << 1;
-  const uint64_t w_base[2] = {reinterpret_cast<uint64_t>(a.packed[0]),
-                              reinterpret_cast<uint64_t>(a.packed2)};
-  const uint64_t s_base[2] = {reinterpret_cast<uint64_t>(a.scale[0]),
-                              reinterpret_cast<uint64_t>(a.scale2)};
+  const int seg_end0 = a.groups[0];
+  const int seg_end1 = a.groups[0] + a.groups[1];
+  const bool one_segment = SWIGLU || a.groups[1] + a.groups[2] == 0;
 
   // per-lane loop constants: byte offsets into a half step of packed bytes / of scales (and
   // their clamped forms for a ragged last step), the x pieces' LDS address, the lane's copy
@@ -1041,24 +1039,34 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
   const uint32_t x_lane = kXsAddr + (static_cast<uint32_t>(lane) << 4);
   const uint32_t lane_off = TERMS == 1 ? static_cast<uint32_t>(lane) << 2
                                        : static_cast<uint32_t>(lane & 31) << 3;
-  const uint64_t all_lanes = ~uint64_t{0};
-  const uint64_t last_lanes = ragged ? ((uint64_t{1} << rem) - 1) : all_lanes;
+  const uint64_t last_lanes = ragged ? ((uint64_t{1} << rem) - 1) : ~uint64_t{0};
 
   // Set-up is written for the number of scalar instructions ahead of the first requests:
   // the 16 wavefronts of a workgroup start together and share four scalar units, so every
-  // instruction here costs four cycles of every wavefront's start.  Only what the own
-  // groups' first requests need comes first; the shared part's cursor is set up behind them.
-  const int passes = a.ring_passes;       // full passes: a whole group per wavefront
-  const int left_base = passes * stride;  // first left-over group; fewer than stride follow
+  // instruction here costs four cycles of every wavefront's start.
+  const int my_groups = a.ring_passes + (first < a.ring_left ? 1 : 0);
 
-  // ---- request cursor over the own groups: piece q_part of group q_group at wq / sq ------
+  // ---- request cursor: piece q_part of group q_group at wq / sq --------------------------
   uint64_t wq[R], sq[R];
-  int q_left = passes * pieces, q_part = 0, q_group = first;
+  int q_left = my_groups * pieces, q_part = 0, q_group = first;
   auto q_locate = [&]() {
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-      wq[r] = w_base[r] + static_cast<uint32_t>(q_group) * row_bytes;
-      sq[r] = s_base[r] + static_cast<uint32_t>(q_group) * row_scale_bytes;
+    if constexpr (SWIGLU) {
+      wq[0] = reinterpret_cast<uint64_t>(a.packed[0]) + static_cast<uint32_t>(q_group) * row_bytes;
+      sq[0] = reinterpret_cast<uint64_t>(a.scale[0]) + static_cast<uint32_t>(q_group) * row_scale_bytes;
+      wq[R - 1] = reinterpret_cast<uint64_t>(a.packed2) + static_cast<uint32_t>(q_group) * row_bytes;
+      sq[R - 1] = reinterpret_cast<uint64_t>(a.scale2) + static_cast<uint32_t>(q_group) * row_scale_bytes;
+    } else {
+      int row = q_group;
+      const uint8_t *pk = a.packed[0];
+      const uint16_t *sc = a.scale[0];
+      if (!one_segment && row >= seg_end0) {
+        const bool third = row >= seg_end1;
+        pk = third ? a.packed[2] : a.packed[1];
+        sc = third ? a.scale[2] : a.scale[1];
+        row -= third ? seg_end1 : seg_end0;
+      }
+      wq[0] = reinterpret_cast<uint64_t>(pk) + static_cast<uint32_t>(row) * row_bytes;
+      sq[0] = reinterpret_cast<uint64_t>(sc) + static_cast<uint32_t>(row) * row_scale_bytes;
     }
   };
   // after the last request of a piece
@@ -1078,63 +1086,6 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
     q_group += stride;
     q_locate();
   };
-
-  // ---- request cursor over the shared half steps [gt, g_end) of group g_group ------------
-  // Once its list is requested it is dead and requests nothing more; the steps from then on
-  // wait for everything in flight instead of for all but the D-1 youngest requests.
-  uint64_t wg[R] = {}, sg[R] = {};
-  int gt = 0, g_end = nsteps, g_group = 0, g_rest = 0;
-  bool g_dead = true;
-  // left-over groups of this workgroup (at most 16) and this wavefront's run of their half
-  // steps: n_shared of them from number sh_k0 on, the first being step sh_t0 of its group
-  int my_left = 0, n_shared = 0, sh_k0 = 0, sh_t0 = 0, sh_end0 = 0;
-  auto g_locate = [&](int grp, int t) {
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-      wg[r] = w_base[r] + static_cast<uint32_t>(grp) * row_bytes + (static_cast<uint32_t>(t) << 9);
-      sg[r] = s_base[r] + static_cast<uint32_t>(grp) * row_scale_bytes +
-              (static_cast<uint32_t>(t) << 5);
-    }
-    g_group = grp;
-    gt = t;
-  };
-  auto g_setup = [&]() {
-    my_left = a.ring_left_div + (block < a.ring_left_mod ? 1 : 0);
-    const int sh_steps = my_left * nsteps;
-    const int sh_run = (sh_steps + waves - 1) / waves;
-    sh_k0 = wave * sh_run;
-    n_shared = max(0, min(sh_run, sh_steps - sh_k0));
-    if (n_shared > 0) {
-      // sh_k0 / nsteps for small operands: the quotient's distance from the next integer is
-      // at least 0.5 / nsteps, far above the rounding of the product
-      const int sh_j0 = static_cast<int>((static_cast<float>(sh_k0) + 0.5f) *
-                                         __builtin_amdgcn_rcpf(static_cast<float>(nsteps)));
-      sh_t0 = sh_k0 - sh_j0 * nsteps;
-      sh_end0 = min(nsteps, sh_t0 + n_shared);  // end of the run's first row piece
-      g_locate(left_base + block + grid * sh_j0, sh_t0);
-      g_end = sh_end0;
-      g_rest = n_shared - (sh_end0 - sh_t0);
-      g_dead = false;
-    }
-  };
-  auto g_advance = [&]() {
-    if (gt + 1 < g_end) {
-      ++gt;
-#pragma unroll
-      for (int r = 0; r < R; ++r) {
-        wg[r] += 512;
-        sg[r] += 32;
-      }
-      return;
-    }
-    if (g_rest > 0) {
-      g_locate(g_group + grid, 0);
-      g_end = min(nsteps, g_rest);
-      g_rest -= g_end;
-      return;
-    }
-    g_dead = true;
-  };
   if (q_left > 0) {
     q_locate();
   }
@@ -1152,8 +1103,8 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
       : "+s"(tok)                                                                         \
       : "v"(VW), "s"(WP), "v"(VS), "s"(SP), "n"((I) * 512), "n"((I) * 32)                 \
       : CLOB);
-  // slot I: half step I of the own piece at wq / sq; LASTP = the piece ends its row
-#define CHR_RING_OWN(I, LASTP)                                                            \
+  // slot I: half step I of the piece at wq / sq; LASTP = the piece ends its row
+#define CHR_RING_REQUEST(I, LASTP)                                                        \
   if constexpr (SWIGLU) {                                                                 \
     if ((I) == NS - 1 && ragged && (LASTP)) {                                             \
       CHR_RING_LOAD(RR2_W(I, 0), RR2_S(I, 0), RR2_CLOB(I, 0), v_wl, v_sl, wq[0], sq[0], I) \
@@ -1169,60 +1120,29 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
       CHR_RING_LOAD(RR1_W(I), RR1_S(I), RR1_CLOB(I), v_w, v_s, wq[0], sq[0], I)           \
     }                                                                                     \
   }
-  // slot I: the general cursor's half step, if it has one left
-#define CHR_RING_GENERAL(I)                                                               \
-  if (!g_dead) {                                                                          \
-    if constexpr (SWIGLU) {                                                               \
-      if (gt == last_t) {                                                                 \
-        CHR_RING_LOAD(RR2_W(I, 0), RR2_S(I, 0), RR2_CLOB(I, 0), v_wl, v_sl, wg[0], sg[0], 0) \
-        CHR_RING_LOAD(RR2_W(I, 1), RR2_S(I, 1), RR2_CLOB(I, 1), v_wl, v_sl, wg[R - 1], sg[R - 1], 0) \
-      } else {                                                                            \
-        CHR_RING_LOAD(RR2_W(I, 0), RR2_S(I, 0), RR2_CLOB(I, 0), v_w, v_s, wg[0], sg[0], 0) \
-        CHR_RING_LOAD(RR2_W(I, 1), RR2_S(I, 1), RR2_CLOB(I, 1), v_w, v_s, wg[R - 1], sg[R - 1], 0) \
-      }                                                                                   \
-    } else {                                                                              \
-      if (gt == last_t) {                                                                 \
-        CHR_RING_LOAD(RR1_W(I), RR1_S(I), RR1_CLOB(I), v_wl, v_sl, wg[0], sg[0], 0)       \
-      } else {                                                                            \
-        CHR_RING_LOAD(RR1_W(I), RR1_S(I), RR1_CLOB(I), v_w, v_s, wg[0], sg[0], 0)         \
-      }                                                                                   \
-    }                                                                                     \
-    g_advance();                                                                          \
-  }
-  // The first NS requests: the first piece of the first own group where there is one (the
-  // usual case: five request instructions and nothing else), otherwise the first shared
-  // half steps.  all_asked says whether all NS were made.
-  bool all_asked = true;
-#define CHR_RING_FILL_OWN(I) \
-  if constexpr (NS > (I)) { CHR_RING_OWN(I, pieces == 1) }
-#define CHR_RING_FILL_GENERAL(I)                                                          \
-  if constexpr (NS > (I)) {                                                               \
-    all_asked = all_asked && !g_dead;                                                     \
-    CHR_RING_GENERAL(I)                                                                   \
-  }
+
+  // The first NS requests: the first piece of the wavefront's first group (five request
+  // instructions and nothing else in the usual case).  A wavefront without work asks for
+  // nothing.
+  const bool any_work = q_left > 0;
+#define CHR_RING_FILL_STEP(I) \
+  if constexpr (NS > (I)) { CHR_RING_REQUEST(I, pieces == 1) }
 #define CHR_RING_FILL                                                                     \
-  if (q_left > 0) {                                                                       \
-    CHR_RING_FILL_OWN(0)                                                                  \
-    CHR_RING_FILL_OWN(1)                                                                  \
-    CHR_RING_FILL_OWN(2)                                                                  \
-    CHR_RING_FILL_OWN(3)                                                                  \
-    CHR_RING_FILL_OWN(4)                                                                  \
-    CHR_RING_FILL_OWN(5)                                                                  \
-    CHR_RING_FILL_OWN(6)                                                                  \
-    CHR_RING_FILL_OWN(7)                                                                  \
+  if (any_work) {                                                                         \
+    CHR_RING_FILL_STEP(0)                                                                 \
+    CHR_RING_FILL_STEP(1)                                                                 \
+    CHR_RING_FILL_STEP(2)                                                                 \
+    CHR_RING_FILL_STEP(3)                                                                 \
+    CHR_RING_FILL_STEP(4)                                                                 \
+    CHR_RING_FILL_STEP(5)                                                                 \
+    CHR_RING_FILL_STEP(6)                                                                 \
+    CHR_RING_FILL_STEP(7)                                                                 \
     q_advance();                                                                          \
-    g_setup();                                                                            \
-  } else {                                                                                \
-    g_setup();                                                                            \
-    CHR_RING_FILL_GENERAL(0)                                                              \
-    CHR_RING_FILL_GENERAL(1)                                                              \
-    CHR_RING_FILL_GENERAL(2)                                                              \
-    CHR_RING_FILL_GENERAL(3)                                                              \
-    CHR_RING_FILL_GENERAL(4)                                                              \
-    CHR_RING_FILL_GENERAL(5)                                                              \
-    CHR_RING_FILL_GENERAL(6)                                                              \
-    CHR_RING_FILL_GENERAL(7)                                                              \
   }
+  // Order of the first requests: x, then the whole ring of weights, and only then the wait
+  // for x: x is the older request, so its (exact) wait does not include the weights, and the
+  // memory system works on the first NS half steps of every wavefront while the level table
+  // is written and x is staged.
   // x travels in registers that the compiler allocates: between its request and its wait
   // there is only this branch's own straight-line code, nothing that could make the compiler
   // move or spill them (hence the two copies of the ring's fill).
@@ -1235,7 +1155,7 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
     } else {
       fill_pair2_table(reinterpret_cast<uint2 *>(dyn_lds), wave, lane);
     }
-    if (!all_asked) {
+    if (!any_work) {
       asm("s_waitcnt vmcnt(0)" : "+s"(tok));
     }
     ring_x_wait<NS * kStepLoads>(xr, tok);
@@ -1258,26 +1178,32 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
     stage_x(a, xs, lds.part);
   }
 #undef CHR_RING_FILL
-#undef CHR_RING_FILL_GENERAL
-#undef CHR_RING_FILL_OWN
+#undef CHR_RING_FILL_STEP
 
   float acc[R] = {};
-  uint16_t *const y_rows = a.y[0];
-  const uint16_t *const add_rows = a.add[0];
   auto finish_group = [&](int grp) {
     if constexpr (SWIGLU) {
       const float gsum = wave_sum(acc[0]);
       const float usum = wave_sum(acc[1]);
       if (lane == 0) {
-        y_rows[grp] = f32_to_bf16(silu(gsum) * usum);
+        a.y[0][grp] = f32_to_bf16(silu(gsum) * usum);
       }
     } else {
+      int row = grp;
+      uint16_t *y = a.y[0];
+      const uint16_t *add = a.add[0];
+      if (!one_segment && row >= seg_end0) {
+        const bool third = row >= seg_end1;
+        y = third ? a.y[2] : a.y[1];
+        add = third ? a.add[2] : a.add[1];
+        row -= third ? seg_end1 : seg_end0;
+      }
       float v = wave_sum(acc[0]);
-      if (add_rows != nullptr) {
-        v += uniform_bf16(add_rows + grp);
+      if (add != nullptr) {
+        v += uniform_bf16(add + row);
       }
       if (lane == 0) {
-        y_rows[grp] = f32_to_bf16(v);
+        y[row] = f32_to_bf16(v);
       }
     }
 #pragma unroll
@@ -1299,12 +1225,12 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
   } else {                                                                                \
     asm("" : "+v"(acc[0]), "+s"(tok));                                                    \
   }
-  // The half step in slot I, its x pieces at XA: wait for it (the D-1 younger half steps
-  // stay in flight), turn its packed bytes into lookup addresses, which frees the slot's
-  // registers, request the slot again at once (REQUEST), and only then look the levels up and
-  // multiply: the new request travels while this half step is computed.  MASK_IF says whether
-  // the lanes past the row's end are to be switched off (LANES_ON the lanes that stay).
-#define CHR_RING_STEP(I, X0, X1, WAIT, REQUEST, MASK_IF, LANES_ON)                        \
+  // The half step in slot I, its x pieces X0 / X1: wait for it (WAIT), turn its packed bytes
+  // into lookup addresses, which frees the slot's registers, request the slot again at once
+  // (REQUEST), and only then look the levels up and multiply: the new request travels while
+  // this half step is computed.  MASK_IF says whether the lanes past the row's end are to be
+  // switched off.
+#define CHR_RING_STEP(I, X0, X1, WAIT, REQUEST, MASK_IF)                                  \
   {                                                                                       \
     const uint4 x0 = X0, x1 = X1;                                                         \
     const uint32_t xw[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};              \
@@ -1316,8 +1242,8 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
       CHR_RING_ADDRESSES(RR2_X(I, 1), RR2_Y(I, 1), RR2_S(I, 1), au, su_, lane_off, tok);  \
       REQUEST                                                                             \
       if (MASK_IF) {                                                                      \
-        CHR_RING_MASKED(sg_, sg_, LANES_ON);                                              \
-        CHR_RING_MASKED(su_, su_, LANES_ON);                                              \
+        CHR_RING_MASKED(sg_, sg_, last_lanes);                                            \
+        CHR_RING_MASKED(su_, su_, last_lanes);                                            \
       }                                                                                   \
       acc[0] = fmaf(sg_, ring_row_dot<TERMS>(ag, xw), acc[0]);                            \
       acc[1] = fmaf(su_, ring_row_dot<TERMS>(au, xw), acc[1]);                            \
@@ -1327,7 +1253,7 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
       CHR_RING_ADDRESSES(RR1_X(I), RR1_Y(I), RR1_S(I), aw, sw_, lane_off, tok);           \
       REQUEST                                                                             \
       if (MASK_IF) {                                                                      \
-        CHR_RING_MASKED(sw_, sw_, LANES_ON);                                              \
+        CHR_RING_MASKED(sw_, sw_, last_lanes);                                            \
       }                                                                                   \
       acc[0] = fmaf(sw_, ring_row_dot<TERMS>(aw, xw), acc[0]);                            \
     }                                                                                     \
@@ -1337,20 +1263,13 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
   // every step so far has requested its slot again: D-1 younger half steps are in flight
 #define CHR_RING_WAIT_FULL \
   asm("s_waitcnt vmcnt(%1)" : "+s"(tok) : "n"((D - 1) * kStepLoads));
-  // the general cursor may have run out: then fewer are, and the wait is for all of them
-#define CHR_RING_WAIT_GENERAL                                                             \
-  if (g_dead) {                                                                           \
-    asm("s_waitcnt vmcnt(0)" : "+s"(tok));                                                \
-  } else {                                                                                \
-    CHR_RING_WAIT_FULL                                                                    \
-  }
+  // the last piece requests nothing: its steps wait for whatever is still on its way
+#define CHR_RING_WAIT_ALL asm("s_waitcnt vmcnt(0)" : "+s"(tok));
 
-  // ---- the own groups, a piece per turn ---------------------------------------------------
-  int c_left = passes * pieces, c_part = 0, c_group = first;
+  // ---- the groups, a piece per turn --------------------------------------------------------
+  int c_left = my_groups * pieces, c_part = 0, c_group = first;
   // XREG (a row is one piece of at most 5 half steps): the lane's x pieces of the whole row
-  // stay in registers for every own group, which takes two 16-byte LDS reads out of each of
-  // their half steps -- 16 of the ~42 cycles that a half step occupies the LDS for, and the
-  // LDS is what bounds the loop.  The shared half steps still read x from the LDS.
+  // stay in registers, which takes two 16-byte LDS reads out of every half step.
   uint4 x_row[XREG ? 2 * NS : 1];
   if constexpr (XREG) {
     if (c_left > 0) {
@@ -1365,10 +1284,10 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
   if constexpr (NS > (I)) {                                                               \
     if constexpr (XREG) {                                                                 \
       CHR_RING_STEP(I, x_row[2 * ((I) % NS)], x_row[2 * ((I) % NS) + 1], WAIT, REQUEST,   \
-                    (I) == NS - 1 && ragged, last_lanes)                                  \
+                    (I) == NS - 1 && ragged)                                              \
     } else {                                                                              \
       CHR_RING_STEP(I, lds0_u128(xa + (I) * 2048), lds0_u128(xa + (I) * 2048 + 1024), WAIT, \
-                    REQUEST, (I) == NS - 1 && ragged && c_last, last_lanes)               \
+                    REQUEST, (I) == NS - 1 && ragged && c_last)                           \
     }                                                                                     \
   }
 #define CHR_RING_PIECE(WAIT, REQUEST_OF, AFTER_REQUESTS)                                  \
@@ -1392,97 +1311,32 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
     } else {                                                                              \
       ++c_part;                                                                           \
     }                                                                                     \
+    (void)xa;                                                                             \
   }
-#define CHR_RING_REQUEST_OWN(I) CHR_RING_OWN(I, q_part == pieces - 1)
-#define CHR_RING_REQUEST_GENERAL(I) CHR_RING_GENERAL(I)
-  // while the piece after this one is an own piece too, every request is an own one
+#define CHR_RING_REQUEST_NEXT(I) CHR_RING_REQUEST(I, q_part == pieces - 1)
+#define CHR_RING_REQUEST_NONE(I)
+  // while a piece is left to request, every step requests its slot again
   while (q_left > 0) {
-    CHR_RING_PIECE(CHR_RING_WAIT_FULL, CHR_RING_REQUEST_OWN, q_advance();)
+    CHR_RING_PIECE(CHR_RING_WAIT_FULL, CHR_RING_REQUEST_NEXT, q_advance();)
   }
-  // the last own piece: its slots go to the shared half steps
-  while (c_left > 0) {
-    CHR_RING_PIECE(CHR_RING_WAIT_GENERAL, CHR_RING_REQUEST_GENERAL, )
-  }
-
-  // ---- the shared half steps: each parks its R sums in LDS --------------------------------
-  {
-    int st = sh_t0, s_end = sh_end0, s_rest = n_shared - (sh_end0 - sh_t0), s_k = sh_k0;
-    int s_todo = n_shared;
-#define CHR_RING_SHARED_STEP(I)                                                           \
-  if constexpr (NS > (I)) {                                                               \
-    if (s_todo > 0) {                                                                     \
-      const uint32_t xa = x_lane + (static_cast<uint32_t>(st) << 11);                     \
-      CHR_RING_STEP(I, lds0_u128(xa), lds0_u128(xa + 1024), CHR_RING_WAIT_GENERAL,        \
-                    CHR_RING_GENERAL(I), ragged && st == last_t, last_lanes)              \
-      _Pragma("unroll") for (int r = 0; r < R; ++r) {                                     \
-        const float v = wave_sum(acc[r]);                                                 \
-        if (lane == 0) {                                                                  \
-          shared_sums[s_k * R + r] = v;                                                   \
-        }                                                                                 \
-        acc[r] = 0.f;                                                                     \
-      }                                                                                   \
-      ++s_k;                                                                              \
-      --s_todo;                                                                           \
-      if (++st == s_end) {                                                                \
-        st = 0;                                                                           \
-        s_end = min(nsteps, s_rest);                                                      \
-        s_rest -= s_end;                                                                  \
-      }                                                                                   \
-    }                                                                                     \
-  }
-    while (s_todo > 0) {
-      CHR_RING_SHARED_STEP(0)
-      CHR_RING_SHARED_STEP(1)
-      CHR_RING_SHARED_STEP(2)
-      CHR_RING_SHARED_STEP(3)
-      CHR_RING_SHARED_STEP(4)
-      CHR_RING_SHARED_STEP(5)
-      CHR_RING_SHARED_STEP(6)
-      CHR_RING_SHARED_STEP(7)
-    }
-#undef CHR_RING_SHARED_STEP
+  // the last piece
+  if (c_left > 0) {
+    CHR_RING_PIECE(CHR_RING_WAIT_ALL, CHR_RING_REQUEST_NONE, )
   }
   // nothing may still be on its way into the fixed registers when the wavefront ends (this
   // statement is volatile: it is what keeps the token chain, and with it every request, alive)
   asm volatile("s_waitcnt vmcnt(0)" : "+s"(tok));
-#undef CHR_RING_REQUEST_GENERAL
-#undef CHR_RING_REQUEST_OWN
+#undef CHR_RING_REQUEST_NONE
+#undef CHR_RING_REQUEST_NEXT
 #undef CHR_RING_PIECE
 #undef CHR_RING_OWN_STEP
-#undef CHR_RING_WAIT_GENERAL
+#undef CHR_RING_WAIT_ALL
 #undef CHR_RING_WAIT_FULL
 #undef CHR_RING_STEP
 #undef CHR_RING_PIN
 #undef CHR_RING_MASKED
-#undef CHR_RING_GENERAL
-#undef CHR_RING_OWN
+#undef CHR_RING_REQUEST
 #undef CHR_RING_LOAD
-
-  // The shared part: wavefront j finishes the workgroup's j-th left-over group (at most 16).
-  if (my_left > 0) {
-    __syncthreads();
-    if (wave < my_left) {
-      const int row = left_base + block + grid * wave;
-      const float *sums = shared_sums + wave * nsteps * R;
-      float s0 = 0.f, s1 = 0.f;
-      for (int t = 0; t < nsteps; ++t) {
-        s0 += sums[t * R];
-        if constexpr (SWIGLU) {
-          s1 += sums[t * R + 1];
-        }
-      }
-      if (lane == 0) {
-        if constexpr (SWIGLU) {
-          y_rows[row] = f32_to_bf16(silu(s0) * s1);
-        } else {
-          if (add_rows != nullptr) {
-            s0 += bf16_to_f32(add_rows[row]);
-          }
-          y_rows[row] = f32_to_bf16(s0);
-        }
-      }
-    }
-  }
 }
 
 // The compiler's VGPR budget stops where the ring's fixed registers begin.  (On this target
@@ -1631,31 +1485,21 @@ int prep_lds(Kern kern, size_t dyn) {
 // more again (10.4, 11.0 us) -- deeper request queues do not pay on this memory system.
 constexpr int kItemSteps = 2;
 
-// pair table, small statics, x pieces, and (ring kernel) the sums of the shared half steps:
-// up to 16 left-over groups of 2 rows per workgroup
+// pair table, small statics, x pieces
 inline size_t staged_lds_bytes(int K_pad) {
-  return kPairTableBytes + kStagedSmallBytes + static_cast<size_t>(x_pieces(K_pad)) * 16 +
-         static_cast<size_t>(x_half_steps(K_pad)) * (kStagedThreads / kWave) * 2 * sizeof(float);
+  return kPairTableBytes + kStagedSmallBytes + static_cast<size_t>(x_pieces(K_pad)) * 16;
 }
 
-// Whether a staged launch of m groups (rows, or gate/up pairs) goes to the ring kernel where
-// that one takes the row length.  The ring kernel streams faster once it runs but starts
-// about a microsecond later (more scalar set-up ahead of its first requests), so it pays
-// where a wavefront walks many rows.  Measured, one-term / two-term levels, ring against
-// pipelined: 13824x5120 11.1 / 12.2 against 10.5 / 12.0 us; 20480x5120 13.2 / 15.4 against
-// 16.0 / 17.3; 27648x5120 18.0 / 21.0 against 19.8 / 21.8; 152064x5120 71 / 78 against
-// 77 / 89.  Rows take it from 20480 up; gate/up pairs (whose kernel has the smaller register
-// budget, and which showed no gain inside a decode step at 13824 pairs) from 32768 up.
-// CHR_NF4_GEMV_RING=0: never; =1: wherever the row length allows (read on every launch).
-constexpr int kRingMinRows = 20480;
-constexpr int kRingMinPairs = 32768;
-
-bool ring_wanted(int m, bool pairs) {
+// Whether staged launches go to the ring kernels where those take the row length: yes.
+// Measured, one-term / two-term levels, ring against pipelined (us): 13824x5120 9.7 / 10.6
+// against 10.8 / 11.6; 5120x13824 10.1 / 10.7 against 11.3 / 11.2; 27648x5120 16.4 / 18.1
+// against 18.6 / 20.7; 152064x5120 72 / 80 against 77 / 89; gate/up 13824x5120 17.3 / 19.4
+// against 20.0 / 21.6; 7168x5120, 5120x5120 and 4096x4096 within 3% either way.
+// CHR_NF4_GEMV_RING=0 keeps every staged launch on the compiler-pipelined kernel (read on
+// every launch).
+bool ring_wanted() {
   const char *e = std::getenv("CHR_NF4_GEMV_RING");
-  if (e != nullptr && e[1] == '\0' && (e[0] == '0' || e[0] == '1')) {
-    return e[0] == '1';
-  }
-  return m >= (pairs ? kRingMinPairs : kRingMinRows);
+  return !(e != nullptr && e[0] == '0' && e[1] == '\0');
 }
 
 // Kernel family for a launch of m_total weight rows: 1 staged, 0 plain, -1 staging is
@@ -1685,7 +1529,7 @@ int staged_rows_for_m(int M, int K_pad, bool pairs) {
   if (f > 0) {
     return f;
   }
-  if (ring_wanted(M, pairs) && ring_piece_steps(x_half_steps(K_pad), pairs) > 0) {
+  if (ring_wanted() && ring_piece_steps(x_half_steps(K_pad), pairs) > 0) {
     return 1;  // the ring kernel walks one row (or one gate/up pair) per group
   }
   return M >= 32768 ? 2 : 1;
@@ -1705,14 +1549,13 @@ int launch_stream(StreamArgs &a, int n_seg, bool staged, hipStream_t st) {
     const int grid = std::min(device_cu_count(), (total + waves - 1) / waves);
     const bool one_term = level_terms() == 1;
     constexpr bool kRingShape = (SWIGLU && R == 2) || (!SWIGLU && R == 1);
-    const int ring_ns = kRingShape && n_seg == 1 && ring_wanted(total, SWIGLU)
+    const int ring_ns = kRingShape && ring_wanted()
                             ? ring_piece_steps(x_half_steps(a.K_pad), SWIGLU) : 0;
     if (ring_ns > 0) {
       const int per_pass = grid * waves;
       a.ring_grid = grid;
       a.ring_passes = total / per_pass;
-      a.ring_left_div = (total % per_pass) / grid;
-      a.ring_left_mod = (total % per_pass) % grid;
+      a.ring_left = total % per_pass;
       if constexpr (kRingShape) {
         auto go = [&](auto kern) {
           if (prep_lds(kern, dyn) != 0) {

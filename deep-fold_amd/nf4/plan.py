@@ -101,12 +101,9 @@ _MAX_DYN_LDS = 150 * 1024
 
 
 def staged_lds_bytes(k_pad_: int) -> int:
-    """LDS of a staged GEMV launch: table, reduction scratch, x in half steps of 1024 codes,
-    and the sums of the half steps that the wavefronts of a workgroup share (up to 16
-    left-over groups of two rows)."""
+    """LDS of a staged GEMV launch: table, reduction scratch, x in half steps of 1024 codes."""
     half_steps = _ceil_div(int(k_pad_) // 16, 64)
-    return (_STAGED_TABLE_BYTES + _STAGED_SMALL_BYTES + half_steps * 128 * 16
-            + half_steps * 16 * 2 * 4)
+    return _STAGED_TABLE_BYTES + _STAGED_SMALL_BYTES + half_steps * 128 * 16
 
 
 def ring_piece_steps(half_steps: int, pairs: bool = False) -> int:
@@ -118,18 +115,10 @@ def ring_piece_steps(half_steps: int, pairs: bool = False) -> int:
     return 0
 
 
-RING_MIN_ROWS = 20480
-RING_MIN_PAIRS = 32768
-
-
-def ring_wanted(m: int, pairs: bool = False) -> bool:
-    """Whether a staged launch of ``m`` groups goes to the ring kernel where it takes the row
-    length: rows from 20480 up, gate/up pairs from 32768 up, or as ``CHR_NF4_GEMV_RING``
-    (0 / 1) says."""
-    e = os.environ.get("CHR_NF4_GEMV_RING")
-    if e in ("0", "1"):
-        return e == "1"
-    return m >= (RING_MIN_PAIRS if pairs else RING_MIN_ROWS)
+def ring_wanted() -> bool:
+    """Whether staged launches go to the ring kernels where those take the row length: yes,
+    unless ``CHR_NF4_GEMV_RING=0``."""
+    return os.environ.get("CHR_NF4_GEMV_RING") != "0"
 
 
 def gemv_is_staged(m: int, k: int, k_pad_: int | None = None) -> bool:
@@ -147,7 +136,7 @@ def gemv_rows_per_wavefront(m: int, forced: int = 0, staged: bool = False,
     if forced in (1, 2, 4):
         return forced
     if staged:
-        if k_pad_ is not None and ring_wanted(m) and ring_piece_steps(_ceil_div(k_pad_ // 16, 64)):
+        if k_pad_ is not None and ring_wanted() and ring_piece_steps(_ceil_div(k_pad_ // 16, 64)):
             return 1
         return 2 if m >= 32768 else 1
     if m >= 32768:

@@ -428,6 +428,40 @@ def test_ring_gemv(m, k, terms, monkeypatch):
 
 
 @pytest.mark.parametrize("terms", [1, 2])
+@pytest.mark.parametrize("mq,mk,k,fused", [(5120, 1024, 5120, True), (4096, 512, 4096, False),
+                                           (130, 33, 6144, True), (3000, 777, 7168, False)])
+def test_ring_qkv(mq, mk, k, fused, terms, monkeypatch):
+    """Three row segments through one ring launch (q/k/v), biases, with and without the folded
+    RMSNorm, against the oracle and against three separate GEMVs."""
+    say("ring qkv", mq, mk, k, fused, terms)
+    monkeypatch.setenv("CHR_NF4_GEMV_STAGED", "1")
+    monkeypatch.setenv("CHR_NF4_GEMV_RING", "1")
+    monkeypatch.setenv("CHR_NF4_GEMV_TERMS", str(terms))
+    mats = [blobs(mq, k, 181), blobs(mk, k, 182), blobs(mk, k, 183)]
+    rng = np.random.default_rng(19)
+    x = rand_x(k, None, 21)
+    g = oc.bf16_round(1 + 0.1 * rng.standard_normal(k).astype(np.float32))
+    biases = [oc.bf16_round(rng.standard_normal(m).astype(np.float32)) for m in (mq, mk, mk)]
+    outs = [torch.empty(m, dtype=torch.bfloat16, device=DEV) for m in (mq, mk, mk)]
+    dx = bf16_tensor(x)
+    rms = (bf16_tensor(g), 1e-6) if fused else (None, 0.0)
+    nf4.nf4_qkv(mats[0][2], mats[0][3], mats[1][2], mats[1][3], mats[2][2], mats[2][3], dx,
+                mq, mk, mk, k, k, outs[0], outs[1], outs[2], *[bf16_tensor(b) for b in biases], *rms)
+    xh = x
+    if fused:
+        h = torch.empty(k, dtype=torch.bfloat16, device=DEV)
+        nf4.nf4_rms(dx, bf16_tensor(g), h, 1e-6)
+        xh = to_f32(h).reshape(-1)
+    for (p, s, dp, ds), m, b, o in zip(mats, (mq, mk, mk), biases, outs):
+        ref = oc.c_matmul_f64(oc.c_decode(p, s, m, k), xh[:, None]).reshape(-1) + b
+        model = staged_gemv_model(p, s, m, k, xh, terms=terms) + b
+        check_linear(o, ref, what="ring qkv", model=model)
+        single = torch.empty(m, dtype=torch.bfloat16, device=DEV)
+        nf4.nf4_gemv(dp, ds, dx, m, k, k, single, bf16_tensor(b), *rms)
+        check_linear(o, to_f32(single), what="ring qkv vs single", ulps=1)
+
+
+@pytest.mark.parametrize("terms", [1, 2])
 @pytest.mark.parametrize("m,k", [(4100, 5120), (520, 4096), (2100, 6208)])
 def test_ring_gemv_fused_rms(m, k, terms, monkeypatch):
     monkeypatch.setenv("CHR_NF4_GEMV_RING", "1")
