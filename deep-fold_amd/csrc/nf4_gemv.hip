@@ -992,10 +992,17 @@ __device__ __forceinline__ float ring_row_dot(const uint32_t (&adr)[8], const ui
 // left-over groups out by half steps, sums meeting in LDS, made all wavefronts finish
 // together and the launch slower: 10.8 against 10.3 us at 13824x5120 -- while the last
 // groups run, the fewer wavefronts still at work are served faster.)
-template <int NS, bool SWIGLU, int TERMS, bool XREG>
+//
+// PAD: a row whose half steps are not a multiple of NS ends in a piece with PAD slots too
+// many.  Those slots are requested like the others (a fixed number of requests per piece is
+// what makes the waits exact), from the piece's first half step, which is there and cached,
+// and never computed.
+template <int NS, bool SWIGLU, int TERMS, bool XREG, int PAD = 0>
 __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
   static_assert(NS >= 2 && NS <= (SWIGLU ? 6 : 8), "slots of the ring that have registers");
   static_assert(!XREG || NS <= 5, "x of a whole row in 8 * NS registers");
+  static_assert(PAD >= 0 && PAD < NS && !(XREG && PAD > 0), "slots left empty in a row's last piece");
+  constexpr int kLastReal = NS - 1 - PAD;  // last slot of a row's last piece that holds a half step
   constexpr int R = SWIGLU ? 2 : 1;
   constexpr int D = NS;                // slots of the ring
   constexpr int kStepLoads = 2 * R;    // vector memory operations of one half step
@@ -1018,8 +1025,8 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
   const int first = wave * grid + block;
   const int stride = grid * waves;
   const int n_half = a.K_pad >> 4;
-  const int nsteps = x_half_steps(a.K_pad);   // a multiple of NS (the host's choice of NS)
-  const int pieces = nsteps / NS;             // pieces of a row
+  const int nsteps = x_half_steps(a.K_pad);   // pieces * NS - PAD (the host's choice of both)
+  const int pieces = (nsteps + PAD) / NS;     // pieces of a row
   const int last_t = nsteps - 1;
   const int rem = n_half - last_t * kWave;  // lanes of a row's last half step that hold a chunk
   const bool ragged = rem < kWave;
@@ -1104,21 +1111,20 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
       : "v"(VW), "s"(WP), "v"(VS), "s"(SP), "n"((I) * 512), "n"((I) * 32)                 \
       : CLOB);
   // slot I: half step I of the piece at wq / sq; LASTP = the piece ends its row
-#define CHR_RING_REQUEST(I, LASTP)                                                        \
+#define CHR_RING_REQUEST_FORM(I, VW, VS, OFF)                                             \
   if constexpr (SWIGLU) {                                                                 \
-    if ((I) == NS - 1 && ragged && (LASTP)) {                                             \
-      CHR_RING_LOAD(RR2_W(I, 0), RR2_S(I, 0), RR2_CLOB(I, 0), v_wl, v_sl, wq[0], sq[0], I) \
-      CHR_RING_LOAD(RR2_W(I, 1), RR2_S(I, 1), RR2_CLOB(I, 1), v_wl, v_sl, wq[R - 1], sq[R - 1], I) \
-    } else {                                                                              \
-      CHR_RING_LOAD(RR2_W(I, 0), RR2_S(I, 0), RR2_CLOB(I, 0), v_w, v_s, wq[0], sq[0], I)  \
-      CHR_RING_LOAD(RR2_W(I, 1), RR2_S(I, 1), RR2_CLOB(I, 1), v_w, v_s, wq[R - 1], sq[R - 1], I) \
-    }                                                                                     \
+    CHR_RING_LOAD(RR2_W(I, 0), RR2_S(I, 0), RR2_CLOB(I, 0), VW, VS, wq[0], sq[0], OFF)    \
+    CHR_RING_LOAD(RR2_W(I, 1), RR2_S(I, 1), RR2_CLOB(I, 1), VW, VS, wq[R - 1], sq[R - 1], OFF) \
   } else {                                                                                \
-    if ((I) == NS - 1 && ragged && (LASTP)) {                                             \
-      CHR_RING_LOAD(RR1_W(I), RR1_S(I), RR1_CLOB(I), v_wl, v_sl, wq[0], sq[0], I)         \
-    } else {                                                                              \
-      CHR_RING_LOAD(RR1_W(I), RR1_S(I), RR1_CLOB(I), v_w, v_s, wq[0], sq[0], I)           \
-    }                                                                                     \
+    CHR_RING_LOAD(RR1_W(I), RR1_S(I), RR1_CLOB(I), VW, VS, wq[0], sq[0], OFF)             \
+  }
+#define CHR_RING_REQUEST(I, LASTP)                                                        \
+  if ((I) > kLastReal && (LASTP)) {                                                       \
+    CHR_RING_REQUEST_FORM(I, v_w, v_s, 0)                                                 \
+  } else if ((I) == kLastReal && ragged && (LASTP)) {                                     \
+    CHR_RING_REQUEST_FORM(I, v_wl, v_sl, I)                                               \
+  } else {                                                                                \
+    CHR_RING_REQUEST_FORM(I, v_w, v_s, I)                                                 \
   }
 
   // The first NS requests: the first piece of the wavefront's first group (five request
@@ -1230,8 +1236,11 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
   // (REQUEST), and only then look the levels up and multiply: the new request travels while
   // this half step is computed.  MASK_IF says whether the lanes past the row's end are to be
   // switched off.
-#define CHR_RING_STEP(I, X0, X1, WAIT, REQUEST, MASK_IF)                                  \
-  {                                                                                       \
+#define CHR_RING_STEP(I, X0, X1, WAIT, REQUEST, MASK_IF, EMPTY_IF)                        \
+  if (EMPTY_IF) {                                                                         \
+    WAIT                                                                                  \
+    REQUEST                                                                               \
+  } else {                                                                                \
     const uint4 x0 = X0, x1 = X1;                                                         \
     const uint32_t xw[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};              \
     WAIT                                                                                  \
@@ -1284,10 +1293,10 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
   if constexpr (NS > (I)) {                                                               \
     if constexpr (XREG) {                                                                 \
       CHR_RING_STEP(I, x_row[2 * ((I) % NS)], x_row[2 * ((I) % NS) + 1], WAIT, REQUEST,   \
-                    (I) == NS - 1 && ragged)                                              \
+                    (I) == NS - 1 && ragged, false)                                       \
     } else {                                                                              \
       CHR_RING_STEP(I, lds0_u128(xa + (I) * 2048), lds0_u128(xa + (I) * 2048 + 1024), WAIT, \
-                    REQUEST, (I) == NS - 1 && ragged && c_last)                           \
+                    REQUEST, (I) == kLastReal && ragged && c_last, (I) > kLastReal && c_last) \
     }                                                                                     \
   }
 #define CHR_RING_PIECE(WAIT, REQUEST_OF, AFTER_REQUESTS)                                  \
@@ -1336,16 +1345,17 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
 #undef CHR_RING_PIN
 #undef CHR_RING_MASKED
 #undef CHR_RING_REQUEST
+#undef CHR_RING_REQUEST_FORM
 #undef CHR_RING_LOAD
 }
 
 // The compiler's VGPR budget stops where the ring's fixed registers begin.  (On this target
 // the attribute counts vector and accumulation registers together and is ignored when the
 // sum exceeds what the launch bounds allow, so it names half the vector registers meant.)
-template <int NS, int TERMS, bool XREG>
+template <int NS, int TERMS, bool XREG, int PAD = 0>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_num_vgpr(52))) void gemv_ring_rows(
     const StreamArgs a) {
-  gemv_ring_body<NS, false, TERMS, XREG>(a);
+  gemv_ring_body<NS, false, TERMS, XREG, PAD>(a);
 }
 
 template <int NS, int TERMS, bool XREG>
@@ -1357,15 +1367,28 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_num_vgpr(46))) void gem
 // Half steps of a piece (= slots of the ring, 512 bytes per row each) for a row of nsteps
 // half steps: the largest divisor the registers hold, at least 4 so that 1.5 KB per row stay
 // in flight (a pure streaming read of a 35 MB matrix by this grid is fastest with 2 KB per
-// wavefront on the way and loses 15% at 4 KB).  0 = the ring kernel does not take this row
-// length (the compiler-pipelined kernel does).
-int ring_piece_steps(int nsteps, bool pairs) {
+// wavefront on the way and loses 15% at 4 KB).  A row kernel also takes a length one half
+// step short of a multiple of 5..8 (11 = 2 * 6 - 1, 27 = 4 * 7 - 1), its last piece ending in
+// one empty slot.  steps == 0: the ring kernel does not take this row length (the
+// compiler-pipelined kernel does).
+struct RingPiece {
+  int steps;
+  int pad;
+};
+RingPiece ring_piece_steps(int nsteps, bool pairs) {
   for (int ns = pairs ? 6 : 8; ns >= 4; --ns) {
     if (nsteps % ns == 0) {
-      return ns;
+      return {ns, 0};
     }
   }
-  return 0;
+  if (!pairs && nsteps > 8) {
+    for (int ns = 8; ns >= 5; --ns) {
+      if ((nsteps + 1) % ns == 0) {
+        return {ns, 1};
+      }
+    }
+  }
+  return {0, 0};
 }
 
 // ---- RMSNorm -----------------------------------------------------------------
@@ -1529,7 +1552,7 @@ int staged_rows_for_m(int M, int K_pad, bool pairs) {
   if (f > 0) {
     return f;
   }
-  if (ring_wanted() && ring_piece_steps(x_half_steps(K_pad), pairs) > 0) {
+  if (ring_wanted() && ring_piece_steps(x_half_steps(K_pad), pairs).steps > 0) {
     return 1;  // the ring kernel walks one row (or one gate/up pair) per group
   }
   return M >= 32768 ? 2 : 1;
@@ -1549,8 +1572,9 @@ int launch_stream(StreamArgs &a, int n_seg, bool staged, hipStream_t st) {
     const int grid = std::min(device_cu_count(), (total + waves - 1) / waves);
     const bool one_term = level_terms() == 1;
     constexpr bool kRingShape = (SWIGLU && R == 2) || (!SWIGLU && R == 1);
-    const int ring_ns = kRingShape && ring_wanted()
-                            ? ring_piece_steps(x_half_steps(a.K_pad), SWIGLU) : 0;
+    const RingPiece ring = kRingShape && ring_wanted()
+                               ? ring_piece_steps(x_half_steps(a.K_pad), SWIGLU) : RingPiece{0, 0};
+    const int ring_ns = ring.steps;
     if (ring_ns > 0) {
       const int per_pass = grid * waves;
       a.ring_grid = grid;
@@ -1581,7 +1605,11 @@ int launch_stream(StreamArgs &a, int n_seg, bool staged, hipStream_t st) {
             case 6: rc = one_term ? go(gemv_ring_pairs<6, 1, false>) : go(gemv_ring_pairs<6, 2, false>); break;
           }
         } else {
-          switch (ring_ns) {
+          switch (ring.pad > 0 ? -ring_ns : ring_ns) {
+            case -5: rc = one_term ? go(gemv_ring_rows<5, 1, false, 1>) : go(gemv_ring_rows<5, 2, false, 1>); break;
+            case -6: rc = one_term ? go(gemv_ring_rows<6, 1, false, 1>) : go(gemv_ring_rows<6, 2, false, 1>); break;
+            case -7: rc = one_term ? go(gemv_ring_rows<7, 1, false, 1>) : go(gemv_ring_rows<7, 2, false, 1>); break;
+            case -8: rc = one_term ? go(gemv_ring_rows<8, 1, false, 1>) : go(gemv_ring_rows<8, 2, false, 1>); break;
             case 4:
               if (one_piece) {
                 rc = one_term ? go(gemv_ring_rows<4, 1, true>) : go(gemv_ring_rows<4, 2, true>);

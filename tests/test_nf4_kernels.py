@@ -388,15 +388,20 @@ def test_swiglu_equals_pair(m, k):
 # half steps of 1024 weights (4..6 for gate/up pairs); by default only from 32768 rows up,
 # CHR_NF4_GEMV_RING=1 sends every such launch to them.
 RING_ROWS = [
-    (4100, 4096),   # 4 half steps, x of the row in registers; one full pass and a shared rest
-    (9000, 5120),   # 5 half steps, two passes
-    (3, 5120),      # fewer rows than wavefronts: shared half steps only
+    (4100, 4096),   # 4 half steps, x of the row in registers; a pass and four rows more
+    (9000, 5120),   # 5 half steps, two passes and a part of a third
+    (3, 5120),      # fewer rows than wavefronts
     (4500, 6144), (4200, 7168), (4100, 8192),
     (700, 13824),   # two pieces of 7 half steps
     (300, 16384),   # two pieces of 8
     (4300, 6208),   # last half step partly filled (4 of 64 lanes)
     (4200, 5056),   # the same with x in registers
     (4100, 4000),   # K below K_pad
+    (4200, 11008),  # 11 half steps: two pieces of 6, the last with an empty slot
+    (600, 27648),   # 27: four pieces of 7, the last with an empty slot
+    (4200, 10950),  # 11 half steps, the last partly filled, then the empty slot
+    (500, 19456),   # 19: four pieces of 5 with an empty slot (x stays in LDS)
+    (400, 23552),   # 23: three pieces of 8 with an empty slot
 ]
 
 
