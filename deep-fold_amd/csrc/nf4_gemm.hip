@@ -40,6 +40,8 @@
 
 #include "nf4_common.h"
 
+#include <type_traits>
+
 #include <atomic>
 
 #include <algorithm>
@@ -103,6 +105,25 @@ constexpr int rows_x_items(int nc, int tps) {
 constexpr int rows_max_tiles(int nc) { return nc == 4 ? 2 : kRowsMaxTiles; }
 constexpr int rows_col_blocks(int N) { return N <= 16 ? 1 : (N <= 32 ? 2 : 4); }
 
+// The stream tile (gemm_stream below): eight wavefronts with 256 registers each on 32 rows and
+// all of K; the pair table, two chunks of x and of weights and the rows' scales in LDS; four
+// chunks of loads in registers.
+constexpr int kStreamBlock = 1024;
+constexpr int kStreamStagers = 512;  // threads of the wavefronts that stage (the other eight multiply)
+constexpr int kStreamRows = 32;
+constexpr int kStreamChunkK = 512;
+constexpr int kStreamRing = 4;
+constexpr int kStreamBodies = 12;   // chunks written out per pass of the loop over K
+constexpr int kStreamMaxGroups = 216;  // K_pad <= 13824: what fits LDS
+constexpr int kStreamXS = kStreamChunkK + kXPad;       // bf16 elements of a token row of one chunk
+constexpr int kStreamXBytes = 32 * kStreamXS * 2;      // one chunk of x, 32 token rows
+constexpr int kStreamWStride = kStreamChunkK / 2 + 16; // bytes of a staged weight row
+constexpr int kStreamWBytes = kStreamRows * kStreamWStride;
+constexpr int kStreamScaleBytes = kStreamMaxGroups * kStreamRows * 2;
+constexpr int kStreamLdsBytes =
+    kPairTableBytes + 2 * kStreamXBytes + 2 * kStreamWBytes + kStreamScaleBytes;
+static_assert(kStreamLdsBytes <= 160 * 1024, "LDS of a compute unit");
+
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
@@ -127,6 +148,21 @@ bool rows_kernel_serves(int N, int tiles_per_split) {
   return on && tiles_per_split <= rows_max_tiles(rows_col_blocks(N));
 }
 
+// The stream tile takes chunks of 8..32 columns in whole 16-byte vectors when K_pad is a
+// multiple of kBK (the four group scales of a row and K tile are then one aligned 8-byte load;
+// gemm_launch checks the pointer), unless a split is forced (it has none).  It is taken where
+// it was measured faster than the split tiles with their reduce: when all its workgroups run
+// at once (no more 32-row blocks than compute units) and K is one pass of its written-out
+// chunks (K_pad <= 6144).  At 14B shapes that is q/k/v (7168x5120: 10.9 / 11.9 / 15.7 us at
+// N = 8 / 16 / 32 against 15.1 / 16.0 / 18.5) and o (10.0 / 11.2 / 14.8 against 12.7 / 13.5 /
+// 15.8), not gate+up (432 workgroups: 28.2 against 24.1 at N = 32) and not down (K = 13824:
+// 29.7 against 23.8).  CHR_NF4_GEMM_STREAM=0 leaves everything to the two older tiles, whose
+// weights are bf16(level * scale) as in the reference's kernel (gpu/nf4/nf4_gemm.cu:312-323).
+bool stream_columns(int N) {
+  static const bool on = env_int("CHR_NF4_GEMM_STREAM", 1) != 0;
+  return on && N >= 8 && N <= 32 && (N & 7) == 0;
+}
+
 Tuning &tuning() {
   static Tuning t = [] {
     Tuning init{};
@@ -148,6 +184,13 @@ int resolved_one_wave() {
 }
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+
+// blocks32: 32-row blocks of the launch (of all its stacked matrices).
+bool stream_kernel_serves(int N, int K_pad, int blocks32) {
+  return stream_columns(N) && tuning().split_k == 0 && K_pad % kBK == 0 &&
+         K_pad <= kStreamBodies * kStreamChunkK && (K_pad >> 6) <= kStreamMaxGroups &&
+         blocks32 <= resolved_one_wave();
+}
 
 // Split-K.  A workgroup is quickest with about three K tiles (measured at every 14B linear
 // shape: fewer tiles leave the fetch latency uncovered, more leave compute units idle), so
@@ -230,7 +273,14 @@ int plan_impl(const chr_nf4_dev_t &h, int32_t N, int32_t have_ws, chr_nf4_plan_t
     p.n_ktiles = ceil_div(h.K_pad, kBK);
     pick_split(p.grid_x, p.n_ktiles, N, have_ws, &p.grid_y, &p.tiles_per_split);
     p.smem_bytes = gemm_lds_bytes(N <= 32 ? 1 : 2);
-    if (rows_kernel_serves(N, p.tiles_per_split)) {
+    if (stream_kernel_serves(N, h.K_pad, ceil_div(h.M, kStreamRows))) {
+      p.bm = kStreamRows;
+      p.block = kStreamBlock;
+      p.grid_x = ceil_div(h.M, kStreamRows);
+      p.grid_y = 1;
+      p.tiles_per_split = p.n_ktiles;
+      p.smem_bytes = kStreamLdsBytes;
+    } else if (rows_kernel_serves(N, p.tiles_per_split)) {
       p.block = kRowsBlock;
       p.smem_bytes = rows_lds_bytes(rows_col_blocks(N), p.tiles_per_split);
     }
@@ -795,6 +845,339 @@ __global__ __launch_bounds__(kRowsBlock) void gemm_rows(const GemmSegs segs,
   }
 }
 
+// ---- stream tile ---------------------------------------------------------------------------
+// The tile for chunks of 8..32 columns in whole 16-byte vectors: a workgroup of sixteen
+// wavefronts owns 32 rows and the WHOLE of K, so a launch has no split-K, no fp32 partials and
+// no second kernel; its epilogue is the reduce's (bias, residual, one rounding to bf16).
+// Eight of the wavefronts multiply, the other eight stage the operands into LDS; a barrier
+// per chunk keeps the two sides one chunk apart.  (One set of wavefronts doing both took the
+// sum of the two times per chunk, 0.7 us at N = 8 and 1.2 us at N = 32 on 7168x5120; two sets
+// take the longer one, 0.6 and 1.1.)
+//
+// Weights never become bf16(level * scale).  A packed byte goes through the GEMV's pair table
+// (byte -> the two levels as a bf16 pair, one v_perm_b32 and one conflict-free LDS read) and
+// the four pairs of a dword are an MFMA A operand as they are.  The k-to-slot map keeps every
+// MFMA inside one 64-wide group: lane l of v_mfma_f32_32x32x16_bf16 supplies eight k of row
+// l % 32 in slots 8 (l / 32) .. + 8, a wavefront step is one group, lane l takes the sixteen
+// bytes (32 codes) of row l % 32 at byte 16 (l / 32) of the group, and the step's four MFMAs
+// take its four dwords: k = 32 (l / 32) + 8 j .. + 8.  Their sum over the group starts from
+// zero and enters the accumulator through one fp32 multiply-add with the group's scale per
+// output row, so the scale is applied once per 64 products instead of once per weight,
+// exactly (fp16 -> fp32), and the only rounding of a weight is bf16(level).
+//
+// K is walked in chunks of 512 (eight groups): multiplying wavefront w works on group w of
+// every chunk, all eight on the same 32 rows, and their eight sums of an output meet in LDS at
+// the end, added in the order of the wavefronts.  Every element of x is therefore read from LDS once
+// per workgroup, and every B operand by one wavefront only.
+//
+// Scales: all of the 32 rows' scales are staged in LDS at the start ([group][row], fp16).  An
+// accumulator lane holds rows 8 b + 4 (l / 32) + i (b, i = 0..3): lane l reads the scale of
+// row 8 ((l % 16) / 4) + 4 (l / 32) + l % 4, which puts the row of accumulator value v at
+// position v of every row of sixteen lanes, where a DPP row broadcast fetches it.
+//
+// Global memory is read with consecutive lanes on consecutive bytes only (a load whose lanes
+// read 64 different rows keeps the memory pipeline's address stage busy for some 140 cycles
+// whatever its width, and the MFMA layout is one row per lane): a chunk of weights, 32 rows x
+// 256 bytes, is one 16-byte load per staging thread, passed through LDS (row stride 272
+// bytes, conflict-free for the 16-byte operand reads); a chunk of x is one or two items per
+// staging thread (two k x eight columns each), interleaved into the transposed chunk buffer.
+//
+// Pipeline: a staging thread keeps its loads of four chunks (three above 16 columns) in
+// flight in registers and stores a chunk to LDS (two buffers) one chunk ahead of its use.  Every request is unconditional --
+// past the end of K it repeats the last chunk, unused -- and kStreamBodies chunks are written
+// out nested (chunk c + 1 inside the "if" of chunk c) inside the loop over K, because vector
+// loads return in order and are waited for by count: only with a fixed number of requests
+// between a request and its use can the compiler wait for the oldest alone, and where a loop
+// closes, or two paths meet, its count starts over (it waits there for nearly everything in
+// flight).  Up to kStreamBodies chunks (K <= 6144) the loop never closes.
+static_assert(8 * 64 * 16 * 4 <= kPairTableBytes, "the wavefronts' sums reuse the table");
+
+// f(0); if (1 < n) { f(1); if (2 < n) { ... } }: chunk C is reached through chunk C - 1 only, so
+// the compiler knows every request of the earlier chunks to have been issued.
+template <int C, int MAX, class F>
+__device__ __forceinline__ void nest_chunks(int n, F &f) {
+  if constexpr (C < MAX) {
+    if (C == 0 || C < n) {
+      f(std::integral_constant<int, C>{});
+      nest_chunks<C + 1, MAX>(n, f);
+    }
+  }
+}
+
+// acc += (position V of this lane's row of sixteen lanes of `mine`) * t
+template <int V>
+__device__ __forceinline__ float scale_into(float acc, float mine, float t) {
+  const int s = __builtin_amdgcn_update_dpp(0, __float_as_int(mine), 0x150 + V, 0xF, 0xF, true);
+  return fmaf(__int_as_float(s), t, acc);
+}
+
+// segs.blocks counts 32-row blocks here.  XI: staging items of x per thread (2 above 16
+// columns).
+template <int XI>
+__global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
+                                                            const uint16_t *__restrict__ x,
+                                                            uint16_t *__restrict__ y,
+                                                            float *__restrict__ partial, int M_all,
+                                                            int K, int K_pad, int N,
+                                                            const uint16_t *__restrict__ bias,
+                                                            const uint16_t *res) {
+  constexpr int XS = kStreamXS;
+  constexpr int CK = kStreamChunkK;
+  constexpr uint32_t kXAddr = kPairTableBytes;
+  constexpr uint32_t kWAddr = kXAddr + 2 * kStreamXBytes;
+  constexpr uint32_t kScaleAddr = kWAddr + 2 * kStreamWBytes;
+  static_assert(kScaleAddr + kStreamScaleBytes == kStreamLdsBytes, "LDS map");
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave16 = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const bool stager = wave16 >= 8;  // wavefronts 8..15 stage, 0..7 multiply
+  const int wave = wave16 & 7;      // group of a chunk (multiplying), or eighth of the staging
+  const int stid = tid & (kStreamStagers - 1);
+  int bx = static_cast<int>(blockIdx.x);
+  int seg = 0;
+  if (bx >= segs.blocks[0]) {
+    bx -= segs.blocks[0];
+    seg = 1;
+    if (bx >= segs.blocks[1]) {
+      bx -= segs.blocks[1];
+      seg = 2;
+    }
+  }
+  const uint8_t *__restrict__ packed = segs.packed[seg];
+  const uint16_t *__restrict__ scale = segs.scale[seg];
+  const int M = segs.M[seg];
+  const int out0 = segs.row0[seg];
+  const int row_base = bx * kStreamRows;
+  const int r = lane & 31;  // row of the A operand, token of the B operand
+  const int h = lane >> 5;  // which half of a group's k
+  const int row_bytes = K_pad >> 1;
+  const int groups = K_pad >> 6;
+  const int n_ch = (K_pad + CK - 1) / CK;
+
+  // ---- requests: a thread's share of one chunk ------------------------------------------------
+  struct Item {
+    uint4 w;             // bytes 16 (stid % 16) .. + 16 of the chunk of row stid / 16
+    uint4 a[XI], b[XI];  // x: rows 2 kp, 2 kp + 1 of the chunk, columns 8 q .. + 8
+  };
+  const uint8_t *wp = packed + static_cast<size_t>(min(row_base + (stid >> 4), M - 1)) * row_bytes;
+  const int w_piece = 16 * (stid & 15);
+  const int nv = N >> 3;
+  const int n_items = (CK / 2) * nv;
+  int xkp[XI], xq[XI];
+#pragma unroll
+  for (int it = 0; it < XI; ++it) {
+    const int idx = min(stid + it * kStreamStagers, n_items - 1);
+    xkp[it] = idx / nv;
+    xq[it] = idx - xkp[it] * nv;
+  }
+  auto load = [&](int c, Item &v) {
+    const int cc = min(c, n_ch - 1);
+    v.w = *reinterpret_cast<const uint4 *>(wp + min(cc * (CK / 2) + w_piece, row_bytes - 16));
+#pragma unroll
+    for (int it = 0; it < XI; ++it) {
+      const int k = cc * CK + 2 * xkp[it];
+      v.a[it] = *reinterpret_cast<const uint4 *>(x + static_cast<size_t>(min(k, K - 1)) * N + 8 * xq[it]);
+      v.b[it] =
+          *reinterpret_cast<const uint4 *>(x + static_cast<size_t>(min(k + 1, K - 1)) * N + 8 * xq[it]);
+    }
+  };
+  auto store = [&](int c, const Item &v) {
+    const int buf = c & 1;
+    // weights: row-major, 272 bytes a row.  A piece past the end of the row (the second half
+    // of a last chunk of 256) repeats the row's last 16 bytes; x is zero there.
+    *reinterpret_cast<uint4 *>(lds_raw + kWAddr + buf * kStreamWBytes + (stid >> 4) * kStreamWStride +
+                               w_piece) = v.w;
+    uint32_t *xd = reinterpret_cast<uint32_t *>(lds_raw + kXAddr + buf * kStreamXBytes);
+#pragma unroll
+    for (int it = 0; it < XI; ++it) {
+      if (stid + it * kStreamStagers < n_items) {
+        const int k = c * CK + 2 * xkp[it];
+        const bool ka = k < K, kb = k + 1 < K;
+        const uint32_t a[4] = {ka ? v.a[it].x : 0u, ka ? v.a[it].y : 0u, ka ? v.a[it].z : 0u,
+                               ka ? v.a[it].w : 0u};
+        const uint32_t b[4] = {kb ? v.b[it].x : 0u, kb ? v.b[it].y : 0u, kb ? v.b[it].z : 0u,
+                               kb ? v.b[it].w : 0u};
+        uint32_t *dst = xd + (8 * xq[it]) * (XS / 2) + xkp[it];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          dst[(2 * e) * (XS / 2)] = (a[e] & 0xFFFFu) | (b[e] << 16);
+          dst[(2 * e + 1) * (XS / 2)] = (a[e] >> 16) | (b[e] & 0xFFFF0000u);
+        }
+      }
+    }
+  };
+
+  // ---- set-up -------------------------------------------------------------------------------
+  // The rows' scales (four groups -- 8 aligned bytes, K_pad being a multiple of 256 -- a
+  // request, a fixed number of requests a thread, the surplus repeating the last one) and
+  // the staging wavefronts' requests in the order the chunks keep them in; the table while
+  // they travel.
+  constexpr int kScaleLoads = (kStreamRows * (kStreamMaxGroups / 4) + kStreamBlock - 1) / kStreamBlock;
+  const int quads = groups >> 2;
+  uint2 sv[kScaleLoads];
+#pragma unroll
+  for (int it = 0; it < kScaleLoads; ++it) {
+    const int i = min(tid + it * kStreamBlock, kStreamRows * quads - 1);
+    const int srow = i / quads;
+    sv[it] = *reinterpret_cast<const uint2 *>(
+        scale + static_cast<size_t>(min(row_base + srow, M - 1)) * groups + 4 * (i - srow * quads));
+  }
+  // chunks a staging thread keeps in flight: with two items of x a chunk, three are what
+  // 128 registers hold
+  constexpr int R = XI == 2 ? 3 : kStreamRing;
+  static_assert(kStreamBodies % R == 0, "slots of the written-out chunks are compile-time");
+  Item ring[R];
+  if (stager) {
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      load(j, ring[j]);
+    }
+  }
+  fill_pair_table(reinterpret_cast<uint32_t *>(lds_raw), wave16, lane);
+  {
+    // token rows N .. 32 of the chunk buffers are never staged: zero them once
+    const int nz = (32 - N) * (XS / 2);
+    for (int b = 0; b < 2; ++b) {
+      uint32_t *z = reinterpret_cast<uint32_t *>(lds_raw + kXAddr + b * kStreamXBytes) + N * (XS / 2);
+      for (int i = tid; i < nz; i += kStreamBlock) {
+        z[i] = 0u;
+      }
+    }
+  }
+  {
+    uint16_t *sl = reinterpret_cast<uint16_t *>(lds_raw + kScaleAddr);  // [group][row of the 32]
+#pragma unroll
+    for (int it = 0; it < kScaleLoads; ++it) {
+      const int i = tid + it * kStreamBlock;
+      if (i < kStreamRows * quads) {
+        const int srow = i / quads;
+        const int gq = i - srow * quads;
+        sl[(4 * gq + 0) * kStreamRows + srow] = static_cast<uint16_t>(sv[it].x);
+        sl[(4 * gq + 1) * kStreamRows + srow] = static_cast<uint16_t>(sv[it].x >> 16);
+        sl[(4 * gq + 2) * kStreamRows + srow] = static_cast<uint16_t>(sv[it].y);
+        sl[(4 * gq + 3) * kStreamRows + srow] = static_cast<uint16_t>(sv[it].y >> 16);
+      }
+    }
+  }
+  if (stager) {
+    store(0, ring[0]);
+    load(R, ring[0]);
+  }
+  __syncthreads();
+
+  // ---- the chunks: one barrier each, in both roles ------------------------------------------
+  f32x16 acc;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    acc[v] = 0.f;
+  }
+  if (stager) {
+    for (int c0 = 0; c0 < n_ch; c0 += kStreamBodies) {
+      auto chunk = [&](auto index) {
+        constexpr int cb = decltype(index)::value;  // kStreamBodies is a multiple of the ring
+        constexpr int j = cb % R;
+        const int c = c0 + cb;
+        // chunk c + 1 goes into the buffers that chunk c - 1 was read from (the multiplying
+        // wavefronts are past those reads: the barrier of chunk c - 1); its registers take
+        // chunk c + 1 + R
+        if (c + 1 < n_ch) {
+          store(c + 1, ring[(j + 1) % R]);
+        }
+        load(c + 1 + R, ring[(j + 1) % R]);
+        __syncthreads();
+      };
+      nest_chunks<0, kStreamBodies>(n_ch - c0, chunk);
+    }
+  } else {
+    const uint32_t lane4 = static_cast<uint32_t>(lane) << 2;
+    const uint32_t x_lane = kXAddr + static_cast<uint32_t>(r * XS + 32 * h + 64 * wave) * 2;
+    const uint32_t w_lane = kWAddr + static_cast<uint32_t>(r * kStreamWStride + 32 * wave + 16 * h);
+    // this lane's scale: row 8 ((l % 16) / 4) + 4 h + l % 4 of the 32, group `wave` of the chunk
+    const uint32_t s_lane =
+        kScaleAddr + static_cast<uint32_t>(wave * kStreamRows + 8 * ((lane & 15) >> 2) + 4 * h + (lane & 3)) * 2;
+    for (int c = 0; c < n_ch; ++c) {
+      const uint32_t buf = static_cast<uint32_t>(c & 1);
+      // a group past the end of K (last chunk of 256) multiplies zeros of x; its scale is read
+      // from the last group that exists
+      const int grp = min(8 * c + wave, groups - 1) - wave;
+      const float mine = f16_to_f32(*reinterpret_cast<const __attribute__((address_space(3))) uint16_t *>(
+          s_lane + static_cast<uint32_t>(grp * kStreamRows * 2)));
+      const uint4 wv = lds0_u128(w_lane + buf * kStreamWBytes);
+      const uint32_t w4[4] = {wv.x, wv.y, wv.z, wv.w};
+      const uint32_t xl = x_lane + buf * kStreamXBytes;
+      f32x16 t;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        t[v] = 0.f;
+      }
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) {
+        const uint4 b = lds0_u128(xl + 16 * jj);
+        const uint4 a = make_uint4(pair_at<0>(w4[jj], lane4), pair_at<1>(w4[jj], lane4),
+                                   pair_at<2>(w4[jj], lane4), pair_at<3>(w4[jj], lane4));
+        t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                    __builtin_bit_cast(bf16x8, b), t, 0, 0, 0);
+      }
+      acc[0] = scale_into<0>(acc[0], mine, t[0]);
+      acc[1] = scale_into<1>(acc[1], mine, t[1]);
+      acc[2] = scale_into<2>(acc[2], mine, t[2]);
+      acc[3] = scale_into<3>(acc[3], mine, t[3]);
+      acc[4] = scale_into<4>(acc[4], mine, t[4]);
+      acc[5] = scale_into<5>(acc[5], mine, t[5]);
+      acc[6] = scale_into<6>(acc[6], mine, t[6]);
+      acc[7] = scale_into<7>(acc[7], mine, t[7]);
+      acc[8] = scale_into<8>(acc[8], mine, t[8]);
+      acc[9] = scale_into<9>(acc[9], mine, t[9]);
+      acc[10] = scale_into<10>(acc[10], mine, t[10]);
+      acc[11] = scale_into<11>(acc[11], mine, t[11]);
+      acc[12] = scale_into<12>(acc[12], mine, t[12]);
+      acc[13] = scale_into<13>(acc[13], mine, t[13]);
+      acc[14] = scale_into<14>(acc[14], mine, t[14]);
+      acc[15] = scale_into<15>(acc[15], mine, t[15]);
+      __syncthreads();
+    }
+  }
+
+  // ---- the eight sums of every output meet in LDS ---------------------------------------------
+  // (the last barrier above has every wavefront past its reads of the table)
+  float *sums = reinterpret_cast<float *>(lds_raw);
+  if (!stager) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      sums[(wave * 16 + v) * kWave + lane] = acc[v];
+    }
+  }
+  __syncthreads();
+  // wavefront w of the sixteen finishes accumulator value w
+  {
+    const int v = wave16;
+    float o32 = 0.f;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      o32 += sums[(q * 16 + v) * kWave + lane];
+    }
+    const int n = r;
+    const int rr = row_base + 8 * (v >> 2) + 4 * h + (v & 3);
+    if (n < N && rr < M) {
+      const size_t at = static_cast<size_t>(out0 + rr) * N + n;
+      if (partial == nullptr) {
+        // the epilogue of reduce_splitk, here (res may alias y: same thread, same element)
+        uint16_t o = f32_to_bf16(o32);
+        if (bias != nullptr) {
+          o = f32_to_bf16(bf16_to_f32(o) + bf16_to_f32(bias[out0 + rr]));
+        }
+        if (res != nullptr) {
+          o = f32_to_bf16(bf16_to_f32(res[at]) + bf16_to_f32(o));
+        }
+        y[at] = o;
+      } else {
+        partial[at] = o32;
+      }
+    }
+  }
+}
+
 struct RowsArgs {
   GemmSegs segs;
   const uint16_t *x;
@@ -1024,6 +1407,15 @@ int gemm_lds_ready() {
         return -6;
       }
     }
+    if (hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_stream<1>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize,
+                            kStreamLdsBytes) != hipSuccess ||
+        hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_stream<2>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize,
+                            kStreamLdsBytes) != hipSuccess) {
+      (void)hipGetLastError();
+      return -6;
+    }
     const RowsArgs none{};
     for (int vec = 0; vec < 2; ++vec) {
       for (int nc = 1; nc <= 4; nc *= 2) {
@@ -1073,21 +1465,35 @@ struct StackPlan {
   GemmSegs segs;
   int M_all, grid_x, grid_y, n_ktiles, tiles_per_split;
   int64_t ws_floats;
+  bool stream;  // the stream tile: 32-row blocks, no split
 };
 
-StackPlan plan_stack(const chr_nf4_dev_t *h, int nseg, int N, int have_ws) {
+// allow_stream: false when the launch cannot take the stream tile for a reason the shape does
+// not show (scales not 8-byte aligned).
+StackPlan plan_stack(const chr_nf4_dev_t *h, int nseg, int N, int have_ws, bool allow_stream = true) {
   StackPlan sp{};
+  int blocks32 = 0;
+  for (int i = 0; i < nseg; ++i) {
+    blocks32 += ceil_div(h[i].M, kStreamRows);
+  }
+  sp.stream = allow_stream && stream_kernel_serves(N, h[0].K_pad, blocks32);
+  const int bm = sp.stream ? kStreamRows : kBM;
   for (int i = 0; i < 3; ++i) {
     const bool on = i < nseg;
     sp.segs.packed[i] = on ? h[i].packed : nullptr;
     sp.segs.scale[i] = on ? h[i].scale : nullptr;
     sp.segs.M[i] = on ? h[i].M : 0;
-    sp.segs.blocks[i] = on ? ceil_div(h[i].M, kBM) : 0;
+    sp.segs.blocks[i] = on ? ceil_div(h[i].M, bm) : 0;
     sp.segs.row0[i] = sp.M_all;
     sp.M_all += sp.segs.M[i];
     sp.grid_x += sp.segs.blocks[i];
   }
   sp.n_ktiles = ceil_div(h[0].K_pad, kBK);
+  if (sp.stream) {
+    sp.grid_y = 1;
+    sp.tiles_per_split = sp.n_ktiles;
+    return sp;
+  }
   pick_split(sp.grid_x, sp.n_ktiles, N, have_ws, &sp.grid_y, &sp.tiles_per_split);
   sp.ws_floats = sp.grid_y > 1 ? static_cast<int64_t>(sp.grid_y) * sp.M_all * N : 0;
   return sp;
@@ -1134,7 +1540,11 @@ int gemm_launch(const chr_nf4_dev_t *const *w, int nseg, const void *x, void *y,
     return gemv_entry(&h[0], x, y, stream, nullptr, nullptr, 0.f);
   }
   const int have_ws = (ws != nullptr && ws_floats > 0) ? 1 : 0;
-  StackPlan sp = plan_stack(h, nseg, N, have_ws);
+  bool scales_aligned8 = true;
+  for (int i = 0; i < nseg; ++i) {
+    scales_aligned8 = scales_aligned8 && (reinterpret_cast<uintptr_t>(h[i].scale) & 7u) == 0;
+  }
+  StackPlan sp = plan_stack(h, nseg, N, have_ws, scales_aligned8);
   if (swiglu) {
     // the activation lives in the reduce, so this launch always goes through fp32 partials
     if (nseg != 2 || h[0].M != h[1].M || bias != nullptr || res != nullptr) {
@@ -1160,7 +1570,15 @@ int gemm_launch(const chr_nf4_dev_t *const *w, int nseg, const void *x, void *y,
   const dim3 block(kGemmBlock);
   const int K = h[0].K, K_pad = h[0].K_pad;
   const int nc = rows_col_blocks(N);
-  if (rows_kernel_serves(N, sp.tiles_per_split)) {
+  if (sp.stream) {
+    if (N <= 16) {
+      gemm_stream<1><<<grid, dim3(kStreamBlock), kStreamLdsBytes, st>>>(
+          sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp);
+    } else {
+      gemm_stream<2><<<grid, dim3(kStreamBlock), kStreamLdsBytes, st>>>(
+          sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp);
+    }
+  } else if (rows_kernel_serves(N, sp.tiles_per_split)) {
     const RowsArgs ra{sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp};
     // the vector staging needs whole 16-byte vectors per row of x
     if (rows_dispatch((N & 7) == 0, nc, sp.tiles_per_split, ra, grid, st, false) != 0) {

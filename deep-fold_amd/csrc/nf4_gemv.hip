@@ -340,16 +340,6 @@ __device__ __forceinline__ void rows_step(const uint32_t (&w)[R][NW], const floa
   }
 }
 
-// ---- pair table (kernels that stage x in LDS) ---------------------------------------
-// One packed byte holds two codes; the table maps a byte to the two levels as a bf16
-// pair, and every lane owns a copy: entry (byte, lane) is the dword at byte address
-// byte*256 + lane*4, so the 64 lookups of a wavefront always fall in 64 different banks
-// whatever the codes are.  The table starts at LDS address 0 (these kernels have no
-// static LDS), which makes a lookup address one v_perm_b32: byte 1 = the packed byte,
-// byte 0 = 4*lane.  A pair meets two activations, kept as the bf16 pair they arrive as,
-// in one v_dot2c_f32_bf16: per two weights one address op, one LDS read and one
-// multiply-add, against two of each with the 16-entry table.
-constexpr int kPairTableBytes = 256 * 64 * 4;
 constexpr int kStagedSmallBytes = 512;  // GemvLds of a staged kernel, after the table
 static_assert(sizeof(GemvLds) <= kStagedSmallBytes, "GemvLds must fit its slot");
 
@@ -358,32 +348,6 @@ typedef __attribute__((ext_vector_type(2))) __bf16 Bf16x2;
 __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float acc) {
   return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(Bf16x2, a),
                                          __builtin_bit_cast(Bf16x2, b), acc, false);
-}
-
-__device__ __forceinline__ uint32_t lds0_u32(uint32_t addr) {
-  return *reinterpret_cast<const __attribute__((address_space(3))) uint32_t *>(addr);
-}
-
-template <int J>
-__device__ __forceinline__ uint32_t pair_at(uint32_t w, uint32_t lane4) {
-  // selector: result byte 0 <- lane4 byte 0, byte 1 <- w byte J, bytes 2..3 <- 0x00
-  constexpr uint32_t sel = 0x0C0C0400u + (static_cast<uint32_t>(J) << 8);
-  return lds0_u32(__builtin_amdgcn_perm(w, lane4, sel));
-}
-
-// bf16 bits (round to nearest even) of a finite binary32 pattern, usable at compile time.
-constexpr uint32_t bf16_bits_rne(uint32_t b) { return (b + 0x7FFFu + ((b >> 16) & 1u)) >> 16; }
-
-// Fill the table from a workgroup of exactly 16 wavefronts; the caller's next barrier
-// publishes it.  Wavefront v writes the bytes whose low code is v: byte = v + 16*j has
-// high code j, a compile-time constant, so an entry costs one OR and one LDS store.
-__device__ __forceinline__ void fill_pair_table(uint32_t *table, int wave, int lane) {
-  const uint32_t lo = bf16_bits_rne(kLutBits[wave]);
-#pragma unroll
-  for (int j = 0; j < 16; ++j) {
-    const uint32_t hi = bf16_bits_rne(kLevelBits[j]) << 16;
-    table[((wave + 16 * j) << 6) + lane] = lo | hi;
-  }
 }
 
 // ---- two-term pair table ----------------------------------------------------------------
@@ -415,11 +379,6 @@ __device__ __forceinline__ void fill_pair2_table(uint2 *table, int wave, int lan
     const uint32_t hi_t = odd ? level_tail_bf16(kLevelBits[2 * jj + 1]) : level_tail_bf16(kLevelBits[2 * jj]);
     table[((wave + 16 * j) << 5) + copy] = make_uint2(lo_h | (hi_h << 16), lo_t | (hi_t << 16));
   }
-}
-
-__device__ __forceinline__ uint4 lds0_u128(uint32_t addr) {
-  const U32x4 v = *reinterpret_cast<const __attribute__((address_space(3))) U32x4 *>(addr);
-  return make_uint4(v.x, v.y, v.z, v.w);
 }
 
 __device__ __forceinline__ uint2 lds0_u64(uint32_t addr) {

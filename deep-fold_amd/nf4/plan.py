@@ -44,6 +44,7 @@ __all__ = [
     "gemv_rows_per_wavefront",
     "gemv_is_staged",
     "staged_lds_bytes",
+    "gemm_streams",
     "gemm_streams_rows",
     "STAGED_MIN_CODES",
     "plan",
@@ -197,6 +198,42 @@ def _rows_kernel_on() -> bool:
     return _ROWS_ON
 
 
+_STREAM_ON: bool | None = None
+_STREAM_ROWS = 32
+_STREAM_MAX_GROUPS = 216
+#: LDS of the stream tile: pair table, two chunks of x (32 token rows of 512 + 8), two chunks of
+#: weights (32 rows of 256 + 16 bytes), the scales of 32 rows
+_STREAM_LDS = 256 * 64 * 4 + 2 * 32 * 520 * 2 + 2 * 32 * 272 + _STREAM_MAX_GROUPS * 32 * 2
+
+
+def _stream_columns(N: int) -> bool:  # noqa: N803
+    """Chunk widths the stream tile takes (8, 16, 24, 32) unless ``CHR_NF4_GEMM_STREAM=0``
+    (read once, like the library does)."""
+    global _STREAM_ON
+    if _STREAM_ON is None:
+        raw = os.environ.get("CHR_NF4_GEMM_STREAM", "")
+        try:
+            _STREAM_ON = int(raw) != 0 if raw.strip() else True
+        except ValueError:
+            _STREAM_ON = False
+    return _STREAM_ON and 8 <= N <= 32 and N % 8 == 0
+
+
+def gemm_streams(M: int, N: int, k_pad_: int, force_split: int = 0,  # noqa: N803
+                 one_wave: int = ONE_WAVE) -> bool:
+    """Whether a launch runs the stream tile (a workgroup of sixteen wavefronts on 32 rows and
+    all of K: no split-K, no partials, no reduce; pair-table lookups, the scale applied per
+    64-wide group): whole-vector chunks of up to 32 columns, no forced split, ``K_pad`` a
+    multiple of 256 and at most 6144, and no more 32-row blocks than compute units.  ``M``
+    counts the rows of all stacked matrices (each a multiple of 32, or count its 32-row blocks
+    and pass 32 times that).  (The library also wants the scales 8-byte aligned, which device
+    allocations are.)"""
+    kp = int(k_pad_)
+    blocks32 = _ceil_div(int(M), _STREAM_ROWS)
+    return (_stream_columns(N) and force_split <= 0 and kp % _BK == 0
+            and kp <= 12 * 512 and blocks32 <= int(one_wave))
+
+
 def _pick_split_rows(grid_x: int, n_ktiles: int, cus: int, fallback: int) -> int:
     """Split for the row-streaming tile (chunks of up to 32 columns): slices of 1..4 K tiles,
     cost = slices of the busiest compute unit x tiles (2 us each; 2.8 when a launch leaves one
@@ -255,6 +292,10 @@ def plan(M: int, K: int, N: int = 1, *, K_pad: int | None = None, have_ws: bool 
     path = PREFILL if N <= 16 else (PREFILL_N32 if N <= 32 else PREFILL_N64)
     grid_x = _ceil_div(M, _BM)
     n_ktiles = _ceil_div(kp, _BK)
+    if gemm_streams(M, N, kp, force_split, one_wave):
+        grid_x = _ceil_div(M, _STREAM_ROWS)
+        return Plan(path, grid_x, 1, 1024, _STREAM_ROWS, _BK, n_ktiles, n_ktiles, grid_x,
+                    _STREAM_LDS, 0)
     split, tps = _pick_split(grid_x, n_ktiles, N, have_ws, force_split, one_wave)
     ws = split * M * N if split > 1 else 0
     if gemm_streams_rows(N, tps):

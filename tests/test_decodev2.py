@@ -228,7 +228,11 @@ def near_tie(logits: np.ndarray) -> bool:
 #: top-1/top-2 gap of ~0.1 and a minimum over 64 picks that is usually below one bf16 step
 #: of the logit, so some streams meet a coin-toss pick; these are the counts measured with
 #: the levels kept as two bf16 terms (fp32-class weights), asserted as floors.
-IDENTICAL_FLOOR = {"plain": 1, "fold_rms": 1, "fp32_levels": 1, "one_term": 1}
+#: One-term (bf16) levels carry 2^-9 of weight rounding into every logit: which side of a
+#: near-tie a stream lands on then changes with the summation order of the kernel that
+#: serves a row length, and no stream is promised to stay identical for 64 picks (every
+#: difference is still checked to sit at a near-tie of the oracle).
+IDENTICAL_FLOOR = {"plain": 1, "fold_rms": 1, "fp32_levels": 1, "one_term": 0}
 
 
 def _streams_64(monkeypatch, form: str) -> tuple[int, list[str]]:

@@ -8,10 +8,13 @@ import pytest
 import torch
 import torch.nn.functional as F
 
+from deepfold_amd import nf4
 from deepfold_amd.chr0.loader import ChrMatrix
 from deepfold_amd.host import CompressedLinear, k_pad, nf4_linear
 from deepfold_amd.ring import HostImage
 from oracle import nf4_oracle as oc
+
+from helpers import staged_gemv_model
 
 
 def blobs(m, k, seed=0, sigma=0.05):
@@ -88,11 +91,25 @@ def test_forward_matches_linear_on_the_decoded_matrix(lead, bias):
     x = torch.randn(*lead, k, generator=g, device="cuda").to(torch.bfloat16)
     y = lin(x)
     assert y.shape == (*lead, m) and y.dtype == torch.bfloat16
-    # the GEMM multiplies bf16-rounded weights (gpu/nf4/nf4_gemm.cu:312-323); one token goes
-    # to the GEMV, which keeps them in fp32
+    # the split-K tiles multiply bf16-rounded weights (gpu/nf4/nf4_gemm.cu:312-323); whole
+    # vectors of up to 32 tokens go to the tile that multiplies bf16(level) and scales each
+    # group's sum; one token goes to the GEMV, which keeps the weights in fp32
+    # (the module feeds the GEMM windows of at most 32 tokens: the expectation goes window by
+    # window too)
     n = int(np.prod(lead))
-    wk = w if n == 1 else w.to(torch.bfloat16).float()
-    want = (x.reshape(n, k).double() @ wk.double().t()).to(torch.bfloat16)
+    x2 = x.reshape(n, k)
+    parts = []
+    for t0 in range(0, n, 32):
+        xw = x2[t0:t0 + 32]
+        nw = xw.shape[0]
+        if nw > 1 and nf4.nf4_plan(m, k, nw)["bm"] == 32:
+            model = staged_gemv_model(p.numpy(), s.numpy().view(np.uint16), m, k,
+                                      xw.float().cpu().numpy().T, terms=1)
+            parts.append(torch.from_numpy(model.T.copy()).cuda().to(torch.bfloat16))
+        else:
+            wk = w if n == 1 else w.to(torch.bfloat16).float()
+            parts.append((xw.double() @ wk.double().t()).to(torch.bfloat16))
+    want = torch.cat(parts, dim=0)
     if bias:
         want = want + b
     want = want.reshape(*lead, m).double()

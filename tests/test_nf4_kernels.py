@@ -526,6 +526,16 @@ def test_rms(n):
 
 
 # ----------------------------------------------------------------------- GEMM
+def gemm_expected(p, s, m, k, x, plan):
+    """What a prefill launch computes, in float64, by the tile its plan names.  The stream
+    tile (the only one with 32-row blocks) multiplies bf16(level) and applies the fp16 scale
+    to each 64-wide group's sum; the two older tiles multiply bf16(level * scale), the
+    reference kernel's weights (gpu/nf4/nf4_gemm.cu:312-323)."""
+    if plan["bm"] == 32:
+        return staged_gemv_model(p, s, m, k, x, terms=1)
+    return oc.c_matmul_f64(oc.bf16_round(oc.c_decode(p, s, m, k)), x)
+
+
 GEMM_SHAPES = [(128, 256), (130, 65), (64, 2048), (300, 5120), (129, 13824), (5120, 512)]
 
 
@@ -538,8 +548,8 @@ def test_gemm_vs_oracle(m, k, n):
     y = nf4.nf4_gemm(dp, ds, bf16_tensor(x), m, k, oc.k_pad(k))
     assert tuple(y.shape) == (m, n)
     w = oc.c_decode(p, s, m, k)
-    # the MFMA path rounds each weight to bf16 before multiplying
-    ref_b = oc.c_matmul_f64(oc.bf16_round(w), x)
+    # against the arithmetic of the tile that ran (each rounds a weight to bf16 once)
+    ref_b = gemm_expected(p, s, m, k, x, nf4.nf4_plan(m, k, n))
     check_linear(y, ref_b, what=f"gemm {m}x{k} n{n} (bf16 weights)")
     # and stays inside the reference's floor-1 bound against unrounded weights
     ref = oc.c_matmul_f64(w, x)
@@ -548,29 +558,39 @@ def test_gemm_vs_oracle(m, k, n):
     assert err.max() / np.abs(ref).max() <= 1e-2
 
 
-def test_gemm_column_subset_equals_padded():
+@pytest.mark.parametrize("wide,narrow", [(16, 8), (32, 16), (7, 3)])
+def test_gemm_column_subset_equals_padded(wide, narrow):
+    """Columns do not mix: a chunk whose extra columns are zero gives the narrower chunk's
+    bits (within one tile family: whole-vector widths run the stream tile, others not)."""
     m, k = 256, 1024
     p, s, dp, ds = blobs(m, k, 301)
-    x = rand_x(k, 16, 13)
-    x3 = x.copy()
-    x3[:, 3:] = 0
-    y16 = nf4.nf4_gemm(dp, ds, bf16_tensor(x3), m, k, k)
-    y3 = nf4.nf4_gemm(dp, ds, bf16_tensor(x[:, :3]), m, k, k)
-    assert (bf16_bits(y3) == bf16_bits(y16[:, :3].contiguous())).all()
-    assert (to_f32(y16[:, 3:]) == 0).all()
+    x = rand_x(k, wide, 13)
+    xz = x.copy()
+    xz[:, narrow:] = 0
+    y_wide = nf4.nf4_gemm(dp, ds, bf16_tensor(xz), m, k, k)
+    y_narrow = nf4.nf4_gemm(dp, ds, bf16_tensor(np.ascontiguousarray(x[:, :narrow])), m, k, k)
+    assert (bf16_bits(y_narrow) == bf16_bits(y_wide[:, :narrow].contiguous())).all()
+    assert (to_f32(y_wide[:, narrow:]) == 0).all()
 
 
-@pytest.mark.parametrize("n", [8, 32])
+@pytest.mark.parametrize("n", [8, 32, 5])
 def test_gemm_every_split_agrees(n):
+    """Forced splits (the two split-K tiles; the stream tile has no split): each against the
+    arithmetic of the tile its plan names, and against each other within two bf16 steps
+    (summation order only)."""
     m, k = 512, 4096
     p, s, dp, ds = blobs(m, k, 302)
-    x = bf16_tensor(rand_x(k, n, 14))
+    xh = rand_x(k, n, 14)
+    x = bf16_tensor(xh)
     outs = []
     try:
         for split in (1, 2, 3, 5, 16):
             nf4.nf4_set_tuning(split_k=split)
-            assert nf4.nf4_plan(m, k, n)["grid_y"] == min(split, 16) or split == 5
-            outs.append(to_f32(nf4.nf4_gemm(dp, ds, x, m, k, k)))
+            plan = nf4.nf4_plan(m, k, n)
+            assert plan["bm"] == 128 and (plan["grid_y"] == min(split, 16) or split == 5)
+            y = nf4.nf4_gemm(dp, ds, x, m, k, k)
+            check_linear(y, gemm_expected(p, s, m, k, xh, plan), what=f"split {split} n{n}")
+            outs.append(to_f32(y))
     finally:
         nf4.nf4_set_tuning()
     for o in outs[1:]:
@@ -578,13 +598,51 @@ def test_gemm_every_split_agrees(n):
         assert (d <= 2.0 ** (np.floor(np.log2(np.maximum(np.abs(outs[0]), 2.0 ** -120))) - 7) + 1e-30).all()
 
 
+STREAM_CASES = [
+    # m, k, n
+    (32, 256, 8), (130, 512, 16), (200, 768, 24),   # a ragged last block; a last chunk of 256
+    (96, 1000, 32),                                  # K below K_pad
+    (256, 5120, 32), (70, 6144, 8),                  # ten and twelve chunks
+    (2048, 2048, 32), (5120, 5120, 8), (7168, 5120, 16),
+    (8192, 1024, 32),                                # as many workgroups as compute units
+]
+
+
+@pytest.mark.parametrize("m,k,n", STREAM_CASES)
+def test_gemm_stream_tile(m, k, n):
+    """The tile without split-K (32 rows and all of K per workgroup, bf16(level) times the
+    activations, the scale applied to each group's sum): against that arithmetic in float64,
+    bit-identical on a second launch, and its fused epilogue against the separate adds."""
+    say("gemm stream", m, k, n)
+    p, s, dp, ds = blobs(m, k, 900 + m + k + n)
+    xh = rand_x(k, n, 19)
+    x = bf16_tensor(xh)
+    kp = oc.k_pad(k)
+    plan = nf4.nf4_plan(m, k, n)
+    assert (plan["bm"], plan["grid_y"], plan["ws_floats"], plan["block"]) == (32, 1, 0, 1024)
+    assert plan["grid_x"] == -(-m // 32)
+    y = nf4.nf4_gemm(dp, ds, x, m, k, kp)
+    check_linear(y, staged_gemv_model(p, s, m, k, xh, terms=1), what=f"stream {m}x{k} n{n}")
+    ref = oc.c_matmul_f64(oc.c_decode(p, s, m, k), xh)
+    err = np.abs(to_f32(y).astype(np.float64) - ref)
+    assert (err <= np.maximum(0.05, 2 ** (np.floor(np.log2(np.maximum(np.abs(ref), 1e-30))) - 8))).all()
+    assert (bf16_bits(nf4.nf4_gemm(dp, ds, x, m, k, kp)) == bf16_bits(y)).all()
+    rng = np.random.default_rng(m + n)
+    bias = bf16_tensor(oc.bf16_round(rng.standard_normal(m).astype(np.float32)))
+    res = bf16_tensor(oc.bf16_round(rng.standard_normal((m, n)).astype(np.float32)))
+    want = res + (y + bias[:, None])
+    got = nf4.nf4_gemm(dp, ds, x, m, k, kp, bias=bias, residual=res)
+    assert (bf16_bits(got) == bf16_bits(want)).all()
+
+
 @pytest.mark.parametrize("n", [5, 8, 16, 24, 32, 40, 64])
 @pytest.mark.parametrize("k,split,tiles", [(1024, 1, 4), (1000, 2, 2), (1024, 4, 1), (768, 1, 3),
                                            (2048, 1, 8), (2048, 8, 1)])
 def test_gemm_every_tile_variant(n, k, split, tiles):
-    """Slice lengths of one to four K tiles (the row-streaming tile, one build per length and
-    per 16-column block count; two tiles at most above 32 columns) and an eight-tile slice
-    (the K-tiled kernel), with whole-vector and ragged column counts and a ragged row block."""
+    """The two split-K tiles under forced splits: slice lengths of one to four K tiles (the
+    row-streaming tile, one build per length and per 16-column block count; two tiles at most
+    above 32 columns) and an eight-tile slice (the K-tiled kernel), with whole-vector and
+    ragged column counts and a ragged row block."""
     m = 200
     say("gemm variant", m, k, n, split)
     p, s, dp, ds = blobs(m, k, 310 + k)
@@ -593,13 +651,12 @@ def test_gemm_every_tile_variant(n, k, split, tiles):
         nf4.nf4_set_tuning(split_k=split)
         plan = nf4.nf4_plan(m, k, n)
         assert (plan["grid_y"], plan["tiles_per_split"]) == (split, tiles)
-        streams = tiles <= (2 if n > 32 else 4)
-        assert plan["block"] == (512 if streams else 256)
+        streams_rows = tiles <= (2 if n > 32 else 4)
+        assert plan["bm"] == 128 and plan["block"] == (512 if streams_rows else 256)
         y = nf4.nf4_gemm(dp, ds, bf16_tensor(x), m, k, oc.k_pad(k), max_n=64)
     finally:
         nf4.nf4_set_tuning()
-    ref = oc.c_matmul_f64(oc.bf16_round(oc.c_decode(p, s, m, k)), x)
-    check_linear(y, ref, what=f"gemm {m}x{k} n{n} split {split}")
+    check_linear(y, gemm_expected(p, s, m, k, x, plan), what=f"gemm {m}x{k} n{n} split {split}")
 
 
 def test_gemm_n1_routes_to_gemv():
@@ -617,14 +674,24 @@ PREFILL_14B = [("qkv", 7168, 5120), ("o", 5120, 5120), ("gate_up", 13824, 5120),
 @pytest.mark.parametrize("name,m,k", PREFILL_14B, ids=[s[0] for s in PREFILL_14B])
 def test_gemm_full_14b_shapes(name, m, k):
     """Every 14B linear shape at N = 8, 16, 32 through ``nf4_gemm`` at full size, all rows
-    against the oracle product on bf16-rounded weights."""
+    against the oracle's weights rounded the way the launch's tile rounds them, and against
+    the unrounded oracle product within the reference's bounds."""
     w, p, s, dp, ds = quantized(m, k, 21 + m % 97)
-    ref_w = oc.bf16_round(oc.c_decode(p, s, m, k))
+    exact_w = oc.c_decode(p, s, m, k)
     for n in (8, 16, 32):
         say("gemm 14B shape", name, m, k, n)
         x = rand_x(k, n, 16 + n)
         y = nf4.nf4_gemm(dp, ds, bf16_tensor(x), m, k, k)
-        check_linear(y, oc.c_matmul_f64(ref_w, x), what=f"prefill {name} n{n}")
+        plan = nf4.nf4_plan(m, k, n)
+        # one workgroup per 32 rows and all of K where that is one round of the GPU and one
+        # pass of its written-out chunks (q/k/v and o); split-K tiles elsewhere
+        streams = -(-m // 32) <= 256 and k <= 6144
+        assert (plan["bm"], plan["grid_y"] == 1) == ((32, True) if streams else (128, False))
+        ref = oc.c_matmul_f64(exact_w, x)
+        err = np.abs(to_f32(y).astype(np.float64) - ref)
+        assert (err <= np.maximum(0.05, 2 ** (np.floor(np.log2(np.maximum(np.abs(ref), 1e-30))) - 8))).all()
+        assert err.max() / np.abs(ref).max() <= 1e-2
+        check_linear(y, gemm_expected(p, s, m, k, x, plan), what=f"prefill {name} n{n} (tile)")
 
 
 # ------------------------------------------------------------------ attention

@@ -45,8 +45,8 @@ def test_noalloc_equals_workspace_entry_twice_second_smaller():
     ws_floats = int(lib.chr_nf4_gemm_noalloc_max_floats())
     assert ws_floats == 4 << 20
     ws = torch.empty(ws_floats, dtype=torch.float32, device="cuda")
-    # first call: a 14B q/k/v chunk, split-K over several slices of partials
-    m, k, n = 7168, 5120, 32
+    # first call: a 14B gate or up chunk, split-K over several slices of partials
+    m, k, n = 13824, 5120, 32
     plan = nf4.nf4_plan(m, k, n)
     assert plan["grid_y"] > 1 and 0 < plan["ws_floats"] <= ws_floats
     rc_ws, rc_na, y_ws, y_na, (packed, scale, x) = _both(lib, m, k, n, 5, ws, ws_floats)
@@ -59,11 +59,15 @@ def test_noalloc_equals_workspace_entry_twice_second_smaller():
     got = y_na[torch.from_numpy(rows).cuda()].double()
     assert float((got - want).abs().max()) <= 1e-2 * float(want.abs().max())
     # second call, smaller, straight after: stale partials of the first must not show
-    m2, k2, n2 = 640, 2048, 8
+    m2, k2, n2 = 640, 2048, 5
     assert nf4.nf4_plan(m2, k2, n2)["grid_y"] > 1
     rc_ws, rc_na, y_ws, y_na, _ = _both(lib, m2, k2, n2, 9, ws, ws_floats)
     assert rc_ws == 0 and rc_na == 0
     assert torch.equal(y_ws.view(torch.int16), y_na.view(torch.int16))
+    # a chunk that the tile without split-K takes (no partials), through both entries alike
+    assert nf4.nf4_plan(7168, 5120, 32)["grid_y"] == 1
+    rc_ws, rc_na, y_ws, y_na, _ = _both(lib, 7168, 5120, 32, 10, ws, ws_floats)
+    assert rc_ws == 0 and rc_na == 0 and torch.equal(y_ws.view(torch.int16), y_na.view(torch.int16))
     # N = 1 goes to the GEMV (no partials at all) through both entries alike
     rc_ws, rc_na, y_ws, y_na, _ = _both(lib, 512, 1024, 1, 11, ws, ws_floats)
     assert rc_ws == 0 and rc_na == 0 and torch.equal(y_ws.view(torch.int16), y_na.view(torch.int16))
