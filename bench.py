@@ -33,7 +33,7 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes one GEMV launch of the primary workload moves, from FETCH_SIZE + WRITE_SIZE
-# hardware counters scaled by a plain device copy (profiles/gemv_staged_13824x5120_pmc.txt
+# hardware counters scaled by a plain device copy (profiles/gemv_ring_rows_13824x5120_pmc.txt
 # has the runs and the arithmetic).  Hardware counters cannot be read inside this process.
 GEMV_TRAFFIC_BYTES = 39_618_434
 MFMA_BF16_PEAK_TFLOPS = 2500.0
@@ -193,15 +193,18 @@ def bench_gemv_shapes(torch, nf4):
     return rows
 
 
-def bench_prefill(torch, nf4):
-    """MFMA GEMM chunks at the 14B linear shapes; weights rotate through > 512 MB."""
+def bench_prefill(torch, nf4, only=None, widths=(8, 16, 32, 64)):
+    """MFMA GEMM chunks at the 14B linear shapes; weights rotate through > 512 MB.  A launch
+    is the tile kernel and, where it splits K, its reduce."""
     shapes = {"qkv": (7168, 5120), "o": (5120, 5120), "gate_up": (13824, 5120), "down": (5120, 13824)}
     rows = []
     for name, (m, k) in shapes.items():
+        if only and name not in only:
+            continue
         by1 = algorithmic_bytes(m, k, 1)
         copies = -(-512 * 1024 * 1024 // by1) + 1
         weights = make_weights(torch, nf4, m, k, copies, seed=4321)
-        for n in (8, 16, 32, 64):  # 64: the chunk width of the feature-major prefill
+        for n in widths:  # 64: the chunk width of the feature-major prefill
             x = (torch.randn((k, n), device="cuda") ).to(torch.bfloat16)
 
             def launch(i):
@@ -210,7 +213,10 @@ def bench_prefill(torch, nf4):
 
             ms = graph_time(torch, launch, 3 * copies, reps=3)
             by = algorithmic_bytes(m, k, n)
-            rows.append({"layer": name, "M": m, "K": k, "N": n, "us": ms * 1e3,
+            plan = nf4.nf4_plan(m, k, n)
+            tile = ("stream (32 rows x all of K, no split)" if plan["bm"] == 32
+                    else f"split-K x{plan['grid_y']} + reduce")
+            rows.append({"layer": name, "M": m, "K": k, "N": n, "us": ms * 1e3, "tile": tile,
                          "gbps": by / (ms * 1e-3) / 1e9,
                          "hbm_frac": by / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                          "mfma_frac": 2.0 * m * k * n / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS})
@@ -450,6 +456,8 @@ def main() -> int:
     ap.add_argument("--no-decode", action="store_true", help="skip the model decode leg")
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill GEMM sweep")
     ap.add_argument("--no-ring", action="store_true", help="skip the host-streaming ring leg")
+    ap.add_argument("--prefill-layers", default="", help="comma list of qkv,o,gate_up,down (default all)")
+    ap.add_argument("--prefill-widths", default="8,16,32,64", help="chunk widths of the prefill sweep")
     ap.add_argument("--decode-models", default="3b,14b,20b,32b", help="comma list of 3b,14b,20b,32b")
     ap.add_argument("--no-shapes", action="store_true", help="skip the GEMV sweep over other shapes")
     ap.add_argument("--schedule", default=None, help="decode launch schedule: plain or fold_rms")
@@ -526,11 +534,11 @@ def main() -> int:
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS,
             "traffic": GEMV_TRAFFIC_BYTES if (M, K) == (13824, 5120) else None,
-            "kernel": "gemv_staged (two-term levels)",
+            "kernel": "gemv_ring_rows<5,2,true> (two-term levels)",
             "algorithmic_bytes_per_launch": by,
         },
         # the same launches on the same copies through the other two kernel forms
-        "roofline_one_term": roofline_of(forms["one_term"], "gemv_staged (one bf16 level)",
+        "roofline_one_term": roofline_of(forms["one_term"], "gemv_ring_rows<5,1,true> (one bf16 level)",
                                          "bf16 levels x bf16 activations"),
         "roofline_fp32_levels": roofline_of(forms["fp32_levels"], "gemv_stream (plain)",
                                             "fp32 levels x fp32-widened activations, 128-bit loads"),
@@ -557,7 +565,9 @@ def main() -> int:
                 rows.append(fast)
         out["decode"] = rows
     if not args.no_prefill:
-        out["prefill"] = bench_prefill(torch, nf4)
+        only = [v.strip() for v in args.prefill_layers.split(",") if v.strip()]
+        widths = tuple(int(v) for v in args.prefill_widths.split(",") if v.strip())
+        out["prefill"] = bench_prefill(torch, nf4, only, widths)
     if not args.no_ring:
         out["ring"] = bench_ring(torch, nf4)
     if not args.no_cpu:

@@ -113,8 +113,8 @@ constexpr int kStreamStagers = 512;  // threads of the wavefronts that stage (th
 constexpr int kStreamRows = 32;
 constexpr int kStreamChunkK = 512;
 constexpr int kStreamRing = 4;
-constexpr int kStreamBodies = 12;   // chunks written out per pass of the loop over K
-constexpr int kStreamMaxGroups = 216;  // K_pad <= 13824: what fits LDS
+constexpr int kStreamBodies = 12;   // chunks of the longest K the tile takes, written out one by one
+constexpr int kStreamMaxGroups = kStreamBodies * kStreamChunkK / 64;  // groups of the longest K
 constexpr int kStreamXS = kStreamChunkK + kXPad;       // bf16 elements of a token row of one chunk
 constexpr int kStreamXBytes = 32 * kStreamXS * 2;      // one chunk of x, 32 token rows
 constexpr int kStreamWStride = kStreamChunkK / 2 + 16; // bytes of a staged weight row
@@ -188,7 +188,7 @@ inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 // blocks32: 32-row blocks of the launch (of all its stacked matrices).
 bool stream_kernel_serves(int N, int K_pad, int blocks32) {
   return stream_columns(N) && tuning().split_k == 0 && K_pad % kBK == 0 &&
-         K_pad <= kStreamBodies * kStreamChunkK && (K_pad >> 6) <= kStreamMaxGroups &&
+         K_pad <= kStreamBodies * kStreamChunkK &&
          blocks32 <= resolved_one_wave();
 }
 
@@ -884,12 +884,13 @@ __global__ __launch_bounds__(kRowsBlock) void gemm_rows(const GemmSegs segs,
 //
 // Pipeline: a staging thread keeps its loads of four chunks (three above 16 columns) in
 // flight in registers and stores a chunk to LDS (two buffers) one chunk ahead of its use.  Every request is unconditional --
-// past the end of K it repeats the last chunk, unused -- and kStreamBodies chunks are written
-// out nested (chunk c + 1 inside the "if" of chunk c) inside the loop over K, because vector
-// loads return in order and are waited for by count: only with a fixed number of requests
-// between a request and its use can the compiler wait for the oldest alone, and where a loop
-// closes, or two paths meet, its count starts over (it waits there for nearly everything in
-// flight).  Up to kStreamBodies chunks (K <= 6144) the loop never closes.
+// past the end of K it repeats the last chunk, unused -- and the chunks of the longest K
+// (kStreamBodies of them: K <= 6144) are written out nested, chunk c + 1 inside the "if" of
+// chunk c, instead of looped over, because vector loads return in order and are waited for by
+// count: only with a fixed number of requests between a request and its use can the compiler
+// wait for the oldest alone, and where a loop closes, or two paths meet, its count starts
+// over (it waits there for nearly everything in flight, and the ring needs as many chunks
+// again to fill).
 static_assert(8 * 64 * 16 * 4 <= kPairTableBytes, "the wavefronts' sums reuse the table");
 
 // f(0); if (1 < n) { f(1); if (2 < n) { ... } }: chunk C is reached through chunk C - 1 only, so
@@ -911,8 +912,25 @@ __device__ __forceinline__ float scale_into(float acc, float mine, float t) {
   return fmaf(__int_as_float(s), t, acc);
 }
 
-// segs.blocks counts 32-row blocks here.  XI: staging items of x per thread (2 above 16
-// columns).
+// Row of a chunk buffer that holds token n.  A staging instruction of 17..32 columns stores
+// tokens 8 q + e for all four vectors q and sixteen consecutive k pairs: with the tokens in
+// order, a token row being 260 dwords = 4 banks on, vectors q and q + 2 would meet in the
+// same banks.  The order below puts the four vectors of an instruction 16 banks apart and
+// still keeps tokens 0..15, and 16..31, in sixteen rows of different banks for the operand
+// reads.  Up to 16 columns (two vectors x 32 k pairs an instruction) the plain order is the
+// one without conflicts.
+template <int XI>
+__device__ __forceinline__ int stream_token_row(int n) {
+  if constexpr (XI != 2) {
+    return n;
+  } else {
+    const int q = n >> 3, e = n & 7;
+    return (n & 16) + ((4 * q + (e & 3) + 8 * (e >> 2)) & 15);
+  }
+}
+
+// segs.blocks counts 32-row blocks here.  XI: how a staging thread fetches x: one item (two
+// k x eight columns) up to 16 columns, two above, four quarter items at exactly 32 columns.
 template <int XI>
 __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
                                                             const uint16_t *__restrict__ x,
@@ -956,41 +974,83 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
   const int n_ch = (K_pad + CK - 1) / CK;
 
   // ---- requests: a thread's share of one chunk ------------------------------------------------
+  // XI = 4 is the form for exactly 32 columns: a k pair of x (rows 2 kp, 2 kp + 1) is then
+  // one 128-byte line, which eight consecutive lanes fetch 16 bytes each -- 1 KB of whole
+  // lines per load instruction -- and the lanes that hold the same columns of the two rows
+  // (j and 7 - j of the eight) swap halves through a DPP half-row mirror before they
+  // interleave: four loads a thread and chunk, each a quarter of an item of the other forms.
+  constexpr bool WIDE = XI == 4;
+  constexpr int NA = WIDE ? 4 : XI, NB = WIDE ? 0 : XI;
+  // a thread's loads of one chunk: w = bytes 16 (stid % 16) .. + 16 of the chunk of row
+  // stid / 16; a, b = x, rows 2 kp and 2 kp + 1 of the chunk, columns 8 q .. + 8
   struct Item {
-    uint4 w;             // bytes 16 (stid % 16) .. + 16 of the chunk of row stid / 16
-    uint4 a[XI], b[XI];  // x: rows 2 kp, 2 kp + 1 of the chunk, columns 8 q .. + 8
+    uint4 a[NA], b[NB > 0 ? NB : 1];
   };
   const uint8_t *wp = packed + static_cast<size_t>(min(row_base + (stid >> 4), M - 1)) * row_bytes;
   const int w_piece = 16 * (stid & 15);
   const int nv = N >> 3;
   const int n_items = (CK / 2) * nv;
-  int xkp[XI], xq[XI];
+  int xkp[NA], xq[NA];
 #pragma unroll
-  for (int it = 0; it < XI; ++it) {
+  for (int it = 0; it < NA; ++it) {
     const int idx = min(stid + it * kStreamStagers, n_items - 1);
     xkp[it] = idx / nv;
     xq[it] = idx - xkp[it] * nv;
   }
-  auto load = [&](int c, Item &v) {
+  // the wide form: lane j of eight holds row 2 kp + (j >> 2), columns 8 q with q = j or 7 - j
+  const int w_half = (lane >> 2) & 1;
+  const int w_q = w_half ? 7 - (lane & 7) : (lane & 7);
+  const int w_kp = (lane >> 3) + 8 * wave;  // + 64 it
+  auto load = [&](int c, U32x4 &w, Item &v) {
     const int cc = min(c, n_ch - 1);
-    v.w = *reinterpret_cast<const uint4 *>(wp + min(cc * (CK / 2) + w_piece, row_bytes - 16));
+    w = *reinterpret_cast<const U32x4 *>(wp + min(cc * (CK / 2) + w_piece, row_bytes - 16));
+    if constexpr (WIDE) {
 #pragma unroll
-    for (int it = 0; it < XI; ++it) {
-      const int k = cc * CK + 2 * xkp[it];
-      v.a[it] = *reinterpret_cast<const uint4 *>(x + static_cast<size_t>(min(k, K - 1)) * N + 8 * xq[it]);
-      v.b[it] =
-          *reinterpret_cast<const uint4 *>(x + static_cast<size_t>(min(k + 1, K - 1)) * N + 8 * xq[it]);
+      for (int it = 0; it < 4; ++it) {
+        const int k = cc * CK + 2 * (w_kp + 64 * it) + w_half;
+        v.a[it] = *reinterpret_cast<const uint4 *>(x + static_cast<size_t>(min(k, K - 1)) * 32 + 8 * w_q);
+      }
+    } else {
+#pragma unroll
+      for (int it = 0; it < NB; ++it) {
+        const int k = cc * CK + 2 * xkp[it];
+        v.a[it] = *reinterpret_cast<const uint4 *>(x + static_cast<size_t>(min(k, K - 1)) * N + 8 * xq[it]);
+        v.b[it] =
+            *reinterpret_cast<const uint4 *>(x + static_cast<size_t>(min(k + 1, K - 1)) * N + 8 * xq[it]);
+      }
     }
   };
-  auto store = [&](int c, const Item &v) {
+  auto store = [&](int c, const U32x4 w, const Item &v) {
     const int buf = c & 1;
     // weights: row-major, 272 bytes a row.  A piece past the end of the row (the second half
     // of a last chunk of 256) repeats the row's last 16 bytes; x is zero there.
-    *reinterpret_cast<uint4 *>(lds_raw + kWAddr + buf * kStreamWBytes + (stid >> 4) * kStreamWStride +
-                               w_piece) = v.w;
+    *reinterpret_cast<U32x4 *>(lds_raw + kWAddr + buf * kStreamWBytes + (stid >> 4) * kStreamWStride +
+                               w_piece) = w;
     uint32_t *xd = reinterpret_cast<uint32_t *>(lds_raw + kXAddr + buf * kStreamXBytes);
+    if constexpr (WIDE) {
 #pragma unroll
-    for (int it = 0; it < XI; ++it) {
+      for (int it = 0; it < 4; ++it) {
+        const int kp = w_kp + 64 * it;
+        const bool live = c * CK + 2 * kp + w_half < K;
+        const uint32_t m0 = live ? v.a[it].x : 0u, m1 = live ? v.a[it].y : 0u;
+        const uint32_t m2 = live ? v.a[it].z : 0u, m3 = live ? v.a[it].w : 0u;
+        // the even row's lane sends columns 4..7, the odd row's lane columns 0..3
+        const int s0 = static_cast<int>(w_half ? m0 : m2), s1 = static_cast<int>(w_half ? m1 : m3);
+        const uint32_t g0 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, s0, 0x141, 0xF, 0xF, true));
+        const uint32_t g1 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, s1, 0x141, 0xF, 0xF, true));
+        // even row's lane: tokens 8 q .. + 4 from its columns 0..3 and the partner's; odd
+        // row's lane: tokens 8 q + 4 .. + 4 from the partner's columns 4..7 and its own
+        const uint32_t a0 = w_half ? g0 : m0, a1 = w_half ? g1 : m1;
+        const uint32_t b0 = w_half ? m2 : g0, b1 = w_half ? m3 : g1;
+        uint32_t *dst = xd + (8 * w_q + 4 * w_half) * (XS / 2) + kp;
+        dst[0] = (a0 & 0xFFFFu) | (b0 << 16);
+        dst[XS / 2] = (a0 >> 16) | (b0 & 0xFFFF0000u);
+        dst[2 * (XS / 2)] = (a1 & 0xFFFFu) | (b1 << 16);
+        dst[3 * (XS / 2)] = (a1 >> 16) | (b1 & 0xFFFF0000u);
+      }
+    } else {
+#pragma unroll
+    for (int it = 0; it < NB; ++it) {
       if (stid + it * kStreamStagers < n_items) {
         const int k = c * CK + 2 * xkp[it];
         const bool ka = k < K, kb = k + 1 < K;
@@ -998,13 +1058,14 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
                                ka ? v.a[it].w : 0u};
         const uint32_t b[4] = {kb ? v.b[it].x : 0u, kb ? v.b[it].y : 0u, kb ? v.b[it].z : 0u,
                                kb ? v.b[it].w : 0u};
-        uint32_t *dst = xd + (8 * xq[it]) * (XS / 2) + xkp[it];
+        uint32_t *dst = xd + xkp[it];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          dst[(2 * e) * (XS / 2)] = (a[e] & 0xFFFFu) | (b[e] << 16);
-          dst[(2 * e + 1) * (XS / 2)] = (a[e] >> 16) | (b[e] & 0xFFFF0000u);
+          dst[stream_token_row<XI>(8 * xq[it] + 2 * e) * (XS / 2)] = (a[e] & 0xFFFFu) | (b[e] << 16);
+          dst[stream_token_row<XI>(8 * xq[it] + 2 * e + 1) * (XS / 2)] = (a[e] >> 16) | (b[e] & 0xFFFF0000u);
         }
       }
+    }
     }
   };
 
@@ -1023,25 +1084,26 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
     sv[it] = *reinterpret_cast<const uint2 *>(
         scale + static_cast<size_t>(min(row_base + srow, M - 1)) * groups + 4 * (i - srow * quads));
   }
-  // chunks a staging thread keeps in flight: with two items of x a chunk, three are what
-  // 128 registers hold
-  constexpr int R = XI == 2 ? 3 : kStreamRing;
-  static_assert(kStreamBodies % R == 0, "slots of the written-out chunks are compile-time");
+  // chunks a staging thread keeps in flight: with 64 bytes of x a chunk, three are what 128
+  // registers hold
+  constexpr int R = XI >= 2 ? 3 : kStreamRing;
   Item ring[R];
+  U32x4 ring_w[R];  // (a native vector: the struct type's assignment would pin it in memory)
   if (stager) {
 #pragma unroll
     for (int j = 0; j < R; ++j) {
-      load(j, ring[j]);
+      load(j, ring_w[j], ring[j]);
     }
   }
   fill_pair_table(reinterpret_cast<uint32_t *>(lds_raw), wave16, lane);
   {
-    // token rows N .. 32 of the chunk buffers are never staged: zero them once
+    // the rows of tokens N .. 32 of the chunk buffers are never staged: zero them once
     const int nz = (32 - N) * (XS / 2);
     for (int b = 0; b < 2; ++b) {
-      uint32_t *z = reinterpret_cast<uint32_t *>(lds_raw + kXAddr + b * kStreamXBytes) + N * (XS / 2);
+      uint32_t *z = reinterpret_cast<uint32_t *>(lds_raw + kXAddr + b * kStreamXBytes);
       for (int i = tid; i < nz; i += kStreamBlock) {
-        z[i] = 0u;
+        const int n = N + i / (XS / 2);
+        z[stream_token_row<XI>(n) * (XS / 2) + (i - (n - N) * (XS / 2))] = 0u;
       }
     }
   }
@@ -1061,8 +1123,8 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
     }
   }
   if (stager) {
-    store(0, ring[0]);
-    load(R, ring[0]);
+    store(0, ring_w[0], ring[0]);
+    load(R, ring_w[0], ring[0]);
   }
   __syncthreads();
 
@@ -1073,25 +1135,25 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
     acc[v] = 0.f;
   }
   if (stager) {
-    for (int c0 = 0; c0 < n_ch; c0 += kStreamBodies) {
+    {
       auto chunk = [&](auto index) {
-        constexpr int cb = decltype(index)::value;  // kStreamBodies is a multiple of the ring
-        constexpr int j = cb % R;
-        const int c = c0 + cb;
+        constexpr int c = decltype(index)::value;
+        constexpr int j = c % R;
         // chunk c + 1 goes into the buffers that chunk c - 1 was read from (the multiplying
         // wavefronts are past those reads: the barrier of chunk c - 1); its registers take
         // chunk c + 1 + R
         if (c + 1 < n_ch) {
-          store(c + 1, ring[(j + 1) % R]);
+          store(c + 1, ring_w[(j + 1) % R], ring[(j + 1) % R]);
         }
-        load(c + 1 + R, ring[(j + 1) % R]);
+        load(c + 1 + R, ring_w[(j + 1) % R], ring[(j + 1) % R]);
         __syncthreads();
       };
-      nest_chunks<0, kStreamBodies>(n_ch - c0, chunk);
+      nest_chunks<0, kStreamBodies>(n_ch, chunk);
     }
   } else {
     const uint32_t lane4 = static_cast<uint32_t>(lane) << 2;
-    const uint32_t x_lane = kXAddr + static_cast<uint32_t>(r * XS + 32 * h + 64 * wave) * 2;
+    const uint32_t x_lane =
+        kXAddr + static_cast<uint32_t>(stream_token_row<XI>(r) * XS + 32 * h + 64 * wave) * 2;
     const uint32_t w_lane = kWAddr + static_cast<uint32_t>(r * kStreamWStride + 32 * wave + 16 * h);
     // this lane's scale: row 8 ((l % 16) / 4) + 4 h + l % 4 of the 32, group `wave` of the chunk
     const uint32_t s_lane =
@@ -1412,6 +1474,9 @@ int gemm_lds_ready() {
                             kStreamLdsBytes) != hipSuccess ||
         hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_stream<2>),
                             hipFuncAttributeMaxDynamicSharedMemorySize,
+                            kStreamLdsBytes) != hipSuccess ||
+        hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_stream<4>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize,
                             kStreamLdsBytes) != hipSuccess) {
       (void)hipGetLastError();
       return -6;
@@ -1573,6 +1638,9 @@ int gemm_launch(const chr_nf4_dev_t *const *w, int nseg, const void *x, void *y,
   if (sp.stream) {
     if (N <= 16) {
       gemm_stream<1><<<grid, dim3(kStreamBlock), kStreamLdsBytes, st>>>(
+          sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp);
+    } else if (N == 32) {
+      gemm_stream<4><<<grid, dim3(kStreamBlock), kStreamLdsBytes, st>>>(
           sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp);
     } else {
       gemm_stream<2><<<grid, dim3(kStreamBlock), kStreamLdsBytes, st>>>(

@@ -200,7 +200,7 @@ def _rows_kernel_on() -> bool:
 
 _STREAM_ON: bool | None = None
 _STREAM_ROWS = 32
-_STREAM_MAX_GROUPS = 216
+_STREAM_MAX_GROUPS = 96
 #: LDS of the stream tile: pair table, two chunks of x (32 token rows of 512 + 8), two chunks of
 #: weights (32 rows of 256 + 16 bytes), the scales of 32 rows
 _STREAM_LDS = 256 * 64 * 4 + 2 * 32 * 520 * 2 + 2 * 32 * 272 + _STREAM_MAX_GROUPS * 32 * 2
