@@ -63,6 +63,12 @@ int chr_nf4_gemm(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N,
                  void *stream);
 
 /* Pure launch math; only M/K/K_pad are read.  N in [1, 64].
+ * Chunks of 8, 16, 24 or 32 columns of a matrix with at most one 32-row block per compute
+ * unit and K_pad a multiple of 256 up to 6144 are planned on the tile that needs no split
+ * (bm 32, grid_y 1, ws_floats 0, block 1024); it multiplies bf16(level) and applies the fp16
+ * scale to each 64-wide group's sum, where the other tiles multiply bf16(level * scale) as
+ * the reference's kernel does.  CHR_NF4_GEMM_STREAM=0 in the environment, a forced split
+ * (chr_nf4_set_tuning) or a scale blob that is not 8-byte aligned keep a launch on those.
  * Replaces chr_nf4_gemm_plan (chr_gpu.h:64-65; nf4_gemm.cu:1656-1667). */
 int chr_nf4_gemm_plan(const chr_nf4_dev_t *w, int32_t N, int32_t have_ws,
                       chr_nf4_plan_t *out);
