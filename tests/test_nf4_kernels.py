@@ -601,6 +601,7 @@ def test_gemm_every_split_agrees(n):
 STREAM_CASES = [
     # m, k, n
     (32, 256, 8), (130, 512, 16), (200, 768, 24),   # a ragged last block; a last chunk of 256
+    (1, 512, 8), (33, 256, 32),                      # one row; one row past a block
     (96, 1000, 32),                                  # K below K_pad
     (256, 5120, 32), (70, 6144, 8),                  # ten and twelve chunks
     (2048, 2048, 32), (5120, 5120, 8), (7168, 5120, 16),
