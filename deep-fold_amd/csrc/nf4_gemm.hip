@@ -105,9 +105,9 @@ constexpr int rows_x_items(int nc, int tps) {
 constexpr int rows_max_tiles(int nc) { return nc == 4 ? 2 : kRowsMaxTiles; }
 constexpr int rows_col_blocks(int N) { return N <= 16 ? 1 : (N <= 32 ? 2 : 4); }
 
-// The stream tile (gemm_stream below): eight wavefronts with 256 registers each on 32 rows and
-// all of K; the pair table, two chunks of x and of weights and the rows' scales in LDS; four
-// chunks of loads in registers.
+// The stream tile (gemm_stream below): sixteen wavefronts, eight staging and eight multiplying,
+// on 32 or 64 rows and all of K; the pair table, two chunks of x and of weights and the rows'
+// scales in LDS; three or four chunks of loads in registers.
 constexpr int kStreamBlock = 1024;
 constexpr int kStreamStagers = 512;  // threads of the wavefronts that stage (the other eight multiply)
 constexpr int kStreamRows = 32;
@@ -118,11 +118,14 @@ constexpr int kStreamMaxGroups = kStreamBodies * kStreamChunkK / 64;  // groups 
 constexpr int kStreamXS = kStreamChunkK + kXPad;       // bf16 elements of a token row of one chunk
 constexpr int kStreamXBytes = 32 * kStreamXS * 2;      // one chunk of x, 32 token rows
 constexpr int kStreamWStride = kStreamChunkK / 2 + 16; // bytes of a staged weight row
-constexpr int kStreamWBytes = kStreamRows * kStreamWStride;
-constexpr int kStreamScaleBytes = kStreamMaxGroups * kStreamRows * 2;
-constexpr int kStreamLdsBytes =
-    kPairTableBytes + 2 * kStreamXBytes + 2 * kStreamWBytes + kStreamScaleBytes;
-static_assert(kStreamLdsBytes <= 160 * 1024, "LDS of a compute unit");
+constexpr int kStreamTableBytes = 256 * 32 * 4;  // the pair table, 32 copies (see fill_pair_table32)
+constexpr int kStreamWBytes = kStreamRows * kStreamWStride;  // a chunk of weights of 32 rows
+// rb: 32-row blocks of a workgroup (1 or 2)
+constexpr int stream_scale_bytes(int rb) { return kStreamMaxGroups * kStreamRows * rb * 2; }
+constexpr int stream_lds_bytes(int rb) {
+  return kStreamTableBytes + 2 * kStreamXBytes + 2 * rb * kStreamWBytes + stream_scale_bytes(rb);
+}
+static_assert(stream_lds_bytes(2) <= 160 * 1024, "LDS of a compute unit");
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -150,14 +153,18 @@ bool rows_kernel_serves(int N, int tiles_per_split) {
 
 // The stream tile takes chunks of 8..32 columns in whole 16-byte vectors when K_pad is a
 // multiple of kBK (the four group scales of a row and K tile are then one aligned 8-byte load;
-// gemm_launch checks the pointer), unless a split is forced (it has none).  It is taken where
-// it was measured faster than the split tiles with their reduce: when all its workgroups run
-// at once (no more 32-row blocks than compute units) and K is one pass of its written-out
-// chunks (K_pad <= 6144).  At 14B shapes that is q/k/v (7168x5120: 10.9 / 11.9 / 15.7 us at
-// N = 8 / 16 / 32 against 15.1 / 16.0 / 18.5) and o (10.0 / 11.2 / 14.8 against 12.7 / 13.5 /
-// 15.8), not gate+up (432 workgroups: 28.2 against 24.1 at N = 32) and not down (K = 13824:
-// 29.7 against 23.8).  CHR_NF4_GEMM_STREAM=0 leaves everything to the two older tiles, whose
-// weights are bf16(level * scale) as in the reference's kernel (gpu/nf4/nf4_gemm.cu:312-323).
+// gemm_launch checks the pointer), unless a split is forced (it has none), and when K is one
+// pass of its written-out chunks (K_pad <= 6144).  Its workgroups hold a compute unit each:
+// 32 rows each while the launch then runs in one round, else 64 rows (every x operand feeds
+// two weight operands) up to two rounds.  Measured at 14B shapes, N = 8 / 16 / 32, against
+// the split tiles with their reduce: q/k/v (7168x5120) 10.9 / 11.9 / 15.7 us against 15.1 /
+// 16.0 / 18.5; o (5120x5120) 10.0 / 11.2 / 14.8 against 12.7 / 13.5 / 15.8; gate or up
+// (13824x5120, 64 rows) 16.6 / 17.1 / 20.3 against 20.9 / 20.9 / 24.0; gate+up stacked
+// (27648 rows, 64 rows, two rounds) 32.8 / 33.6 / 40.2 against 33.6 / 37.0 / 42.6.  Not down
+// (K = 13824).  With 64 rows where 32 fill one round q/k/v takes 14.9 / 15.6 / 18.8 (half
+// the compute units idle).  CHR_NF4_GEMM_STREAM=0 leaves everything to the two older tiles,
+// whose weights are bf16(level * scale) as in the reference's kernel
+// (gpu/nf4/nf4_gemm.cu:312-323).
 bool stream_columns(int N) {
   static const bool on = env_int("CHR_NF4_GEMM_STREAM", 1) != 0;
   return on && N >= 8 && N <= 32 && (N & 7) == 0;
@@ -185,11 +192,23 @@ int resolved_one_wave() {
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
-// blocks32: 32-row blocks of the launch (of all its stacked matrices).
-bool stream_kernel_serves(int N, int K_pad, int blocks32) {
-  return stream_columns(N) && tuning().split_k == 0 && K_pad % kBK == 0 &&
-         K_pad <= kStreamBodies * kStreamChunkK &&
-         blocks32 <= resolved_one_wave();
+// 32-row blocks of a workgroup of the stream tile for this launch, 0: another tile serves it.
+// blocks32, blocks64: 32- and 64-row blocks of the launch (summed over its stacked matrices).
+// 32 rows each while one round of workgroups (one a compute unit) covers the launch, else 64
+// rows up to two rounds.  CHR_NF4_GEMM_STREAM_ROWS=32 or 64 allows only that form.
+int stream_row_blocks(int N, int K_pad, int blocks32, int blocks64) {
+  static const int only = env_int("CHR_NF4_GEMM_STREAM_ROWS", 0);
+  if (!stream_columns(N) || tuning().split_k != 0 || K_pad % kBK != 0 ||
+      K_pad > kStreamBodies * kStreamChunkK) {
+    return 0;
+  }
+  if (blocks32 <= resolved_one_wave() && only != 64) {
+    return 1;
+  }
+  if (blocks64 <= 2 * resolved_one_wave() && only != 32) {
+    return 2;
+  }
+  return 0;
 }
 
 // Split-K.  A workgroup is quickest with about three K tiles (measured at every 14B linear
@@ -273,13 +292,13 @@ int plan_impl(const chr_nf4_dev_t &h, int32_t N, int32_t have_ws, chr_nf4_plan_t
     p.n_ktiles = ceil_div(h.K_pad, kBK);
     pick_split(p.grid_x, p.n_ktiles, N, have_ws, &p.grid_y, &p.tiles_per_split);
     p.smem_bytes = gemm_lds_bytes(N <= 32 ? 1 : 2);
-    if (stream_kernel_serves(N, h.K_pad, ceil_div(h.M, kStreamRows))) {
-      p.bm = kStreamRows;
+    if (const int rb = stream_row_blocks(N, h.K_pad, ceil_div(h.M, kStreamRows), ceil_div(h.M, 2 * kStreamRows))) {
+      p.bm = kStreamRows * rb;
       p.block = kStreamBlock;
-      p.grid_x = ceil_div(h.M, kStreamRows);
+      p.grid_x = ceil_div(h.M, p.bm);
       p.grid_y = 1;
       p.tiles_per_split = p.n_ktiles;
-      p.smem_bytes = kStreamLdsBytes;
+      p.smem_bytes = stream_lds_bytes(rb);
     } else if (rows_kernel_serves(N, p.tiles_per_split)) {
       p.block = kRowsBlock;
       p.smem_bytes = rows_lds_bytes(rows_col_blocks(N), p.tiles_per_split);
@@ -891,7 +910,29 @@ __global__ __launch_bounds__(kRowsBlock) void gemm_rows(const GemmSegs segs,
 // wait for the oldest alone, and where a loop closes, or two paths meet, its count starts
 // over (it waits there for nearly everything in flight, and the ring needs as many chunks
 // again to fill).
-static_assert(8 * 64 * 16 * 4 <= kPairTableBytes, "the wavefronts' sums reuse the table");
+
+// The pair table of this tile: entry (byte, copy) at byte * 128 + copy * 4, 32 copies.  The
+// LDS serves a 4-byte read of a wavefront in two halves of 32 lanes, so lane & 31 picking the
+// copy keeps the lookups free of bank conflicts in 32 KB instead of the GEMV's 64 KB (measured:
+// the same conflict count and the same time); the address costs a shift and an and-or instead
+// of one v_perm_b32.  Filled by sixteen wavefronts: wavefront v writes the bytes whose low
+// code is v, lanes 0..31 / 32..63 the even / odd high codes.
+__device__ __forceinline__ void fill_pair_table32(uint32_t *table, int wave16, int lane) {
+  const uint32_t lo = bf16_bits_rne(kLutBits[wave16]);
+  const int copy = lane & 31, half = lane >> 5;
+#pragma unroll
+  for (int jj = 0; jj < 8; ++jj) {
+    const int j = 2 * jj + half;
+    const uint32_t hi = (half ? bf16_bits_rne(kLevelBits[2 * jj + 1]) : bf16_bits_rne(kLevelBits[2 * jj])) << 16;
+    table[((wave16 + 16 * j) << 5) + copy] = lo | hi;
+  }
+}
+// the pair of byte J of w; copy4 = 4 * (lane & 31)
+template <int J>
+__device__ __forceinline__ uint32_t pair32_at(uint32_t w, uint32_t copy4) {
+  const uint32_t sh = J == 0 ? (w << 7) : (w >> (8 * J - 7));
+  return lds0_u32((sh & 0x7F80u) | copy4);
+}
 
 // f(0); if (1 < n) { f(1); if (2 < n) { ... } }: chunk C is reached through chunk C - 1 only, so
 // the compiler knows every request of the earlier chunks to have been issued.
@@ -929,9 +970,11 @@ __device__ __forceinline__ int stream_token_row(int n) {
   }
 }
 
-// segs.blocks counts 32-row blocks here.  XI: how a staging thread fetches x: one item (two
-// k x eight columns) up to 16 columns, two above, four quarter items at exactly 32 columns.
-template <int XI>
+// XI: how a staging thread fetches x: one item (two k x eight columns) up to 16 columns, two
+// above, four quarter items at exactly 32 columns.  RB: 32-row blocks of a workgroup, 1 or 2
+// (segs.blocks counts blocks of 32 RB rows): with two, a multiplying wavefront feeds every B
+// operand it reads to two A operands, and x is staged once per 64 rows.
+template <int XI, int RB>
 __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
                                                             const uint16_t *__restrict__ x,
                                                             uint16_t *__restrict__ y,
@@ -941,10 +984,13 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
                                                             const uint16_t *res) {
   constexpr int XS = kStreamXS;
   constexpr int CK = kStreamChunkK;
-  constexpr uint32_t kXAddr = kPairTableBytes;
+  constexpr int ROWS = kStreamRows * RB;
+  constexpr uint32_t kWBuf = RB * kStreamWBytes;
+  constexpr uint32_t kXAddr = kStreamTableBytes;
   constexpr uint32_t kWAddr = kXAddr + 2 * kStreamXBytes;
-  constexpr uint32_t kScaleAddr = kWAddr + 2 * kStreamWBytes;
-  static_assert(kScaleAddr + kStreamScaleBytes == kStreamLdsBytes, "LDS map");
+  constexpr uint32_t kScaleAddr = kWAddr + 2 * kWBuf;
+  static_assert(kScaleAddr + stream_scale_bytes(RB) == stream_lds_bytes(RB), "LDS map");
+  static_assert(8 * 64 * 16 * RB * 4 <= kWAddr, "the wavefronts' sums reuse the table and x");
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1);
@@ -966,7 +1012,7 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
   const uint16_t *__restrict__ scale = segs.scale[seg];
   const int M = segs.M[seg];
   const int out0 = segs.row0[seg];
-  const int row_base = bx * kStreamRows;
+  const int row_base = bx * ROWS;
   const int r = lane & 31;  // row of the A operand, token of the B operand
   const int h = lane >> 5;  // which half of a group's k
   const int row_bytes = K_pad >> 1;
@@ -986,7 +1032,11 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
   struct Item {
     uint4 a[NA], b[NB > 0 ? NB : 1];
   };
-  const uint8_t *wp = packed + static_cast<size_t>(min(row_base + (stid >> 4), M - 1)) * row_bytes;
+  const uint8_t *wp[RB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    wp[rb] = packed + static_cast<size_t>(min(row_base + 32 * rb + (stid >> 4), M - 1)) * row_bytes;
+  }
   const int w_piece = 16 * (stid & 15);
   const int nv = N >> 3;
   const int n_items = (CK / 2) * nv;
@@ -1001,9 +1051,12 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
   const int w_half = (lane >> 2) & 1;
   const int w_q = w_half ? 7 - (lane & 7) : (lane & 7);
   const int w_kp = (lane >> 3) + 8 * wave;  // + 64 it
-  auto load = [&](int c, U32x4 &w, Item &v) {
+  auto load = [&](int c, U32x4 &w0, U32x4 &w1, Item &v) {
     const int cc = min(c, n_ch - 1);
-    w = *reinterpret_cast<const U32x4 *>(wp + min(cc * (CK / 2) + w_piece, row_bytes - 16));
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      (rb ? w1 : w0) = *reinterpret_cast<const U32x4 *>(wp[rb] + min(cc * (CK / 2) + w_piece, row_bytes - 16));
+    }
     if constexpr (WIDE) {
 #pragma unroll
       for (int it = 0; it < 4; ++it) {
@@ -1020,12 +1073,15 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
       }
     }
   };
-  auto store = [&](int c, const U32x4 w, const Item &v) {
+  auto store = [&](int c, const U32x4 w0, const U32x4 w1, const Item &v) {
     const int buf = c & 1;
     // weights: row-major, 272 bytes a row.  A piece past the end of the row (the second half
     // of a last chunk of 256) repeats the row's last 16 bytes; x is zero there.
-    *reinterpret_cast<U32x4 *>(lds_raw + kWAddr + buf * kStreamWBytes + (stid >> 4) * kStreamWStride +
-                               w_piece) = w;
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      *reinterpret_cast<U32x4 *>(lds_raw + kWAddr + buf * kWBuf + (32 * rb + (stid >> 4)) * kStreamWStride +
+                                 w_piece) = rb ? w1 : w0;
+    }
     uint32_t *xd = reinterpret_cast<uint32_t *>(lds_raw + kXAddr + buf * kStreamXBytes);
     if constexpr (WIDE) {
 #pragma unroll
@@ -1074,28 +1130,31 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
   // request, a fixed number of requests a thread, the surplus repeating the last one) and
   // the staging wavefronts' requests in the order the chunks keep them in; the table while
   // they travel.
-  constexpr int kScaleLoads = (kStreamRows * (kStreamMaxGroups / 4) + kStreamBlock - 1) / kStreamBlock;
+  constexpr int kScaleLoads = (ROWS * (kStreamMaxGroups / 4) + kStreamBlock - 1) / kStreamBlock;
   const int quads = groups >> 2;
   uint2 sv[kScaleLoads];
 #pragma unroll
   for (int it = 0; it < kScaleLoads; ++it) {
-    const int i = min(tid + it * kStreamBlock, kStreamRows * quads - 1);
+    const int i = min(tid + it * kStreamBlock, ROWS * quads - 1);
     const int srow = i / quads;
     sv[it] = *reinterpret_cast<const uint2 *>(
         scale + static_cast<size_t>(min(row_base + srow, M - 1)) * groups + 4 * (i - srow * quads));
   }
   // chunks a staging thread keeps in flight: with 64 bytes of x a chunk, three are what 128
   // registers hold
+  // (deeper rings measured slower in every form: 6 / 4 chunks with 32 rows, 5 / 4 with 64)
   constexpr int R = XI >= 2 ? 3 : kStreamRing;
   Item ring[R];
-  U32x4 ring_w[R];  // (a native vector: the struct type's assignment would pin it in memory)
+  // (native vectors: the struct type's assignment would pin them in memory; the second block's
+  // are idle with one block)
+  U32x4 ring_w[R], ring_w1[R];
   if (stager) {
 #pragma unroll
     for (int j = 0; j < R; ++j) {
-      load(j, ring_w[j], ring[j]);
+      load(j, ring_w[j], ring_w1[j], ring[j]);
     }
   }
-  fill_pair_table(reinterpret_cast<uint32_t *>(lds_raw), wave16, lane);
+  fill_pair_table32(reinterpret_cast<uint32_t *>(lds_raw), wave16, lane);
   {
     // the rows of tokens N .. 32 of the chunk buffers are never staged: zero them once
     const int nz = (32 - N) * (XS / 2);
@@ -1108,32 +1167,30 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
     }
   }
   {
-    uint16_t *sl = reinterpret_cast<uint16_t *>(lds_raw + kScaleAddr);  // [group][row of the 32]
+    uint16_t *sl = reinterpret_cast<uint16_t *>(lds_raw + kScaleAddr);  // [group][row of the block]
 #pragma unroll
     for (int it = 0; it < kScaleLoads; ++it) {
       const int i = tid + it * kStreamBlock;
-      if (i < kStreamRows * quads) {
+      if (i < ROWS * quads) {
         const int srow = i / quads;
         const int gq = i - srow * quads;
-        sl[(4 * gq + 0) * kStreamRows + srow] = static_cast<uint16_t>(sv[it].x);
-        sl[(4 * gq + 1) * kStreamRows + srow] = static_cast<uint16_t>(sv[it].x >> 16);
-        sl[(4 * gq + 2) * kStreamRows + srow] = static_cast<uint16_t>(sv[it].y);
-        sl[(4 * gq + 3) * kStreamRows + srow] = static_cast<uint16_t>(sv[it].y >> 16);
+        sl[(4 * gq + 0) * ROWS + srow] = static_cast<uint16_t>(sv[it].x);
+        sl[(4 * gq + 1) * ROWS + srow] = static_cast<uint16_t>(sv[it].x >> 16);
+        sl[(4 * gq + 2) * ROWS + srow] = static_cast<uint16_t>(sv[it].y);
+        sl[(4 * gq + 3) * ROWS + srow] = static_cast<uint16_t>(sv[it].y >> 16);
       }
     }
   }
   if (stager) {
-    store(0, ring_w[0], ring[0]);
-    load(R, ring_w[0], ring[0]);
+    store(0, ring_w[0], ring_w1[0], ring[0]);
+    load(R, ring_w[0], ring_w1[0], ring[0]);
   }
   __syncthreads();
 
   // ---- the chunks: one barrier each, in both roles ------------------------------------------
-  f32x16 acc;
-#pragma unroll
-  for (int v = 0; v < 16; ++v) {
-    acc[v] = 0.f;
-  }
+  // (the multiplying wavefronts' sums live and die inside their branch, so that the staging
+  // wavefronts' registers hold the ring alone)
+  float *sums = reinterpret_cast<float *>(lds_raw);
   if (stager) {
     {
       auto chunk = [&](auto index) {
@@ -1143,84 +1200,115 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
         // wavefronts are past those reads: the barrier of chunk c - 1); its registers take
         // chunk c + 1 + R
         if (c + 1 < n_ch) {
-          store(c + 1, ring_w[(j + 1) % R], ring[(j + 1) % R]);
+          store(c + 1, ring_w[(j + 1) % R], ring_w1[(j + 1) % R], ring[(j + 1) % R]);
         }
-        load(c + 1 + R, ring_w[(j + 1) % R], ring[(j + 1) % R]);
+        load(c + 1 + R, ring_w[(j + 1) % R], ring_w1[(j + 1) % R], ring[(j + 1) % R]);
         __syncthreads();
       };
       nest_chunks<0, kStreamBodies>(n_ch, chunk);
     }
-  } else {
-    const uint32_t lane4 = static_cast<uint32_t>(lane) << 2;
+  }
+  // (a second question of its own, not an else: the staging wavefronts' ring is then dead
+  // before the multiplying wavefronts' sums are born, and the two roles share registers)
+  int role;
+  asm volatile("s_mov_b32 %0, %1" : "=s"(role) : "s"(wave16));
+  if (role < 8) {
+    f32x16 acc[RB];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        acc[rb][v] = 0.f;
+      }
+    }
+    const uint32_t copy4 = static_cast<uint32_t>(lane & 31) << 2;
     const uint32_t x_lane =
         kXAddr + static_cast<uint32_t>(stream_token_row<XI>(r) * XS + 32 * h + 64 * wave) * 2;
     const uint32_t w_lane = kWAddr + static_cast<uint32_t>(r * kStreamWStride + 32 * wave + 16 * h);
     // this lane's scale: row 8 ((l % 16) / 4) + 4 h + l % 4 of the 32, group `wave` of the chunk
     const uint32_t s_lane =
-        kScaleAddr + static_cast<uint32_t>(wave * kStreamRows + 8 * ((lane & 15) >> 2) + 4 * h + (lane & 3)) * 2;
+        kScaleAddr + static_cast<uint32_t>(wave * ROWS + 8 * ((lane & 15) >> 2) + 4 * h + (lane & 3)) * 2;
     for (int c = 0; c < n_ch; ++c) {
       const uint32_t buf = static_cast<uint32_t>(c & 1);
       // a group past the end of K (last chunk of 256) multiplies zeros of x; its scale is read
       // from the last group that exists
       const int grp = min(8 * c + wave, groups - 1) - wave;
-      const float mine = f16_to_f32(*reinterpret_cast<const __attribute__((address_space(3))) uint16_t *>(
-          s_lane + static_cast<uint32_t>(grp * kStreamRows * 2)));
-      const uint4 wv = lds0_u128(w_lane + buf * kStreamWBytes);
-      const uint32_t w4[4] = {wv.x, wv.y, wv.z, wv.w};
-      const uint32_t xl = x_lane + buf * kStreamXBytes;
-      f32x16 t;
+      float mine[RB];
+      uint32_t w4[RB][4];
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        t[v] = 0.f;
+      for (int rb = 0; rb < RB; ++rb) {
+        mine[rb] = f16_to_f32(*reinterpret_cast<const __attribute__((address_space(3))) uint16_t *>(
+            s_lane + static_cast<uint32_t>((grp * ROWS + 32 * rb) * 2)));
+        const uint4 wv = lds0_u128(w_lane + buf * kWBuf + rb * kStreamWBytes);
+        w4[rb][0] = wv.x;
+        w4[rb][1] = wv.y;
+        w4[rb][2] = wv.z;
+        w4[rb][3] = wv.w;
+      }
+      const uint32_t xl = x_lane + buf * kStreamXBytes;
+      f32x16 t[RB];
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          t[rb][v] = 0.f;
+        }
       }
 #pragma unroll
       for (int jj = 0; jj < 4; ++jj) {
         const uint4 b = lds0_u128(xl + 16 * jj);
-        const uint4 a = make_uint4(pair_at<0>(w4[jj], lane4), pair_at<1>(w4[jj], lane4),
-                                   pair_at<2>(w4[jj], lane4), pair_at<3>(w4[jj], lane4));
-        t = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
-                                                    __builtin_bit_cast(bf16x8, b), t, 0, 0, 0);
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb) {
+          const uint32_t w = w4[rb][jj];
+          const uint4 a = make_uint4(pair32_at<0>(w, copy4), pair32_at<1>(w, copy4), pair32_at<2>(w, copy4),
+                                     pair32_at<3>(w, copy4));
+          t[rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                          __builtin_bit_cast(bf16x8, b), t[rb], 0, 0, 0);
+        }
       }
-      acc[0] = scale_into<0>(acc[0], mine, t[0]);
-      acc[1] = scale_into<1>(acc[1], mine, t[1]);
-      acc[2] = scale_into<2>(acc[2], mine, t[2]);
-      acc[3] = scale_into<3>(acc[3], mine, t[3]);
-      acc[4] = scale_into<4>(acc[4], mine, t[4]);
-      acc[5] = scale_into<5>(acc[5], mine, t[5]);
-      acc[6] = scale_into<6>(acc[6], mine, t[6]);
-      acc[7] = scale_into<7>(acc[7], mine, t[7]);
-      acc[8] = scale_into<8>(acc[8], mine, t[8]);
-      acc[9] = scale_into<9>(acc[9], mine, t[9]);
-      acc[10] = scale_into<10>(acc[10], mine, t[10]);
-      acc[11] = scale_into<11>(acc[11], mine, t[11]);
-      acc[12] = scale_into<12>(acc[12], mine, t[12]);
-      acc[13] = scale_into<13>(acc[13], mine, t[13]);
-      acc[14] = scale_into<14>(acc[14], mine, t[14]);
-      acc[15] = scale_into<15>(acc[15], mine, t[15]);
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        acc[rb][0] = scale_into<0>(acc[rb][0], mine[rb], t[rb][0]);
+        acc[rb][1] = scale_into<1>(acc[rb][1], mine[rb], t[rb][1]);
+        acc[rb][2] = scale_into<2>(acc[rb][2], mine[rb], t[rb][2]);
+        acc[rb][3] = scale_into<3>(acc[rb][3], mine[rb], t[rb][3]);
+        acc[rb][4] = scale_into<4>(acc[rb][4], mine[rb], t[rb][4]);
+        acc[rb][5] = scale_into<5>(acc[rb][5], mine[rb], t[rb][5]);
+        acc[rb][6] = scale_into<6>(acc[rb][6], mine[rb], t[rb][6]);
+        acc[rb][7] = scale_into<7>(acc[rb][7], mine[rb], t[rb][7]);
+        acc[rb][8] = scale_into<8>(acc[rb][8], mine[rb], t[rb][8]);
+        acc[rb][9] = scale_into<9>(acc[rb][9], mine[rb], t[rb][9]);
+        acc[rb][10] = scale_into<10>(acc[rb][10], mine[rb], t[rb][10]);
+        acc[rb][11] = scale_into<11>(acc[rb][11], mine[rb], t[rb][11]);
+        acc[rb][12] = scale_into<12>(acc[rb][12], mine[rb], t[rb][12]);
+        acc[rb][13] = scale_into<13>(acc[rb][13], mine[rb], t[rb][13]);
+        acc[rb][14] = scale_into<14>(acc[rb][14], mine[rb], t[rb][14]);
+        acc[rb][15] = scale_into<15>(acc[rb][15], mine[rb], t[rb][15]);
+      }
       __syncthreads();
     }
-  }
-
-  // ---- the eight sums of every output meet in LDS ---------------------------------------------
-  // (the last barrier above has every wavefront past its reads of the table)
-  float *sums = reinterpret_cast<float *>(lds_raw);
-  if (!stager) {
+    // ---- the eight sums of every output meet in LDS -------------------------------------------
+    // (the last barrier above has every wavefront past its reads of the table and of x)
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-      sums[(wave * 16 + v) * kWave + lane] = acc[v];
+    for (int rb = 0; rb < RB; ++rb) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        sums[((rb * 8 + wave) * 16 + v) * kWave + lane] = acc[rb][v];
+      }
     }
   }
   __syncthreads();
-  // wavefront w of the sixteen finishes accumulator value w
-  {
+  // wavefront w of the sixteen finishes accumulator value w of every 32-row block
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
     const int v = wave16;
     float o32 = 0.f;
 #pragma unroll
     for (int q = 0; q < 8; ++q) {
-      o32 += sums[(q * 16 + v) * kWave + lane];
+      o32 += sums[((rb * 8 + q) * 16 + v) * kWave + lane];
     }
     const int n = r;
-    const int rr = row_base + 8 * (v >> 2) + 4 * h + (v & 3);
+    const int rr = row_base + 32 * rb + 8 * (v >> 2) + 4 * h + (v & 3);
     if (n < N && rr < M) {
       const size_t at = static_cast<size_t>(out0 + rr) * N + n;
       if (partial == nullptr) {
@@ -1469,17 +1557,19 @@ int gemm_lds_ready() {
         return -6;
       }
     }
-    if (hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_stream<1>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize,
-                            kStreamLdsBytes) != hipSuccess ||
-        hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_stream<2>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize,
-                            kStreamLdsBytes) != hipSuccess ||
-        hipFuncSetAttribute(reinterpret_cast<const void *>(gemm_stream<4>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize,
-                            kStreamLdsBytes) != hipSuccess) {
-      (void)hipGetLastError();
-      return -6;
+    const std::pair<const void *, int> streams[6] = {
+        {reinterpret_cast<const void *>(gemm_stream<1, 1>), stream_lds_bytes(1)},
+        {reinterpret_cast<const void *>(gemm_stream<2, 1>), stream_lds_bytes(1)},
+        {reinterpret_cast<const void *>(gemm_stream<4, 1>), stream_lds_bytes(1)},
+        {reinterpret_cast<const void *>(gemm_stream<1, 2>), stream_lds_bytes(2)},
+        {reinterpret_cast<const void *>(gemm_stream<2, 2>), stream_lds_bytes(2)},
+        {reinterpret_cast<const void *>(gemm_stream<4, 2>), stream_lds_bytes(2)}};
+    for (const auto &k : streams) {
+      if (hipFuncSetAttribute(k.first, hipFuncAttributeMaxDynamicSharedMemorySize, k.second) !=
+          hipSuccess) {
+        (void)hipGetLastError();
+        return -6;
+      }
     }
     const RowsArgs none{};
     for (int vec = 0; vec < 2; ++vec) {
@@ -1530,19 +1620,20 @@ struct StackPlan {
   GemmSegs segs;
   int M_all, grid_x, grid_y, n_ktiles, tiles_per_split;
   int64_t ws_floats;
-  bool stream;  // the stream tile: 32-row blocks, no split
+  int stream;  // 32-row blocks of a workgroup of the stream tile (no split), 0: another tile
 };
 
 // allow_stream: false when the launch cannot take the stream tile for a reason the shape does
 // not show (scales not 8-byte aligned).
 StackPlan plan_stack(const chr_nf4_dev_t *h, int nseg, int N, int have_ws, bool allow_stream = true) {
   StackPlan sp{};
-  int blocks32 = 0;
+  int blocks32 = 0, blocks64 = 0;
   for (int i = 0; i < nseg; ++i) {
     blocks32 += ceil_div(h[i].M, kStreamRows);
+    blocks64 += ceil_div(h[i].M, 2 * kStreamRows);
   }
-  sp.stream = allow_stream && stream_kernel_serves(N, h[0].K_pad, blocks32);
-  const int bm = sp.stream ? kStreamRows : kBM;
+  sp.stream = allow_stream ? stream_row_blocks(N, h[0].K_pad, blocks32, blocks64) : 0;
+  const int bm = sp.stream ? kStreamRows * sp.stream : kBM;
   for (int i = 0; i < 3; ++i) {
     const bool on = i < nseg;
     sp.segs.packed[i] = on ? h[i].packed : nullptr;
@@ -1635,15 +1726,26 @@ int gemm_launch(const chr_nf4_dev_t *const *w, int nseg, const void *x, void *y,
   const dim3 block(kGemmBlock);
   const int K = h[0].K, K_pad = h[0].K_pad;
   const int nc = rows_col_blocks(N);
-  if (sp.stream) {
+  if (sp.stream == 1) {
     if (N <= 16) {
-      gemm_stream<1><<<grid, dim3(kStreamBlock), kStreamLdsBytes, st>>>(
+      gemm_stream<1, 1><<<grid, dim3(kStreamBlock), stream_lds_bytes(1), st>>>(
           sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp);
     } else if (N == 32) {
-      gemm_stream<4><<<grid, dim3(kStreamBlock), kStreamLdsBytes, st>>>(
+      gemm_stream<4, 1><<<grid, dim3(kStreamBlock), stream_lds_bytes(1), st>>>(
           sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp);
     } else {
-      gemm_stream<2><<<grid, dim3(kStreamBlock), kStreamLdsBytes, st>>>(
+      gemm_stream<2, 1><<<grid, dim3(kStreamBlock), stream_lds_bytes(1), st>>>(
+          sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp);
+    }
+  } else if (sp.stream == 2) {
+    if (N <= 16) {
+      gemm_stream<1, 2><<<grid, dim3(kStreamBlock), stream_lds_bytes(2), st>>>(
+          sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp);
+    } else if (N == 32) {
+      gemm_stream<4, 2><<<grid, dim3(kStreamBlock), stream_lds_bytes(2), st>>>(
+          sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp);
+    } else {
+      gemm_stream<2, 2><<<grid, dim3(kStreamBlock), stream_lds_bytes(2), st>>>(
           sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp);
     }
   } else if (rows_kernel_serves(N, sp.tiles_per_split)) {

@@ -199,11 +199,25 @@ def _rows_kernel_on() -> bool:
 
 
 _STREAM_ON: bool | None = None
+_STREAM_ONLY: int | None = None
 _STREAM_ROWS = 32
 _STREAM_MAX_GROUPS = 96
-#: LDS of the stream tile: pair table, two chunks of x (32 token rows of 512 + 8), two chunks of
-#: weights (32 rows of 256 + 16 bytes), the scales of 32 rows
-_STREAM_LDS = 256 * 64 * 4 + 2 * 32 * 520 * 2 + 2 * 32 * 272 + _STREAM_MAX_GROUPS * 32 * 2
+
+
+def stream_lds_bytes(row_blocks: int) -> int:
+    """LDS of the stream tile with ``row_blocks`` (1 or 2) 32-row blocks a workgroup: the pair
+    table (32 copies of 256 entries), two chunks of x (32 token rows of 512 + 8), two chunks
+    of weights (rows of 256 + 16 bytes), the rows' scales."""
+    rows = _STREAM_ROWS * row_blocks
+    return 256 * 32 * 4 + 2 * 32 * 520 * 2 + 2 * rows * 272 + _STREAM_MAX_GROUPS * rows * 2
+
+
+def _env_int_once(name: str, dflt: int) -> int:
+    raw = os.environ.get(name, "")
+    try:
+        return int(raw) if raw.strip() else dflt
+    except ValueError:
+        return 0                 # atoi() of a non-number is 0
 
 
 def _stream_columns(N: int) -> bool:  # noqa: N803
@@ -211,27 +225,33 @@ def _stream_columns(N: int) -> bool:  # noqa: N803
     (read once, like the library does)."""
     global _STREAM_ON
     if _STREAM_ON is None:
-        raw = os.environ.get("CHR_NF4_GEMM_STREAM", "")
-        try:
-            _STREAM_ON = int(raw) != 0 if raw.strip() else True
-        except ValueError:
-            _STREAM_ON = False
+        _STREAM_ON = _env_int_once("CHR_NF4_GEMM_STREAM", 1) != 0
     return _STREAM_ON and 8 <= N <= 32 and N % 8 == 0
 
 
-def gemm_streams(M: int, N: int, k_pad_: int, force_split: int = 0,  # noqa: N803
-                 one_wave: int = ONE_WAVE) -> bool:
-    """Whether a launch runs the stream tile (a workgroup of sixteen wavefronts on 32 rows and
-    all of K: no split-K, no partials, no reduce; pair-table lookups, the scale applied per
-    64-wide group): whole-vector chunks of up to 32 columns, no forced split, ``K_pad`` a
-    multiple of 256 and at most 6144, and no more 32-row blocks than compute units.  ``M``
-    counts the rows of all stacked matrices (each a multiple of 32, or count its 32-row blocks
-    and pass 32 times that).  (The library also wants the scales 8-byte aligned, which device
-    allocations are.)"""
+def gemm_streams(M, N: int, k_pad_: int, force_split: int = 0,  # noqa: N803
+                 one_wave: int = ONE_WAVE) -> int:
+    """32-row blocks of a workgroup (1 or 2) when a launch runs the stream tile, else 0.  The
+    tile is a workgroup of sixteen wavefronts on 32 or 64 rows and all of K: no split-K, no
+    partials, no reduce; pair-table lookups, the scale applied per 64-wide group.  It takes
+    whole-vector chunks of up to 32 columns, no forced split, ``K_pad`` a multiple of 256 and
+    at most 6144; 32 rows a workgroup while the launch has no more 32-row blocks than compute
+    units, else 64 rows up to two workgroups a compute unit.  ``M``: the rows, or the rows of
+    each stacked matrix (blocks do not straddle matrices).  ``CHR_NF4_GEMM_STREAM_ROWS=32`` or
+    ``64`` allows only that form.  (The library also wants the scales 8-byte aligned, which
+    device allocations are.)"""
+    global _STREAM_ONLY
+    if _STREAM_ONLY is None:
+        _STREAM_ONLY = _env_int_once("CHR_NF4_GEMM_STREAM_ROWS", 0)
     kp = int(k_pad_)
-    blocks32 = _ceil_div(int(M), _STREAM_ROWS)
-    return (_stream_columns(N) and force_split <= 0 and kp % _BK == 0
-            and kp <= 12 * 512 and blocks32 <= int(one_wave))
+    rows = [int(M)] if isinstance(M, int) else [int(m) for m in M]
+    if not (_stream_columns(N) and force_split <= 0 and kp % _BK == 0 and kp <= 12 * 512):
+        return 0
+    if sum(_ceil_div(m, _STREAM_ROWS) for m in rows) <= int(one_wave) and _STREAM_ONLY != 64:
+        return 1
+    if sum(_ceil_div(m, 2 * _STREAM_ROWS) for m in rows) <= 2 * int(one_wave) and _STREAM_ONLY != 32:
+        return 2
+    return 0
 
 
 def _pick_split_rows(grid_x: int, n_ktiles: int, cus: int, fallback: int) -> int:
@@ -292,10 +312,12 @@ def plan(M: int, K: int, N: int = 1, *, K_pad: int | None = None, have_ws: bool 
     path = PREFILL if N <= 16 else (PREFILL_N32 if N <= 32 else PREFILL_N64)
     grid_x = _ceil_div(M, _BM)
     n_ktiles = _ceil_div(kp, _BK)
-    if gemm_streams(M, N, kp, force_split, one_wave):
-        grid_x = _ceil_div(M, _STREAM_ROWS)
-        return Plan(path, grid_x, 1, 1024, _STREAM_ROWS, _BK, n_ktiles, n_ktiles, grid_x,
-                    _STREAM_LDS, 0)
+    row_blocks = gemm_streams(M, N, kp, force_split, one_wave)
+    if row_blocks:
+        bm = _STREAM_ROWS * row_blocks
+        grid_x = _ceil_div(M, bm)
+        return Plan(path, grid_x, 1, 1024, bm, _BK, n_ktiles, n_ktiles, grid_x,
+                    stream_lds_bytes(row_blocks), 0)
     split, tps = _pick_split(grid_x, n_ktiles, N, have_ws, force_split, one_wave)
     ws = split * M * N if split > 1 else 0
     if gemm_streams_rows(N, tps):

@@ -528,10 +528,10 @@ def test_rms(n):
 # ----------------------------------------------------------------------- GEMM
 def gemm_expected(p, s, m, k, x, plan):
     """What a prefill launch computes, in float64, by the tile its plan names.  The stream
-    tile (the only one with 32-row blocks) multiplies bf16(level) and applies the fp16 scale
+    tile (the only one with 32- or 64-row blocks) multiplies bf16(level) and applies the fp16 scale
     to each 64-wide group's sum; the two older tiles multiply bf16(level * scale), the
     reference kernel's weights (gpu/nf4/nf4_gemm.cu:312-323)."""
-    if plan["bm"] == 32:
+    if plan["bm"] in (32, 64):
         return staged_gemv_model(p, s, m, k, x, terms=1)
     return oc.c_matmul_f64(oc.bf16_round(oc.c_decode(p, s, m, k)), x)
 
@@ -606,12 +606,15 @@ STREAM_CASES = [
     (256, 5120, 32), (70, 6144, 8),                  # ten and twelve chunks
     (2048, 2048, 32), (5120, 5120, 8), (7168, 5120, 16),
     (8192, 1024, 32),                                # as many workgroups as compute units
+    # 64 rows a workgroup: more 32-row blocks than compute units
+    (8224, 256, 8), (8193, 512, 32), (9000, 1000, 24), (13824, 5120, 16),
+    (32768, 768, 32),                                # two workgroups for every compute unit
 ]
 
 
 @pytest.mark.parametrize("m,k,n", STREAM_CASES)
 def test_gemm_stream_tile(m, k, n):
-    """The tile without split-K (32 rows and all of K per workgroup, bf16(level) times the
+    """The tile without split-K (32 or 64 rows and all of K per workgroup, bf16(level) times the
     activations, the scale applied to each group's sum): against that arithmetic in float64,
     bit-identical on a second launch, and its fused epilogue against the separate adds."""
     say("gemm stream", m, k, n)
@@ -620,8 +623,10 @@ def test_gemm_stream_tile(m, k, n):
     x = bf16_tensor(xh)
     kp = oc.k_pad(k)
     plan = nf4.nf4_plan(m, k, n)
-    assert (plan["bm"], plan["grid_y"], plan["ws_floats"], plan["block"]) == (32, 1, 0, 1024)
-    assert plan["grid_x"] == -(-m // 32)
+    bm = 32 if -(-m // 32) <= 256 else 64
+    assert (plan["bm"], plan["grid_y"], plan["ws_floats"], plan["block"]) == (bm, 1, 0, 1024)
+    assert plan["grid_x"] == -(-m // bm)
+    assert plan["smem_bytes"] == 32768 + 2 * 33280 + 2 * bm * 272 + 96 * bm * 2
     y = nf4.nf4_gemm(dp, ds, x, m, k, kp)
     check_linear(y, staged_gemv_model(p, s, m, k, xh, terms=1), what=f"stream {m}x{k} n{n}")
     ref = oc.c_matmul_f64(oc.c_decode(p, s, m, k), xh)
@@ -684,10 +689,11 @@ def test_gemm_full_14b_shapes(name, m, k):
         x = rand_x(k, n, 16 + n)
         y = nf4.nf4_gemm(dp, ds, bf16_tensor(x), m, k, k)
         plan = nf4.nf4_plan(m, k, n)
-        # one workgroup per 32 rows and all of K where that is one round of the GPU and one
-        # pass of its written-out chunks (q/k/v and o); split-K tiles elsewhere
-        streams = -(-m // 32) <= 256 and k <= 6144
-        assert (plan["bm"], plan["grid_y"] == 1) == ((32, True) if streams else (128, False))
+        # one workgroup per 32 rows and all of K where that is one round of the GPU (q/k/v and
+        # o), per 64 rows otherwise (gate, up), K being one pass of the tile's written-out
+        # chunks; split-K tiles elsewhere (down)
+        bm = 128 if k > 6144 else (32 if -(-m // 32) <= 256 else 64)
+        assert (plan["bm"], plan["grid_y"] == 1) == (bm, bm != 128)
         ref = oc.c_matmul_f64(exact_w, x)
         err = np.abs(to_f32(y).astype(np.float64) - ref)
         assert (err <= np.maximum(0.05, 2 ** (np.floor(np.log2(np.maximum(np.abs(ref), 1e-30))) - 8))).all()

@@ -45,8 +45,8 @@ def test_noalloc_equals_workspace_entry_twice_second_smaller():
     ws_floats = int(lib.chr_nf4_gemm_noalloc_max_floats())
     assert ws_floats == 4 << 20
     ws = torch.empty(ws_floats, dtype=torch.float32, device="cuda")
-    # first call: a 14B gate or up chunk, split-K over several slices of partials
-    m, k, n = 13824, 5120, 32
+    # first call: a 14B down chunk, split-K over several slices of partials
+    m, k, n = 5120, 13824, 32
     plan = nf4.nf4_plan(m, k, n)
     assert plan["grid_y"] > 1 and 0 < plan["ws_floats"] <= ws_floats
     rc_ws, rc_na, y_ws, y_na, (packed, scale, x) = _both(lib, m, k, n, 5, ws, ws_floats)
