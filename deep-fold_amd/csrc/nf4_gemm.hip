@@ -43,6 +43,7 @@
 #include <type_traits>
 
 #include <atomic>
+#include <mutex>
 
 #include <algorithm>
 #include <cstdlib>
@@ -165,9 +166,19 @@ bool rows_kernel_serves(int N, int tiles_per_split) {
 // the compute units idle).  CHR_NF4_GEMM_STREAM=0 leaves everything to the two older tiles,
 // whose weights are bf16(level * scale) as in the reference's kernel
 // (gpu/nf4/nf4_gemm.cu:312-323).
+// -1: never, 0: where the cost model below prefers it to the split tiles, 1: wherever it fits.
+// Starts from CHR_NF4_GEMM_STREAM (0: never, 2: wherever it fits); chr_nf4_gemm_stream_policy
+// changes it.
+std::atomic<int> &stream_policy() {
+  static std::atomic<int> policy{[] {
+    const int e = env_int("CHR_NF4_GEMM_STREAM", 1);
+    return e == 0 ? -1 : (e == 2 ? 1 : 0);
+  }()};
+  return policy;
+}
+
 bool stream_columns(int N) {
-  static const bool on = env_int("CHR_NF4_GEMM_STREAM", 1) != 0;
-  return on && N >= 8 && N <= 32 && (N & 7) == 0;
+  return stream_policy().load(std::memory_order_relaxed) >= 0 && N >= 8 && N <= 32 && (N & 7) == 0;
 }
 
 Tuning &tuning() {
@@ -192,23 +203,78 @@ int resolved_one_wave() {
 
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
-// 32-row blocks of a workgroup of the stream tile for this launch, 0: another tile serves it.
+// How the stream tile takes a launch: rb = 32-row blocks of a workgroup (0: another tile
+// serves the launch), split = workgroups that share a row block's K (grid.y), chunks = 512-wide
+// chunks of the longest split.
+struct StreamPlan {
+  int rb, split, chunks;
+};
+
+constexpr int64_t kStreamMinCodes = int64_t{1} << 24;
+constexpr int kArriveSlots = 32;     // launches that may overlap in time (one a stream)
+constexpr int kArriveBlocks = 1024;  // row blocks of a launch whose splits meet in the tile
+
 // blocks32, blocks64: 32- and 64-row blocks of the launch (summed over its stacked matrices).
-// 32 rows each while one round of workgroups (one a compute unit) covers the launch, else 64
-// rows up to two rounds.  CHR_NF4_GEMM_STREAM_ROWS=32 or 64 allows only that form.
-int stream_row_blocks(int N, int K_pad, int blocks32, int blocks64) {
+// Picks, among the forms that fit (at most 12 chunks a workgroup; splits only when all
+// workgroups run at once and the caller brought a workspace; at most two rounds of
+// workgroups, and two only with 8 chunks or more to spread a round's fixed time over), the one a cost model fitted to measurements calls cheapest, in hundredths of a
+// microsecond: a round of 32-row workgroups 5.2 us + 0.55 / 0.67 / 0.86 / 1.06 us a chunk at
+// 8 / 16 / 24 / 32 columns, of 64-row workgroups 6.5 us + 1.00 / 1.06 / 1.22 / 1.38 us a chunk,
+// 2.3 us for the meeting of a split's partials (at most 8 splits; a split has to win by 3%).
+// codes: weights of the launch; with 2^24 or fewer the split tiles keep it (measured at
+// 8 / 32 columns, this tile against those: 256x5120 8.2 / 8.8 us against 7.5 / 8.5, 2048x2048
+// 6.9 / 9.0 against 7.2 / 8.2, 4096x4096 9.0 / 12.2 against 8.9 / 11.5, 1024x13824 10.6 /
+// 18.7 against 10.5 / 12.4; above, 3072x8192 11.0 / 15.2 against 12.1 / 15.1 and the 14B
+// shapes below).  At the 14B shapes:
+// q/k/v 32 rows x all of K up to 24 columns and 64 rows x 2 splits at 32; o 32 rows x all of K
+// up to 16 columns, 64 rows x 3 splits above; gate or up 64 rows; gate+up stacked 64 rows in two
+// rounds; down (K = 13824) 64 rows x 3 splits.  CHR_NF4_GEMM_STREAM_ROWS=32 or 64 allows only
+// that form, CHR_NF4_GEMM_STREAM_SPLIT=0 no splits.
+StreamPlan stream_plan(int N, int K_pad, int blocks32, int blocks64, int have_ws, int64_t codes) {
   static const int only = env_int("CHR_NF4_GEMM_STREAM_ROWS", 0);
-  if (!stream_columns(N) || tuning().split_k != 0 || K_pad % kBK != 0 ||
-      K_pad > kStreamBodies * kStreamChunkK) {
-    return 0;
+  static const bool splits = env_int("CHR_NF4_GEMM_STREAM_SPLIT", 1) != 0;
+  StreamPlan best{0, 1, 0};
+  if (!stream_columns(N) || tuning().split_k != 0 || K_pad % kBK != 0) {
+    return best;
   }
-  if (blocks32 <= resolved_one_wave() && only != 64) {
-    return 1;
+  static constexpr int kFixed[2] = {520, 650};
+  static constexpr int kChunk[2][4] = {{55, 67, 86, 106}, {100, 106, 122, 138}};
+  constexpr int kMeet = 230, kMaxSplit = 8;
+  const int cus = resolved_one_wave();
+  const int n_ch = ceil_div(K_pad, kStreamChunkK);
+  int best_cost = 0;
+  for (int rb = 1; rb <= 2; ++rb) {
+    if (only != 0 && only != kStreamRows * rb) {
+      continue;
+    }
+    const int blocks = rb == 1 ? blocks32 : blocks64;
+    for (int split = 1; split <= std::min(n_ch, kMaxSplit); ++split) {
+      const int chunks = ceil_div(n_ch, split);
+      if (ceil_div(n_ch, chunks) != split || chunks > kStreamBodies) {
+        continue;  // (the same chunks with fewer workgroups comes first; too long a K)
+      }
+      const int rounds = ceil_div(blocks * split, cus);
+      if (rounds > 2 || (split > 1 && (rounds > 1 || !splits || !have_ws || blocks > kArriveBlocks))) {
+        continue;
+      }
+      if (rounds == 2 && chunks < 8) {
+        continue;  // (22016x2048 in two rounds of 4 chunks: 18.1 / 22.1 us against 14.1 / 20.3)
+      }
+      int cost = rounds * (kFixed[rb - 1] + chunks * kChunk[rb - 1][N / 8 - 1]);
+      if (split > 1) {
+        cost += kMeet;
+        cost += cost / 32;
+      }
+      if (best.rb == 0 || cost < best_cost) {
+        best = StreamPlan{rb, split, chunks};
+        best_cost = cost;
+      }
+    }
   }
-  if (blocks64 <= 2 * resolved_one_wave() && only != 32) {
-    return 2;
+  if (codes <= kStreamMinCodes && only == 0 && stream_policy().load(std::memory_order_relaxed) == 0) {
+    best.rb = 0;
   }
-  return 0;
+  return best;
 }
 
 // Split-K.  A workgroup is quickest with about three K tiles (measured at every 14B linear
@@ -292,13 +358,16 @@ int plan_impl(const chr_nf4_dev_t &h, int32_t N, int32_t have_ws, chr_nf4_plan_t
     p.n_ktiles = ceil_div(h.K_pad, kBK);
     pick_split(p.grid_x, p.n_ktiles, N, have_ws, &p.grid_y, &p.tiles_per_split);
     p.smem_bytes = gemm_lds_bytes(N <= 32 ? 1 : 2);
-    if (const int rb = stream_row_blocks(N, h.K_pad, ceil_div(h.M, kStreamRows), ceil_div(h.M, 2 * kStreamRows))) {
-      p.bm = kStreamRows * rb;
+    const StreamPlan st =
+        stream_plan(N, h.K_pad, ceil_div(h.M, kStreamRows), ceil_div(h.M, 2 * kStreamRows), have_ws,
+                    static_cast<int64_t>(h.M) * h.K_pad);
+    if (st.rb != 0) {
+      p.bm = kStreamRows * st.rb;
       p.block = kStreamBlock;
       p.grid_x = ceil_div(h.M, p.bm);
-      p.grid_y = 1;
-      p.tiles_per_split = p.n_ktiles;
-      p.smem_bytes = stream_lds_bytes(rb);
+      p.grid_y = st.split;
+      p.tiles_per_split = std::min(2 * st.chunks, p.n_ktiles);
+      p.smem_bytes = stream_lds_bytes(st.rb);
     } else if (rows_kernel_serves(N, p.tiles_per_split)) {
       p.block = kRowsBlock;
       p.smem_bytes = rows_lds_bytes(rows_col_blocks(N), p.tiles_per_split);
@@ -974,6 +1043,12 @@ __device__ __forceinline__ int stream_token_row(int n) {
 // above, four quarter items at exactly 32 columns.  RB: 32-row blocks of a workgroup, 1 or 2
 // (segs.blocks counts blocks of 32 RB rows): with two, a multiplying wavefront feeds every B
 // operand it reads to two A operands, and x is staged once per 64 rows.
+// Arrival counts of the stream tile's K splits, one word a row block: the workgroup that finds
+// the others of its row block already counted adds up the partials.  All zero when the library
+// is loaded, and every launch leaves them zero.  A launch uses one slot; launches that may
+// overlap in time must use different slots (the host deals a slot to every stream).
+static __device__ unsigned int stream_arrivals[kArriveSlots][kArriveBlocks];
+
 template <int XI, int RB>
 __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
                                                             const uint16_t *__restrict__ x,
@@ -981,7 +1056,7 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
                                                             float *__restrict__ partial, int M_all,
                                                             int K, int K_pad, int N,
                                                             const uint16_t *__restrict__ bias,
-                                                            const uint16_t *res) {
+                                                            const uint16_t *res, int arrive_slot) {
   constexpr int XS = kStreamXS;
   constexpr int CK = kStreamChunkK;
   constexpr int ROWS = kStreamRows * RB;
@@ -1015,9 +1090,18 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
   const int row_base = bx * ROWS;
   const int r = lane & 31;  // row of the A operand, token of the B operand
   const int h = lane >> 5;  // which half of a group's k
-  const int row_bytes = K_pad >> 1;
-  const int groups = K_pad >> 6;
-  const int n_ch = (K_pad + CK - 1) / CK;
+  // grid.y splits K by whole chunks: this workgroup takes n_ch of them from chunk c0 on, and
+  // from here on x, K, row_bytes and groups describe what is left of K from that chunk on
+  const int n_ch_all = (K_pad + CK - 1) / CK;
+  const int per_split = (n_ch_all + static_cast<int>(gridDim.y) - 1) / static_cast<int>(gridDim.y);
+  const int c0 = static_cast<int>(blockIdx.y) * per_split;
+  const int n_ch = min(per_split, n_ch_all - c0);
+  const int row_stride = K_pad >> 1;  // bytes of a packed row
+  const int row_bytes = row_stride - c0 * (CK / 2);
+  const int groups_all = K_pad >> 6;
+  const int groups = min(8 * n_ch, groups_all - 8 * c0);
+  x += static_cast<size_t>(c0) * CK * N;
+  K -= c0 * CK;
 
   // ---- requests: a thread's share of one chunk ------------------------------------------------
   // XI = 4 is the form for exactly 32 columns: a k pair of x (rows 2 kp, 2 kp + 1) is then
@@ -1035,7 +1119,8 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
   const uint8_t *wp[RB];
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
-    wp[rb] = packed + static_cast<size_t>(min(row_base + 32 * rb + (stid >> 4), M - 1)) * row_bytes;
+    wp[rb] = packed + static_cast<size_t>(min(row_base + 32 * rb + (stid >> 4), M - 1)) * row_stride +
+             c0 * (CK / 2);
   }
   const int w_piece = 16 * (stid & 15);
   const int nv = N >> 3;
@@ -1138,7 +1223,7 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
     const int i = min(tid + it * kStreamBlock, ROWS * quads - 1);
     const int srow = i / quads;
     sv[it] = *reinterpret_cast<const uint2 *>(
-        scale + static_cast<size_t>(min(row_base + srow, M - 1)) * groups + 4 * (i - srow * quads));
+        scale + static_cast<size_t>(min(row_base + srow, M - 1)) * groups_all + 8 * c0 + 4 * (i - srow * quads));
   }
   // chunks a staging thread keeps in flight: with 64 bytes of x a chunk, three are what 128
   // registers hold
@@ -1299,31 +1384,97 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
   }
   __syncthreads();
   // wavefront w of the sixteen finishes accumulator value w of every 32-row block
+  float o32[RB];
+  size_t at[RB];
+  bool live[RB];
+  int orow[RB];
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
     const int v = wave16;
-    float o32 = 0.f;
+    o32[rb] = 0.f;
 #pragma unroll
     for (int q = 0; q < 8; ++q) {
-      o32 += sums[((rb * 8 + q) * 16 + v) * kWave + lane];
+      o32[rb] += sums[((rb * 8 + q) * 16 + v) * kWave + lane];
     }
-    const int n = r;
     const int rr = row_base + 32 * rb + 8 * (v >> 2) + 4 * h + (v & 3);
-    if (n < N && rr < M) {
-      const size_t at = static_cast<size_t>(out0 + rr) * N + n;
-      if (partial == nullptr) {
-        // the epilogue of reduce_splitk, here (res may alias y: same thread, same element)
-        uint16_t o = f32_to_bf16(o32);
-        if (bias != nullptr) {
-          o = f32_to_bf16(bf16_to_f32(o) + bf16_to_f32(bias[out0 + rr]));
+    live[rb] = r < N && rr < M;
+    orow[rb] = out0 + min(rr, M - 1);
+    at[rb] = static_cast<size_t>(orow[rb]) * N + min(r, N - 1);
+  }
+  if (partial != nullptr) {
+    // this split's slab of the partials
+    const size_t slab = static_cast<size_t>(M_all) * N;
+    if (arrive_slot < 0) {
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        if (live[rb]) {
+          partial[blockIdx.y * slab + at[rb]] = o32[rb];
         }
-        if (res != nullptr) {
-          o = f32_to_bf16(bf16_to_f32(res[at]) + bf16_to_f32(o));
-        }
-        y[at] = o;
-      } else {
-        partial[at] = o32;
       }
+      return;  // a reduce kernel adds the slabs up
+    }
+    // The last of this row block's splits to arrive adds them up, in split order whoever it
+    // is; nobody waits for anybody.  The compute dies' L2 caches do not see each other's
+    // lines, and a fence that makes them (write back and invalidate the whole cache) costs
+    // tens of microseconds with a few hundred workgroups at it.  So the partials and the
+    // count go past the caches one access at a time instead: device-scope stores that write
+    // through, waited for by every thread before the barrier after which thread 0 counts the
+    // workgroup in, and device-scope loads that do not take a cached line for an answer.
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      if (live[rb]) {
+        __hip_atomic_store(partial + blockIdx.y * slab + at[rb], o32[rb], __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    int *last = reinterpret_cast<int *>(lds_raw + kScaleAddr);  // (the scales are done with)
+    if (tid == 0) {
+      unsigned int *count = &stream_arrivals[arrive_slot][blockIdx.x];
+      const unsigned int before =
+          __hip_atomic_fetch_add(count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const bool all_in = before + 1 == gridDim.y;
+      if (all_in) {
+        __hip_atomic_store(count, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      *last = all_in ? 1 : 0;
+    }
+    __syncthreads();
+    if (*last == 0) {
+      return;
+    }
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      // (four requests at a time: a loop of single ones waits a round trip for each)
+      float sum = 0.f;
+      for (unsigned int j0 = 0; j0 < gridDim.y; j0 += 4) {
+        float v[4];
+#pragma unroll
+        for (unsigned int u = 0; u < 4; ++u) {
+          v[u] = __hip_atomic_load(partial + min(j0 + u, gridDim.y - 1) * slab + at[rb], __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+        }
+#pragma unroll
+        for (unsigned int u = 0; u < 4; ++u) {
+          sum = j0 + u == 0 ? v[0] : (j0 + u < gridDim.y ? sum + v[u] : sum);
+        }
+      }
+      o32[rb] = sum;
+    }
+  }
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    if (live[rb]) {
+      // the epilogue of reduce_splitk, here (res may alias y: same thread, same element)
+      uint16_t o = f32_to_bf16(o32[rb]);
+      if (bias != nullptr) {
+        o = f32_to_bf16(bf16_to_f32(o) + bf16_to_f32(bias[orow[rb]]));
+      }
+      if (res != nullptr) {
+        o = f32_to_bf16(bf16_to_f32(res[at[rb]]) + bf16_to_f32(o));
+      }
+      y[at[rb]] = o;
     }
   }
 }
@@ -1592,6 +1743,10 @@ int gemm_lds_ready() {
 
 using namespace chr;
 
+extern "C" void chr_nf4_gemm_stream_policy(int32_t policy) {
+  chr::stream_policy().store(policy < 0 ? -1 : (policy > 0 ? 1 : 0), std::memory_order_relaxed);
+}
+
 extern "C" void chr_nf4_set_tuning(int32_t path, int32_t split_k, int32_t one_wave) {
   Tuning &t = tuning();
   t.path = (path >= 0 && path <= 2) ? path : 0;
@@ -1620,8 +1775,33 @@ struct StackPlan {
   GemmSegs segs;
   int M_all, grid_x, grid_y, n_ktiles, tiles_per_split;
   int64_t ws_floats;
-  int stream;  // 32-row blocks of a workgroup of the stream tile (no split), 0: another tile
+  int stream;  // 32-row blocks of a workgroup of the stream tile, 0: another tile
 };
+
+// The slot of arrival counts for launches on this stream of the current device; -1 when all
+// slots are taken by other streams (the splits then meet in a reduce kernel).  Launches on one
+// stream run one after the other, so they can share a slot.
+int arrival_slot(hipStream_t st) {
+  static std::mutex mu;
+  static std::pair<int, hipStream_t> owner[kArriveSlots];
+  static int used = 0;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    (void)hipGetLastError();
+    return -1;
+  }
+  const std::lock_guard<std::mutex> lock(mu);
+  for (int i = 0; i < used; ++i) {
+    if (owner[i].first == dev && owner[i].second == st) {
+      return i;
+    }
+  }
+  if (used == kArriveSlots) {
+    return -1;
+  }
+  owner[used] = {dev, st};
+  return used++;
+}
 
 // allow_stream: false when the launch cannot take the stream tile for a reason the shape does
 // not show (scales not 8-byte aligned).
@@ -1632,7 +1812,13 @@ StackPlan plan_stack(const chr_nf4_dev_t *h, int nseg, int N, int have_ws, bool 
     blocks32 += ceil_div(h[i].M, kStreamRows);
     blocks64 += ceil_div(h[i].M, 2 * kStreamRows);
   }
-  sp.stream = allow_stream ? stream_row_blocks(N, h[0].K_pad, blocks32, blocks64) : 0;
+  int64_t codes = 0;
+  for (int i = 0; i < nseg; ++i) {
+    codes += static_cast<int64_t>(h[i].M) * h[i].K_pad;
+  }
+  const StreamPlan stp = allow_stream ? stream_plan(N, h[0].K_pad, blocks32, blocks64, have_ws, codes)
+                                      : StreamPlan{0, 1, 0};
+  sp.stream = stp.rb;
   const int bm = sp.stream ? kStreamRows * sp.stream : kBM;
   for (int i = 0; i < 3; ++i) {
     const bool on = i < nseg;
@@ -1646,8 +1832,9 @@ StackPlan plan_stack(const chr_nf4_dev_t *h, int nseg, int N, int have_ws, bool 
   }
   sp.n_ktiles = ceil_div(h[0].K_pad, kBK);
   if (sp.stream) {
-    sp.grid_y = 1;
-    sp.tiles_per_split = sp.n_ktiles;
+    sp.grid_y = stp.split;
+    sp.tiles_per_split = std::min(2 * stp.chunks, sp.n_ktiles);
+    sp.ws_floats = sp.grid_y > 1 ? static_cast<int64_t>(sp.grid_y) * sp.M_all * N : 0;
     return sp;
   }
   pick_split(sp.grid_x, sp.n_ktiles, N, have_ws, &sp.grid_y, &sp.tiles_per_split);
@@ -1726,27 +1913,33 @@ int gemm_launch(const chr_nf4_dev_t *const *w, int nseg, const void *x, void *y,
   const dim3 block(kGemmBlock);
   const int K = h[0].K, K_pad = h[0].K_pad;
   const int nc = rows_col_blocks(N);
+  // the stream tile's splits meet in the tile itself unless the reduce has more to do
+  // (SwiGLU, the column sums of squares)
+  int slot = -1;
+  if (sp.stream != 0 && sp.grid_y > 1 && !swiglu && !(colsq != nullptr && 256 % N == 0)) {
+    slot = sp.grid_x <= kArriveBlocks ? arrival_slot(st) : -1;
+  }
   if (sp.stream == 1) {
     if (N <= 16) {
       gemm_stream<1, 1><<<grid, dim3(kStreamBlock), stream_lds_bytes(1), st>>>(
-          sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp);
+          sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp, slot);
     } else if (N == 32) {
       gemm_stream<4, 1><<<grid, dim3(kStreamBlock), stream_lds_bytes(1), st>>>(
-          sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp);
+          sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp, slot);
     } else {
       gemm_stream<2, 1><<<grid, dim3(kStreamBlock), stream_lds_bytes(1), st>>>(
-          sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp);
+          sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp, slot);
     }
   } else if (sp.stream == 2) {
     if (N <= 16) {
       gemm_stream<1, 2><<<grid, dim3(kStreamBlock), stream_lds_bytes(2), st>>>(
-          sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp);
+          sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp, slot);
     } else if (N == 32) {
       gemm_stream<4, 2><<<grid, dim3(kStreamBlock), stream_lds_bytes(2), st>>>(
-          sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp);
+          sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp, slot);
     } else {
       gemm_stream<2, 2><<<grid, dim3(kStreamBlock), stream_lds_bytes(2), st>>>(
-          sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp);
+          sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp, slot);
     }
   } else if (rows_kernel_serves(N, sp.tiles_per_split)) {
     const RowsArgs ra{sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp};
@@ -1775,7 +1968,7 @@ int gemm_launch(const chr_nf4_dev_t *const *w, int nseg, const void *x, void *y,
     const int half_rows = h[0].M * N;
     reduce_swiglu<<<dim3(static_cast<unsigned>(ceil_div(half_rows, 256))), dim3(256), 0, st>>>(
         partial, yp, half_rows, sp.grid_y);
-  } else if (partial != nullptr) {
+  } else if (partial != nullptr && slot < 0) {
     const int rows = sp.M_all * N;
     if (colsq != nullptr && 256 % N == 0) {
       reduce_splitk_sq<<<dim3(static_cast<unsigned>(ceil_div(rows, kSqElems))), dim3(kSqElems),

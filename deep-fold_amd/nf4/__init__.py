@@ -113,6 +113,7 @@ EXPORTS = (
     ("chr_nf4_gemm_noalloc", ctypes.c_int, [_DP, _P, _P, _I, _P]),
     ("chr_nf4_gemm_noalloc_max_floats", ctypes.c_int64, []),
     ("chr_nf4_set_tuning", None, [_I, _I, _I]),
+    ("chr_nf4_gemm_stream_policy", None, [_I]),
     ("chr_nf4_gemv", ctypes.c_int, [_DP, _P, _P, _P, _P, _P, _F]),
     ("chr_nf4_gemv_qkv", ctypes.c_int, [_DP, _DP, _DP, _P, _P, _P, _P, _P, _P, _P, _P, _P, _F]),
     ("chr_nf4_gemv_swiglu", ctypes.c_int, [_DP, _DP, _P, _P, _P, _P, _F]),
@@ -275,6 +276,14 @@ def nf4_set_tuning(path: int = 0, split_k: int = 0, one_wave: int = 0) -> None:
     """Override the planner for this process (``gpu/nf4/__init__.py:361-372``):
     ``split_k`` 0 = auto, >0 forced; ``one_wave`` 0 = this GPU's compute units."""
     _load_ext().chr_nf4_set_tuning(int(path), int(split_k), int(one_wave))
+
+
+def nf4_gemm_stream_policy(policy: int = 0) -> None:
+    """Which prefill launches run the tile whose workgroups finish their rows themselves
+    (no reduce launch): 0 where the planner's cost model prefers it to the split tiles (the
+    default unless ``CHR_NF4_GEMM_STREAM`` says otherwise), 1 wherever it fits, -1 never.  No
+    counterpart in the reference."""
+    _load_ext().chr_nf4_gemm_stream_policy(int(policy))
 
 
 def nf4_gemm(packed: torch.Tensor, scale: torch.Tensor, x: torch.Tensor, M: int, K: int,  # noqa: N803

@@ -198,7 +198,7 @@ def _rows_kernel_on() -> bool:
     return _ROWS_ON
 
 
-_STREAM_ON: bool | None = None
+_STREAM_ON: int | None = None
 _STREAM_ONLY: int | None = None
 _STREAM_ROWS = 32
 _STREAM_MAX_GROUPS = 96
@@ -220,38 +220,85 @@ def _env_int_once(name: str, dflt: int) -> int:
         return 0                 # atoi() of a non-number is 0
 
 
-def _stream_columns(N: int) -> bool:  # noqa: N803
-    """Chunk widths the stream tile takes (8, 16, 24, 32) unless ``CHR_NF4_GEMM_STREAM=0``
-    (read once, like the library does)."""
+def stream_policy_default() -> int:
+    """-1 never, 0 where the cost model prefers the stream tile, 1 wherever it fits: from
+    ``CHR_NF4_GEMM_STREAM`` (0: never, 2: wherever it fits), read once like the library does
+    (``nf4_gemm_stream_policy`` changes the library's; pass the same to ``plan``)."""
     global _STREAM_ON
     if _STREAM_ON is None:
-        _STREAM_ON = _env_int_once("CHR_NF4_GEMM_STREAM", 1) != 0
-    return _STREAM_ON and 8 <= N <= 32 and N % 8 == 0
+        e = _env_int_once("CHR_NF4_GEMM_STREAM", 1)
+        _STREAM_ON = -1 if e == 0 else (1 if e == 2 else 0)
+    return _STREAM_ON
+
+
+def _stream_columns(N: int, policy: int) -> bool:  # noqa: N803
+    """Chunk widths the stream tile takes (8, 16, 24, 32)."""
+    return policy >= 0 and 8 <= N <= 32 and N % 8 == 0
+
+
+_STREAM_SPLITS: bool | None = None
+#: the stream tile's cost model, hundredths of a microsecond: a round of workgroups of 32 / 64
+#: rows, a 512-wide chunk at 8 / 16 / 24 / 32 columns, the meeting of a split's partials
+_STREAM_FIXED = (520, 650)
+_STREAM_CHUNK = ((55, 67, 86, 106), (100, 106, 122, 138))
+_STREAM_MEET = 230
+_STREAM_MAX_SPLIT = 8
+_STREAM_MIN_CODES = 1 << 24
+_ARRIVE_BLOCKS = 1024
 
 
 def gemm_streams(M, N: int, k_pad_: int, force_split: int = 0,  # noqa: N803
-                 one_wave: int = ONE_WAVE) -> int:
-    """32-row blocks of a workgroup (1 or 2) when a launch runs the stream tile, else 0.  The
-    tile is a workgroup of sixteen wavefronts on 32 or 64 rows and all of K: no split-K, no
-    partials, no reduce; pair-table lookups, the scale applied per 64-wide group.  It takes
-    whole-vector chunks of up to 32 columns, no forced split, ``K_pad`` a multiple of 256 and
-    at most 6144; 32 rows a workgroup while the launch has no more 32-row blocks than compute
-    units, else 64 rows up to two workgroups a compute unit.  ``M``: the rows, or the rows of
-    each stacked matrix (blocks do not straddle matrices).  ``CHR_NF4_GEMM_STREAM_ROWS=32`` or
-    ``64`` allows only that form.  (The library also wants the scales 8-byte aligned, which
-    device allocations are.)"""
-    global _STREAM_ONLY
+                 one_wave: int = ONE_WAVE, have_ws: bool = True,
+                 policy: int | None = None) -> tuple[int, int, int]:
+    """``(row_blocks, split, chunks)`` of the stream tile for a launch, ``row_blocks`` 0 when
+    another tile serves it.  The tile is a workgroup of sixteen wavefronts on 32 or 64 rows
+    (``row_blocks`` 1 or 2) and ``chunks`` 512-wide chunks of K; ``split`` workgroups share a
+    row block's K and the last of them to finish adds up their fp32 partials (no reduce
+    launch); pair-table lookups, the scale applied per 64-wide group.  It takes whole-vector
+    chunks of up to 32 columns, no forced split, ``K_pad`` a multiple of 256, at most 12
+    chunks a workgroup, splits only when all workgroups run at once and there is a workspace,
+    at most 8 splits, at most two rounds of workgroups (two only with 8 chunks or more) --
+    and of the forms that fit, the cheapest by the cost model above (a split has to win by
+    3%), if the launch has more than 2^24 weights (``policy`` 0; 1: wherever it fits; -1:
+    never; None: the process default).  ``M``: the rows, or the rows of each stacked matrix
+    (blocks do not straddle matrices).  ``CHR_NF4_GEMM_STREAM_ROWS=32`` or ``64`` allows only
+    that form and skips the weight count, ``CHR_NF4_GEMM_STREAM_SPLIT=0`` allows no splits.
+    (The library also wants the scales 8-byte aligned, which device allocations are.)"""
+    global _STREAM_ONLY, _STREAM_SPLITS
     if _STREAM_ONLY is None:
         _STREAM_ONLY = _env_int_once("CHR_NF4_GEMM_STREAM_ROWS", 0)
+        _STREAM_SPLITS = _env_int_once("CHR_NF4_GEMM_STREAM_SPLIT", 1) != 0
     kp = int(k_pad_)
     rows = [int(M)] if isinstance(M, int) else [int(m) for m in M]
-    if not (_stream_columns(N) and force_split <= 0 and kp % _BK == 0 and kp <= 12 * 512):
-        return 0
-    if sum(_ceil_div(m, _STREAM_ROWS) for m in rows) <= int(one_wave) and _STREAM_ONLY != 64:
-        return 1
-    if sum(_ceil_div(m, 2 * _STREAM_ROWS) for m in rows) <= 2 * int(one_wave) and _STREAM_ONLY != 32:
-        return 2
-    return 0
+    best, best_cost = (0, 1, 0), 0
+    policy = stream_policy_default() if policy is None else int(policy)
+    if not (_stream_columns(N, policy) and force_split <= 0 and kp % _BK == 0):
+        return best
+    cus = int(one_wave)
+    n_ch = _ceil_div(kp, 512)
+    for rb in (1, 2):
+        if _STREAM_ONLY not in (0, _STREAM_ROWS * rb):
+            continue
+        blocks = sum(_ceil_div(m, _STREAM_ROWS * rb) for m in rows)
+        for split in range(1, min(n_ch, _STREAM_MAX_SPLIT) + 1):
+            chunks = _ceil_div(n_ch, split)
+            if _ceil_div(n_ch, chunks) != split or chunks > 12:
+                continue
+            rounds = _ceil_div(blocks * split, cus)
+            if rounds > 2 or (split > 1 and (rounds > 1 or not _STREAM_SPLITS or not have_ws
+                                             or blocks > _ARRIVE_BLOCKS)):
+                continue
+            if rounds == 2 and chunks < 8:
+                continue
+            cost = rounds * (_STREAM_FIXED[rb - 1] + chunks * _STREAM_CHUNK[rb - 1][N // 8 - 1])
+            if split > 1:
+                cost += _STREAM_MEET
+                cost += cost // 32
+            if best[0] == 0 or cost < best_cost:
+                best, best_cost = (rb, split, chunks), cost
+    if policy == 0 and _STREAM_ONLY == 0 and sum(rows) * kp <= _STREAM_MIN_CODES:
+        return (0, 1, 0)
+    return best
 
 
 def _pick_split_rows(grid_x: int, n_ktiles: int, cus: int, fallback: int) -> int:
@@ -287,7 +334,8 @@ def _pick_split(grid_x: int, n_ktiles: int, N: int, have_ws: bool, force_split: 
 
 
 def plan(M: int, K: int, N: int = 1, *, K_pad: int | None = None, have_ws: bool = True,  # noqa: N803
-         force_split: int = 0, one_wave: int = ONE_WAVE, gemv_rows: int = 0) -> Plan:
+         force_split: int = 0, one_wave: int = ONE_WAVE, gemv_rows: int = 0,
+         stream_policy: int | None = None) -> Plan:
     M, K, N = int(M), int(K), int(N)
     if M < 1 or K < 1:
         raise ValueError(f"M and K must be >= 1, got M={M} K={K}")
@@ -312,12 +360,12 @@ def plan(M: int, K: int, N: int = 1, *, K_pad: int | None = None, have_ws: bool 
     path = PREFILL if N <= 16 else (PREFILL_N32 if N <= 32 else PREFILL_N64)
     grid_x = _ceil_div(M, _BM)
     n_ktiles = _ceil_div(kp, _BK)
-    row_blocks = gemm_streams(M, N, kp, force_split, one_wave)
+    row_blocks, split, chunks = gemm_streams(M, N, kp, force_split, one_wave, have_ws, stream_policy)
     if row_blocks:
         bm = _STREAM_ROWS * row_blocks
         grid_x = _ceil_div(M, bm)
-        return Plan(path, grid_x, 1, 1024, bm, _BK, n_ktiles, n_ktiles, grid_x,
-                    stream_lds_bytes(row_blocks), 0)
+        return Plan(path, grid_x, split, 1024, bm, _BK, n_ktiles, min(2 * chunks, n_ktiles),
+                    grid_x * split, stream_lds_bytes(row_blocks), split * M * N if split > 1 else 0)
     split, tps = _pick_split(grid_x, n_ktiles, N, have_ws, force_split, one_wave)
     ws = split * M * N if split > 1 else 0
     if gemm_streams_rows(N, tps):

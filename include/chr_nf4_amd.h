@@ -63,12 +63,16 @@ int chr_nf4_gemm(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N,
                  void *stream);
 
 /* Pure launch math; only M/K/K_pad are read.  N in [1, 64].
- * Chunks of 8, 16, 24 or 32 columns of a matrix with at most one 32-row block per compute
- * unit and K_pad a multiple of 256 up to 6144 are planned on the tile that needs no split
- * (bm 32, grid_y 1, ws_floats 0, block 1024); it multiplies bf16(level) and applies the fp16
- * scale to each 64-wide group's sum, where the other tiles multiply bf16(level * scale) as
- * the reference's kernel does.  CHR_NF4_GEMM_STREAM=0 in the environment, a forced split
- * (chr_nf4_set_tuning) or a scale blob that is not 8-byte aligned keep a launch on those.
+ * Chunks of 8, 16, 24 or 32 columns with K_pad a multiple of 256 can run the tile whose
+ * workgroups finish their rows themselves (block 1024; bm 32 or 64 rows a workgroup; grid_y
+ * workgroups share a row block's K in 512-wide chunks, at most 12 each, and the last of them
+ * to finish adds their fp32 partials up in split order: ws_floats = grid_y * M * N when
+ * grid_y > 1, no reduce launch).  The planner takes it where its cost model prefers it to
+ * the split tiles (at 14B shapes: all of them); chr_nf4_gemm_stream_policy and
+ * CHR_NF4_GEMM_STREAM (0 never, 2 wherever it fits) change that, a forced split
+ * (chr_nf4_set_tuning) or a scale blob that is not 8-byte aligned keep a launch on the split
+ * tiles.  It multiplies bf16(level) and applies the fp16 scale to each 64-wide group's sum,
+ * where the other tiles multiply bf16(level * scale) as the reference's kernel does.
  * Replaces chr_nf4_gemm_plan (chr_gpu.h:64-65; nf4_gemm.cu:1656-1667). */
 int chr_nf4_gemm_plan(const chr_nf4_dev_t *w, int32_t N, int32_t have_ws,
                       chr_nf4_plan_t *out);
@@ -106,6 +110,15 @@ int64_t chr_nf4_gemm_noalloc_max_floats(void);
  * Initial values come from CHR_NF4_PATH / CHR_NF4_SPLIT_K / CHR_NF4_ONE_WAVE.
  * Replaces chr_nf4_set_tuning (chr_gpu.h:84; nf4_gemm.cu:1648-1654). */
 void chr_nf4_set_tuning(int32_t path, int32_t split_k, int32_t one_wave);
+
+/* Which prefill launches run the tile whose workgroups finish their rows themselves:
+ * 0 where the planner's cost model prefers it (the default), > 0 wherever it fits, < 0 never.
+ * Process-wide, like chr_nf4_set_tuning.  Launches of that tile that split K count their
+ * arrivals in a table the library owns, one slot per stream (32 streams; further streams get
+ * a reduce launch instead): launches that may overlap in time must be made on different
+ * streams, and graphs captured from one stream must not be replayed concurrently.
+ * No counterpart in the reference. */
+void chr_nf4_gemm_stream_policy(int32_t policy);
 
 /* N=1 GEMV.  x bf16 [K], y bf16 [M].  add: optional bf16 [M] residual, may
  * alias y.  rms_w: optional bf16 [K]; when set, RMSNorm(x, rms_w, rms_eps),

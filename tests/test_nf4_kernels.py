@@ -8,6 +8,7 @@ import torch
 import torch.nn.functional as F
 
 from deepfold_amd import nf4
+from deepfold_amd.nf4 import plan as pyplan
 from oracle import nf4_oracle as oc
 
 from helpers import (DEV, MAX_REL, bf16_bits, bf16_tensor, check_linear, rand_x, to_f32, ulp_bf16, up,
@@ -609,23 +610,39 @@ STREAM_CASES = [
     # 64 rows a workgroup: more 32-row blocks than compute units
     (8224, 256, 8), (8193, 512, 32), (9000, 1000, 24), (13824, 5120, 16),
     (32768, 768, 32),                                # two workgroups for every compute unit
+    # K split over workgroups that meet in the tile: 5 to 8, 3 and 2 splits
+    (256, 5120, 32), (1024, 5120, 8), (5120, 13824, 8), (5120, 5120, 32), (3072, 8192, 16),
+    (5000, 13560, 16),                               # ragged rows, K below K_pad, a last chunk of 256
 ]
 
 
 @pytest.mark.parametrize("m,k,n", STREAM_CASES)
 def test_gemm_stream_tile(m, k, n):
-    """The tile without split-K (32 or 64 rows and all of K per workgroup, bf16(level) times the
-    activations, the scale applied to each group's sum): against that arithmetic in float64,
-    bit-identical on a second launch, and its fused epilogue against the separate adds."""
+    """The tile without a reduce launch (32 or 64 rows per workgroup and all of K, or K split
+    over workgroups of which the last to finish adds up the partials in split order; bf16(level)
+    times the activations, the scale applied to each group's sum): against that arithmetic in
+    float64, bit-identical on a second launch, and its fused epilogue against the separate
+    adds."""
     say("gemm stream", m, k, n)
     p, s, dp, ds = blobs(m, k, 900 + m + k + n)
     xh = rand_x(k, n, 19)
     x = bf16_tensor(xh)
     kp = oc.k_pad(k)
+    nf4.nf4_gemm_stream_policy(1)  # wherever it fits: the planner leaves small launches to the split tiles
+    try:
+        _stream_tile_case(m, k, n, p, s, dp, ds, xh, x, kp)
+    finally:
+        nf4.nf4_gemm_stream_policy(0)
+
+
+def _stream_tile_case(m, k, n, p, s, dp, ds, xh, x, kp):
     plan = nf4.nf4_plan(m, k, n)
-    bm = 32 if -(-m // 32) <= 256 else 64
-    assert (plan["bm"], plan["grid_y"], plan["ws_floats"], plan["block"]) == (bm, 1, 0, 1024)
-    assert plan["grid_x"] == -(-m // bm)
+    want = pyplan.plan(m, k, n, one_wave=256, stream_policy=1)
+    assert all(plan[key] == getattr(want, key) for key in plan), (plan, want)
+    bm, split = plan["bm"], plan["grid_y"]
+    assert bm in (32, 64) and plan["block"] == 1024 and plan["grid_x"] == -(-m // bm)
+    assert plan["ws_floats"] == (split * m * n if split > 1 else 0)
+    assert -(-kp // 512) <= split * 12 and (split == 1 or plan["ctas"] <= 256)
     assert plan["smem_bytes"] == 32768 + 2 * 33280 + 2 * bm * 272 + 96 * bm * 2
     y = nf4.nf4_gemm(dp, ds, x, m, k, kp)
     check_linear(y, staged_gemv_model(p, s, m, k, xh, terms=1), what=f"stream {m}x{k} n{n}")
@@ -689,11 +706,12 @@ def test_gemm_full_14b_shapes(name, m, k):
         x = rand_x(k, n, 16 + n)
         y = nf4.nf4_gemm(dp, ds, bf16_tensor(x), m, k, k)
         plan = nf4.nf4_plan(m, k, n)
-        # one workgroup per 32 rows and all of K where that is one round of the GPU (q/k/v and
-        # o), per 64 rows otherwise (gate, up), K being one pass of the tile's written-out
-        # chunks; split-K tiles elsewhere (down)
-        bm = 128 if k > 6144 else (32 if -(-m // 32) <= 256 else 64)
-        assert (plan["bm"], plan["grid_y"] == 1) == (bm, bm != 128)
+        # every one of them on the tile whose workgroups finish their rows themselves: 32 rows
+        # and all of K (q/k/v, o to 24 columns), 64 rows (gate, up), 64 rows and K over three
+        # workgroups (o at 32 columns, down)
+        form = {"qkv": (32, 1), "o": (64, 3) if n == 32 else (32, 1), "gate_up": (64, 1), "down": (64, 3)}
+        assert (plan["bm"], plan["grid_y"]) == form[name], name
+        assert plan["block"] == 1024
         ref = oc.c_matmul_f64(exact_w, x)
         err = np.abs(to_f32(y).astype(np.float64) - ref)
         assert (err <= np.maximum(0.05, 2 ** (np.floor(np.log2(np.maximum(np.abs(ref), 1e-30))) - 8))).all()

@@ -282,11 +282,21 @@ def test_wide_chunk_equals_two_narrow_ones(m, k, n):
         nf4.nf4_gemm(dp, ds, x, m, k, kp)  # the reference's ceiling without max_n
 
 
+@pytest.fixture
+def stream_wherever_it_fits():
+    """The planner leaves launches of few weights to the split tiles; these cases want the
+    tile whose workgroups finish their rows themselves on small stacks too."""
+    nf4.nf4_gemm_stream_policy(1)
+    yield
+    nf4.nf4_gemm_stream_policy(0)
+
+
 @pytest.mark.parametrize("mq,mk,k,n,bias", [(256, 64, 512, 8, True), (5120, 1024, 5120, 64, True),
                                             (130, 70, 1088, 5, False), (2048, 256, 2048, 32, False),
-                                            (130, 70, 1024, 16, True),   # ragged 32-row blocks, no split
-                                            (6000, 1500, 512, 16, True)])  # ragged 64-row blocks, no split
-def test_stacked_qkv_equals_three_gemms(mq, mk, k, n, bias):
+                                            (130, 70, 1024, 16, True),   # ragged 32-row blocks
+                                            (6000, 1500, 512, 16, True),  # ragged 64-row blocks
+                                            (600, 200, 4096, 32, False)])  # K over several workgroups
+def test_stacked_qkv_equals_three_gemms(mq, mk, k, n, bias, stream_wherever_it_fits):
     say("gemm_qkv", mq, mk, k, n, bias)
     rng = np.random.default_rng(mq + n)
     mats = []
@@ -314,8 +324,9 @@ def test_stacked_qkv_equals_three_gemms(mq, mk, k, n, bias):
 
 @pytest.mark.parametrize("m,k,n", [(256, 512, 8), (13824, 5120, 64), (130, 1088, 5), (384, 256, 2),
                                    (130, 1024, 24), (2048, 2048, 32),
-                                   (4500, 512, 8), (13824, 5120, 32)])  # 64-row blocks, no split
-def test_stacked_gate_up_with_swiglu_in_the_reduce(m, k, n):
+                                   (4500, 512, 8), (13824, 5120, 32),  # 64-row blocks
+                                   (512, 6144, 16)])                   # K over several workgroups
+def test_stacked_gate_up_with_swiglu_in_the_reduce(m, k, n, stream_wherever_it_fits):
     say("gemm_swiglu", m, k, n)
     rng = np.random.default_rng(m + n)
     mats = []

@@ -64,9 +64,9 @@ def test_noalloc_equals_workspace_entry_twice_second_smaller():
     rc_ws, rc_na, y_ws, y_na, _ = _both(lib, m2, k2, n2, 9, ws, ws_floats)
     assert rc_ws == 0 and rc_na == 0
     assert torch.equal(y_ws.view(torch.int16), y_na.view(torch.int16))
-    # a chunk that the tile without split-K takes (no partials), through both entries alike
-    assert nf4.nf4_plan(7168, 5120, 32)["grid_y"] == 1
-    rc_ws, rc_na, y_ws, y_na, _ = _both(lib, 7168, 5120, 32, 10, ws, ws_floats)
+    # a chunk that needs no partials (a workgroup takes all of K), through both entries alike
+    assert nf4.nf4_plan(7168, 5120, 8)["grid_y"] == 1
+    rc_ws, rc_na, y_ws, y_na, _ = _both(lib, 7168, 5120, 8, 10, ws, ws_floats)
     assert rc_ws == 0 and rc_na == 0 and torch.equal(y_ws.view(torch.int16), y_na.view(torch.int16))
     # N = 1 goes to the GEMV (no partials at all) through both entries alike
     rc_ws, rc_na, y_ws, y_na, _ = _both(lib, 512, 1024, 1, 11, ws, ws_floats)
