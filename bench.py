@@ -214,8 +214,11 @@ def bench_prefill(torch, nf4, only=None, widths=(8, 16, 32, 64)):
             ms = graph_time(torch, launch, 3 * copies, reps=3)
             by = algorithmic_bytes(m, k, n)
             plan = nf4.nf4_plan(m, k, n)
-            tile = (f"stream ({plan['bm']} rows x all of K, no split)" if plan["bm"] in (32, 64)
-                    else f"split-K x{plan['grid_y']} + reduce")
+            if plan["bm"] in (32, 64):
+                tile = (f"stream ({plan['bm']} rows x all of K, no split)" if plan["grid_y"] == 1 else
+                        f"stream ({plan['bm']} rows, K over {plan['grid_y']} workgroups that meet in the tile)")
+            else:
+                tile = f"split-K x{plan['grid_y']} + reduce"
             rows.append({"layer": name, "M": m, "K": k, "N": n, "us": ms * 1e3, "tile": tile,
                          "gbps": by / (ms * 1e-3) / 1e9,
                          "hbm_frac": by / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,

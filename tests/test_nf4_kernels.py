@@ -609,7 +609,7 @@ STREAM_CASES = [
     (8192, 1024, 32),                                # as many workgroups as compute units
     # 64 rows a workgroup: more 32-row blocks than compute units
     (8224, 256, 8), (8193, 512, 32), (9000, 1000, 24), (13824, 5120, 16),
-    (32768, 768, 32),                                # two workgroups for every compute unit
+    (32768, 4096, 8),                                # two workgroups for every compute unit
     # K split over workgroups that meet in the tile: 5 to 8, 3 and 2 splits
     (256, 5120, 32), (1024, 5120, 8), (5120, 13824, 8), (5120, 5120, 32), (3072, 8192, 16),
     (5000, 13560, 16),                               # ragged rows, K below K_pad, a last chunk of 256
