@@ -658,6 +658,56 @@ def _stream_tile_case(m, k, n, p, s, dp, ds, xh, x, kp):
     assert (bf16_bits(got) == bf16_bits(want)).all()
 
 
+def test_gemm_stream_splits_on_many_streams():
+    """Launches whose workgroups share K count their arrivals in a slot of a table the library
+    owns, one slot per stream; streams beyond its 32 slots get the reduce kernel on the same
+    partials.  Forty streams, each launching twice: every result equals the first bit for bit."""
+    m, k, n = 5120, 13824, 8
+    say("gemm stream, many streams", m, k, n)
+    assert nf4.nf4_plan(m, k, n)["grid_y"] == 3 and nf4.nf4_plan(m, k, n)["block"] == 1024
+    p, s, dp, ds = blobs(m, k, 77)
+    x = bf16_tensor(rand_x(k, n, 5))
+    first = bf16_bits(nf4.nf4_gemm(dp, ds, x, m, k, k))
+    torch.cuda.synchronize()
+    outs = []
+    for _ in range(40):
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            outs.append(nf4.nf4_gemm(dp, ds, x, m, k, k))
+            outs.append(nf4.nf4_gemm(dp, ds, x, m, k, k))
+    torch.cuda.synchronize()
+    for o in outs:
+        assert (bf16_bits(o) == first).all()
+
+
+def test_gemm_stream_splits_in_a_replayed_graph():
+    """Three launches with K shared by workgroups, captured in one graph: every replay, with
+    eager launches of the same tile between the replays, gives the eager results bit for bit
+    (the arrival counts must be back at zero after every launch)."""
+    shapes = [(5120, 13824, 8), (5120, 5120, 32), (3072, 8192, 16)]
+    mats, xs, eager = [], [], []
+    for i, (m, k, n) in enumerate(shapes):
+        say("gemm stream, graph", m, k, n)
+        assert nf4.nf4_plan(m, k, n)["grid_y"] > 1 and nf4.nf4_plan(m, k, n)["block"] == 1024
+        p, s, dp, ds = blobs(m, k, 31 + i)
+        mats.append((dp, ds))
+        xs.append(bf16_tensor(rand_x(k, n, 40 + i)))
+        eager.append(bf16_bits(nf4.nf4_gemm(dp, ds, xs[i], m, k, k)))
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = [nf4.nf4_gemm(mats[i][0], mats[i][1], xs[i], m, k, k) for i, (m, k, n) in enumerate(shapes)]
+    for _ in range(4):
+        for o in outs:
+            o.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        for o, want in zip(outs, eager):
+            assert (bf16_bits(o) == want).all()
+        m, k, n = shapes[0]
+        assert (bf16_bits(nf4.nf4_gemm(mats[0][0], mats[0][1], xs[0], m, k, k)) == eager[0]).all()
+
+
 @pytest.mark.parametrize("n", [5, 8, 16, 24, 32, 40, 64])
 @pytest.mark.parametrize("k,split,tiles", [(1024, 1, 4), (1000, 2, 2), (1024, 4, 1), (768, 1, 3),
                                            (2048, 1, 8), (2048, 8, 1)])
