@@ -127,6 +127,18 @@ constexpr int stream_lds_bytes(int rb) {
   return kStreamTableBytes + 2 * kStreamXBytes + 2 * rb * kStreamWBytes + stream_scale_bytes(rb);
 }
 static_assert(stream_lds_bytes(2) <= 160 * 1024, "LDS of a compute unit");
+// The same tile at exactly 64 columns (gemm_stream64 below): 64 rows, chunks of 256.
+constexpr int kWideChunkK = 256;
+constexpr int kWideBodies = 20;  // chunks of the longest K (of one split) the tile takes
+constexpr int kWideRows = 64;
+constexpr int kWideXS = kWideChunkK + kXPad;           // bf16 elements of a token row of one chunk
+constexpr int kWideXBytes = 64 * kWideXS * 2;          // one chunk of x, 64 token rows
+constexpr int kWideWStride = kWideChunkK / 2 + 16;     // bytes of a staged weight row
+constexpr int kWideWBytes = kWideRows * kWideWStride;  // a chunk of weights
+constexpr int kWideMaxGroups = kWideBodies * kWideChunkK / 64;
+constexpr int kWideScaleBytes = kWideMaxGroups * kWideRows * 2;
+constexpr int kWideLdsBytes = kStreamTableBytes + 2 * kWideXBytes + 2 * kWideWBytes + kWideScaleBytes;
+static_assert(kWideLdsBytes <= 160 * 1024, "LDS of a compute unit");
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -178,7 +190,8 @@ std::atomic<int> &stream_policy() {
 }
 
 bool stream_columns(int N) {
-  return stream_policy().load(std::memory_order_relaxed) >= 0 && N >= 8 && N <= 32 && (N & 7) == 0;
+  return stream_policy().load(std::memory_order_relaxed) >= 0 &&
+         ((N >= 8 && N <= 32 && (N & 7) == 0) || N == 64);
 }
 
 Tuning &tuning() {
@@ -239,28 +252,31 @@ StreamPlan stream_plan(int N, int K_pad, int blocks32, int blocks64, int have_ws
   }
   static constexpr int kFixed[2] = {520, 650};
   static constexpr int kChunk[2][4] = {{55, 67, 86, 106}, {100, 106, 122, 138}};
+  constexpr int kWideChunk = 110;  // a 256-wide chunk of the 64-column form
   constexpr int kMeet = 230, kMaxSplit = 8;
   const int cus = resolved_one_wave();
-  const int n_ch = ceil_div(K_pad, kStreamChunkK);
+  const bool wide = N == 64;  // 64 rows and chunks of 256 only
+  const int n_ch = ceil_div(K_pad, wide ? kWideChunkK : kStreamChunkK);
+  const int bodies = wide ? kWideBodies : kStreamBodies;
   int best_cost = 0;
-  for (int rb = 1; rb <= 2; ++rb) {
+  for (int rb = wide ? 2 : 1; rb <= 2; ++rb) {
     if (only != 0 && only != kStreamRows * rb) {
       continue;
     }
     const int blocks = rb == 1 ? blocks32 : blocks64;
     for (int split = 1; split <= std::min(n_ch, kMaxSplit); ++split) {
       const int chunks = ceil_div(n_ch, split);
-      if (ceil_div(n_ch, chunks) != split || chunks > kStreamBodies) {
+      if (ceil_div(n_ch, chunks) != split || chunks > bodies) {
         continue;  // (the same chunks with fewer workgroups comes first; too long a K)
       }
       const int rounds = ceil_div(blocks * split, cus);
       if (rounds > 2 || (split > 1 && (rounds > 1 || !splits || !have_ws || blocks > kArriveBlocks))) {
         continue;
       }
-      if (rounds == 2 && chunks < 8) {
+      if (rounds == 2 && chunks * (wide ? kWideChunkK : kStreamChunkK) < 8 * kStreamChunkK) {
         continue;  // (22016x2048 in two rounds of 4 chunks: 18.1 / 22.1 us against 14.1 / 20.3)
       }
-      int cost = rounds * (kFixed[rb - 1] + chunks * kChunk[rb - 1][N / 8 - 1]);
+      int cost = rounds * (kFixed[rb - 1] + chunks * (wide ? kWideChunk : kChunk[rb - 1][N / 8 - 1]));
       if (split > 1) {
         cost += kMeet;
         cost += cost / 32;
@@ -366,8 +382,8 @@ int plan_impl(const chr_nf4_dev_t &h, int32_t N, int32_t have_ws, chr_nf4_plan_t
       p.block = kStreamBlock;
       p.grid_x = ceil_div(h.M, p.bm);
       p.grid_y = st.split;
-      p.tiles_per_split = std::min(2 * st.chunks, p.n_ktiles);
-      p.smem_bytes = stream_lds_bytes(st.rb);
+      p.tiles_per_split = N == 64 ? st.chunks : std::min(2 * st.chunks, p.n_ktiles);
+      p.smem_bytes = N == 64 ? kWideLdsBytes : stream_lds_bytes(st.rb);
     } else if (rows_kernel_serves(N, p.tiles_per_split)) {
       p.block = kRowsBlock;
       p.smem_bytes = rows_lds_bytes(rows_col_blocks(N), p.tiles_per_split);
@@ -1183,11 +1199,15 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
         // row's lane: tokens 8 q + 4 .. + 4 from the partner's columns 4..7 and its own
         const uint32_t a0 = w_half ? g0 : m0, a1 = w_half ? g1 : m1;
         const uint32_t b0 = w_half ? m2 : g0, b1 = w_half ? m3 : g1;
-        uint32_t *dst = xd + (8 * w_q + 4 * w_half) * (XS / 2) + kp;
+        // token 4 u + e lives in row 8 e + u of the chunk buffer: the eight lanes of a k pair
+        // (u = 2 q + half) store into eight consecutive rows, 4 banks apart, and the four k
+        // pairs of 32 lanes fill the banks between -- no two lanes on a bank, where rows in
+        // token order (eight rows 4 apart, 16 banks apart) put four there
+        uint32_t *dst = xd + (2 * w_q + w_half) * (XS / 2) + kp;
         dst[0] = (a0 & 0xFFFFu) | (b0 << 16);
-        dst[XS / 2] = (a0 >> 16) | (b0 & 0xFFFF0000u);
-        dst[2 * (XS / 2)] = (a1 & 0xFFFFu) | (b1 << 16);
-        dst[3 * (XS / 2)] = (a1 >> 16) | (b1 & 0xFFFF0000u);
+        dst[8 * (XS / 2)] = (a0 >> 16) | (b0 & 0xFFFF0000u);
+        dst[16 * (XS / 2)] = (a1 & 0xFFFFu) | (b1 << 16);
+        dst[24 * (XS / 2)] = (a1 >> 16) | (b1 & 0xFFFF0000u);
       }
     } else {
 #pragma unroll
@@ -1399,7 +1419,9 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
     const int rr = row_base + 32 * rb + 8 * (v >> 2) + 4 * h + (v & 3);
     live[rb] = r < N && rr < M;
     orow[rb] = out0 + min(rr, M - 1);
-    at[rb] = static_cast<size_t>(orow[rb]) * N + min(r, N - 1);
+    // (at 32 columns row r of the chunk buffers, the B operand's column r, holds token
+    // 4 (r % 8) + r / 8)
+    at[rb] = static_cast<size_t>(orow[rb]) * N + (WIDE ? 4 * (r & 7) + (r >> 3) : min(r, N - 1));
   }
   if (partial != nullptr) {
     // this split's slab of the partials
@@ -1475,6 +1497,348 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
         o = f32_to_bf16(bf16_to_f32(res[at[rb]]) + bf16_to_f32(o));
       }
       y[at[rb]] = o;
+    }
+  }
+}
+
+// ---- the same tile for chunks of exactly 64 columns -------------------------------------------
+// Two 32-column B operands per A operand: what a wavefront looks up once multiplies 64 tokens.
+// A workgroup owns 64 rows; K is walked in chunks of 256 (four groups), multiplying wavefront
+// w takes group w % 4 of row block w / 4 and both halves of the tokens, so every weight goes
+// through the table once per workgroup and every element of x is read from LDS by two
+// wavefronts.  A row of x is then exactly one 128-byte line: eight lanes fetch it 16 bytes
+// each, the next eight the row after it, and lanes eight apart (same tokens, rows k and
+// k + 1) swap halves through a DPP rotation of their row of sixteen before they interleave.
+// The chunk buffers hold the tokens in an order that spreads those stores over the banks
+// (the B operand's column l of block cb is token 4 (l % 16) + 2 cb + l / 16).
+// Everything else -- the pair table, the scales in LDS and their DPP broadcast, the ring of
+// requests and the nested chunks, the splits of K that meet in the tile -- is gemm_stream's.
+__global__ __launch_bounds__(kStreamBlock) void gemm_stream64(GemmSegs segs,
+                                                              const uint16_t *__restrict__ x,
+                                                              uint16_t *__restrict__ y,
+                                                              float *__restrict__ partial, int M_all,
+                                                              int K, int K_pad,
+                                                              const uint16_t *__restrict__ bias,
+                                                              const uint16_t *res, int arrive_slot) {
+  constexpr int XS = kWideXS;
+  constexpr int CK = kWideChunkK;
+  constexpr int ROWS = kWideRows;
+  constexpr int N = 64;
+  constexpr uint32_t kXAddr = kStreamTableBytes;
+  constexpr uint32_t kWAddr = kXAddr + 2 * kWideXBytes;
+  constexpr uint32_t kScaleAddr = kWAddr + 2 * kWideWBytes;
+  static_assert(kScaleAddr + kWideScaleBytes == kWideLdsBytes, "LDS map");
+  static_assert(8 * 2 * 16 * 64 * 4 <= kWAddr, "the wavefronts' sums reuse the table and x");
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave16 = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const bool stager = wave16 >= 8;  // wavefronts 8..15 stage, 0..7 multiply
+  const int wave = wave16 & 7;
+  const int stid = tid & (kStreamStagers - 1);
+  int bx = static_cast<int>(blockIdx.x);
+  int seg = 0;
+  if (bx >= segs.blocks[0]) {
+    bx -= segs.blocks[0];
+    seg = 1;
+    if (bx >= segs.blocks[1]) {
+      bx -= segs.blocks[1];
+      seg = 2;
+    }
+  }
+  const uint8_t *__restrict__ packed = segs.packed[seg];
+  const uint16_t *__restrict__ scale = segs.scale[seg];
+  const int M = segs.M[seg];
+  const int out0 = segs.row0[seg];
+  const int row_base = bx * ROWS;
+  const int r = lane & 31;  // row of the A operand, token of the B operand
+  const int h = lane >> 5;  // which half of a group's k
+  // grid.y splits K by whole chunks (see gemm_stream): from here on x, K, row_bytes and groups
+  // describe what is left of K from this workgroup's first chunk on
+  const int n_ch_all = (K_pad + CK - 1) / CK;
+  const int per_split = (n_ch_all + static_cast<int>(gridDim.y) - 1) / static_cast<int>(gridDim.y);
+  const int c0 = static_cast<int>(blockIdx.y) * per_split;
+  const int n_ch = min(per_split, n_ch_all - c0);
+  const int row_stride = K_pad >> 1;
+  const int row_bytes = row_stride - c0 * (CK / 2);
+  const int groups_all = K_pad >> 6;
+  const int groups = min(4 * n_ch, groups_all - 4 * c0);
+  x += static_cast<size_t>(c0) * CK * N;
+  K -= c0 * CK;
+
+  // ---- requests: a thread's share of one chunk ------------------------------------------------
+  // w = bytes 16 (stid % 8) .. + 16 of the chunk of row stid / 8 (a row's 128 bytes of a chunk
+  // are one line); a[it] = x, row 2 kp + half of the chunk, tokens 8 q .. + 8, with kp =
+  // lane / 16 + 4 wave + 32 it, half = (lane / 8) % 2, q = lane % 8
+  struct Item {
+    uint4 a[4];
+  };
+  const uint8_t *wp = packed + static_cast<size_t>(min(row_base + (stid >> 3), M - 1)) * row_stride +
+                      c0 * (CK / 2);
+  const int w_piece = 16 * (stid & 7);
+  const int w_half = (lane >> 3) & 1;
+  const int w_q = lane & 7;
+  const int w_kp = (lane >> 4) + 4 * wave;  // + 32 it
+  auto load = [&](int c, U32x4 &w, Item &v) {
+    const int cc = min(c, n_ch - 1);
+    w = *reinterpret_cast<const U32x4 *>(wp + min(cc * (CK / 2) + w_piece, row_bytes - 16));
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+      const int k = cc * CK + 2 * (w_kp + 32 * it) + w_half;
+      v.a[it] = *reinterpret_cast<const uint4 *>(x + static_cast<size_t>(min(k, K - 1)) * N + 8 * w_q);
+    }
+  };
+  auto store = [&](int c, const U32x4 w, const Item &v) {
+    const int buf = c & 1;
+    *reinterpret_cast<U32x4 *>(lds_raw + kWAddr + buf * kWideWBytes + (stid >> 3) * kWideWStride + w_piece) = w;
+    uint32_t *xd = reinterpret_cast<uint32_t *>(lds_raw + kXAddr + buf * kWideXBytes);
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+      const int kp = w_kp + 32 * it;
+      const bool live = c * CK + 2 * kp + w_half < K;
+      const uint32_t m0 = live ? v.a[it].x : 0u, m1 = live ? v.a[it].y : 0u;
+      const uint32_t m2 = live ? v.a[it].z : 0u, m3 = live ? v.a[it].w : 0u;
+      // the even row's lane sends tokens 4..7 of its eight, the odd row's lane tokens 0..3
+      const int s0 = static_cast<int>(w_half ? m0 : m2), s1 = static_cast<int>(w_half ? m1 : m3);
+      const uint32_t g0 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, s0, 0x128, 0xF, 0xF, true));
+      const uint32_t g1 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, s1, 0x128, 0xF, 0xF, true));
+      // even row's lane: tokens 8 q .. + 4 from its own and the partner's; odd row's lane:
+      // tokens 8 q + 4 .. + 4 from the partner's and its own
+      const uint32_t a0 = w_half ? g0 : m0, a1 = w_half ? g1 : m1;
+      const uint32_t b0 = w_half ? m2 : g0, b1 = w_half ? m3 : g1;
+      // token 4 u + e lives in row 16 e + u of the chunk buffer: the sixteen lanes of a k pair
+      // (u = 2 q + half) then store into sixteen consecutive rows, 4 banks apart -- two lanes
+      // a bank, where rows in token order (sixteen rows 4 apart, 16 banks apart) put eight
+      // lanes on a bank
+      uint32_t *dst = xd + (2 * w_q + w_half) * (XS / 2) + kp;
+      dst[0] = (a0 & 0xFFFFu) | (b0 << 16);
+      dst[16 * (XS / 2)] = (a0 >> 16) | (b0 & 0xFFFF0000u);
+      dst[32 * (XS / 2)] = (a1 & 0xFFFFu) | (b1 << 16);
+      dst[48 * (XS / 2)] = (a1 >> 16) | (b1 & 0xFFFF0000u);
+    }
+  };
+
+  // ---- set-up -------------------------------------------------------------------------------
+  constexpr int kScaleLoads = (ROWS * (kWideMaxGroups / 4) + kStreamBlock - 1) / kStreamBlock;
+  const int quads = groups >> 2;
+  uint2 sv[kScaleLoads];
+#pragma unroll
+  for (int it = 0; it < kScaleLoads; ++it) {
+    const int i = min(tid + it * kStreamBlock, ROWS * quads - 1);
+    const int srow = i / quads;
+    sv[it] = *reinterpret_cast<const uint2 *>(
+        scale + static_cast<size_t>(min(row_base + srow, M - 1)) * groups_all + 4 * c0 + 4 * (i - srow * quads));
+  }
+  constexpr int R = 3;
+  Item ring[R];
+  U32x4 ring_w[R];
+  if (stager) {
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      load(j, ring_w[j], ring[j]);
+    }
+  }
+  fill_pair_table32(reinterpret_cast<uint32_t *>(lds_raw), wave16, lane);
+  {
+    uint16_t *sl = reinterpret_cast<uint16_t *>(lds_raw + kScaleAddr);  // [group][row of the block]
+#pragma unroll
+    for (int it = 0; it < kScaleLoads; ++it) {
+      const int i = tid + it * kStreamBlock;
+      if (i < ROWS * quads) {
+        const int srow = i / quads;
+        const int gq = i - srow * quads;
+        sl[(4 * gq + 0) * ROWS + srow] = static_cast<uint16_t>(sv[it].x);
+        sl[(4 * gq + 1) * ROWS + srow] = static_cast<uint16_t>(sv[it].x >> 16);
+        sl[(4 * gq + 2) * ROWS + srow] = static_cast<uint16_t>(sv[it].y);
+        sl[(4 * gq + 3) * ROWS + srow] = static_cast<uint16_t>(sv[it].y >> 16);
+      }
+    }
+  }
+  if (stager) {
+    store(0, ring_w[0], ring[0]);
+    load(R, ring_w[0], ring[0]);
+  }
+  __syncthreads();
+
+  // ---- the chunks: one barrier each, in both roles (two questions, not an else: see
+  // gemm_stream) ------------------------------------------------------------------------------
+  float *sums = reinterpret_cast<float *>(lds_raw);
+  if (stager) {
+    auto chunk = [&](auto index) {
+      constexpr int c = decltype(index)::value;
+      constexpr int j = c % R;
+      if (c + 1 < n_ch) {
+        store(c + 1, ring_w[(j + 1) % R], ring[(j + 1) % R]);
+      }
+      load(c + 1 + R, ring_w[(j + 1) % R], ring[(j + 1) % R]);
+      __syncthreads();
+    };
+    nest_chunks<0, kWideBodies>(n_ch, chunk);
+  }
+  int role;
+  asm volatile("s_mov_b32 %0, %1" : "=s"(role) : "s"(wave16));
+  if (role < 8) {
+    const int g = wave & 3;    // group of a chunk
+    const int rb = wave >> 2;  // 32-row block of the workgroup's 64 rows
+    f32x16 acc[2];
+#pragma unroll
+    for (int cb = 0; cb < 2; ++cb) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        acc[cb][v] = 0.f;
+      }
+    }
+    const uint32_t copy4 = static_cast<uint32_t>(lane & 31) << 2;
+    const uint32_t x_lane = kXAddr + static_cast<uint32_t>(r * XS + 32 * h + 64 * g) * 2;
+    const uint32_t w_lane =
+        kWAddr + static_cast<uint32_t>((32 * rb + r) * kWideWStride + 32 * g + 16 * h);
+    const uint32_t s_lane =
+        kScaleAddr +
+        static_cast<uint32_t>(g * ROWS + 32 * rb + 8 * ((lane & 15) >> 2) + 4 * h + (lane & 3)) * 2;
+    for (int c = 0; c < n_ch; ++c) {
+      const uint32_t buf = static_cast<uint32_t>(c & 1);
+      const int grp = min(4 * c + g, groups - 1) - g;
+      const float mine = f16_to_f32(*reinterpret_cast<const __attribute__((address_space(3))) uint16_t *>(
+          s_lane + static_cast<uint32_t>(grp * ROWS * 2)));
+      const uint4 wv = lds0_u128(w_lane + buf * kWideWBytes);
+      const uint32_t w4[4] = {wv.x, wv.y, wv.z, wv.w};
+      const uint32_t xl = x_lane + buf * kWideXBytes;
+      f32x16 t[2];
+#pragma unroll
+      for (int cb = 0; cb < 2; ++cb) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          t[cb][v] = 0.f;
+        }
+      }
+#pragma unroll
+      for (int jj = 0; jj < 4; ++jj) {
+        const uint32_t w = w4[jj];
+        const uint4 a = make_uint4(pair32_at<0>(w, copy4), pair32_at<1>(w, copy4), pair32_at<2>(w, copy4),
+                                   pair32_at<3>(w, copy4));
+#pragma unroll
+        for (int cb = 0; cb < 2; ++cb) {
+          const uint4 b = lds0_u128(xl + static_cast<uint32_t>(cb * 32 * XS * 2) + 16 * jj);
+          t[cb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                          __builtin_bit_cast(bf16x8, b), t[cb], 0, 0, 0);
+        }
+      }
+#pragma unroll
+      for (int cb = 0; cb < 2; ++cb) {
+        acc[cb][0] = scale_into<0>(acc[cb][0], mine, t[cb][0]);
+        acc[cb][1] = scale_into<1>(acc[cb][1], mine, t[cb][1]);
+        acc[cb][2] = scale_into<2>(acc[cb][2], mine, t[cb][2]);
+        acc[cb][3] = scale_into<3>(acc[cb][3], mine, t[cb][3]);
+        acc[cb][4] = scale_into<4>(acc[cb][4], mine, t[cb][4]);
+        acc[cb][5] = scale_into<5>(acc[cb][5], mine, t[cb][5]);
+        acc[cb][6] = scale_into<6>(acc[cb][6], mine, t[cb][6]);
+        acc[cb][7] = scale_into<7>(acc[cb][7], mine, t[cb][7]);
+        acc[cb][8] = scale_into<8>(acc[cb][8], mine, t[cb][8]);
+        acc[cb][9] = scale_into<9>(acc[cb][9], mine, t[cb][9]);
+        acc[cb][10] = scale_into<10>(acc[cb][10], mine, t[cb][10]);
+        acc[cb][11] = scale_into<11>(acc[cb][11], mine, t[cb][11]);
+        acc[cb][12] = scale_into<12>(acc[cb][12], mine, t[cb][12]);
+        acc[cb][13] = scale_into<13>(acc[cb][13], mine, t[cb][13]);
+        acc[cb][14] = scale_into<14>(acc[cb][14], mine, t[cb][14]);
+        acc[cb][15] = scale_into<15>(acc[cb][15], mine, t[cb][15]);
+      }
+      __syncthreads();
+    }
+    // the four sums of every output (one per group of a chunk) meet in LDS
+#pragma unroll
+    for (int cb = 0; cb < 2; ++cb) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        sums[((cb * 8 + wave) * 16 + v) * kWave + lane] = acc[cb][v];
+      }
+    }
+  }
+  __syncthreads();
+  // wavefront w of the sixteen finishes accumulator value w of both row blocks and both
+  // halves of the tokens
+  float o32[4];
+  size_t at[4];
+  bool live[4];
+  int orow[4];
+#pragma unroll
+  for (int o = 0; o < 4; ++o) {
+    const int rb = o >> 1, cb = o & 1, v = wave16;
+    o32[o] = 0.f;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      o32[o] += sums[((cb * 8 + 4 * rb + g) * 16 + v) * kWave + lane];
+    }
+    const int rr = row_base + 32 * rb + 8 * (v >> 2) + 4 * h + (v & 3);
+    live[o] = rr < M;
+    orow[o] = out0 + min(rr, M - 1);
+    // (row 32 cb + r of the chunk buffers holds token 4 (r % 16) + 2 cb + r / 16)
+    at[o] = static_cast<size_t>(orow[o]) * N + 4 * (r & 15) + 2 * cb + (r >> 4);
+  }
+  if (partial != nullptr) {
+    const size_t slab = static_cast<size_t>(M_all) * N;
+    if (arrive_slot < 0) {
+#pragma unroll
+      for (int o = 0; o < 4; ++o) {
+        if (live[o]) {
+          partial[blockIdx.y * slab + at[o]] = o32[o];
+        }
+      }
+      return;  // a reduce kernel adds the slabs up
+    }
+    // the splits meet here: see gemm_stream
+#pragma unroll
+    for (int o = 0; o < 4; ++o) {
+      if (live[o]) {
+        __hip_atomic_store(partial + blockIdx.y * slab + at[o], o32[o], __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    int *last = reinterpret_cast<int *>(lds_raw + kScaleAddr);  // (the scales are done with)
+    if (tid == 0) {
+      unsigned int *count = &stream_arrivals[arrive_slot][blockIdx.x];
+      const unsigned int before =
+          __hip_atomic_fetch_add(count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const bool all_in = before + 1 == gridDim.y;
+      if (all_in) {
+        __hip_atomic_store(count, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      *last = all_in ? 1 : 0;
+    }
+    __syncthreads();
+    if (*last == 0) {
+      return;
+    }
+#pragma unroll
+    for (int o = 0; o < 4; ++o) {
+      float sum = 0.f;
+      for (unsigned int j0 = 0; j0 < gridDim.y; j0 += 4) {
+        float v[4];
+#pragma unroll
+        for (unsigned int u = 0; u < 4; ++u) {
+          v[u] = __hip_atomic_load(partial + min(j0 + u, gridDim.y - 1) * slab + at[o], __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+        }
+#pragma unroll
+        for (unsigned int u = 0; u < 4; ++u) {
+          sum = j0 + u == 0 ? v[0] : (j0 + u < gridDim.y ? sum + v[u] : sum);
+        }
+      }
+      o32[o] = sum;
+    }
+  }
+#pragma unroll
+  for (int o = 0; o < 4; ++o) {
+    if (live[o]) {
+      uint16_t out = f32_to_bf16(o32[o]);
+      if (bias != nullptr) {
+        out = f32_to_bf16(bf16_to_f32(out) + bf16_to_f32(bias[orow[o]]));
+      }
+      if (res != nullptr) {
+        out = f32_to_bf16(bf16_to_f32(res[at[o]]) + bf16_to_f32(out));
+      }
+      y[at[o]] = out;
     }
   }
 }
@@ -1708,7 +2072,8 @@ int gemm_lds_ready() {
         return -6;
       }
     }
-    const std::pair<const void *, int> streams[6] = {
+    const std::pair<const void *, int> streams[7] = {
+        {reinterpret_cast<const void *>(gemm_stream64), kWideLdsBytes},
         {reinterpret_cast<const void *>(gemm_stream<1, 1>), stream_lds_bytes(1)},
         {reinterpret_cast<const void *>(gemm_stream<2, 1>), stream_lds_bytes(1)},
         {reinterpret_cast<const void *>(gemm_stream<4, 1>), stream_lds_bytes(1)},
@@ -1833,7 +2198,7 @@ StackPlan plan_stack(const chr_nf4_dev_t *h, int nseg, int N, int have_ws, bool 
   sp.n_ktiles = ceil_div(h[0].K_pad, kBK);
   if (sp.stream) {
     sp.grid_y = stp.split;
-    sp.tiles_per_split = std::min(2 * stp.chunks, sp.n_ktiles);
+    sp.tiles_per_split = N == 64 ? stp.chunks : std::min(2 * stp.chunks, sp.n_ktiles);
     sp.ws_floats = sp.grid_y > 1 ? static_cast<int64_t>(sp.grid_y) * sp.M_all * N : 0;
     return sp;
   }
@@ -1930,6 +2295,9 @@ int gemm_launch(const chr_nf4_dev_t *const *w, int nseg, const void *x, void *y,
       gemm_stream<2, 1><<<grid, dim3(kStreamBlock), stream_lds_bytes(1), st>>>(
           sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp, slot);
     }
+  } else if (sp.stream == 2 && N == 64) {
+    gemm_stream64<<<grid, dim3(kStreamBlock), kWideLdsBytes, st>>>(sp.segs, xp, yp, partial, sp.M_all, K,
+                                                                    K_pad, bp, rp, slot);
   } else if (sp.stream == 2) {
     if (N <= 16) {
       gemm_stream<1, 2><<<grid, dim3(kStreamBlock), stream_lds_bytes(2), st>>>(

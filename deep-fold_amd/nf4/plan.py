@@ -212,6 +212,11 @@ def stream_lds_bytes(row_blocks: int) -> int:
     return 256 * 32 * 4 + 2 * 32 * 520 * 2 + 2 * rows * 272 + _STREAM_MAX_GROUPS * rows * 2
 
 
+#: LDS of the 64-column form: the pair table, two chunks of x (64 token rows of 256 + 8), two
+#: chunks of weights (64 rows of 128 + 16 bytes), the scales of 64 rows and 80 groups
+_STREAM_LDS_64 = 256 * 32 * 4 + 2 * 64 * 264 * 2 + 2 * 64 * 144 + 80 * 64 * 2
+
+
 def _env_int_once(name: str, dflt: int) -> int:
     raw = os.environ.get(name, "")
     try:
@@ -232,8 +237,8 @@ def stream_policy_default() -> int:
 
 
 def _stream_columns(N: int, policy: int) -> bool:  # noqa: N803
-    """Chunk widths the stream tile takes (8, 16, 24, 32)."""
-    return policy >= 0 and 8 <= N <= 32 and N % 8 == 0
+    """Chunk widths the stream tile takes (8, 16, 24, 32, and 64 in a form of its own)."""
+    return policy >= 0 and ((8 <= N <= 32 and N % 8 == 0) or N == 64)
 
 
 _STREAM_SPLITS: bool | None = None
@@ -241,6 +246,7 @@ _STREAM_SPLITS: bool | None = None
 #: rows, a 512-wide chunk at 8 / 16 / 24 / 32 columns, the meeting of a split's partials
 _STREAM_FIXED = (520, 650)
 _STREAM_CHUNK = ((55, 67, 86, 106), (100, 106, 122, 138))
+_STREAM_CHUNK_64 = 110      # a 256-wide chunk of the 64-column form (64 rows a workgroup)
 _STREAM_MEET = 230
 _STREAM_MAX_SPLIT = 8
 _STREAM_MIN_CODES = 1 << 24
@@ -255,7 +261,8 @@ def gemm_streams(M, N: int, k_pad_: int, force_split: int = 0,  # noqa: N803
     (``row_blocks`` 1 or 2) and ``chunks`` 512-wide chunks of K; ``split`` workgroups share a
     row block's K and the last of them to finish adds up their fp32 partials (no reduce
     launch); pair-table lookups, the scale applied per 64-wide group.  It takes whole-vector
-    chunks of up to 32 columns, no forced split, ``K_pad`` a multiple of 256, at most 12
+    chunks of up to 32 columns (and, with 64 rows and 256-wide chunks, at most 20 of them a
+    workgroup, chunks of exactly 64), no forced split, ``K_pad`` a multiple of 256, at most 12
     chunks a workgroup, splits only when all workgroups run at once and there is a workspace,
     at most 8 splits, at most two rounds of workgroups (two only with 8 chunks or more) --
     and of the forms that fit, the cheapest by the cost model above (a split has to win by
@@ -275,22 +282,25 @@ def gemm_streams(M, N: int, k_pad_: int, force_split: int = 0,  # noqa: N803
     if not (_stream_columns(N, policy) and force_split <= 0 and kp % _BK == 0):
         return best
     cus = int(one_wave)
-    n_ch = _ceil_div(kp, 512)
-    for rb in (1, 2):
+    wide = N == 64              # 64 rows and chunks of 256 only, at most 20 a workgroup
+    chunk_k, bodies = (256, 20) if wide else (512, 12)
+    n_ch = _ceil_div(kp, chunk_k)
+    for rb in ((2,) if wide else (1, 2)):
         if _STREAM_ONLY not in (0, _STREAM_ROWS * rb):
             continue
         blocks = sum(_ceil_div(m, _STREAM_ROWS * rb) for m in rows)
         for split in range(1, min(n_ch, _STREAM_MAX_SPLIT) + 1):
             chunks = _ceil_div(n_ch, split)
-            if _ceil_div(n_ch, chunks) != split or chunks > 12:
+            if _ceil_div(n_ch, chunks) != split or chunks > bodies:
                 continue
             rounds = _ceil_div(blocks * split, cus)
             if rounds > 2 or (split > 1 and (rounds > 1 or not _STREAM_SPLITS or not have_ws
                                              or blocks > _ARRIVE_BLOCKS)):
                 continue
-            if rounds == 2 and chunks < 8:
+            if rounds == 2 and chunks * chunk_k < 8 * 512:
                 continue
-            cost = rounds * (_STREAM_FIXED[rb - 1] + chunks * _STREAM_CHUNK[rb - 1][N // 8 - 1])
+            per_chunk = _STREAM_CHUNK_64 if wide else _STREAM_CHUNK[rb - 1][N // 8 - 1]
+            cost = rounds * (_STREAM_FIXED[rb - 1] + chunks * per_chunk)
             if split > 1:
                 cost += _STREAM_MEET
                 cost += cost // 32
@@ -364,8 +374,10 @@ def plan(M: int, K: int, N: int = 1, *, K_pad: int | None = None, have_ws: bool 
     if row_blocks:
         bm = _STREAM_ROWS * row_blocks
         grid_x = _ceil_div(M, bm)
-        return Plan(path, grid_x, split, 1024, bm, _BK, n_ktiles, min(2 * chunks, n_ktiles),
-                    grid_x * split, stream_lds_bytes(row_blocks), split * M * N if split > 1 else 0)
+        tps = chunks if N == 64 else min(2 * chunks, n_ktiles)
+        lds = _STREAM_LDS_64 if N == 64 else stream_lds_bytes(row_blocks)
+        return Plan(path, grid_x, split, 1024, bm, _BK, n_ktiles, tps, grid_x * split, lds,
+                    split * M * N if split > 1 else 0)
     split, tps = _pick_split(grid_x, n_ktiles, N, have_ws, force_split, one_wave)
     ws = split * M * N if split > 1 else 0
     if gemm_streams_rows(N, tps):

@@ -613,6 +613,10 @@ STREAM_CASES = [
     # K split over workgroups that meet in the tile: 5 to 8, 3 and 2 splits
     (256, 5120, 32), (1024, 5120, 8), (5120, 13824, 8), (5120, 5120, 32), (3072, 8192, 16),
     (5000, 13560, 16),                               # ragged rows, K below K_pad, a last chunk of 256
+    # 64 columns: 64 rows a workgroup, chunks of 256
+    (64, 256, 64), (100, 2304, 64), (130, 1000, 64),  # one chunk; ragged rows; K below K_pad
+    (200, 5120, 64), (70, 10240, 64),                 # twenty chunks; splits of twenty
+    (5120, 5120, 64), (7168, 5120, 64), (13824, 5120, 64), (5120, 13824, 64),
 ]
 
 
@@ -642,19 +646,24 @@ def _stream_tile_case(m, k, n, p, s, dp, ds, xh, x, kp):
     bm, split = plan["bm"], plan["grid_y"]
     assert bm in (32, 64) and plan["block"] == 1024 and plan["grid_x"] == -(-m // bm)
     assert plan["ws_floats"] == (split * m * n if split > 1 else 0)
-    assert -(-kp // 512) <= split * 12 and (split == 1 or plan["ctas"] <= 256)
-    assert plan["smem_bytes"] == 32768 + 2 * 33280 + 2 * bm * 272 + 96 * bm * 2
-    y = nf4.nf4_gemm(dp, ds, x, m, k, kp)
+    assert split == 1 or plan["ctas"] <= 256
+    if n == 64:
+        assert bm == 64 and -(-kp // 256) <= split * 20
+        assert plan["smem_bytes"] == 32768 + 2 * 64 * 264 * 2 + 2 * 64 * 144 + 80 * 64 * 2
+    else:
+        assert -(-kp // 512) <= split * 12
+        assert plan["smem_bytes"] == 32768 + 2 * 33280 + 2 * bm * 272 + 96 * bm * 2
+    y = nf4.nf4_gemm(dp, ds, x, m, k, kp, 64)
     check_linear(y, staged_gemv_model(p, s, m, k, xh, terms=1), what=f"stream {m}x{k} n{n}")
     ref = oc.c_matmul_f64(oc.c_decode(p, s, m, k), xh)
     err = np.abs(to_f32(y).astype(np.float64) - ref)
     assert (err <= np.maximum(0.05, 2 ** (np.floor(np.log2(np.maximum(np.abs(ref), 1e-30))) - 8))).all()
-    assert (bf16_bits(nf4.nf4_gemm(dp, ds, x, m, k, kp)) == bf16_bits(y)).all()
+    assert (bf16_bits(nf4.nf4_gemm(dp, ds, x, m, k, kp, 64)) == bf16_bits(y)).all()
     rng = np.random.default_rng(m + n)
     bias = bf16_tensor(oc.bf16_round(rng.standard_normal(m).astype(np.float32)))
     res = bf16_tensor(oc.bf16_round(rng.standard_normal((m, n)).astype(np.float32)))
     want = res + (y + bias[:, None])
-    got = nf4.nf4_gemm(dp, ds, x, m, k, kp, bias=bias, residual=res)
+    got = nf4.nf4_gemm(dp, ds, x, m, k, kp, 64, bias=bias, residual=res)
     assert (bf16_bits(got) == bf16_bits(want)).all()
 
 

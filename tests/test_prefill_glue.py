@@ -264,10 +264,10 @@ def test_wide_chunk_equals_two_narrow_ones(m, k, n):
     first = min(32, n - 2)  # at least two columns: one alone would go to the GEMV
     hi = nf4.nf4_gemm(dp, ds, x[:, first:].contiguous(), m, k, kp)
     assert tuple(wide.shape) == (m, n)
-    # the same split by the same kernel (block size and rows per block tell the tiles apart;
-    # chunks of 8, 16, 24 or 32 columns run the stream tile, which rounds weights differently)
+    # the same split by the same kernel (block size, rows per block and LDS bytes tell the
+    # tiles and their forms apart)
     plans = [nf4.nf4_plan(m, k, c) for c in (n, 32, n - first)]
-    same_split = len({(q["grid_y"], q["block"], q["bm"]) for q in plans}) == 1
+    same_split = len({(q["grid_y"], q["block"], q["bm"], q["smem_bytes"]) for q in plans}) == 1
     for got, want_ in ((wide[:, :32].contiguous(), lo), (wide[:, first:].contiguous(), hi.view(m, n - first))):
         if same_split:  # same K order, same partial sums: the same bits
             assert (bf16_bits(got) == bf16_bits(want_)).all()
