@@ -290,6 +290,9 @@ StreamPlan stream_plan(int N, int K_pad, int blocks32, int blocks64, int have_ws
   if (codes <= kStreamMinCodes && only == 0 && stream_policy().load(std::memory_order_relaxed) == 0) {
     best.rb = 0;
   }
+  if (codes >= (int64_t{1} << 33)) {
+    best.rb = 0;  // (the tile addresses a matrix's packed bytes with 32-bit offsets)
+  }
   return best;
 }
 
@@ -1031,11 +1034,39 @@ __device__ __forceinline__ void nest_chunks(int n, F &f) {
   }
 }
 
-// acc += (position V of this lane's row of sixteen lanes of `mine`) * t
+// acc += (position V of this lane's row of sixteen lanes of `mine`) * t, as one instruction
+// (the compiler keeps the broadcast and the multiply-add apart)
 template <int V>
 __device__ __forceinline__ float scale_into(float acc, float mine, float t) {
-  const int s = __builtin_amdgcn_update_dpp(0, __float_as_int(mine), 0x150 + V, 0xF, 0xF, true);
-  return fmaf(__int_as_float(s), t, acc);
+  asm("v_fmac_f32_dpp %0, %1, %2 row_newbcast:%3 row_mask:0xf bank_mask:0xf"
+      : "+v"(acc)
+      : "v"(mine), "v"(t), "n"(V));
+  return acc;
+}
+
+// The matrix core's result registers may be read by hand-written instructions only after it
+// has finished writing them (up to 18 wait states after the last MFMA was issued); the
+// compiler counts those for its own instructions, not for what an asm statement reads.  This
+// stands between the MFMAs that write t and the scale_into statements that read it.
+__device__ __forceinline__ void mfma_results_settled(f32x16 &t) {
+  asm volatile("s_nop 15\n\ts_nop 7" : "+v"(t));
+}
+
+// The low halves of a and b as one dword, a below b; the high halves likewise: a byte
+// permute each.
+__device__ __forceinline__ uint32_t low_halves(uint32_t a, uint32_t b) {
+  return __builtin_amdgcn_perm(b, a, 0x05040100u);
+}
+__device__ __forceinline__ uint32_t high_halves(uint32_t a, uint32_t b) {
+  return __builtin_amdgcn_perm(b, a, 0x07060302u);
+}
+
+// `own` in the lanes of the banks (fours of a row of sixteen lanes) that MASK leaves out, what
+// the DPP pattern CTRL brings of `other` in the rest.
+template <int CTRL, int MASK>
+__device__ __forceinline__ uint32_t dpp_into(uint32_t own, uint32_t other) {
+  return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(static_cast<int>(own), static_cast<int>(other),
+                                                           CTRL, 0xF, MASK, false));
 }
 
 // Row of a chunk buffer that holds token n.  A staging instruction of 17..32 columns stores
@@ -1132,12 +1163,6 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
   struct Item {
     uint4 a[NA], b[NB > 0 ? NB : 1];
   };
-  const uint8_t *wp[RB];
-#pragma unroll
-  for (int rb = 0; rb < RB; ++rb) {
-    wp[rb] = packed + static_cast<size_t>(min(row_base + 32 * rb + (stid >> 4), M - 1)) * row_stride +
-             c0 * (CK / 2);
-  }
   const int w_piece = 16 * (stid & 15);
   const int nv = N >> 3;
   const int n_items = (CK / 2) * nv;
@@ -1152,25 +1177,35 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
   const int w_half = (lane >> 2) & 1;
   const int w_q = w_half ? 7 - (lane & 7) : (lane & 7);
   const int w_kp = (lane >> 3) + 8 * wave;  // + 64 it
+  // Requests take a base that is the same in every lane (it moves from chunk to chunk on the
+  // scalar side) and a 32-bit offset of the lane: what does not depend on the chunk is in
+  // registers, and a request costs the clamp that keeps the tail of K inside x and the row.
+  uint32_t w_off[RB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    w_off[rb] = static_cast<uint32_t>(min(row_base + 32 * rb + (stid >> 4), M - 1)) * row_stride + c0 * (CK / 2);
+  }
+  const uint32_t x_row = 2u * N;  // bytes of a row of x
+  uint32_t xk_off[NA], xq_off[NA];
+#pragma unroll
+  for (int it = 0; it < NA; ++it) {
+    xk_off[it] = WIDE ? (2 * (w_kp + 64 * it) + w_half) * x_row : 2 * xkp[it] * x_row;
+    xq_off[it] = 16u * (WIDE ? w_q : xq[it]);
+  }
   auto load = [&](int c, U32x4 &w0, U32x4 &w1, Item &v) {
     const int cc = min(c, n_ch - 1);
+    const uint32_t w_at = min(static_cast<uint32_t>(cc * (CK / 2) + w_piece), static_cast<uint32_t>(row_bytes - 16));
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
-      (rb ? w1 : w0) = *reinterpret_cast<const U32x4 *>(wp[rb] + min(cc * (CK / 2) + w_piece, row_bytes - 16));
+      (rb ? w1 : w0) = *reinterpret_cast<const U32x4 *>(packed + (w_off[rb] + w_at));
     }
-    if constexpr (WIDE) {
+    const unsigned char *xb = reinterpret_cast<const unsigned char *>(x) + static_cast<size_t>(cc) * CK * x_row;
+    const uint32_t k_last = static_cast<uint32_t>(K - 1 - cc * CK) * x_row;  // offset of the last row of x
 #pragma unroll
-      for (int it = 0; it < 4; ++it) {
-        const int k = cc * CK + 2 * (w_kp + 64 * it) + w_half;
-        v.a[it] = *reinterpret_cast<const uint4 *>(x + static_cast<size_t>(min(k, K - 1)) * 32 + 8 * w_q);
-      }
-    } else {
-#pragma unroll
-      for (int it = 0; it < NB; ++it) {
-        const int k = cc * CK + 2 * xkp[it];
-        v.a[it] = *reinterpret_cast<const uint4 *>(x + static_cast<size_t>(min(k, K - 1)) * N + 8 * xq[it]);
-        v.b[it] =
-            *reinterpret_cast<const uint4 *>(x + static_cast<size_t>(min(k + 1, K - 1)) * N + 8 * xq[it]);
+    for (int it = 0; it < NA; ++it) {
+      v.a[it] = *reinterpret_cast<const uint4 *>(xb + (min(xk_off[it], k_last) + xq_off[it]));
+      if constexpr (!WIDE) {
+        v.b[it] = *reinterpret_cast<const uint4 *>(xb + (min(xk_off[it] + x_row, k_last) + xq_off[it]));
       }
     }
   };
@@ -1184,49 +1219,61 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
                                  w_piece) = rb ? w1 : w0;
     }
     uint32_t *xd = reinterpret_cast<uint32_t *>(lds_raw + kXAddr + buf * kStreamXBytes);
+    const bool tail = (c + 1) * CK > K;  // only the chunk at the end of K has rows of x to blank
     if constexpr (WIDE) {
 #pragma unroll
       for (int it = 0; it < 4; ++it) {
         const int kp = w_kp + 64 * it;
-        const bool live = c * CK + 2 * kp + w_half < K;
-        const uint32_t m0 = live ? v.a[it].x : 0u, m1 = live ? v.a[it].y : 0u;
-        const uint32_t m2 = live ? v.a[it].z : 0u, m3 = live ? v.a[it].w : 0u;
-        // the even row's lane sends columns 4..7, the odd row's lane columns 0..3
-        const int s0 = static_cast<int>(w_half ? m0 : m2), s1 = static_cast<int>(w_half ? m1 : m3);
-        const uint32_t g0 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, s0, 0x141, 0xF, 0xF, true));
-        const uint32_t g1 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, s1, 0x141, 0xF, 0xF, true));
-        // even row's lane: tokens 8 q .. + 4 from its columns 0..3 and the partner's; odd
-        // row's lane: tokens 8 q + 4 .. + 4 from the partner's columns 4..7 and its own
-        const uint32_t a0 = w_half ? g0 : m0, a1 = w_half ? g1 : m1;
-        const uint32_t b0 = w_half ? m2 : g0, b1 = w_half ? m3 : g1;
+        uint32_t m0 = v.a[it].x, m1 = v.a[it].y, m2 = v.a[it].z, m3 = v.a[it].w;
+        if (tail) {
+          asm volatile("" ::: "memory");  // (a branch, not four selects in every chunk)
+          const bool live = c * CK + 2 * kp + w_half < K;
+          m0 = live ? m0 : 0u;
+          m1 = live ? m1 : 0u;
+          m2 = live ? m2 : 0u;
+          m3 = live ? m3 : 0u;
+        }
+        // Lanes 0..3 of eight hold the even row of a k pair, lanes 4..7 the odd one, mirrored:
+        // partners hold the same eight tokens.  The even row's lane makes tokens 8 q .. + 4
+        // (a = its own tokens 0..3, b = the partner's), the odd row's lane tokens 8 q + 4 ..
+        // + 4 (a = the partner's tokens 4..7, b = its own): the half-row mirror brings the
+        // partner's dwords into the lanes of banks 1 and 3 (odd rows), or 0 and 2.
+        const uint32_t a0 = dpp_into<0x141, 0xA>(m0, m2), a1 = dpp_into<0x141, 0xA>(m1, m3);
+        const uint32_t b0 = dpp_into<0x141, 0x5>(m2, m0), b1 = dpp_into<0x141, 0x5>(m3, m1);
         // token 4 u + e lives in row 8 e + u of the chunk buffer: the eight lanes of a k pair
         // (u = 2 q + half) store into eight consecutive rows, 4 banks apart, and the four k
         // pairs of 32 lanes fill the banks between -- no two lanes on a bank, where rows in
         // token order (eight rows 4 apart, 16 banks apart) put four there
         uint32_t *dst = xd + (2 * w_q + w_half) * (XS / 2) + kp;
-        dst[0] = (a0 & 0xFFFFu) | (b0 << 16);
-        dst[8 * (XS / 2)] = (a0 >> 16) | (b0 & 0xFFFF0000u);
-        dst[16 * (XS / 2)] = (a1 & 0xFFFFu) | (b1 << 16);
-        dst[24 * (XS / 2)] = (a1 >> 16) | (b1 & 0xFFFF0000u);
+        dst[0] = low_halves(a0, b0);
+        dst[8 * (XS / 2)] = high_halves(a0, b0);
+        dst[16 * (XS / 2)] = low_halves(a1, b1);
+        dst[24 * (XS / 2)] = high_halves(a1, b1);
       }
     } else {
 #pragma unroll
-    for (int it = 0; it < NB; ++it) {
-      if (stid + it * kStreamStagers < n_items) {
-        const int k = c * CK + 2 * xkp[it];
-        const bool ka = k < K, kb = k + 1 < K;
-        const uint32_t a[4] = {ka ? v.a[it].x : 0u, ka ? v.a[it].y : 0u, ka ? v.a[it].z : 0u,
-                               ka ? v.a[it].w : 0u};
-        const uint32_t b[4] = {kb ? v.b[it].x : 0u, kb ? v.b[it].y : 0u, kb ? v.b[it].z : 0u,
-                               kb ? v.b[it].w : 0u};
-        uint32_t *dst = xd + xkp[it];
+      for (int it = 0; it < NB; ++it) {
+        if (stid + it * kStreamStagers < n_items) {
+          uint32_t a[4] = {v.a[it].x, v.a[it].y, v.a[it].z, v.a[it].w};
+          uint32_t b[4] = {v.b[it].x, v.b[it].y, v.b[it].z, v.b[it].w};
+          if (tail) {
+            asm volatile("" ::: "memory");  // (a branch, not eight selects in every chunk)
+            const int k = c * CK + 2 * xkp[it];
+            const bool ka = k < K, kb = k + 1 < K;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          dst[stream_token_row<XI>(8 * xq[it] + 2 * e) * (XS / 2)] = (a[e] & 0xFFFFu) | (b[e] << 16);
-          dst[stream_token_row<XI>(8 * xq[it] + 2 * e + 1) * (XS / 2)] = (a[e] >> 16) | (b[e] & 0xFFFF0000u);
+            for (int e = 0; e < 4; ++e) {
+              a[e] = ka ? a[e] : 0u;
+              b[e] = kb ? b[e] : 0u;
+            }
+          }
+          uint32_t *dst = xd + xkp[it];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            dst[stream_token_row<XI>(8 * xq[it] + 2 * e) * (XS / 2)] = low_halves(a[e], b[e]);
+            dst[stream_token_row<XI>(8 * xq[it] + 2 * e + 1) * (XS / 2)] = high_halves(a[e], b[e]);
+          }
         }
       }
-    }
     }
   };
 
@@ -1373,6 +1420,7 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
       }
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
+        mfma_results_settled(t[rb]);
         acc[rb][0] = scale_into<0>(acc[rb][0], mine[rb], t[rb][0]);
         acc[rb][1] = scale_into<1>(acc[rb][1], mine[rb], t[rb][1]);
         acc[rb][2] = scale_into<2>(acc[rb][2], mine[rb], t[rb][2]);
@@ -1573,48 +1621,64 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream64(GemmSegs segs,
   struct Item {
     uint4 a[4];
   };
-  const uint8_t *wp = packed + static_cast<size_t>(min(row_base + (stid >> 3), M - 1)) * row_stride +
-                      c0 * (CK / 2);
   const int w_piece = 16 * (stid & 7);
+  // (a base that is the same in every lane and a 32-bit offset of the lane: see gemm_stream)
+  const uint32_t w_off =
+      static_cast<uint32_t>(min(row_base + (stid >> 3), M - 1)) * row_stride + c0 * (CK / 2);
   const int w_half = (lane >> 3) & 1;
   const int w_q = lane & 7;
   const int w_kp = (lane >> 4) + 4 * wave;  // + 32 it
+  constexpr uint32_t x_row = 2u * N;  // bytes of a row of x
+  uint32_t xk_off[4];
+#pragma unroll
+  for (int it = 0; it < 4; ++it) {
+    xk_off[it] = (2 * (w_kp + 32 * it) + w_half) * x_row;
+  }
+  const uint32_t xq_off = 16u * w_q;
   auto load = [&](int c, U32x4 &w, Item &v) {
     const int cc = min(c, n_ch - 1);
-    w = *reinterpret_cast<const U32x4 *>(wp + min(cc * (CK / 2) + w_piece, row_bytes - 16));
+    const uint32_t w_at = min(static_cast<uint32_t>(cc * (CK / 2) + w_piece), static_cast<uint32_t>(row_bytes - 16));
+    w = *reinterpret_cast<const U32x4 *>(packed + (w_off + w_at));
+    const unsigned char *xb = reinterpret_cast<const unsigned char *>(x) + static_cast<size_t>(cc) * CK * x_row;
+    const uint32_t k_last = static_cast<uint32_t>(K - 1 - cc * CK) * x_row;  // offset of the last row of x
 #pragma unroll
     for (int it = 0; it < 4; ++it) {
-      const int k = cc * CK + 2 * (w_kp + 32 * it) + w_half;
-      v.a[it] = *reinterpret_cast<const uint4 *>(x + static_cast<size_t>(min(k, K - 1)) * N + 8 * w_q);
+      v.a[it] = *reinterpret_cast<const uint4 *>(xb + (min(xk_off[it], k_last) + xq_off));
     }
   };
   auto store = [&](int c, const U32x4 w, const Item &v) {
     const int buf = c & 1;
     *reinterpret_cast<U32x4 *>(lds_raw + kWAddr + buf * kWideWBytes + (stid >> 3) * kWideWStride + w_piece) = w;
     uint32_t *xd = reinterpret_cast<uint32_t *>(lds_raw + kXAddr + buf * kWideXBytes);
+    const bool tail = (c + 1) * CK > K;  // only the chunk at the end of K has rows of x to blank
 #pragma unroll
     for (int it = 0; it < 4; ++it) {
       const int kp = w_kp + 32 * it;
-      const bool live = c * CK + 2 * kp + w_half < K;
-      const uint32_t m0 = live ? v.a[it].x : 0u, m1 = live ? v.a[it].y : 0u;
-      const uint32_t m2 = live ? v.a[it].z : 0u, m3 = live ? v.a[it].w : 0u;
-      // the even row's lane sends tokens 4..7 of its eight, the odd row's lane tokens 0..3
-      const int s0 = static_cast<int>(w_half ? m0 : m2), s1 = static_cast<int>(w_half ? m1 : m3);
-      const uint32_t g0 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, s0, 0x128, 0xF, 0xF, true));
-      const uint32_t g1 = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, s1, 0x128, 0xF, 0xF, true));
-      // even row's lane: tokens 8 q .. + 4 from its own and the partner's; odd row's lane:
-      // tokens 8 q + 4 .. + 4 from the partner's and its own
-      const uint32_t a0 = w_half ? g0 : m0, a1 = w_half ? g1 : m1;
-      const uint32_t b0 = w_half ? m2 : g0, b1 = w_half ? m3 : g1;
+      uint32_t m0 = v.a[it].x, m1 = v.a[it].y, m2 = v.a[it].z, m3 = v.a[it].w;
+      if (tail) {
+        asm volatile("" ::: "memory");  // (a branch, not four selects in every chunk)
+        const bool live = c * CK + 2 * kp + w_half < K;
+        m0 = live ? m0 : 0u;
+        m1 = live ? m1 : 0u;
+        m2 = live ? m2 : 0u;
+        m3 = live ? m3 : 0u;
+      }
+      // Lanes 0..7 of sixteen hold the even row of a k pair, lanes 8..15 the odd one, the same
+      // tokens eight lanes apart.  The even row's lane makes tokens 8 q .. + 4 (a = its own
+      // tokens 0..3, b = the partner's), the odd row's lane tokens 8 q + 4 .. + 4 (a = the
+      // partner's tokens 4..7, b = its own): a rotation by eight brings the partner's dwords
+      // into the lanes of banks 2 and 3 (odd rows), or 0 and 1.
+      const uint32_t a0 = dpp_into<0x128, 0xC>(m0, m2), a1 = dpp_into<0x128, 0xC>(m1, m3);
+      const uint32_t b0 = dpp_into<0x128, 0x3>(m2, m0), b1 = dpp_into<0x128, 0x3>(m3, m1);
       // token 4 u + e lives in row 16 e + u of the chunk buffer: the sixteen lanes of a k pair
       // (u = 2 q + half) then store into sixteen consecutive rows, 4 banks apart -- two lanes
       // a bank, where rows in token order (sixteen rows 4 apart, 16 banks apart) put eight
       // lanes on a bank
       uint32_t *dst = xd + (2 * w_q + w_half) * (XS / 2) + kp;
-      dst[0] = (a0 & 0xFFFFu) | (b0 << 16);
-      dst[16 * (XS / 2)] = (a0 >> 16) | (b0 & 0xFFFF0000u);
-      dst[32 * (XS / 2)] = (a1 & 0xFFFFu) | (b1 << 16);
-      dst[48 * (XS / 2)] = (a1 >> 16) | (b1 & 0xFFFF0000u);
+      dst[0] = low_halves(a0, b0);
+      dst[16 * (XS / 2)] = high_halves(a0, b0);
+      dst[32 * (XS / 2)] = low_halves(a1, b1);
+      dst[48 * (XS / 2)] = high_halves(a1, b1);
     }
   };
 
@@ -1725,6 +1789,7 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream64(GemmSegs segs,
       }
 #pragma unroll
       for (int cb = 0; cb < 2; ++cb) {
+        mfma_results_settled(t[cb]);
         acc[cb][0] = scale_into<0>(acc[cb][0], mine, t[cb][0]);
         acc[cb][1] = scale_into<1>(acc[cb][1], mine, t[cb][1]);
         acc[cb][2] = scale_into<2>(acc[cb][2], mine, t[cb][2]);

@@ -308,6 +308,8 @@ def gemm_streams(M, N: int, k_pad_: int, force_split: int = 0,  # noqa: N803
                 best, best_cost = (rb, split, chunks), cost
     if policy == 0 and _STREAM_ONLY == 0 and sum(rows) * kp <= _STREAM_MIN_CODES:
         return (0, 1, 0)
+    if sum(rows) * kp >= 1 << 33:   # the tile addresses the packed bytes with 32-bit offsets
+        return (0, 1, 0)
     return best
 
 
