@@ -63,9 +63,10 @@ int chr_nf4_gemm(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N,
                  void *stream);
 
 /* Pure launch math; only M/K/K_pad are read.  N in [1, 64].
- * Chunks of 8, 16, 24 or 32 columns with K_pad a multiple of 256 can run the tile whose
- * workgroups finish their rows themselves (block 1024; bm 32 or 64 rows a workgroup; grid_y
- * workgroups share a row block's K in 512-wide chunks, at most 12 each, and the last of them
+ * Chunks of 8, 16, 24, 32 or exactly 64 columns with K_pad a multiple of 256 can run the tile
+ * whose workgroups finish their rows themselves (block 1024; bm 32 or 64 rows a workgroup;
+ * grid_y workgroups share a row block's K in 512-wide chunks, at most 12 each -- 256-wide and
+ * at most 20 at 64 columns, where tiles_per_split counts those -- and the last of them
  * to finish adds their fp32 partials up in split order: ws_floats = grid_y * M * N when
  * grid_y > 1, no reduce launch).  The planner takes it where its cost model prefers it to
  * the split tiles (at 14B shapes: all of them); chr_nf4_gemm_stream_policy and
