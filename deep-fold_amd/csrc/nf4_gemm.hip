@@ -1047,9 +1047,12 @@ __device__ __forceinline__ float scale_into(float acc, float mine, float t) {
 // The matrix core's result registers may be read by hand-written instructions only after it
 // has finished writing them (up to 18 wait states after the last MFMA was issued); the
 // compiler counts those for its own instructions, not for what an asm statement reads.  This
-// stands between the MFMAs that write t and the scale_into statements that read it.
-__device__ __forceinline__ void mfma_results_settled(f32x16 &t) {
-  asm volatile("s_nop 15\n\ts_nop 7" : "+v"(t));
+// stands between the MFMAs that write t and the scale_into statements that read it.  The
+// scale goes through it too: a DPP operand must have been written two instructions or more
+// before it is read, and an asm statement's operand may otherwise be computed right in front
+// of it.
+__device__ __forceinline__ void mfma_results_settled(f32x16 &t, float &scale) {
+  asm volatile("s_nop 15\n\ts_nop 7" : "+v"(t), "+v"(scale));
 }
 
 // The low halves of a and b as one dword, a below b; the high halves likewise: a byte
@@ -1103,7 +1106,8 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
                                                             float *__restrict__ partial, int M_all,
                                                             int K, int K_pad, int N,
                                                             const uint16_t *__restrict__ bias,
-                                                            const uint16_t *res, int arrive_slot) {
+                                                            const uint16_t *res, int arrive_slot,
+                                                            float *__restrict__ colsq) {
   constexpr int XS = kStreamXS;
   constexpr int CK = kStreamChunkK;
   constexpr int ROWS = kStreamRows * RB;
@@ -1420,7 +1424,7 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
       }
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
-        mfma_results_settled(t[rb]);
+        mfma_results_settled(t[rb], mine[rb]);
         acc[rb][0] = scale_into<0>(acc[rb][0], mine[rb], t[rb][0]);
         acc[rb][1] = scale_into<1>(acc[rb][1], mine[rb], t[rb][1]);
         acc[rb][2] = scale_into<2>(acc[rb][2], mine[rb], t[rb][2]);
@@ -1533,8 +1537,10 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
       o32[rb] = sum;
     }
   }
+  float square[RB];
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
+    square[rb] = 0.f;
     if (live[rb]) {
       // the epilogue of reduce_splitk, here (res may alias y: same thread, same element)
       uint16_t o = f32_to_bf16(o32[rb]);
@@ -1545,6 +1551,34 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
         o = f32_to_bf16(bf16_to_f32(res[at[rb]]) + bf16_to_f32(o));
       }
       y[at[rb]] = o;
+      square[rb] = bf16_to_f32(o) * bf16_to_f32(o);
+    }
+  }
+  if constexpr (WIDE) {
+    // What reduce_splitk_sq leaves for the RMSNorm that reads y next, here: the column sums
+    // of squares of the values as stored, per block of 1024 / 32 = 32 rows -- a 32-row block
+    // of this workgroup, whose 32 contributions to a column (sixteen wavefronts, two lanes)
+    // meet in LDS and are added in a fixed order.  One matrix only (rows from 0).
+    if (colsq != nullptr) {
+      __syncthreads();  // every wavefront is past its reads of `sums`
+#pragma unroll
+      for (int rb = 0; rb < RB; ++rb) {
+        sums[(rb * 16 + wave16) * kWave + lane] = square[rb];
+      }
+      __syncthreads();
+      if (tid < 32 * RB) {
+        const int b = tid >> 5, col = tid & 31;
+        const int rcol = (col >> 2) + 8 * (col & 3);  // the B operand's column that holds token col
+        float sum = 0.f;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          sum += sums[(b * 16 + v) * kWave + rcol];
+          sum += sums[(b * 16 + v) * kWave + rcol + 32];
+        }
+        if (row_base + 32 * b < M) {
+          colsq[static_cast<size_t>((row_base >> 5) + b) * 32 + col] = sum;
+        }
+      }
     }
   }
 }
@@ -1567,7 +1601,8 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream64(GemmSegs segs,
                                                               float *__restrict__ partial, int M_all,
                                                               int K, int K_pad,
                                                               const uint16_t *__restrict__ bias,
-                                                              const uint16_t *res, int arrive_slot) {
+                                                              const uint16_t *res, int arrive_slot,
+                                                              float *__restrict__ colsq) {
   constexpr int XS = kWideXS;
   constexpr int CK = kWideChunkK;
   constexpr int ROWS = kWideRows;
@@ -1762,7 +1797,7 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream64(GemmSegs segs,
     for (int c = 0; c < n_ch; ++c) {
       const uint32_t buf = static_cast<uint32_t>(c & 1);
       const int grp = min(4 * c + g, groups - 1) - g;
-      const float mine = f16_to_f32(*reinterpret_cast<const __attribute__((address_space(3))) uint16_t *>(
+      float mine = f16_to_f32(*reinterpret_cast<const __attribute__((address_space(3))) uint16_t *>(
           s_lane + static_cast<uint32_t>(grp * ROWS * 2)));
       const uint4 wv = lds0_u128(w_lane + buf * kWideWBytes);
       const uint32_t w4[4] = {wv.x, wv.y, wv.z, wv.w};
@@ -1789,7 +1824,7 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream64(GemmSegs segs,
       }
 #pragma unroll
       for (int cb = 0; cb < 2; ++cb) {
-        mfma_results_settled(t[cb]);
+        mfma_results_settled(t[cb], mine);
         acc[cb][0] = scale_into<0>(acc[cb][0], mine, t[cb][0]);
         acc[cb][1] = scale_into<1>(acc[cb][1], mine, t[cb][1]);
         acc[cb][2] = scale_into<2>(acc[cb][2], mine, t[cb][2]);
@@ -1893,8 +1928,10 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream64(GemmSegs segs,
       o32[o] = sum;
     }
   }
+  float square[4];
 #pragma unroll
   for (int o = 0; o < 4; ++o) {
+    square[o] = 0.f;
     if (live[o]) {
       uint16_t out = f32_to_bf16(o32[o]);
       if (bias != nullptr) {
@@ -1904,6 +1941,33 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream64(GemmSegs segs,
         out = f32_to_bf16(bf16_to_f32(res[at[o]]) + bf16_to_f32(out));
       }
       y[at[o]] = out;
+      square[o] = bf16_to_f32(out) * bf16_to_f32(out);
+    }
+  }
+  // The column sums of squares of what was stored, per block of 1024 / 64 = 16 rows (see
+  // gemm_stream): rows 16 b .. + 16 of the workgroup's 64 are accumulator values 8 (b % 2) ..
+  // + 8 of row block b / 2, in both halves of the lanes.
+  if (colsq != nullptr) {
+    __syncthreads();  // every wavefront is past its reads of `sums`
+#pragma unroll
+    for (int o = 0; o < 4; ++o) {
+      sums[(o * 16 + wave16) * kWave + lane] = square[o];
+    }
+    __syncthreads();
+    if (tid < 256) {
+      const int b = tid >> 6, col = tid & 63;
+      const int cb = (col >> 1) & 1;
+      const int rcol = (col >> 2) + 16 * (col & 1);  // the B operand's column of block cb that holds token col
+      const int o = 2 * (b >> 1) + cb;
+      float sum = 0.f;
+#pragma unroll
+      for (int v = 0; v < 8; ++v) {
+        sum += sums[(o * 16 + 8 * (b & 1) + v) * kWave + rcol];
+        sum += sums[(o * 16 + 8 * (b & 1) + v) * kWave + rcol + 32];
+      }
+      if (row_base + 16 * b < M) {
+        colsq[static_cast<size_t>((row_base >> 4) + b) * 64 + col] = sum;
+      }
     }
   }
 }
@@ -2345,34 +2409,37 @@ int gemm_launch(const chr_nf4_dev_t *const *w, int nseg, const void *x, void *y,
   const int nc = rows_col_blocks(N);
   // the stream tile's splits meet in the tile itself unless the reduce has more to do
   // (SwiGLU, the column sums of squares)
+  // (at 32 and 64 columns the tile leaves the column sums of squares itself)
+  const bool sq_in_tile = colsq != nullptr && nseg == 1 && sp.stream != 0 && (N == 32 || N == 64);
+  float *tile_sq = sq_in_tile ? colsq : nullptr;
   int slot = -1;
-  if (sp.stream != 0 && sp.grid_y > 1 && !swiglu && !(colsq != nullptr && 256 % N == 0)) {
+  if (sp.stream != 0 && sp.grid_y > 1 && !swiglu && (sq_in_tile || !(colsq != nullptr && 256 % N == 0))) {
     slot = sp.grid_x <= kArriveBlocks ? arrival_slot(st) : -1;
   }
   if (sp.stream == 1) {
     if (N <= 16) {
       gemm_stream<1, 1><<<grid, dim3(kStreamBlock), stream_lds_bytes(1), st>>>(
-          sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp, slot);
+          sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp, slot, tile_sq);
     } else if (N == 32) {
       gemm_stream<4, 1><<<grid, dim3(kStreamBlock), stream_lds_bytes(1), st>>>(
-          sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp, slot);
+          sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp, slot, tile_sq);
     } else {
       gemm_stream<2, 1><<<grid, dim3(kStreamBlock), stream_lds_bytes(1), st>>>(
-          sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp, slot);
+          sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp, slot, tile_sq);
     }
   } else if (sp.stream == 2 && N == 64) {
     gemm_stream64<<<grid, dim3(kStreamBlock), kWideLdsBytes, st>>>(sp.segs, xp, yp, partial, sp.M_all, K,
-                                                                    K_pad, bp, rp, slot);
+                                                                    K_pad, bp, rp, slot, tile_sq);
   } else if (sp.stream == 2) {
     if (N <= 16) {
       gemm_stream<1, 2><<<grid, dim3(kStreamBlock), stream_lds_bytes(2), st>>>(
-          sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp, slot);
+          sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp, slot, tile_sq);
     } else if (N == 32) {
       gemm_stream<4, 2><<<grid, dim3(kStreamBlock), stream_lds_bytes(2), st>>>(
-          sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp, slot);
+          sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp, slot, tile_sq);
     } else {
       gemm_stream<2, 2><<<grid, dim3(kStreamBlock), stream_lds_bytes(2), st>>>(
-          sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp, slot);
+          sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp, slot, tile_sq);
     }
   } else if (rows_kernel_serves(N, sp.tiles_per_split)) {
     const RowsArgs ra{sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp};
@@ -2412,6 +2479,9 @@ int gemm_launch(const chr_nf4_dev_t *const *w, int nseg, const void *x, void *y,
         partial, yp, rows, sp.grid_y, N, bp, rp);
   }
   const int rc = launch_rc();
+  if (sq_in_tile && (partial == nullptr || slot >= 0)) {
+    return rc;  // the tile wrote them
+  }
   // a caller that asked for the column sums learns that this launch did not write them
   return rc == 0 && colsq != nullptr ? 1 : rc;
 }
