@@ -229,8 +229,9 @@ constexpr int kArriveBlocks = 1024;  // row blocks of a launch whose splits meet
 
 // blocks32, blocks64: 32- and 64-row blocks of the launch (summed over its stacked matrices).
 // Picks, among the forms that fit (at most 12 chunks a workgroup; splits only when all
-// workgroups run at once and the caller brought a workspace; at most two rounds of
-// workgroups, and two only with 8 chunks or more to spread a round's fixed time over), the one a cost model fitted to measurements calls cheapest, in hundredths of a
+// the caller brought a workspace; at most four rounds of workgroups, and more than one only
+// with 3072 of K or more to spread a round's fixed time over and the rounds four fifths full,
+// and splits over several rounds only from 24 columns on), the one a cost model fitted to measurements calls cheapest, in hundredths of a
 // microsecond: a round of 32-row workgroups 5.2 us + 0.55 / 0.67 / 0.86 / 1.06 us a chunk at
 // 8 / 16 / 24 / 32 columns, of 64-row workgroups 6.5 us + 1.00 / 1.06 / 1.22 / 1.38 us a chunk,
 // 2.3 us for the meeting of a split's partials (at most 8 splits; a split has to win by 3%).
@@ -270,11 +271,14 @@ StreamPlan stream_plan(int N, int K_pad, int blocks32, int blocks64, int have_ws
         continue;  // (the same chunks with fewer workgroups comes first; too long a K)
       }
       const int rounds = ceil_div(blocks * split, cus);
-      if (rounds > 2 || (split > 1 && (rounds > 1 || !splits || !have_ws || blocks > kArriveBlocks))) {
+      if (rounds > 4 || (split > 1 && (!splits || !have_ws || blocks > kArriveBlocks))) {
         continue;
       }
-      if (rounds == 2 && chunks * (wide ? kWideChunkK : kStreamChunkK) < 8 * kStreamChunkK) {
-        continue;  // (22016x2048 in two rounds of 4 chunks: 18.1 / 22.1 us against 14.1 / 20.3)
+      // more than one round of workgroups: only long ones (22016x2048 in two rounds of 4
+      // chunks: 18.1 / 22.1 us against 14.1 / 20.3) that fill the rounds to four fifths
+      if (rounds > 1 && (chunks * (wide ? kWideChunkK : kStreamChunkK) < 6 * kStreamChunkK ||
+                         blocks * split * 5 < rounds * cus * 4 || (split > 1 && N < 24))) {
+        continue;  // (6144x16384 at 8 columns, 5 splits in two rounds: 28.2 us against 23.8)
       }
       int cost = rounds * (kFixed[rb - 1] + chunks * (wide ? kWideChunk : kChunk[rb - 1][N / 8 - 1]));
       if (split > 1) {

@@ -263,8 +263,9 @@ def gemm_streams(M, N: int, k_pad_: int, force_split: int = 0,  # noqa: N803
     launch); pair-table lookups, the scale applied per 64-wide group.  It takes whole-vector
     chunks of up to 32 columns (and, with 64 rows and 256-wide chunks, at most 20 of them a
     workgroup, chunks of exactly 64), no forced split, ``K_pad`` a multiple of 256, at most 12
-    chunks a workgroup, splits only when all workgroups run at once and there is a workspace,
-    at most 8 splits, at most two rounds of workgroups (two only with 8 chunks or more) --
+    chunks a workgroup, splits only with a workspace and at most 8 of them, at most four rounds
+    of workgroups (more than one only with 3072 of K or more a workgroup and the rounds four
+    fifths full, and with splits only from 24 columns on) --
     and of the forms that fit, the cheapest by the cost model above (a split has to win by
     3%), if the launch has more than 2^24 weights (``policy`` 0; 1: wherever it fits; -1:
     never; None: the process default).  ``M``: the rows, or the rows of each stacked matrix
@@ -294,10 +295,11 @@ def gemm_streams(M, N: int, k_pad_: int, force_split: int = 0,  # noqa: N803
             if _ceil_div(n_ch, chunks) != split or chunks > bodies:
                 continue
             rounds = _ceil_div(blocks * split, cus)
-            if rounds > 2 or (split > 1 and (rounds > 1 or not _STREAM_SPLITS or not have_ws
+            if rounds > 4 or (split > 1 and (not _STREAM_SPLITS or not have_ws
                                              or blocks > _ARRIVE_BLOCKS)):
                 continue
-            if rounds == 2 and chunks * chunk_k < 8 * 512:
+            if rounds > 1 and (chunks * chunk_k < 6 * 512 or blocks * split * 5 < rounds * cus * 4
+                               or (split > 1 and N < 24)):
                 continue
             per_chunk = _STREAM_CHUNK_64 if wide else _STREAM_CHUNK[rb - 1][N // 8 - 1]
             cost = rounds * (_STREAM_FIXED[rb - 1] + chunks * per_chunk)
