@@ -224,6 +224,7 @@ struct StreamPlan {
 };
 
 constexpr int64_t kStreamMinCodes = int64_t{1} << 24;
+constexpr int64_t kStreamMinCodes64 = int64_t{1} << 20;  // at 64 columns
 constexpr int kArriveSlots = 32;     // launches that may overlap in time (one a stream)
 constexpr int kArriveBlocks = 1024;  // row blocks of a launch whose splits meet in the tile
 
@@ -239,7 +240,9 @@ constexpr int kArriveBlocks = 1024;  // row blocks of a launch whose splits meet
 // 8 / 32 columns, this tile against those: 256x5120 8.2 / 8.8 us against 7.5 / 8.5, 2048x2048
 // 6.9 / 9.0 against 7.2 / 8.2, 4096x4096 9.0 / 12.2 against 8.9 / 11.5, 1024x13824 10.6 /
 // 18.7 against 10.5 / 12.4; above, 3072x8192 11.0 / 15.2 against 12.1 / 15.1 and the 14B
-// shapes below).  At the 14B shapes:
+// shapes below).  At 64 columns, where the split tiles are slower, above 2^20 weights
+// (512x2048 14.9 us against 17.7, 2560x2048 13.6 against 19.1, 4096x4096 16.3 against 20.5;
+// 256x1024 10.9 against 10.4).  At the 14B shapes:
 // q/k/v 32 rows x all of K up to 24 columns and 64 rows x 2 splits at 32; o 32 rows x all of K
 // up to 16 columns, 64 rows x 3 splits above; gate or up 64 rows; gate+up stacked 64 rows in two
 // rounds; down (K = 13824) 64 rows x 3 splits.  CHR_NF4_GEMM_STREAM_ROWS=32 or 64 allows only
@@ -291,7 +294,8 @@ StreamPlan stream_plan(int N, int K_pad, int blocks32, int blocks64, int have_ws
       }
     }
   }
-  if (codes <= kStreamMinCodes && only == 0 && stream_policy().load(std::memory_order_relaxed) == 0) {
+  if (codes <= (wide ? kStreamMinCodes64 : kStreamMinCodes) && only == 0 &&
+      stream_policy().load(std::memory_order_relaxed) == 0) {
     best.rb = 0;
   }
   if (codes >= (int64_t{1} << 33)) {

@@ -250,6 +250,7 @@ _STREAM_CHUNK_64 = 110      # a 256-wide chunk of the 64-column form (64 rows a 
 _STREAM_MEET = 230
 _STREAM_MAX_SPLIT = 8
 _STREAM_MIN_CODES = 1 << 24
+_STREAM_MIN_CODES_64 = 1 << 20    # at 64 columns the split tiles are slower
 _ARRIVE_BLOCKS = 1024
 
 
@@ -267,7 +268,7 @@ def gemm_streams(M, N: int, k_pad_: int, force_split: int = 0,  # noqa: N803
     of workgroups (more than one only with 3072 of K or more a workgroup and the rounds four
     fifths full, and with splits only from 24 columns on) --
     and of the forms that fit, the cheapest by the cost model above (a split has to win by
-    3%), if the launch has more than 2^24 weights (``policy`` 0; 1: wherever it fits; -1:
+    3%), if the launch has more than 2^24 weights, or 2^20 at 64 columns (``policy`` 0; 1: wherever it fits; -1:
     never; None: the process default).  ``M``: the rows, or the rows of each stacked matrix
     (blocks do not straddle matrices).  ``CHR_NF4_GEMM_STREAM_ROWS=32`` or ``64`` allows only
     that form and skips the weight count, ``CHR_NF4_GEMM_STREAM_SPLIT=0`` allows no splits.
@@ -308,7 +309,8 @@ def gemm_streams(M, N: int, k_pad_: int, force_split: int = 0,  # noqa: N803
                 cost += cost // 32
             if best[0] == 0 or cost < best_cost:
                 best, best_cost = (rb, split, chunks), cost
-    if policy == 0 and _STREAM_ONLY == 0 and sum(rows) * kp <= _STREAM_MIN_CODES:
+    if policy == 0 and _STREAM_ONLY == 0 and sum(rows) * kp <= (_STREAM_MIN_CODES_64 if wide
+                                                                else _STREAM_MIN_CODES):
         return (0, 1, 0)
     if sum(rows) * kp >= 1 << 33:   # the tile addresses the packed bytes with 32-bit offsets
         return (0, 1, 0)
