@@ -1107,7 +1107,10 @@ __device__ __forceinline__ int stream_token_row(int n) {
 // overlap in time must use different slots (the host deals a slot to every stream).
 static __device__ unsigned int stream_arrivals[kArriveSlots][kArriveBlocks];
 
-template <int XI, int RB>
+// PAIR (with two row blocks): they are rows 32 b .. + 32 of two matrices of the same shape,
+// gate (segs' first) and up (second), and the epilogue stores silu(gate) * up, [M, N], with
+// reduce_swiglu's roundings: no partials and no reduce launch.  grid.y must be 1.
+template <int XI, int RB, bool PAIR = false>
 __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
                                                             const uint16_t *__restrict__ x,
                                                             uint16_t *__restrict__ y,
@@ -1132,21 +1135,24 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
   const bool stager = wave16 >= 8;  // wavefronts 8..15 stage, 0..7 multiply
   const int wave = wave16 & 7;      // group of a chunk (multiplying), or eighth of the staging
   const int stid = tid & (kStreamStagers - 1);
+  static_assert(!PAIR || RB == 2, "a pair is two row blocks");
   int bx = static_cast<int>(blockIdx.x);
   int seg = 0;
-  if (bx >= segs.blocks[0]) {
-    bx -= segs.blocks[0];
-    seg = 1;
-    if (bx >= segs.blocks[1]) {
-      bx -= segs.blocks[1];
-      seg = 2;
+  if constexpr (!PAIR) {
+    if (bx >= segs.blocks[0]) {
+      bx -= segs.blocks[0];
+      seg = 1;
+      if (bx >= segs.blocks[1]) {
+        bx -= segs.blocks[1];
+        seg = 2;
+      }
     }
   }
   const uint8_t *__restrict__ packed = segs.packed[seg];
   const uint16_t *__restrict__ scale = segs.scale[seg];
   const int M = segs.M[seg];
   const int out0 = segs.row0[seg];
-  const int row_base = bx * ROWS;
+  const int row_base = bx * (PAIR ? kStreamRows : ROWS);  // first row, of each matrix when PAIR
   const int r = lane & 31;  // row of the A operand, token of the B operand
   const int h = lane >> 5;  // which half of a group's k
   // grid.y splits K by whole chunks: this workgroup takes n_ch of them from chunk c0 on, and
@@ -1195,7 +1201,8 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
   uint32_t w_off[RB];
 #pragma unroll
   for (int rb = 0; rb < RB; ++rb) {
-    w_off[rb] = static_cast<uint32_t>(min(row_base + 32 * rb + (stid >> 4), M - 1)) * row_stride + c0 * (CK / 2);
+    w_off[rb] = static_cast<uint32_t>(min(row_base + (PAIR ? 0 : 32 * rb) + (stid >> 4), M - 1)) * row_stride +
+                c0 * (CK / 2);
   }
   const uint32_t x_row = 2u * N;  // bytes of a row of x
   uint32_t xk_off[NA], xq_off[NA];
@@ -1209,7 +1216,8 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
     const uint32_t w_at = min(static_cast<uint32_t>(cc * (CK / 2) + w_piece), static_cast<uint32_t>(row_bytes - 16));
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
-      (rb ? w1 : w0) = *reinterpret_cast<const U32x4 *>(packed + (w_off[rb] + w_at));
+      (rb ? w1 : w0) =
+          *reinterpret_cast<const U32x4 *>((PAIR && rb ? segs.packed[1] : packed) + (w_off[rb] + w_at));
     }
     const unsigned char *xb = reinterpret_cast<const unsigned char *>(x) + static_cast<size_t>(cc) * CK * x_row;
     const uint32_t k_last = static_cast<uint32_t>(K - 1 - cc * CK) * x_row;  // offset of the last row of x
@@ -1301,8 +1309,10 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
   for (int it = 0; it < kScaleLoads; ++it) {
     const int i = min(tid + it * kStreamBlock, ROWS * quads - 1);
     const int srow = i / quads;
+    const uint16_t *sc = PAIR && srow >= 32 ? segs.scale[1] : scale;
     sv[it] = *reinterpret_cast<const uint2 *>(
-        scale + static_cast<size_t>(min(row_base + srow, M - 1)) * groups_all + 8 * c0 + 4 * (i - srow * quads));
+        sc + static_cast<size_t>(min(row_base + (PAIR ? srow & 31 : srow), M - 1)) * groups_all + 8 * c0 +
+        4 * (i - srow * quads));
   }
   // chunks a staging thread keeps in flight: with 64 bytes of x a chunk, three are what 128
   // registers hold
@@ -1476,12 +1486,21 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
     for (int q = 0; q < 8; ++q) {
       o32[rb] += sums[((rb * 8 + q) * 16 + v) * kWave + lane];
     }
-    const int rr = row_base + 32 * rb + 8 * (v >> 2) + 4 * h + (v & 3);
+    const int rr = row_base + (PAIR ? 0 : 32 * rb) + 8 * (v >> 2) + 4 * h + (v & 3);
     live[rb] = r < N && rr < M;
     orow[rb] = out0 + min(rr, M - 1);
     // (at 32 columns row r of the chunk buffers, the B operand's column r, holds token
     // 4 (r % 8) + r / 8)
     at[rb] = static_cast<size_t>(orow[rb]) * N + (WIDE ? 4 * (r & 7) + (r >> 3) : min(r, N - 1));
+  }
+  if constexpr (PAIR) {
+    // output 0 is the gate's, output 1 the up's, at the same row and token
+    if (live[0]) {
+      const float a = bf16_to_f32(f32_to_bf16(o32[0]));
+      const float act = bf16_to_f32(f32_to_bf16(a / (1.f + expf(-a))));
+      y[at[0]] = f32_to_bf16(act * bf16_to_f32(f32_to_bf16(o32[1])));
+    }
+    return;
   }
   if (partial != nullptr) {
     // this split's slab of the partials
@@ -1603,6 +1622,10 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
 // (the B operand's column l of block cb is token 4 (l % 16) + 2 cb + l / 16).
 // Everything else -- the pair table, the scales in LDS and their DPP broadcast, the ring of
 // requests and the nested chunks, the splits of K that meet in the tile -- is gemm_stream's.
+// PAIR: the two 32-row blocks of a workgroup are rows 32 b .. + 32 of two matrices of the same
+// shape, gate (segs' first) and up (second), and the epilogue stores silu(gate) * up, [M, 64],
+// with reduce_swiglu's roundings: no partials and no reduce launch.  grid.y must be 1.
+template <bool PAIR>
 __global__ __launch_bounds__(kStreamBlock) void gemm_stream64(GemmSegs segs,
                                                               const uint16_t *__restrict__ x,
                                                               uint16_t *__restrict__ y,
@@ -1629,19 +1652,22 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream64(GemmSegs segs,
   const int stid = tid & (kStreamStagers - 1);
   int bx = static_cast<int>(blockIdx.x);
   int seg = 0;
-  if (bx >= segs.blocks[0]) {
-    bx -= segs.blocks[0];
-    seg = 1;
-    if (bx >= segs.blocks[1]) {
-      bx -= segs.blocks[1];
-      seg = 2;
+  if constexpr (!PAIR) {
+    if (bx >= segs.blocks[0]) {
+      bx -= segs.blocks[0];
+      seg = 1;
+      if (bx >= segs.blocks[1]) {
+        bx -= segs.blocks[1];
+        seg = 2;
+      }
     }
   }
-  const uint8_t *__restrict__ packed = segs.packed[seg];
+  // (PAIR: the staging wavefronts 8..11 fetch gate rows, 12..15 up rows)
+  const uint8_t *__restrict__ packed = segs.packed[PAIR ? (wave16 >= 12 ? 1 : 0) : seg];
   const uint16_t *__restrict__ scale = segs.scale[seg];
   const int M = segs.M[seg];
   const int out0 = segs.row0[seg];
-  const int row_base = bx * ROWS;
+  const int row_base = bx * (PAIR ? 32 : ROWS);  // first row, of each matrix when PAIR
   const int r = lane & 31;  // row of the A operand, token of the B operand
   const int h = lane >> 5;  // which half of a group's k
   // grid.y splits K by whole chunks (see gemm_stream): from here on x, K, row_bytes and groups
@@ -1667,7 +1693,8 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream64(GemmSegs segs,
   const int w_piece = 16 * (stid & 7);
   // (a base that is the same in every lane and a 32-bit offset of the lane: see gemm_stream)
   const uint32_t w_off =
-      static_cast<uint32_t>(min(row_base + (stid >> 3), M - 1)) * row_stride + c0 * (CK / 2);
+      static_cast<uint32_t>(min(row_base + (PAIR ? (stid >> 3) & 31 : stid >> 3), M - 1)) * row_stride +
+      c0 * (CK / 2);
   const int w_half = (lane >> 3) & 1;
   const int w_q = lane & 7;
   const int w_kp = (lane >> 4) + 4 * wave;  // + 32 it
@@ -1733,8 +1760,10 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream64(GemmSegs segs,
   for (int it = 0; it < kScaleLoads; ++it) {
     const int i = min(tid + it * kStreamBlock, ROWS * quads - 1);
     const int srow = i / quads;
+    const uint16_t *sc = PAIR && srow >= 32 ? segs.scale[1] : scale;
     sv[it] = *reinterpret_cast<const uint2 *>(
-        scale + static_cast<size_t>(min(row_base + srow, M - 1)) * groups_all + 4 * c0 + 4 * (i - srow * quads));
+        sc + static_cast<size_t>(min(row_base + (PAIR ? srow & 31 : srow), M - 1)) * groups_all + 4 * c0 +
+        4 * (i - srow * quads));
   }
   constexpr int R = 3;
   Item ring[R];
@@ -1876,11 +1905,23 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream64(GemmSegs segs,
     for (int g = 0; g < 4; ++g) {
       o32[o] += sums[((cb * 8 + 4 * rb + g) * 16 + v) * kWave + lane];
     }
-    const int rr = row_base + 32 * rb + 8 * (v >> 2) + 4 * h + (v & 3);
+    const int rr = row_base + (PAIR ? 0 : 32 * rb) + 8 * (v >> 2) + 4 * h + (v & 3);
     live[o] = rr < M;
     orow[o] = out0 + min(rr, M - 1);
     // (row 32 cb + r of the chunk buffers holds token 4 (r % 16) + 2 cb + r / 16)
     at[o] = static_cast<size_t>(orow[o]) * N + 4 * (r & 15) + 2 * cb + (r >> 4);
+  }
+  if constexpr (PAIR) {
+    // outputs 0, 1 are the gate's two token halves, 2, 3 the up's, at the same rows
+#pragma unroll
+    for (int cb = 0; cb < 2; ++cb) {
+      if (live[cb]) {
+        const float a = bf16_to_f32(f32_to_bf16(o32[cb]));
+        const float act = bf16_to_f32(f32_to_bf16(a / (1.f + expf(-a))));
+        y[at[cb]] = f32_to_bf16(act * bf16_to_f32(f32_to_bf16(o32[2 + cb])));
+      }
+    }
+    return;
   }
   if (partial != nullptr) {
     const size_t slab = static_cast<size_t>(M_all) * N;
@@ -2209,8 +2250,12 @@ int gemm_lds_ready() {
         return -6;
       }
     }
-    const std::pair<const void *, int> streams[7] = {
-        {reinterpret_cast<const void *>(gemm_stream64), kWideLdsBytes},
+    const std::pair<const void *, int> streams[11] = {
+        {reinterpret_cast<const void *>(gemm_stream<1, 2, true>), stream_lds_bytes(2)},
+        {reinterpret_cast<const void *>(gemm_stream<2, 2, true>), stream_lds_bytes(2)},
+        {reinterpret_cast<const void *>(gemm_stream<4, 2, true>), stream_lds_bytes(2)},
+        {reinterpret_cast<const void *>(gemm_stream64<false>), kWideLdsBytes},
+        {reinterpret_cast<const void *>(gemm_stream64<true>), kWideLdsBytes},
         {reinterpret_cast<const void *>(gemm_stream<1, 1>), stream_lds_bytes(1)},
         {reinterpret_cast<const void *>(gemm_stream<2, 1>), stream_lds_bytes(1)},
         {reinterpret_cast<const void *>(gemm_stream<4, 1>), stream_lds_bytes(1)},
@@ -2344,6 +2389,10 @@ StackPlan plan_stack(const chr_nf4_dev_t *h, int nseg, int N, int have_ws, bool 
   return sp;
 }
 
+// Whether a stacked gate+up launch pairs the rows inside the tile (its unsplit 64-row forms):
+// then there are no partials and no reduce launch.
+bool swiglu_pairs(const StackPlan &sp, int /*N*/) { return sp.stream == 2 && sp.grid_y == 1; }
+
 // live_max: widest chunk the entry launches.  The reference's entries stop at 32 columns
 // (wider ones are described by the planner only); the chr_dv2_gemm_* entries go to 64.
 // w[0..nseg) share K and x; y, bias and res cover the stacked rows.
@@ -2390,17 +2439,28 @@ int gemm_launch(const chr_nf4_dev_t *const *w, int nseg, const void *x, void *y,
     scales_aligned8 = scales_aligned8 && (reinterpret_cast<uintptr_t>(h[i].scale) & 7u) == 0;
   }
   StackPlan sp = plan_stack(h, nseg, N, have_ws, scales_aligned8);
+  bool pair = false;
   if (swiglu) {
-    // the activation lives in the reduce, so this launch always goes through fp32 partials
     if (nseg != 2 || h[0].M != h[1].M || bias != nullptr || res != nullptr) {
       return -3;
     }
-    sp.ws_floats = static_cast<int64_t>(sp.grid_y) * sp.M_all * N;
+    pair = swiglu_pairs(sp, N);
+    if (pair) {
+      // a workgroup takes 32 gate rows and the 32 up rows that go with them, and stores the
+      // activation itself
+      sp.grid_x = ceil_div(h[0].M, kStreamRows);
+      sp.segs.blocks[0] = sp.grid_x;
+      sp.segs.blocks[1] = 0;
+      sp.ws_floats = 0;
+    } else {
+      // the activation lives in the reduce, so the launch goes through fp32 partials
+      sp.ws_floats = static_cast<int64_t>(sp.grid_y) * sp.M_all * N;
+    }
   }
   if (sp.ws_floats > 0 && (!have_ws || ws_floats < sp.ws_floats)) {
     return -7;
   }
-  float *partial = (sp.grid_y > 1 || swiglu) ? ws : nullptr;
+  float *partial = (sp.grid_y > 1 || (swiglu && !pair)) ? ws : nullptr;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const dim3 grid(static_cast<unsigned>(sp.grid_x), static_cast<unsigned>(sp.grid_y));
   // 16-byte activation vectors need N in {8, 16, 32, 64}; x is 16-byte aligned (checked above)
@@ -2436,8 +2496,26 @@ int gemm_launch(const chr_nf4_dev_t *const *w, int nseg, const void *x, void *y,
           sp.segs, xp, yp, partial, sp.M_all, K, K_pad, N, bp, rp, slot, tile_sq);
     }
   } else if (sp.stream == 2 && N == 64) {
-    gemm_stream64<<<grid, dim3(kStreamBlock), kWideLdsBytes, st>>>(sp.segs, xp, yp, partial, sp.M_all, K,
-                                                                    K_pad, bp, rp, slot, tile_sq);
+    if (pair) {
+      gemm_stream64<true><<<grid, dim3(kStreamBlock), kWideLdsBytes, st>>>(sp.segs, xp, yp, nullptr, sp.M_all,
+                                                                            K, K_pad, nullptr, nullptr, -1,
+                                                                            nullptr);
+      return launch_rc();
+    }
+    gemm_stream64<false><<<grid, dim3(kStreamBlock), kWideLdsBytes, st>>>(sp.segs, xp, yp, partial, sp.M_all,
+                                                                           K, K_pad, bp, rp, slot, tile_sq);
+  } else if (sp.stream == 2 && pair) {
+    if (N <= 16) {
+      gemm_stream<1, 2, true><<<grid, dim3(kStreamBlock), stream_lds_bytes(2), st>>>(
+          sp.segs, xp, yp, nullptr, sp.M_all, K, K_pad, N, nullptr, nullptr, -1, nullptr);
+    } else if (N == 32) {
+      gemm_stream<4, 2, true><<<grid, dim3(kStreamBlock), stream_lds_bytes(2), st>>>(
+          sp.segs, xp, yp, nullptr, sp.M_all, K, K_pad, N, nullptr, nullptr, -1, nullptr);
+    } else {
+      gemm_stream<2, 2, true><<<grid, dim3(kStreamBlock), stream_lds_bytes(2), st>>>(
+          sp.segs, xp, yp, nullptr, sp.M_all, K, K_pad, N, nullptr, nullptr, -1, nullptr);
+    }
+    return launch_rc();
   } else if (sp.stream == 2) {
     if (N <= 16) {
       gemm_stream<1, 2><<<grid, dim3(kStreamBlock), stream_lds_bytes(2), st>>>(
@@ -2615,8 +2693,10 @@ extern "C" int64_t chr_dv2_gemm_swiglu_ws(const chr_nf4_dev_t *gate, const chr_n
   if (h[0].M < 1 || h[0].M != h[1].M || h[0].K < 1 || !k_pad_ok(h[0].K, h[0].K_pad)) {
     return -1;
   }
-  const StackPlan sp = plan_stack(h, 2, N, 1);
-  return static_cast<int64_t>(sp.grid_y) * sp.M_all * N;
+  // (as the launch decides: the tile wants the scale blobs 8-byte aligned)
+  const bool aligned = ((reinterpret_cast<uintptr_t>(h[0].scale) | reinterpret_cast<uintptr_t>(h[1].scale)) & 7u) == 0;
+  const StackPlan sp = plan_stack(h, 2, N, 1, aligned);
+  return swiglu_pairs(sp, N) ? 0 : static_cast<int64_t>(sp.grid_y) * sp.M_all * N;
 }
 
 extern "C" int chr_dv2_gemm_swiglu(const chr_nf4_dev_t *gate, const chr_nf4_dev_t *up,

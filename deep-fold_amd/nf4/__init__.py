@@ -961,10 +961,11 @@ def dv2_gemm_swiglu(gate, up, x: torch.Tensor) -> torch.Tensor:
     _need(devs[0].M == devs[1].M, "gate and up must have the same number of rows")
     lib = _load_ext()
     need = int(lib.chr_dv2_gemm_swiglu_ws(ctypes.byref(devs[0]), ctypes.byref(devs[1]), n))
-    _need(need > 0, "chr_dv2_gemm_swiglu_ws refused the shapes")
-    ws = torch.empty(need, dtype=torch.float32, device=x.device)
+    _need(need >= 0, "chr_dv2_gemm_swiglu_ws refused the shapes")
+    # (0: the launch pairs gate and up rows inside the tile and stores the activation itself)
+    ws = torch.empty(need, dtype=torch.float32, device=x.device) if need > 0 else None
     y = torch.empty((devs[0].M, n), dtype=torch.bfloat16, device=x.device)
     rc = lib.chr_dv2_gemm_swiglu(ctypes.byref(devs[0]), ctypes.byref(devs[1]), x.data_ptr(), y.data_ptr(),
-                                 n, ws.data_ptr(), need, _stream())
+                                 n, None if ws is None else ws.data_ptr(), need, _stream())
     _check_rc("chr_dv2_gemm_swiglu", rc)
     return y

@@ -336,8 +336,12 @@ int chr_dv2_gemm_qkv(const chr_nf4_dev_t *q, const chr_nf4_dev_t *k, const chr_n
  * of chr_nf4_gemv_swiglu; gpu/decodev2/prefill.py:133 runs two GEMMs, F.silu and a product):
  * y [M, N] = silu(gate x) * (up x), gate and up rounded to bf16 first and the activation
  * rounded to bf16 before the product, as those separate bf16 ops round.  Both matrices are
- * M x K.  N = 2..64.  The launch always goes through fp32 partials: chr_dv2_gemm_swiglu_ws
- * gives the workspace elements it needs (-1: bad arguments).  No reference counterpart. */
+ * M x K.  N = 2..64.  The launch goes through fp32 partials and a reduce that applies the
+ * activation -- chr_dv2_gemm_swiglu_ws gives the workspace elements it needs (-1: bad
+ * arguments) -- or, at 64 columns where the planner takes the unsplit tile that finishes its
+ * rows itself, pairs 32 gate rows with their up rows in a workgroup, which stores the
+ * activation: then chr_dv2_gemm_swiglu_ws gives 0 and ws may be NULL.  No reference
+ * counterpart. */
 int64_t chr_dv2_gemm_swiglu_ws(const chr_nf4_dev_t *gate, const chr_nf4_dev_t *up, int32_t N);
 int chr_dv2_gemm_swiglu(const chr_nf4_dev_t *gate, const chr_nf4_dev_t *up, const void *x,
                         void *y, int32_t N, float *ws, int64_t ws_floats, void *stream);
