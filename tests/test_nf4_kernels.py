@@ -669,6 +669,39 @@ def _stream_tile_case(m, k, n, p, s, dp, ds, xh, x, kp):
     assert (bf16_bits(got) == bf16_bits(want)).all()
 
 
+def test_gemm_stream_tile_random_shapes():
+    """Sixty seeded random launches of the tile that finishes its rows itself, taken wherever it
+    fits (rows 1..12000, K_pad 256..9984 with K at or below it, every chunk width it has):
+    each against its arithmetic in float64 and bit-identical on a second launch."""
+    rng = np.random.default_rng(2024)
+    nf4.nf4_gemm_stream_policy(1)
+    try:
+        forms, done = set(), 0
+        while done < 60:
+            n = int(rng.choice([8, 16, 24, 32, 64]))
+            kp = int(rng.integers(1, 40)) * 256
+            k = kp - int(rng.integers(0, 64)) if rng.random() < 0.5 else kp
+            m = int(rng.integers(1, 3000)) if rng.random() < 0.7 else int(rng.integers(3000, 12000))
+            if m * kp > 40_000_000:
+                continue
+            plan = nf4.nf4_plan(m, k, n)
+            if plan["block"] != 1024 or plan["bm"] not in (32, 64):
+                continue
+            say("gemm stream, random", m, k, n, plan["bm"], plan["grid_x"], plan["grid_y"])
+            p, s = oc.toy_blobs(m, k, int(rng.integers(1 << 30)))
+            dp, ds = up(p), up_scale(s)
+            xh = rand_x(k, n, int(rng.integers(1000)))
+            x = bf16_tensor(xh)
+            y = nf4.nf4_gemm(dp, ds, x, m, k, oc.k_pad(k), 64)
+            assert (bf16_bits(nf4.nf4_gemm(dp, ds, x, m, k, oc.k_pad(k), 64)) == bf16_bits(y)).all()
+            check_linear(y, staged_gemv_model(p, s, m, k, xh, terms=1), what=f"stream {m}x{k} n{n}")
+            forms.add((plan["bm"], plan["grid_y"] > 1, n == 64))
+            done += 1
+        assert len(forms) >= 5, forms  # 32 and 64 rows, split and not, the 64-column form
+    finally:
+        nf4.nf4_gemm_stream_policy(0)
+
+
 def test_gemm_stream_splits_on_many_streams():
     """Launches whose workgroups share K count their arrivals in a slot of a table the library
     owns, one slot per stream; streams beyond its 32 slots get the reduce kernel on the same
