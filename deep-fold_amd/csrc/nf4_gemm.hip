@@ -961,51 +961,55 @@ __global__ __launch_bounds__(kRowsBlock) void gemm_rows(const GemmSegs segs,
 }
 
 // ---- stream tile ---------------------------------------------------------------------------
-// The tile for chunks of 8..32 columns in whole 16-byte vectors: a workgroup of sixteen
-// wavefronts owns 32 rows and the WHOLE of K, so a launch has no split-K, no fp32 partials and
-// no second kernel; its epilogue is the reduce's (bias, residual, one rounding to bf16).
-// Eight of the wavefronts multiply, the other eight stage the operands into LDS; a barrier
-// per chunk keeps the two sides one chunk apart.  (One set of wavefronts doing both took the
-// sum of the two times per chunk, 0.7 us at N = 8 and 1.2 us at N = 32 on 7168x5120; two sets
-// take the longer one, 0.6 and 1.1.)
+// The tile for chunks of 8..32 columns in whole 16-byte vectors (gemm_stream64 further down is
+// its form for exactly 64): a workgroup of sixteen wavefronts owns 32 or 64 rows and all of K,
+// or a share of K in whole chunks (grid.y) whose partials the last workgroup of a row block to
+// finish adds up -- either way a launch has no second kernel; the epilogue is the reduce's
+// (bias, residual, one rounding to bf16).  Eight of the wavefronts multiply, the other eight
+// stage the operands into LDS; a barrier per chunk keeps the two sides one chunk apart.  (One
+// set of wavefronts doing both took the sum of the two times per chunk, 0.7 us at N = 8 and
+// 1.2 us at N = 32 on 7168x5120; two sets take the longer one.)
 //
-// Weights never become bf16(level * scale).  A packed byte goes through the GEMV's pair table
-// (byte -> the two levels as a bf16 pair, one v_perm_b32 and one conflict-free LDS read) and
-// the four pairs of a dword are an MFMA A operand as they are.  The k-to-slot map keeps every
-// MFMA inside one 64-wide group: lane l of v_mfma_f32_32x32x16_bf16 supplies eight k of row
-// l % 32 in slots 8 (l / 32) .. + 8, a wavefront step is one group, lane l takes the sixteen
-// bytes (32 codes) of row l % 32 at byte 16 (l / 32) of the group, and the step's four MFMAs
-// take its four dwords: k = 32 (l / 32) + 8 j .. + 8.  Their sum over the group starts from
-// zero and enters the accumulator through one fp32 multiply-add with the group's scale per
-// output row, so the scale is applied once per 64 products instead of once per weight,
-// exactly (fp16 -> fp32), and the only rounding of a weight is bf16(level).
+// Weights never become bf16(level * scale).  A packed byte goes through a pair table (byte ->
+// the two levels as a bf16 pair, one conflict-free LDS read) and the four pairs of a dword are
+// an MFMA A operand as they are.  The k-to-slot map keeps every MFMA inside one 64-wide group:
+// lane l of v_mfma_f32_32x32x16_bf16 supplies eight k of row l % 32 in slots 8 (l / 32) .. + 8,
+// a wavefront step is one group, lane l takes the sixteen bytes (32 codes) of row l % 32 at
+// byte 16 (l / 32) of the group, and the step's four MFMAs take its four dwords: k =
+// 32 (l / 32) + 8 j .. + 8.  Their sum over the group starts from zero and enters the
+// accumulator through one fp32 multiply-add with the group's scale per output row, so the
+// scale is applied once per 64 products instead of once per weight, exactly (fp16 -> fp32),
+// and the only rounding of a weight is bf16(level).
 //
 // K is walked in chunks of 512 (eight groups): multiplying wavefront w works on group w of
-// every chunk, all eight on the same 32 rows, and their eight sums of an output meet in LDS at
-// the end, added in the order of the wavefronts.  Every element of x is therefore read from LDS once
-// per workgroup, and every B operand by one wavefront only.
+// every chunk, all eight on the same rows (with 64 rows a workgroup every B operand it reads
+// feeds two A operands), and their eight sums of an output meet in LDS at the end, added in
+// the order of the wavefronts.  Every element of x is therefore read from LDS once per
+// workgroup, and every B operand by one wavefront only.
 //
-// Scales: all of the 32 rows' scales are staged in LDS at the start ([group][row], fp16).  An
-// accumulator lane holds rows 8 b + 4 (l / 32) + i (b, i = 0..3): lane l reads the scale of
-// row 8 ((l % 16) / 4) + 4 (l / 32) + l % 4, which puts the row of accumulator value v at
-// position v of every row of sixteen lanes, where a DPP row broadcast fetches it.
+// Scales: all of the rows' scales are staged in LDS at the start ([group][row], fp16).  An
+// accumulator lane holds rows 8 b + 4 (l / 32) + i (b, i = 0..3) of a 32-row block: lane l
+// reads the scale of row 8 ((l % 16) / 4) + 4 (l / 32) + l % 4, which puts the row of
+// accumulator value v at position v of every row of sixteen lanes, where a DPP row broadcast
+// fetches it.
 //
 // Global memory is read with consecutive lanes on consecutive bytes only (a load whose lanes
 // read 64 different rows keeps the memory pipeline's address stage busy for some 140 cycles
 // whatever its width, and the MFMA layout is one row per lane): a chunk of weights, 32 rows x
 // 256 bytes, is one 16-byte load per staging thread, passed through LDS (row stride 272
 // bytes, conflict-free for the 16-byte operand reads); a chunk of x is one or two items per
-// staging thread (two k x eight columns each), interleaved into the transposed chunk buffer.
+// staging thread (two k x eight columns each), or at 32 columns four whole-line pieces,
+// interleaved into the transposed chunk buffer.
 //
 // Pipeline: a staging thread keeps its loads of four chunks (three above 16 columns) in
-// flight in registers and stores a chunk to LDS (two buffers) one chunk ahead of its use.  Every request is unconditional --
-// past the end of K it repeats the last chunk, unused -- and the chunks of the longest K
-// (kStreamBodies of them: K <= 6144) are written out nested, chunk c + 1 inside the "if" of
-// chunk c, instead of looped over, because vector loads return in order and are waited for by
-// count: only with a fixed number of requests between a request and its use can the compiler
-// wait for the oldest alone, and where a loop closes, or two paths meet, its count starts
-// over (it waits there for nearly everything in flight, and the ring needs as many chunks
-// again to fill).
+// flight in registers and stores a chunk to LDS (two buffers) one chunk ahead of its use.
+// Every request is unconditional -- past the end of K it repeats the last chunk, unused --
+// and the chunks of a workgroup (at most kStreamBodies) are written out nested, chunk c + 1
+// inside the "if" of chunk c, instead of looped over, because vector loads return in order
+// and are waited for by count: only with a fixed number of requests between a request and its
+// use can the compiler wait for the oldest alone, and where a loop closes, or two paths meet,
+// its count starts over (it waits there for nearly everything in flight, and the ring needs
+// as many chunks again to fill).
 
 // The pair table of this tile: entry (byte, copy) at byte * 128 + copy * 4, 32 copies.  The
 // LDS serves a 4-byte read of a wavefront in two halves of 32 lanes, so lane & 31 picking the
