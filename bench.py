@@ -60,14 +60,20 @@ def make_weights(torch, nf4, m: int, k: int, copies: int, seed: int):
     return out
 
 
-def graph_time(torch, launch, n_launches: int, reps: int = 5) -> float:
+#: a timed window holds at least this many launches (a graph of fewer is replayed back to back)
+MIN_WINDOW_LAUNCHES = 200
+
+
+def graph_time(torch, launch, n_launches: int, reps: int = 5, min_window: int = MIN_WINDOW_LAUNCHES) -> float:
     """Capture ``n_launches`` calls of ``launch(i)`` into a HIP graph, once per timed window
     with ``i`` running on from where the window before stopped (so a window never starts on
     the copies the one before it has just left in the caches), and return the median over
-    the ``reps`` windows of the average milliseconds per launch.  Events on the capture
-    stream bracket each replay."""
+    the ``reps`` windows of the average milliseconds per launch.  A window is the graph
+    replayed back to back until it holds at least ``min_window`` launches (a window of a few
+    launches is mostly its own start and end); events on the capture stream bracket it."""
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
+    replays = max(1, -(-min_window // n_launches))
     with torch.cuda.stream(side):
         for i in range(min(n_launches, 32)):
             launch(i)
@@ -86,16 +92,31 @@ def graph_time(torch, launch, n_launches: int, reps: int = 5) -> float:
         side.synchronize()
         e0 = torch.cuda.Event(enable_timing=True)
         e1 = torch.cuda.Event(enable_timing=True)
+        # untimed: a card that has been idle runs its first milliseconds at a lower clock; replay
+        # until two windows in a row agree to 2% (at most 0.3 s)
+        t_spin = time.perf_counter()
+        last = None
+        while time.perf_counter() - t_spin < 0.3:
+            e0.record(side)
+            for _ in range(replays):
+                graphs[0].replay()
+            e1.record(side)
+            side.synchronize()
+            now = e0.elapsed_time(e1)
+            if last is not None and abs(now - last) <= 0.02 * last:
+                break
+            last = now
         windows = []
         for graph in graphs[1:]:
             e0.record(side)
-            graph.replay()
+            for _ in range(replays):
+                graph.replay()
             e1.record(side)
             side.synchronize()
             windows.append(e0.elapsed_time(e1))
     torch.cuda.current_stream().wait_stream(side)
     windows.sort()
-    return windows[len(windows) // 2] / n_launches
+    return windows[len(windows) // 2] / (n_launches * replays)
 
 
 #: kernel forms of the N=1 path, by the environment switches the library reads per launch
@@ -539,6 +560,16 @@ def main() -> int:
             "traffic": GEMV_TRAFFIC_BYTES if (M, K) == (13824, 5120) else None,
             "kernel": "gemv_ring_rows<5,2,true> (two-term levels)",
             "algorithmic_bytes_per_launch": by,
+            # the figures of the other legs that belong beside this one (each is also given in
+            # full further down the line): fractions of 8 TB/s for the same launches through the
+            # other two kernel forms, and of each model's bandwidth roofline for the decode legs
+            "other": {
+                "one_term_frac": by / (forms["one_term"] * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                "one_term_us_per_launch": forms["one_term"] * 1e3,
+                "fp32_levels_frac": by / (forms["fp32_levels"] * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                "fp32_levels_us_per_launch": forms["fp32_levels"] * 1e3,
+                "window_launches": max(args.steps, MIN_WINDOW_LAUNCHES),
+            },
         },
         # the same launches on the same copies through the other two kernel forms
         "roofline_one_term": roofline_of(forms["one_term"], "gemv_ring_rows<5,1,true> (one bf16 level)",
@@ -548,6 +579,8 @@ def main() -> int:
     }
     if not args.no_shapes:
         out["gemv_shapes"] = bench_gemv_shapes(torch, nf4)
+        for row in out["gemv_shapes"]:
+            out["roofline"]["other"][f"gemv_{row['M']}x{row['K']}_frac"] = row["hbm_frac"]
     if not args.no_decode:
         rows = []
         for name in (n.strip() for n in args.decode_models.split(",")):
@@ -567,6 +600,12 @@ def main() -> int:
                 fast["gemv_levels"] = "one bf16 term (CHR_NF4_GEMV_TERMS=1)"
                 rows.append(fast)
         out["decode"] = rows
+        for row in rows:
+            key = row["model"].lower().replace(" ", "_").replace(".", "")
+            if row["gemv_levels"].startswith("one"):
+                key += "_one_term"
+            out["roofline"]["other"][f"decode_{key}_roofline_frac"] = row["roofline_frac"]
+            out["roofline"]["other"][f"decode_{key}_tok_s"] = row["tok_s"]
     if not args.no_prefill:
         only = [v.strip() for v in args.prefill_layers.split(",") if v.strip()]
         widths = tuple(int(v) for v in args.prefill_widths.split(",") if v.strip())

@@ -71,6 +71,7 @@ def build(force: bool = True, verbose: bool = False) -> str:
 
     ring_asm_check.check_source(hipcc(), HIPCC_FLAGS, os.path.join(CSRC, "nf4_gemv.hip"))
     build_host_check()
+    build_launch_probe()
     return LIB
 
 
@@ -91,6 +92,25 @@ def build_host_check() -> str | None:
     if proc.returncode != 0:
         raise RuntimeError(f"hipcc failed on host_check.cpp ({proc.returncode}):\n{proc.stderr}")
     return HOST_CHECK
+
+
+#: A stand-alone measurement program (no library code, no torch): launch floor, streaming-read
+#: ceiling, where the time before a launch's first product goes, and chains of launches that
+#: overlap through device words.  ``profiles/launch_*.txt`` are its output.
+LAUNCH_PROBE_SRC = os.path.join(CSRC, "launch_probe.hip")
+LAUNCH_PROBE = os.path.splitext(LAUNCH_PROBE_SRC)[0]
+
+
+def build_launch_probe() -> str:
+    cmd = [hipcc(), "--offload-arch=gfx950", "-O3", "-std=c++17",
+           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           # scalar kernel arguments arrive in registers (one of the things the program measures)
+           "-mllvm", "-amdgpu-kernarg-preload-count=16",
+           "-o", LAUNCH_PROBE, LAUNCH_PROBE_SRC]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed on launch_probe.hip ({proc.returncode}):\n{proc.stderr}")
+    return LAUNCH_PROBE
 
 
 if __name__ == "__main__":
