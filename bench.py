@@ -121,8 +121,11 @@ def graph_time(torch, launch, n_launches: int, reps: int = 5, min_window: int = 
 
 #: kernel forms of the N=1 path, by the environment switches the library reads per launch
 GEMV_FORMS = {
-    # levels as head + tail bf16 (17 significant bits), exact products, fp32 accumulation
-    "two_term": {"CHR_NF4_GEMV_STAGED": None, "CHR_NF4_GEMV_TERMS": None},
+    # levels rounded to binary16 (11 significant bits) against x staged as binary16 times a power
+    # of two (exact for bf16 x), exact products, fp32 accumulation: the default
+    "f16_levels": {"CHR_NF4_GEMV_STAGED": None, "CHR_NF4_GEMV_TERMS": None},
+    # levels as head + tail bf16 (17 significant bits): 8-byte lookups
+    "two_term": {"CHR_NF4_GEMV_STAGED": None, "CHR_NF4_GEMV_TERMS": "2"},
     # levels rounded to one bf16
     "one_term": {"CHR_NF4_GEMV_STAGED": None, "CHR_NF4_GEMV_TERMS": "1"},
     # 16 fp32 levels, x widened to fp32, 128-bit loads (the plain kernel)
@@ -179,7 +182,7 @@ def bench_gemv(torch, nf4, steps: int, warmup: int, copies: int):
     eager_ms = (time.perf_counter() - t0) * 1e3 / steps
     ms = graph_time(torch, launch, steps)
     forms = {}
-    for name in ("one_term", "fp32_levels"):
+    for name in ("two_term", "one_term", "fp32_levels"):
         with gemv_form(name):
             forms[name] = graph_time(torch, launch, steps)
     del weights
@@ -348,7 +351,7 @@ def bench_decode(torch, spec_name: str, prompt_len: int, new_tokens: int, schedu
         "roofline_ms_per_token": roof_ms, "roofline_tok_s": 1e3 / roof_ms,
         "roofline_frac": roof_ms / ms_tok, "achieved_gbps": bytes_tok / (ms_tok * 1e-3) / 1e9,
         "weights_load_s": load_s,
-        "gemv_levels": "two bf16 terms (default)",
+        "gemv_levels": "binary16 levels (default)",
     }
     del graph, state, weights
     torch.cuda.empty_cache()
@@ -539,10 +542,11 @@ def main() -> int:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        # what the timed kernel multiplies: NF4 levels kept as two bf16 terms (head + tail,
-        # 17 significant bits) times bf16 activations, exact products, fp32 accumulation
-        "dtype": "bf16",
-        "dtype_note": "levels as head+tail bf16 pairs x bf16 activations (v_dot2c_f32_bf16), "
+        # what the timed kernel multiplies: NF4 levels rounded to binary16 times the bf16
+        # activations held as binary16 (exactly: a power of two puts the largest in range),
+        # exact products, fp32 accumulation; bf16 in, bf16 out
+        "dtype": "f16",
+        "dtype_note": "binary16 level pairs x bf16 activations staged as binary16 (v_dot2c_f32_f16), "
                       "fp32 accumulate, one bf16 rounding of y",
         "data": "synthetic",
         "config": {
@@ -558,12 +562,14 @@ def main() -> int:
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS,
             "traffic": GEMV_TRAFFIC_BYTES if (M, K) == (13824, 5120) else None,
-            "kernel": "gemv_ring_rows<5,2,true> (two-term levels)",
+            "kernel": "gemv_ring_rows<5,3,true> (binary16 levels)",
             "algorithmic_bytes_per_launch": by,
             # the figures of the other legs that belong beside this one (each is also given in
             # full further down the line): fractions of 8 TB/s for the same launches through the
             # other two kernel forms, and of each model's bandwidth roofline for the decode legs
             "other": {
+                "two_term_frac": by / (forms["two_term"] * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                "two_term_us_per_launch": forms["two_term"] * 1e3,
                 "one_term_frac": by / (forms["one_term"] * 1e-3) / 1e9 / HBM_PEAK_GBPS,
                 "one_term_us_per_launch": forms["one_term"] * 1e3,
                 "fp32_levels_frac": by / (forms["fp32_levels"] * 1e-3) / 1e9 / HBM_PEAK_GBPS,
@@ -571,7 +577,9 @@ def main() -> int:
                 "window_launches": max(args.steps, MIN_WINDOW_LAUNCHES),
             },
         },
-        # the same launches on the same copies through the other two kernel forms
+        # the same launches on the same copies through the other kernel forms
+        "roofline_two_term": roofline_of(forms["two_term"], "gemv_ring_rows<5,2,true> (head + tail bf16 levels)",
+                                         "two bf16 terms per level x bf16 activations"),
         "roofline_one_term": roofline_of(forms["one_term"], "gemv_ring_rows<5,1,true> (one bf16 level)",
                                          "bf16 levels x bf16 activations"),
         "roofline_fp32_levels": roofline_of(forms["fp32_levels"], "gemv_stream (plain)",
@@ -593,17 +601,21 @@ def main() -> int:
             rows.append(bench_decode(torch, name, prompt, new, args.schedule, width,
                                      torch_glue=(name == "14b")))
             if name == "14b":
-                # the same model with one-term (bf16) levels in the GEMVs: the faster,
-                # less exact form a caller can opt into
-                with gemv_form("one_term"):
-                    fast = bench_decode(torch, name, prompt, new, args.schedule, width, torch_glue=False)
-                fast["gemv_levels"] = "one bf16 term (CHR_NF4_GEMV_TERMS=1)"
-                rows.append(fast)
+                # the same model with the other two forms of the levels: two bf16 terms (more
+                # exact, 8-byte lookups) and one bf16 term (less exact)
+                for form, label in (("two_term", "two bf16 terms (CHR_NF4_GEMV_TERMS=2)"),
+                                    ("one_term", "one bf16 term (CHR_NF4_GEMV_TERMS=1)")):
+                    with gemv_form(form):
+                        other = bench_decode(torch, name, prompt, new, args.schedule, width, torch_glue=False)
+                    other["gemv_levels"] = label
+                    rows.append(other)
         out["decode"] = rows
         for row in rows:
             key = row["model"].lower().replace(" ", "_").replace(".", "")
             if row["gemv_levels"].startswith("one"):
                 key += "_one_term"
+            elif row["gemv_levels"].startswith("two"):
+                key += "_two_term"
             out["roofline"]["other"][f"decode_{key}_roofline_frac"] = row["roofline_frac"]
             out["roofline"]["other"][f"decode_{key}_tok_s"] = row["tok_s"]
     if not args.no_prefill:

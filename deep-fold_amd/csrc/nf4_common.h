@@ -33,19 +33,19 @@ __device__ __forceinline__ float bf16_to_f32(uint16_t h) {
   return bits_to_f32(static_cast<uint32_t>(h) << 16);
 }
 
-// f32 -> bf16 bits, round to nearest even; NaN stays NaN
-// (same closed form as internal/f16/f16.go:93-106).
+// f32 -> bf16 bits, round to nearest even, NaN stays NaN: the conversion instruction of gfx950
+// (v_cvt_pk_bf16_f32), which rounds every finite value as the closed form of
+// internal/f16/f16.go:93-106 does.
 __device__ __forceinline__ uint16_t f32_to_bf16(float f) {
-  uint32_t b = f32_to_bits(f);
-  if ((b & 0x7FFFFFFFu) > 0x7F800000u) {
-    uint32_t n = b >> 16;
-    if ((n & 0x7Fu) == 0) {
-      n |= 1u;
-    }
-    return static_cast<uint16_t>(n);
-  }
-  b += 0x7FFFu + ((b >> 16) & 1u);
-  return static_cast<uint16_t>(b >> 16);
+  return __builtin_bit_cast(uint16_t, static_cast<__bf16>(f));
+}
+
+// two values in one instruction: lo in bits 0..15, hi in bits 16..31
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2(float lo, float hi) {
+  typedef __attribute__((ext_vector_type(2))) float F32x2;
+  typedef __attribute__((ext_vector_type(2))) __bf16 Bf16x2Bits;
+  const F32x2 f = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, Bf16x2Bits));
 }
 
 // binary16 bits -> f32, exact (v_cvt_f32_f16 widens subnormals exactly).

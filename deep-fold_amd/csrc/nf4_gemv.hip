@@ -21,10 +21,14 @@
 // where the staged kernel's set-up costs more than its inner loop returns.
 //
 // Numerics.  Plain: weight = fp32 LUT * fp32(scale) never rounded below fp32, x widened
-// bf16->fp32 (gpu/nf4/nf4_gemv.cu:70-101, 217-245).  Staged: levels rounded to bf16,
-// exact products, the fp16 scale applied in fp32 to each 16-weight partial: the
-// precision class of the reference's tensor-core path (gpu/nf4/nf4_gemm.cu:322).  Both:
-// fp32 accumulation, residual / bias added in fp32, one bf16 rounding at the store.
+// bf16->fp32 (gpu/nf4/nf4_gemv.cu:70-101, 217-245).  Staged and ring kernels, by the form of
+// the levels (CHR_NF4_GEMV_TERMS): 3, the default: levels rounded to binary16 (2^-12 relative)
+// against x staged as binary16 times a power of two, which holds every bf16 element within
+// 2^-29 of the largest exactly; 2: levels as two bf16 terms (below 2^-17), 8-byte lookups;
+// 1: levels rounded to bf16 (2^-9), the precision class of the reference's tensor-core path
+// (gpu/nf4/nf4_gemm.cu:322).  In all three the products are exact and the fp16 scale is
+// applied in fp32 to each 16-weight partial.  Both families: fp32 accumulation, residual /
+// bias added in fp32, one bf16 rounding at the store.
 
 #include "nf4_common.h"
 #include "nf4_gemv_ring_regs.h"
@@ -44,6 +48,12 @@ struct GemvLds {
   float lut[16];
   float part[kMaxWaves];
   float ksum[kMaxWaves][4];  // K-split: per-wavefront partial dot products of a row group
+};
+
+// The kernels that stage x in LDS keep two things more in their slot of small statics.
+struct StagedLds : GemvLds {
+  float vmax[kMaxWaves];  // per-wavefront maxima (x staged as binary16)
+  int xexp;               // x staged as binary16: the power of two it was multiplied by
 };
 
 __device__ __forceinline__ float fma8(const Levels8 &v, const float *xf, float acc) {
@@ -92,6 +102,94 @@ __device__ __forceinline__ float block_sum(float v, float *part) {
   }
   __syncthreads();
   return s;
+}
+
+// ---- largest magnitude of a staged vector, on the bf16 bit patterns ------------------------
+// The magnitude bits of a bf16 value order like the value's magnitude, so the largest element is
+// an unsigned 16-bit maximum: one packed instruction per two elements.
+typedef uint16_t U16x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
+  return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(U16x2, a),
+                                                                __builtin_bit_cast(U16x2, b)));
+}
+
+// running maximum of the magnitudes of two bf16 values, per half of the dword
+__device__ __forceinline__ uint32_t mag_max(uint32_t acc, uint32_t pair) {
+  return pk_max_u16(acc, pair & 0x7FFF7FFFu);
+}
+
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_u32(uint32_t v) {
+  return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), CTRL, 0xF, 0xF, true));
+}
+
+// maximum per 16-bit half over each row of 16 lanes, in every lane of the row
+__device__ __forceinline__ uint32_t row_pk_max(uint32_t v) {
+  v = pk_max_u16(v, dpp_u32<kDppQuadXor1>(v));
+  v = pk_max_u16(v, dpp_u32<kDppQuadXor2>(v));
+  v = pk_max_u16(v, dpp_u32<kDppRowHalfMirror>(v));
+  v = pk_max_u16(v, dpp_u32<kDppRowMirror>(v));
+  return v;
+}
+
+// Sum of `sum` and per-half maximum of `pk` over the workgroup (16 wavefronts), the same in
+// every thread, with one barrier: wavefront totals go to LDS, lane l reads the total of
+// wavefront l % 16, and a row of 16 lanes folds them.  The caller's next barrier is what
+// separates this use of the two arrays from any later one.
+template <bool WITH_SUM>
+__device__ __forceinline__ void block_fold(float &sum, uint32_t &pk, float *part, float *vmax) {
+  static_assert(kStagedThreads == 16 * kWave, "one total per lane of a 16-lane row");
+  uint32_t *vm = reinterpret_cast<uint32_t *>(vmax);
+  if constexpr (WITH_SUM) {
+    sum = wave_sum(sum);
+  }
+  pk = row_pk_max(pk);
+  const uint32_t r0 = __builtin_amdgcn_readlane(pk, 0), r1 = __builtin_amdgcn_readlane(pk, 16);
+  const uint32_t r2 = __builtin_amdgcn_readlane(pk, 32), r3 = __builtin_amdgcn_readlane(pk, 48);
+  pk = pk_max_u16(pk_max_u16(r0, r1), pk_max_u16(r2, r3));
+  const int lane = threadIdx.x & (kWave - 1);
+  if (lane == 0) {
+    if constexpr (WITH_SUM) {
+      part[threadIdx.x >> 6] = sum;
+    }
+    vm[threadIdx.x >> 6] = pk;
+  }
+  __syncthreads();
+  if constexpr (WITH_SUM) {
+    sum = group_sum<16>(part[lane & 15]);
+  }
+  pk = row_pk_max(vm[lane & 15]);
+}
+
+// the larger half of a packed pair of bf16 magnitudes, as a float
+__device__ __forceinline__ float larger_half_bf16(uint32_t pk) {
+  return bits_to_f32(max(pk & 0xFFFFu, pk >> 16) << 16);
+}
+
+// ---- x as binary16 -------------------------------------------------------------------
+// With levels kept as binary16 (11 significant bits against bf16's 8) the products need x as
+// binary16 too.  A bf16 value has 8 significant bits, so it is a binary16 value exactly
+// whenever its exponent fits; the staged vector is therefore multiplied by the power of two
+// that puts its largest magnitude in [2^14, 2^15): every element within 2^-29 of the largest
+// converts exactly, smaller ones land on binary16's subnormal grid (absolute error below
+// 2^-39 of the largest element: far under the fp32 accumulation's own rounding).  The row
+// sums are multiplied by the inverse power at the end.  Largest magnitude 0 (or not finite):
+// power 0 (what is not finite stays so through the products).
+__device__ __forceinline__ int x_power_for(float largest) {
+  const uint32_t b = f32_to_bits(largest) & 0x7FFFFFFFu;
+  if (b == 0u || b >= 0x7F800000u) {
+    return 0;
+  }
+  // -113 (the largest bf16) .. 141 (a subnormal reads as exponent -127 and ends up below 2^15 too)
+  return 14 - (static_cast<int>(b >> 23) - 127);
+}
+
+// two bf16 values (one dword) -> the same two values times 2^power as a binary16 pair
+__device__ __forceinline__ uint32_t bf16x2_to_f16x2(uint32_t pair, int power) {
+  const float lo = __builtin_ldexpf(bf16_lo(pair), power);
+  const float hi = __builtin_ldexpf(bf16_hi(pair), power);
+  return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo, hi));
 }
 
 // ---- activations staged in LDS ------------------------------------------------------
@@ -181,9 +279,7 @@ __device__ __forceinline__ uint4 merged_attn_piece(const StreamArgs &a, int i) {
   uint32_t r[4];
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
-    const uint32_t lo16 = f32_to_bf16(o[2 * q] * inv);
-    const uint32_t hi16 = f32_to_bf16(o[2 * q + 1] * inv);
-    r[q] = lo16 | (hi16 << 16);
+    r[q] = f32x2_to_bf16x2(o[2 * q] * inv, o[2 * q + 1] * inv);
   }
   return make_uint4(r[0], r[1], r[2], r[3]);
 }
@@ -221,29 +317,60 @@ __device__ __forceinline__ void x_request(const StreamArgs &a, uint4 (&v)[kXKeep
 
 // Fast staging, second half: normalise if asked, store the pieces, barrier.  With rms_w
 // the value stored is bf16( (w*x) * rsqrt(mean(x^2)+eps) ), i.e. what a separate RMSNorm
-// launch would have handed over (gpu/nf4/nf4_gemv.cu:264-289).
-__device__ __forceinline__ void x_store(const StreamArgs &a, uint4 *xs, float *part,
+// launch would have handed over (gpu/nf4/nf4_gemv.cu:264-289).  F16: those bf16 values are
+// stored as binary16 times a power of two (x_power_for), which lds.xexp then holds.
+template <bool F16>
+__device__ __forceinline__ void x_store(const StreamArgs &a, uint4 *xs, StagedLds &lds,
                                         const uint4 (&v)[kXKeep], const uint4 (&g)[kXKeep]) {
   const int nk = a.K >> 3;
   const int nvec = a.K_pad >> 3;
   zero_unused_slots(xs, a.K_pad);
   float inv = 1.f;
+  int power = 0;
   if (a.rms_w != nullptr) {
     float ss = 0.f;
+    uint32_t xm = 0u, gm = 0u;  // largest magnitudes of x and of the norm weights, per dword half
 #pragma unroll
     for (int j = 0; j < kXKeep; ++j) {
       const int i = threadIdx.x + j * kStagedThreads;
       const uint32_t u[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
+      const uint32_t gw[4] = {g[j].x, g[j].y, g[j].z, g[j].w};
       float s4 = 0.f;
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         s4 = fmaf(bf16_lo(u[q]), bf16_lo(u[q]), s4);
         s4 = fmaf(bf16_hi(u[q]), bf16_hi(u[q]), s4);
+        if constexpr (F16) {
+          // (a vector past the end repeats the last one: the same maxima)
+          xm = mag_max(xm, u[q]);
+          gm = mag_max(gm, gw[q]);
+        }
       }
       ss += i < nk ? s4 : 0.f;
     }
-    ss = block_sum(ss, part);
-    inv = rsqrtf(ss / static_cast<float>(a.K) + a.rms_eps);
+    if constexpr (F16) {
+      // one word: the weights' maximum in the high half, x's in the low half
+      uint32_t pk = (max(gm & 0xFFFFu, gm >> 16) << 16) | max(xm & 0xFFFFu, xm >> 16);
+      block_fold<true>(ss, pk, lds.part, lds.vmax);
+      inv = rsqrtf(ss / static_cast<float>(a.K) + a.rms_eps);
+      // No normalised value is larger than bf16((G * X) * inv) with G, X the two maxima: the
+      // product of two bf16 values is exact in fp32, and multiplying by inv and the two
+      // roundings keep the order of magnitudes.
+      const float bound = (bits_to_f32(pk & 0xFFFF0000u) * bits_to_f32(pk << 16)) * inv;
+      power = x_power_for(bf16_to_f32(f32_to_bf16(bound)));
+    } else {
+      ss = block_sum(ss, lds.part);
+      inv = rsqrtf(ss / static_cast<float>(a.K) + a.rms_eps);
+    }
+  } else if constexpr (F16) {
+    uint32_t xm = 0u;
+#pragma unroll
+    for (int j = 0; j < kXKeep; ++j) {
+      xm = mag_max(mag_max(mag_max(mag_max(xm, v[j].x), v[j].y), v[j].z), v[j].w);
+    }
+    float none = 0.f;
+    block_fold<false>(none, xm, lds.part, lds.vmax);
+    power = x_power_for(larger_half_bf16(xm));
   }
 #pragma unroll
   for (int j = 0; j < kXKeep; ++j) {
@@ -256,26 +383,61 @@ __device__ __forceinline__ void x_store(const StreamArgs &a, uint4 *xs, float *p
         uint32_t r[4];
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          const uint32_t lo = f32_to_bf16((bf16_lo(gw[q]) * bf16_lo(u[q])) * inv);
-          const uint32_t hi = f32_to_bf16((bf16_hi(gw[q]) * bf16_hi(u[q])) * inv);
-          r[q] = lo | (hi << 16);
+          r[q] = f32x2_to_bf16x2((bf16_lo(gw[q]) * bf16_lo(u[q])) * inv, (bf16_hi(gw[q]) * bf16_hi(u[q])) * inv);
         }
         o = make_uint4(r[0], r[1], r[2], r[3]);
       }
+      if constexpr (F16) {
+        o = make_uint4(bf16x2_to_f16x2(o.x, power), bf16x2_to_f16x2(o.y, power),
+                       bf16x2_to_f16x2(o.z, power), bf16x2_to_f16x2(o.w, power));
+      }
       xs[x_slot(i)] = o;
+    }
+  }
+  if constexpr (F16) {
+    if (threadIdx.x == 0) {
+      lds.xexp = power;
     }
   }
   __syncthreads();
 }
 
+// F16 staging of what the loops below left as bf16: the largest magnitude, then the conversion,
+// every thread on the pieces it alone touches.
+__device__ __forceinline__ void staged_to_f16(const StreamArgs &a, uint4 *xs, StagedLds &lds) {
+  const int nvec = a.K_pad >> 3;
+  uint32_t xm = 0u;
+  for (int i = threadIdx.x; i < nvec; i += kStagedThreads) {
+    const uint4 q = xs[x_slot(i)];
+    xm = mag_max(mag_max(mag_max(mag_max(xm, q.x), q.y), q.z), q.w);
+  }
+  float none = 0.f;
+  block_fold<false>(none, xm, lds.part, lds.vmax);
+  const int power = x_power_for(larger_half_bf16(xm));
+  for (int i = threadIdx.x; i < nvec; i += kStagedThreads) {
+    const uint4 q = xs[x_slot(i)];
+    xs[x_slot(i)] = make_uint4(bf16x2_to_f16x2(q.x, power), bf16x2_to_f16x2(q.y, power),
+                               bf16x2_to_f16x2(q.z, power), bf16x2_to_f16x2(q.w, power));
+  }
+  if (threadIdx.x == 0) {
+    lds.xexp = power;
+  }
+  __syncthreads();
+}
+
 // Staging for the other cases: the attention merge, a ragged K, unaligned pointers.
-__device__ __forceinline__ void stage_x(const StreamArgs &a, uint4 *xs, float *part) {
+template <bool F16>
+__device__ __forceinline__ void stage_x(const StreamArgs &a, uint4 *xs, StagedLds &lds) {
+  float *part = lds.part;
   zero_unused_slots(xs, a.K_pad);
   if (a.attn_state != nullptr) {
     for (int i = threadIdx.x; i < (a.K_pad >> 3); i += kStagedThreads) {
       xs[x_slot(i)] = merged_attn_piece(a, i);
     }
     __syncthreads();
+    if constexpr (F16) {
+      staged_to_f16(a, xs, lds);
+    }
     return;
   }
   {
@@ -302,6 +464,9 @@ __device__ __forceinline__ void stage_x(const StreamArgs &a, uint4 *xs, float *p
     }
   }
   __syncthreads();
+  if constexpr (F16) {
+    staged_to_f16(a, xs, lds);
+  }
 }
 
 __device__ __forceinline__ void widen8(const uint4 v, float *xf) {
@@ -341,13 +506,55 @@ __device__ __forceinline__ void rows_step(const uint32_t (&w)[R][NW], const floa
 }
 
 constexpr int kStagedSmallBytes = 512;  // GemvLds of a staged kernel, after the table
-static_assert(sizeof(GemvLds) <= kStagedSmallBytes, "GemvLds must fit its slot");
+static_assert(sizeof(StagedLds) <= kStagedSmallBytes, "the small statics must fit their slot");
 
 typedef __attribute__((ext_vector_type(2))) __bf16 Bf16x2;
 
 __device__ __forceinline__ float dot2_bf16(uint32_t a, uint32_t b, float acc) {
   return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(Bf16x2, a),
                                          __builtin_bit_cast(Bf16x2, b), acc, false);
+}
+
+typedef __attribute__((ext_vector_type(2))) _Float16 F16x2v;
+
+__device__ __forceinline__ float dot2_f16(uint32_t a, uint32_t b, float acc) {
+  return __builtin_amdgcn_fdot2(__builtin_bit_cast(F16x2v, a), __builtin_bit_cast(F16x2v, b), acc, false);
+}
+
+// Products of one level pair with one pair of x for the single-lookup forms: bf16 levels times
+// bf16 x (LEVELS 1), binary16 levels times x staged as binary16 (LEVELS 3).
+template <int LEVELS>
+__device__ __forceinline__ float dot2_levels(uint32_t a, uint32_t b, float acc) {
+  if constexpr (LEVELS == 3) {
+    return dot2_f16(a, b, acc);
+  } else {
+    return dot2_bf16(a, b, acc);
+  }
+}
+
+// ---- binary16 pair table --------------------------------------------------------------
+// The pair table of nf4_common.h with the levels rounded to binary16 instead of bf16: 11
+// significant bits, 2^-12 relative weight error against 2^-9, same table size, same single
+// 4-byte lookup per two weights.  Filled by a workgroup of exactly 16 wavefronts.
+constexpr uint32_t f16_bits_rne(uint32_t b) {  // finite, zero or of a magnitude binary16 holds as a normal number
+  if ((b & 0x7FFFFFFFu) == 0u) {
+    return (b >> 16) & 0x8000u;
+  }
+  uint32_t half = ((b >> 16) & 0x8000u) | ((((b >> 23) & 0xFFu) - 112u) << 10) | ((b & 0x7FFFFFu) >> 13);
+  const uint32_t rem = b & 0x1FFFu;
+  if (rem > 0x1000u || (rem == 0x1000u && (half & 1u) != 0u)) {
+    ++half;
+  }
+  return half;
+}
+
+__device__ __forceinline__ void fill_pair_table_f16(uint32_t *table, int wave, int lane) {
+  const uint32_t lo = __builtin_bit_cast(uint16_t, static_cast<_Float16>(bits_to_f32(kLutBits[wave])));
+#pragma unroll
+  for (int j = 0; j < 16; ++j) {
+    const uint32_t hi = f16_bits_rne(kLevelBits[j]) << 16;
+    table[((wave + 16 * j) << 6) + lane] = lo | hi;
+  }
 }
 
 // ---- two-term pair table ----------------------------------------------------------------
@@ -587,6 +794,28 @@ __global__ __launch_bounds__(256) void gemv_stream(const StreamArgs a) {
   }
 }
 
+// The level table of a kernel that stages x in LDS, by the form of its levels.
+template <int TERMS>
+__device__ __forceinline__ void fill_level_table(uint4 *dyn_lds, int wave, int lane) {
+  if constexpr (TERMS == 1) {
+    fill_pair_table(reinterpret_cast<uint32_t *>(dyn_lds), wave, lane);
+  } else if constexpr (TERMS == 3) {
+    fill_pair_table_f16(reinterpret_cast<uint32_t *>(dyn_lds), wave, lane);
+  } else {
+    fill_pair2_table(reinterpret_cast<uint2 *>(dyn_lds), wave, lane);
+  }
+}
+
+// A row sum of the binary16 form is the sum over x * 2^power: divide the power out again.
+template <int TERMS>
+__device__ __forceinline__ float unscaled(float sum, int power) {
+  if constexpr (TERMS == 3) {
+    return __builtin_ldexpf(sum, -power);
+  } else {
+    return sum;
+  }
+}
+
 // ---- staged kernel: x in LDS, pair table, weight requests one item ahead -----------
 // Request half step t of R rows: 8 packed bytes per lane.  Lanes past the end of the row
 // read the row's last half chunk instead (in bounds, one instruction form for every
@@ -604,7 +833,8 @@ __device__ __forceinline__ void load_step(const uint8_t *const (&prow)[R],
 }
 
 // TERMS == 1: levels as one bf16 (pair table of dwords, 64 copies).  TERMS == 2: levels as
-// head + tail (two-term table, 32 copies of 8-byte entries).
+// head + tail (two-term table, 32 copies of 8-byte entries).  TERMS == 3: levels as one
+// binary16 against x staged as binary16 (same table shape as TERMS == 1).
 template <int R, int TERMS>
 __device__ __forceinline__ void dot_step(const uint2 (&w)[R], const uint16_t (&sc)[R],
                                          const uint4 *xs, int n_half, int t, int lane,
@@ -612,19 +842,19 @@ __device__ __forceinline__ void dot_step(const uint2 (&w)[R], const uint16_t (&s
   const bool on = (t << 6) + lane < n_half;
   const uint4 *xp = xs + (t << 7) + lane;
   const uint4 x0 = xp[0], x1 = xp[64];
-  if constexpr (TERMS == 1) {
+  if constexpr (TERMS != 2) {
     const uint32_t lane4 = static_cast<uint32_t>(lane) << 2;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       float pa = 0.f, pb = 0.f;
-      pa = dot2_bf16(pair_at<0>(w[r].x, lane4), x0.x, pa);
-      pb = dot2_bf16(pair_at<1>(w[r].x, lane4), x0.y, pb);
-      pa = dot2_bf16(pair_at<2>(w[r].x, lane4), x0.z, pa);
-      pb = dot2_bf16(pair_at<3>(w[r].x, lane4), x0.w, pb);
-      pa = dot2_bf16(pair_at<0>(w[r].y, lane4), x1.x, pa);
-      pb = dot2_bf16(pair_at<1>(w[r].y, lane4), x1.y, pb);
-      pa = dot2_bf16(pair_at<2>(w[r].y, lane4), x1.z, pa);
-      pb = dot2_bf16(pair_at<3>(w[r].y, lane4), x1.w, pb);
+      pa = dot2_levels<TERMS>(pair_at<0>(w[r].x, lane4), x0.x, pa);
+      pb = dot2_levels<TERMS>(pair_at<1>(w[r].x, lane4), x0.y, pb);
+      pa = dot2_levels<TERMS>(pair_at<2>(w[r].x, lane4), x0.z, pa);
+      pb = dot2_levels<TERMS>(pair_at<3>(w[r].x, lane4), x0.w, pb);
+      pa = dot2_levels<TERMS>(pair_at<0>(w[r].y, lane4), x1.x, pa);
+      pb = dot2_levels<TERMS>(pair_at<1>(w[r].y, lane4), x1.y, pb);
+      pa = dot2_levels<TERMS>(pair_at<2>(w[r].y, lane4), x1.z, pa);
+      pb = dot2_levels<TERMS>(pair_at<3>(w[r].y, lane4), x1.w, pb);
       const float scale = on ? f16_to_f32(sc[r]) : 0.f;
       acc[r] = fmaf(scale, pa + pb, acc[r]);
     }
@@ -681,7 +911,7 @@ template <int R, int S, bool SWIGLU, int TERMS>
 __global__ __launch_bounds__(1024) void gemv_staged(const StreamArgs a) {
   extern __shared__ uint4 dyn_lds[];  // [pair table][GemvLds][x pieces], table at address 0
   char *base = reinterpret_cast<char *>(dyn_lds);
-  GemvLds &lds = *reinterpret_cast<GemvLds *>(base + kPairTableBytes);
+  StagedLds &lds = *reinterpret_cast<StagedLds *>(base + kPairTableBytes);
   uint4 *xs = reinterpret_cast<uint4 *>(base + kPairTableBytes + kStagedSmallBytes);
   constexpr int U = SWIGLU ? R / 2 : R;
   const int lane = threadIdx.x & (kWave - 1);
@@ -718,13 +948,7 @@ __global__ __launch_bounds__(1024) void gemv_staged(const StreamArgs a) {
     }                                                                   \
   }
 
-  auto fill_table = [&]() {
-    if constexpr (TERMS == 1) {
-      fill_pair_table(reinterpret_cast<uint32_t *>(dyn_lds), wave, lane);
-    } else {
-      fill_pair2_table(reinterpret_cast<uint2 *>(dyn_lds), wave, lane);
-    }
-  };
+  auto fill_table = [&]() { fill_level_table<TERMS>(dyn_lds, wave, lane); };
 
   // Order of the first requests: x, then the first item of weights, and only then the
   // wait for x.  Vector loads return in order, so x must be the older request or its wait
@@ -738,10 +962,10 @@ __global__ __launch_bounds__(1024) void gemv_staged(const StreamArgs a) {
       group_pointers<R, SWIGLU>(a, first, prow, srow);
       CHR_REQUEST(wa, sa)
       fill_table();
-      x_store(a, xs, lds.part, xv, xg);
+      x_store<TERMS == 3>(a, xs, lds, xv, xg);
     } else {
       fill_table();
-      x_store(a, xs, lds.part, xv, xg);
+      x_store<TERMS == 3>(a, xs, lds, xv, xg);
     }
   } else {
     // The other staging forms read what they need in loops of their own; the first item
@@ -752,8 +976,10 @@ __global__ __launch_bounds__(1024) void gemv_staged(const StreamArgs a) {
       CHR_REQUEST(wa, sa)
     }
     fill_table();
-    stage_x(a, xs, lds.part);
+    stage_x<TERMS == 3>(a, xs, lds);
   }
+  // binary16 x: the power of two the row sums are divided by again
+  const int xexp = TERMS == 3 ? __builtin_amdgcn_readfirstlane(lds.xexp) : 0;
 
   // compute cursor: half step ci of the list = step ct of group cg
   int ci = 0, cg = first, ct = 0;
@@ -765,8 +991,8 @@ __global__ __launch_bounds__(1024) void gemv_staged(const StreamArgs a) {
     if constexpr (SWIGLU) {
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const float gsum = wave_sum(acc[u]);
-        const float usum = wave_sum(acc[U + u]);
+        const float gsum = unscaled<TERMS>(wave_sum(acc[u]), xexp);
+        const float usum = unscaled<TERMS>(wave_sum(acc[U + u]), xexp);
         const int r = row0 + u;
         if (lane == u && r < M) {
           a.y[0][r] = f32_to_bf16(silu(gsum) * usum);
@@ -777,7 +1003,7 @@ __global__ __launch_bounds__(1024) void gemv_staged(const StreamArgs a) {
       uint16_t *y = a.y[seg];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        float v = wave_sum(acc[u]);
+        float v = unscaled<TERMS>(wave_sum(acc[u]), xexp);
         const int r = row0 + u;
         if (add != nullptr) {
           v += uniform_bf16(add + min(r, M - 1));
@@ -910,12 +1136,12 @@ __device__ __forceinline__ void ring_x_wait(XRegs &x, uint32_t &tok) {
 // bf16 pairs of x (xw), the scale applied to the 16-weight partial.
 template <int TERMS>
 __device__ __forceinline__ float ring_row_dot(const uint32_t (&adr)[8], const uint32_t (&xw)[8]) {
-  if constexpr (TERMS == 1) {
+  if constexpr (TERMS != 2) {
     float pa = 0.f, pb = 0.f;
 #pragma unroll
     for (int j = 0; j < 8; j += 2) {
-      pa = dot2_bf16(lds0_u32(adr[j]), xw[j], pa);
-      pb = dot2_bf16(lds0_u32(adr[j + 1]), xw[j + 1], pb);
+      pa = dot2_levels<TERMS>(lds0_u32(adr[j]), xw[j], pa);
+      pb = dot2_levels<TERMS>(lds0_u32(adr[j + 1]), xw[j + 1], pb);
     }
     return pa + pb;
   } else {
@@ -969,7 +1195,7 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
   constexpr uint32_t kXsAddr = kPairTableBytes + kStagedSmallBytes;
   extern __shared__ uint4 dyn_lds[];  // [pair table][GemvLds][x pieces]
   char *base = reinterpret_cast<char *>(dyn_lds);
-  GemvLds &lds = *reinterpret_cast<GemvLds *>(base + kPairTableBytes);
+  StagedLds &lds = *reinterpret_cast<StagedLds *>(base + kPairTableBytes);
   uint4 *xs = reinterpret_cast<uint4 *>(base + kXsAddr);
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
@@ -1003,7 +1229,7 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
   const uint32_t v_wl = static_cast<uint32_t>(min(lane, rem - 1)) << 3;
   const uint32_t v_sl = static_cast<uint32_t>(min(lane, rem - 1) >> 2) << 1;
   const uint32_t x_lane = kXsAddr + (static_cast<uint32_t>(lane) << 4);
-  const uint32_t lane_off = TERMS == 1 ? static_cast<uint32_t>(lane) << 2
+  const uint32_t lane_off = TERMS != 2 ? static_cast<uint32_t>(lane) << 2
                                        : static_cast<uint32_t>(lane & 31) << 3;
   const uint64_t last_lanes = ragged ? ((uint64_t{1} << rem) - 1) : ~uint64_t{0};
 
@@ -1092,18 +1318,41 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
   const bool any_work = q_left > 0;
 #define CHR_RING_FILL_STEP(I) \
   if constexpr (NS > (I)) { CHR_RING_REQUEST(I, pieces == 1) }
-#define CHR_RING_FILL                                                                     \
+  // The first kRingEarlySlots slots are requested right after x, the others after the level
+  // table has been written: x then queues behind two half steps per wavefront instead of the
+  // whole ring (all slots at once: 7168x5120 7.2-7.4 us and 5120x5120 6.1 us against 7.0 and
+  // 5.8 us; one early slot is no better than two).
+  constexpr int kRingEarlySlots = 2;
+#define CHR_RING_FILL_A_STEP(I) \
+  if constexpr ((I) < kRingEarlySlots) { CHR_RING_FILL_STEP(I) }
+#define CHR_RING_FILL_B_STEP(I) \
+  if constexpr ((I) >= kRingEarlySlots) { CHR_RING_FILL_STEP(I) }
+#define CHR_RING_FILL_A                                                                   \
   if (any_work) {                                                                         \
-    CHR_RING_FILL_STEP(0)                                                                 \
-    CHR_RING_FILL_STEP(1)                                                                 \
-    CHR_RING_FILL_STEP(2)                                                                 \
-    CHR_RING_FILL_STEP(3)                                                                 \
-    CHR_RING_FILL_STEP(4)                                                                 \
-    CHR_RING_FILL_STEP(5)                                                                 \
-    CHR_RING_FILL_STEP(6)                                                                 \
-    CHR_RING_FILL_STEP(7)                                                                 \
+    CHR_RING_FILL_A_STEP(0)                                                               \
+    CHR_RING_FILL_A_STEP(1)                                                               \
+    CHR_RING_FILL_A_STEP(2)                                                               \
+    CHR_RING_FILL_A_STEP(3)                                                               \
+    CHR_RING_FILL_A_STEP(4)                                                               \
+    CHR_RING_FILL_A_STEP(5)                                                               \
+    CHR_RING_FILL_A_STEP(6)                                                               \
+    CHR_RING_FILL_A_STEP(7)                                                               \
+  }
+#define CHR_RING_FILL_B                                                                   \
+  if (any_work) {                                                                         \
+    CHR_RING_FILL_B_STEP(0)                                                               \
+    CHR_RING_FILL_B_STEP(1)                                                               \
+    CHR_RING_FILL_B_STEP(2)                                                               \
+    CHR_RING_FILL_B_STEP(3)                                                               \
+    CHR_RING_FILL_B_STEP(4)                                                               \
+    CHR_RING_FILL_B_STEP(5)                                                               \
+    CHR_RING_FILL_B_STEP(6)                                                               \
+    CHR_RING_FILL_B_STEP(7)                                                               \
     q_advance();                                                                          \
   }
+#define CHR_RING_FILL CHR_RING_FILL_A CHR_RING_FILL_B
+  // nothing of the compiler's own memory traffic crosses this, nor any statement of the chain
+#define CHR_RING_FENCE asm volatile("" : "+s"(tok)::"memory");
   // Order of the first requests: x, then the whole ring of weights, and only then the wait
   // for x: x is the older request, so its (exact) wait does not include the weights, and the
   // memory system works on the first NS half steps of every wavefront while the level table
@@ -1114,12 +1363,11 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
   if (stage_fast_ok(a)) {
     XRegs xr;
     ring_x_request(a, xr, tok);
-    CHR_RING_FILL
-    if constexpr (TERMS == 1) {
-      fill_pair_table(reinterpret_cast<uint32_t *>(dyn_lds), wave, lane);
-    } else {
-      fill_pair2_table(reinterpret_cast<uint2 *>(dyn_lds), wave, lane);
-    }
+    CHR_RING_FILL_A
+    if constexpr (kRingEarlySlots < NS) { CHR_RING_FENCE }
+    fill_level_table<TERMS>(dyn_lds, wave, lane);
+    if constexpr (kRingEarlySlots < NS) { CHR_RING_FENCE }
+    CHR_RING_FILL_B
     if (!any_work) {
       asm("s_waitcnt vmcnt(0)" : "+s"(tok));
     }
@@ -1130,26 +1378,29 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
       xv[j] = make_uint4(xr.v[j].x, xr.v[j].y, xr.v[j].z, xr.v[j].w);
       xg[j] = make_uint4(xr.g[j].x, xr.g[j].y, xr.g[j].z, xr.g[j].w);
     }
-    x_store(a, xs, lds.part, xv, xg);
+    x_store<TERMS == 3>(a, xs, lds, xv, xg);
   } else {
     // The other staging forms read what they need in loops of their own (loads the compiler
     // counts: its waits then also cover the half steps requested here, which are older).
     CHR_RING_FILL
-    if constexpr (TERMS == 1) {
-      fill_pair_table(reinterpret_cast<uint32_t *>(dyn_lds), wave, lane);
-    } else {
-      fill_pair2_table(reinterpret_cast<uint2 *>(dyn_lds), wave, lane);
-    }
-    stage_x(a, xs, lds.part);
+    fill_level_table<TERMS>(dyn_lds, wave, lane);
+    stage_x<TERMS == 3>(a, xs, lds);
   }
+  // binary16 x: the power of two the row sums are divided by again
+  const int xexp = TERMS == 3 ? __builtin_amdgcn_readfirstlane(lds.xexp) : 0;
+#undef CHR_RING_FENCE
 #undef CHR_RING_FILL
+#undef CHR_RING_FILL_B
+#undef CHR_RING_FILL_A
+#undef CHR_RING_FILL_B_STEP
+#undef CHR_RING_FILL_A_STEP
 #undef CHR_RING_FILL_STEP
 
   float acc[R] = {};
   auto finish_group = [&](int grp) {
     if constexpr (SWIGLU) {
-      const float gsum = wave_sum(acc[0]);
-      const float usum = wave_sum(acc[1]);
+      const float gsum = unscaled<TERMS>(wave_sum(acc[0]), xexp);
+      const float usum = unscaled<TERMS>(wave_sum(acc[1]), xexp);
       if (lane == 0) {
         a.y[0][grp] = f32_to_bf16(silu(gsum) * usum);
       }
@@ -1163,7 +1414,7 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
         add = third ? a.add[2] : a.add[1];
         row -= third ? seg_end1 : seg_end0;
       }
-      float v = wave_sum(acc[0]);
+      float v = unscaled<TERMS>(wave_sum(acc[0]), xexp);
       if (add != nullptr) {
         v += uniform_bf16(add + row);
       }
@@ -1436,11 +1687,26 @@ int forced_staged() {
   return -1;
 }
 
-// Terms a level is kept as in the staged kernel: 2 (head + tail bf16, the default) or 1
-// (one bf16, 2^-9 relative weight error; CHR_NF4_GEMV_TERMS=1, read on every launch).
+// Form of the levels in the kernels that stage x in LDS (CHR_NF4_GEMV_TERMS, read on every
+// launch): 3 = one binary16 against x staged as binary16 (2^-12 relative weight error; "3" or
+// "f16"), 2 = head + tail bf16 (below 2^-17; "2"), 1 = one bf16 (2^-9; "1").
+#ifndef CHR_NF4_DEFAULT_TERMS
+#define CHR_NF4_DEFAULT_TERMS 3
+#endif
 int level_terms() {
   const char *e = std::getenv("CHR_NF4_GEMV_TERMS");
-  return e != nullptr && e[0] == '1' && e[1] == '\0' ? 1 : 2;
+  if (e != nullptr && e[0] != '\0') {
+    if (e[0] == '1' && e[1] == '\0') {
+      return 1;
+    }
+    if (e[0] == '2' && e[1] == '\0') {
+      return 2;
+    }
+    if ((e[0] == '3' && e[1] == '\0') || (e[0] == 'f' && e[1] == '1' && e[2] == '6' && e[3] == '\0')) {
+      return 3;
+    }
+  }
+  return CHR_NF4_DEFAULT_TERMS;
 }
 
 constexpr int kThreads = 256;
@@ -1529,7 +1795,7 @@ int launch_stream(StreamArgs &a, int n_seg, bool staged, hipStream_t st) {
     const size_t dyn = staged_lds_bytes(a.K_pad);
     const int waves = kStagedThreads / kWave;
     const int grid = std::min(device_cu_count(), (total + waves - 1) / waves);
-    const bool one_term = level_terms() == 1;
+    const int terms = level_terms();
     constexpr bool kRingShape = (SWIGLU && R == 2) || (!SWIGLU && R == 1);
     const RingPiece ring = kRingShape && ring_wanted()
                                ? ring_piece_steps(x_half_steps(a.K_pad), SWIGLU) : RingPiece{0, 0};
@@ -1549,51 +1815,49 @@ int launch_stream(StreamArgs &a, int n_seg, bool staged, hipStream_t st) {
         };
         int rc = -6;
         // a row that is one piece of at most 5 half steps keeps its x in registers (the pair
-        // kernel only with one-term levels: two rows of two-term lookups leave no room)
+        // kernel only with single-lookup levels: two rows of two-term lookups leave no room)
         const bool one_piece = x_half_steps(a.K_pad) == ring_ns && ring_ns <= 5;
+        // the kernel for NS slots by the form of the levels
+#define CHR_GO_ROWS(NS, XREG, PAD)                                                        \
+  (terms == 1 ? go(gemv_ring_rows<NS, 1, XREG, PAD>)                                      \
+   : terms == 3 ? go(gemv_ring_rows<NS, 3, XREG, PAD>) : go(gemv_ring_rows<NS, 2, XREG, PAD>))
+#define CHR_GO_PAIRS(NS, XREG_OK)                                                         \
+  (terms == 2 ? go(gemv_ring_pairs<NS, 2, false>)                                         \
+   : terms == 1 ? ((XREG_OK) && one_piece ? go(gemv_ring_pairs<NS, 1, XREG_OK>) : go(gemv_ring_pairs<NS, 1, false>)) \
+                : ((XREG_OK) && one_piece ? go(gemv_ring_pairs<NS, 3, XREG_OK>) : go(gemv_ring_pairs<NS, 3, false>)))
         if constexpr (SWIGLU) {
           switch (ring_ns) {
-            case 4:
-              rc = !one_term ? go(gemv_ring_pairs<4, 2, false>)
-                   : one_piece ? go(gemv_ring_pairs<4, 1, true>) : go(gemv_ring_pairs<4, 1, false>);
-              break;
-            case 5:
-              rc = !one_term ? go(gemv_ring_pairs<5, 2, false>)
-                   : one_piece ? go(gemv_ring_pairs<5, 1, true>) : go(gemv_ring_pairs<5, 1, false>);
-              break;
-            case 6: rc = one_term ? go(gemv_ring_pairs<6, 1, false>) : go(gemv_ring_pairs<6, 2, false>); break;
+            case 4: rc = CHR_GO_PAIRS(4, true); break;
+            case 5: rc = CHR_GO_PAIRS(5, true); break;
+            case 6: rc = CHR_GO_PAIRS(6, false); break;
           }
         } else {
           switch (ring.pad > 0 ? -ring_ns : ring_ns) {
-            case -5: rc = one_term ? go(gemv_ring_rows<5, 1, false, 1>) : go(gemv_ring_rows<5, 2, false, 1>); break;
-            case -6: rc = one_term ? go(gemv_ring_rows<6, 1, false, 1>) : go(gemv_ring_rows<6, 2, false, 1>); break;
-            case -7: rc = one_term ? go(gemv_ring_rows<7, 1, false, 1>) : go(gemv_ring_rows<7, 2, false, 1>); break;
-            case -8: rc = one_term ? go(gemv_ring_rows<8, 1, false, 1>) : go(gemv_ring_rows<8, 2, false, 1>); break;
-            case 4:
-              if (one_piece) {
-                rc = one_term ? go(gemv_ring_rows<4, 1, true>) : go(gemv_ring_rows<4, 2, true>);
-              } else {
-                rc = one_term ? go(gemv_ring_rows<4, 1, false>) : go(gemv_ring_rows<4, 2, false>);
-              }
-              break;
-            case 5:
-              if (one_piece) {
-                rc = one_term ? go(gemv_ring_rows<5, 1, true>) : go(gemv_ring_rows<5, 2, true>);
-              } else {
-                rc = one_term ? go(gemv_ring_rows<5, 1, false>) : go(gemv_ring_rows<5, 2, false>);
-              }
-              break;
-            case 6: rc = one_term ? go(gemv_ring_rows<6, 1, false>) : go(gemv_ring_rows<6, 2, false>); break;
-            case 7: rc = one_term ? go(gemv_ring_rows<7, 1, false>) : go(gemv_ring_rows<7, 2, false>); break;
-            case 8: rc = one_term ? go(gemv_ring_rows<8, 1, false>) : go(gemv_ring_rows<8, 2, false>); break;
+            case -5: rc = CHR_GO_ROWS(5, false, 1); break;
+            case -6: rc = CHR_GO_ROWS(6, false, 1); break;
+            case -7: rc = CHR_GO_ROWS(7, false, 1); break;
+            case -8: rc = CHR_GO_ROWS(8, false, 1); break;
+            case 4: rc = one_piece ? CHR_GO_ROWS(4, true, 0) : CHR_GO_ROWS(4, false, 0); break;
+            case 5: rc = one_piece ? CHR_GO_ROWS(5, true, 0) : CHR_GO_ROWS(5, false, 0); break;
+            case 6: rc = CHR_GO_ROWS(6, false, 0); break;
+            case 7: rc = CHR_GO_ROWS(7, false, 0); break;
+            case 8: rc = CHR_GO_ROWS(8, false, 0); break;
           }
         }
+#undef CHR_GO_PAIRS
+#undef CHR_GO_ROWS
         if (rc != 0) {
           return rc;
         }
       }
-    } else if (one_term) {
+    } else if (terms == 1) {
       constexpr auto kern = gemv_staged<R, kItemSteps, SWIGLU, 1>;
+      if (prep_lds(kern, dyn) != 0) {
+        return -6;
+      }
+      kern<<<dim3(grid), dim3(kStagedThreads), dyn, st>>>(a);
+    } else if (terms == 3) {
+      constexpr auto kern = gemv_staged<R, kItemSteps, SWIGLU, 3>;
       if (prep_lds(kern, dyn) != 0) {
         return -6;
       }

@@ -57,18 +57,30 @@ def ulp_bf16(v: np.ndarray) -> np.ndarray:
 def takes_staged_gemv(m: int, k: int, *, fused: bool = False) -> bool:
     """Whether a GEMV launch of m rows takes the staged kernel (x in LDS: fused RMSNorm,
     ragged K, attention merge, and every matrix from 16M codes up).  That kernel multiplies
-    bf16-rounded levels, as the reference's tensor-core path does with the whole dequantised
-    weight (gpu/nf4/nf4_gemm.cu:322)."""
+    levels rounded to binary16 (or kept as two bf16 terms, or rounded to bf16:
+    ``staged_levels``); the reference's tensor-core path rounds the whole dequantised weight to
+    bf16 (gpu/nf4/nf4_gemm.cu:322)."""
     return fused or pyplan.gemv_is_staged(m, k)
 
 
+#: form of the levels the library takes when CHR_NF4_GEMV_TERMS is not set
+DEFAULT_TERMS = 3
+
+
+def env_terms() -> int:
+    return {"1": 1, "2": 2, "3": 3, "f16": 3}.get(os.environ.get("CHR_NF4_GEMV_TERMS", ""), DEFAULT_TERMS)
+
+
 def staged_levels(terms: int | None = None) -> np.ndarray:
-    """The 16 levels as the staged GEMV multiplies them, in float64: head = bf16(level) plus
-    tail = bf16(level - head) (two terms, the default), or the head alone
-    (CHR_NF4_GEMV_TERMS=1)."""
+    """The 16 levels as the staged GEMV multiplies them, in float64: rounded to binary16
+    (form 3, the default; x is staged as binary16 times a power of two, which is exact for every
+    element within 2^-29 of the largest, so the model leaves x alone), head = bf16(level) plus
+    tail = bf16(level - head) (form 2), or the head alone (form 1)."""
     if terms is None:
-        terms = 1 if os.environ.get("CHR_NF4_GEMV_TERMS") == "1" else 2
+        terms = env_terms()
     lut32 = oc.LUT.astype(np.float32)
+    if terms == 3:
+        return lut32.astype(np.float16).astype(np.float64)
     head = oc.bf16_round(lut32)
     if terms == 1:
         return head.astype(np.float64)

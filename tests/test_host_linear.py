@@ -14,7 +14,7 @@ from deepfold_amd.host import CompressedLinear, k_pad, nf4_linear
 from deepfold_amd.ring import HostImage
 from oracle import nf4_oracle as oc
 
-from helpers import staged_gemv_model
+from helpers import staged_gemv_model, takes_staged_gemv
 
 
 def blobs(m, k, seed=0, sigma=0.05):
@@ -106,15 +106,21 @@ def test_forward_matches_linear_on_the_decoded_matrix(lead, bias):
             model = staged_gemv_model(p.numpy(), s.numpy().view(np.uint16), m, k,
                                       xw.float().cpu().numpy().T, terms=1)
             parts.append(torch.from_numpy(model.T.copy()).cuda().to(torch.bfloat16))
+        elif n == 1:
+            # K = 200 is ragged, so the one-token launch stages x in LDS and multiplies the
+            # levels as that kernel keeps them (tests/helpers.py staged_levels)
+            assert takes_staged_gemv(m, k, fused=k % 64 != 0)
+            model = staged_gemv_model(p.numpy(), s.numpy().view(np.uint16), m, k, xw.float().cpu().numpy().T)
+            parts.append(torch.from_numpy(model.T.copy()).cuda().to(torch.bfloat16))
         else:
-            wk = w if n == 1 else w.to(torch.bfloat16).float()
+            wk = w.to(torch.bfloat16).float()
             parts.append((xw.double() @ wk.double().t()).to(torch.bfloat16))
-    want = torch.cat(parts, dim=0)
-    if bias:
-        want = want + b
-    want = want.reshape(*lead, m).double()
+    want0 = torch.cat(parts, dim=0)
+    want = want0 + b if bias else want0
+    want0, want = want0.reshape(*lead, m).double(), want.reshape(*lead, m).double()
     err = (y.double() - want).abs()
-    ulp = 2.0 ** (torch.floor(torch.log2(want.abs().clamp_min(2.0 ** -126))) - 7)
+    # a step of the product before the bias is added may be larger than a step of the sum
+    ulp = 2.0 ** (torch.floor(torch.log2(torch.maximum(want.abs(), want0.abs()).clamp_min(2.0 ** -126))) - 7)
     assert bool((err <= 2 * ulp + 1e-3 * want.pow(2).mean().sqrt()).all()), float((err / ulp).max())
     # the same through the functional form and torch's own linear on the decoded weight
     y2 = nf4_linear(x, lin.packed, lin.scale, m, k, k_pad(k), lin.bias if bias else None)

@@ -385,9 +385,9 @@ def test_swiglu_equals_pair(m, k):
 
 
 # ----------------------------------------------------------------- ring GEMV kernels
-# The ring kernels take staged launches of one segment whose row length is a multiple of 4..8
-# half steps of 1024 weights (4..6 for gate/up pairs); by default only from 32768 rows up,
-# CHR_NF4_GEMV_RING=1 sends every such launch to them.
+# The ring kernels take every staged launch whose row length is a multiple of 4..8 half steps
+# of 1024 weights (4..6 for gate/up pairs) or, for single rows, one half step short of a
+# multiple of 5..8; CHR_NF4_GEMV_RING=0 keeps such launches on the compiler-pipelined kernel.
 RING_ROWS = [
     (4100, 4096),   # 4 half steps, x of the row in registers; a pass and four rows more
     (9000, 5120),   # 5 half steps, two passes and a part of a third
@@ -406,7 +406,7 @@ RING_ROWS = [
 ]
 
 
-@pytest.mark.parametrize("terms", [1, 2])
+@pytest.mark.parametrize("terms", [1, 2, 3])
 @pytest.mark.parametrize("m,k", RING_ROWS)
 def test_ring_gemv(m, k, terms, monkeypatch):
     say("ring gemv", m, k, terms)
@@ -433,7 +433,66 @@ def test_ring_gemv(m, k, terms, monkeypatch):
     check_linear(y, to_f32(y0), what=f"ring {m}x{k} vs pipelined", ulps=1)
 
 
-@pytest.mark.parametrize("terms", [1, 2])
+# Form 3 stages x as binary16 times the power of two that puts its largest magnitude in
+# [2^14, 2^15).  Every element within 2^-29 of the largest converts exactly; the cases below are
+# the ones a fixed binary16 conversion would break (overflow above 65504, underflow of a vector
+# that is tiny as a whole) and the ones the scaling itself could (all zero, one huge outlier among
+# tiny elements, elements so far below the largest that they land on the subnormal grid).
+def _x_cases(k):
+    rng = np.random.default_rng(5)
+    base = rng.standard_normal(k).astype(np.float32)
+    spike = base * 1e-3
+    spike[k // 3] = 3.0e6
+    wide = base * np.exp2(rng.integers(-40, 10, k)).astype(np.float32)
+    return {
+        "large": base * 4.0e5,            # far above binary16's 65504
+        "tiny": base * 1.0e-20,           # far below binary16's smallest subnormal
+        "zero": np.zeros(k, np.float32),
+        "spike": spike,                   # one element 2^30 above the rest
+        "wide": wide,                     # fifty binades in one vector
+        "bf16_max": np.where(np.arange(k) % 97 == 0, 1.0e38, base).astype(np.float32),  # near the end of the range
+    }
+
+
+@pytest.mark.parametrize("case", ["large", "tiny", "zero", "spike", "wide", "bf16_max"])
+@pytest.mark.parametrize("m,k,ring", [(4100, 4096, "1"), (300, 16384, "1"), (200, 2048, "0"), (130, 200, "0")])
+def test_binary16_staging_range(m, k, ring, case, monkeypatch):
+    say("binary16 staging", m, k, ring, case)
+    monkeypatch.setenv("CHR_NF4_GEMV_STAGED", "1")
+    monkeypatch.setenv("CHR_NF4_GEMV_RING", ring)
+    monkeypatch.setenv("CHR_NF4_GEMV_TERMS", "3")
+    p, s, dp, ds = blobs(m, k, 900 + m)
+    x = oc.bf16_round(_x_cases(k)[case])
+    y = nf4.nf4_gemv(dp, ds, bf16_tensor(x), m, k, oc.k_pad(k))
+    got = to_f32(y).astype(np.float64).reshape(-1)
+    model = staged_gemv_model(p, s, m, k, x, terms=3).reshape(-1)
+    if case == "zero":
+        assert (got == 0).all()
+        return
+    assert np.isfinite(got).all()
+    # relative to the output's own size (the absolute floors of check_linear mean nothing at
+    # 1e-20 or 1e5): one bf16 step, plus 1e-3 of the rms for rows that cancel
+    rms = np.sqrt((model ** 2).mean())
+    assert rms > 0
+    assert (np.abs(got - model) <= ulp_bf16(model) + 1e-3 * rms).all(), (
+        case, float(np.max(np.abs(got - model) / (ulp_bf16(model) + 1e-3 * rms))))
+    # and the fused norm on the same vector (the largest normalised value is bounded from the
+    # two maxima, not searched for): against the same model on the normalised vector
+    if case in ("large", "wide") and k % 64 == 0:
+        g = oc.bf16_round((1 + 0.25 * np.random.default_rng(2).standard_normal(k)).astype(np.float32) * 37.0)
+        eps = 1e-6
+        y2 = nf4.nf4_gemv(dp, ds, bf16_tensor(x), m, k, oc.k_pad(k), rms_w=bf16_tensor(g), rms_eps=eps)
+        x64 = x.astype(np.float64)
+        inv = np.float32(1.0) / np.sqrt(np.float32((x64 ** 2).sum() / k + eps))
+        xh = oc.bf16_round(((g * x).astype(np.float32) * np.float32(inv)).astype(np.float32))
+        m2 = staged_gemv_model(p, s, m, k, xh, terms=3).reshape(-1)
+        got2 = to_f32(y2).astype(np.float64).reshape(-1)
+        rms2 = np.sqrt((m2 ** 2).mean())
+        assert np.isfinite(got2).all() and rms2 > 0
+        assert (np.abs(got2 - m2) <= 4 * ulp_bf16(m2) + 4e-3 * rms2).all(), case
+
+
+@pytest.mark.parametrize("terms", [1, 2, 3])
 @pytest.mark.parametrize("mq,mk,k,fused", [(5120, 1024, 5120, True), (4096, 512, 4096, False),
                                            (130, 33, 6144, True), (3000, 777, 7168, False)])
 def test_ring_qkv(mq, mk, k, fused, terms, monkeypatch):
@@ -467,7 +526,7 @@ def test_ring_qkv(mq, mk, k, fused, terms, monkeypatch):
         check_linear(o, to_f32(single), what="ring qkv vs single", ulps=1)
 
 
-@pytest.mark.parametrize("terms", [1, 2])
+@pytest.mark.parametrize("terms", [1, 2, 3])
 @pytest.mark.parametrize("m,k", [(4100, 5120), (520, 4096), (2100, 6208)])
 def test_ring_gemv_fused_rms(m, k, terms, monkeypatch):
     monkeypatch.setenv("CHR_NF4_GEMV_RING", "1")
@@ -488,7 +547,7 @@ def test_ring_gemv_fused_rms(m, k, terms, monkeypatch):
     check_linear(y, to_f32(y2), what="ring fused rms vs rms+gemv", ulps=1)
 
 
-@pytest.mark.parametrize("terms", [1, 2])
+@pytest.mark.parametrize("terms", [1, 2, 3])
 @pytest.mark.parametrize("m,k", [(4100, 4096), (4400, 5120), (20, 5120), (2300, 6144), (1100, 12288),
                                  (2100, 5056)])
 def test_ring_swiglu(m, k, terms, monkeypatch):
