@@ -225,7 +225,7 @@ struct StreamPlan {
 
 constexpr int64_t kStreamMinCodes = int64_t{1} << 24;
 constexpr int64_t kStreamMinCodes64 = int64_t{1} << 20;  // at 64 columns
-constexpr int kArriveSlots = 32;     // launches that may overlap in time (one a stream)
+constexpr int kArriveSlots = 512;    // owners of a row of arrival counts: streams, and captures in progress
 constexpr int kArriveBlocks = 1024;  // row blocks of a launch whose splits meet in the tile
 
 // blocks32, blocks64: 32- and 64-row blocks of the launch (summed over its stacked matrices).
@@ -1046,26 +1046,48 @@ __device__ __forceinline__ void nest_chunks(int n, F &f) {
   }
 }
 
-// acc += (position V of this lane's row of sixteen lanes of `mine`) * t, as one instruction
-// (the compiler keeps the broadcast and the multiply-add apart)
-template <int V>
-__device__ __forceinline__ float scale_into(float acc, float mine, float t) {
-  asm("v_fmac_f32_dpp %0, %1, %2 row_newbcast:%3 row_mask:0xf bank_mask:0xf"
-      : "+v"(acc)
-      : "v"(mine), "v"(t), "n"(V));
-  return acc;
+// acc[v] += (position v of this lane's row of sixteen lanes of `mine`) * t[v] for the sixteen
+// values of a 32x32 result, one v_fmac_f32_dpp each (the compiler keeps the broadcast and the
+// multiply-add apart), written as two statements of eight so that nothing the compiler emits
+// can stand where a hazard would be:
+//  - the matrix core's result registers may be read by hand-written instructions only after it
+//    has finished writing them (up to 18 wait states after the last MFMA was issued); the
+//    compiler counts those for its own instructions, not for what an asm statement reads: the
+//    first statement opens with the wait states, and t goes through it as a whole;
+//  - a DPP operand must have been written two instructions or more before it is read, and the
+//    compiler may compute or copy an asm operand right in front of the statement (seen once: a
+//    stale value in accumulator 0 of every block): both statements open with wait states for
+//    that too.
+#define CHR_FMAC8(FIRST)                                                                  \
+  "v_fmac_f32_dpp %0, %16, %8 row_newbcast:" #FIRST "+0 row_mask:0xf bank_mask:0xf\n\t"    \
+  "v_fmac_f32_dpp %1, %16, %9 row_newbcast:" #FIRST "+1 row_mask:0xf bank_mask:0xf\n\t"    \
+  "v_fmac_f32_dpp %2, %16, %10 row_newbcast:" #FIRST "+2 row_mask:0xf bank_mask:0xf\n\t"   \
+  "v_fmac_f32_dpp %3, %16, %11 row_newbcast:" #FIRST "+3 row_mask:0xf bank_mask:0xf\n\t"   \
+  "v_fmac_f32_dpp %4, %16, %12 row_newbcast:" #FIRST "+4 row_mask:0xf bank_mask:0xf\n\t"   \
+  "v_fmac_f32_dpp %5, %16, %13 row_newbcast:" #FIRST "+5 row_mask:0xf bank_mask:0xf\n\t"   \
+  "v_fmac_f32_dpp %6, %16, %14 row_newbcast:" #FIRST "+6 row_mask:0xf bank_mask:0xf\n\t"   \
+  "v_fmac_f32_dpp %7, %16, %15 row_newbcast:" #FIRST "+7 row_mask:0xf bank_mask:0xf"
+__device__ __forceinline__ void scale_into_all(f32x16 &acc, float mine, const f32x16 &t) {
+  float a[16], v[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    a[i] = acc[i];
+    v[i] = t[i];
+  }
+  asm volatile("s_nop 15\n\ts_nop 7\n\t" CHR_FMAC8(0)
+               : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(a[6]), "+v"(a[7])
+               : "v"(v[0]), "v"(v[1]), "v"(v[2]), "v"(v[3]), "v"(v[4]), "v"(v[5]), "v"(v[6]), "v"(v[7]), "v"(mine));
+  asm volatile("s_nop 1\n\t" CHR_FMAC8(8)
+               : "+v"(a[8]), "+v"(a[9]), "+v"(a[10]), "+v"(a[11]), "+v"(a[12]), "+v"(a[13]), "+v"(a[14]),
+                 "+v"(a[15])
+               : "v"(v[8]), "v"(v[9]), "v"(v[10]), "v"(v[11]), "v"(v[12]), "v"(v[13]), "v"(v[14]), "v"(v[15]),
+                 "v"(mine));
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    acc[i] = a[i];
+  }
 }
-
-// The matrix core's result registers may be read by hand-written instructions only after it
-// has finished writing them (up to 18 wait states after the last MFMA was issued); the
-// compiler counts those for its own instructions, not for what an asm statement reads.  This
-// stands between the MFMAs that write t and the scale_into statements that read it.  The
-// scale goes through it too: a DPP operand must have been written two instructions or more
-// before it is read, and an asm statement's operand may otherwise be computed right in front
-// of it.
-__device__ __forceinline__ void mfma_results_settled(f32x16 &t, float &scale) {
-  asm volatile("s_nop 15\n\ts_nop 7" : "+v"(t), "+v"(scale));
-}
+#undef CHR_FMAC8
 
 // The low halves of a and b as one dword, a below b; the high halves likewise: a byte
 // permute each.
@@ -1446,23 +1468,7 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
       }
 #pragma unroll
       for (int rb = 0; rb < RB; ++rb) {
-        mfma_results_settled(t[rb], mine[rb]);
-        acc[rb][0] = scale_into<0>(acc[rb][0], mine[rb], t[rb][0]);
-        acc[rb][1] = scale_into<1>(acc[rb][1], mine[rb], t[rb][1]);
-        acc[rb][2] = scale_into<2>(acc[rb][2], mine[rb], t[rb][2]);
-        acc[rb][3] = scale_into<3>(acc[rb][3], mine[rb], t[rb][3]);
-        acc[rb][4] = scale_into<4>(acc[rb][4], mine[rb], t[rb][4]);
-        acc[rb][5] = scale_into<5>(acc[rb][5], mine[rb], t[rb][5]);
-        acc[rb][6] = scale_into<6>(acc[rb][6], mine[rb], t[rb][6]);
-        acc[rb][7] = scale_into<7>(acc[rb][7], mine[rb], t[rb][7]);
-        acc[rb][8] = scale_into<8>(acc[rb][8], mine[rb], t[rb][8]);
-        acc[rb][9] = scale_into<9>(acc[rb][9], mine[rb], t[rb][9]);
-        acc[rb][10] = scale_into<10>(acc[rb][10], mine[rb], t[rb][10]);
-        acc[rb][11] = scale_into<11>(acc[rb][11], mine[rb], t[rb][11]);
-        acc[rb][12] = scale_into<12>(acc[rb][12], mine[rb], t[rb][12]);
-        acc[rb][13] = scale_into<13>(acc[rb][13], mine[rb], t[rb][13]);
-        acc[rb][14] = scale_into<14>(acc[rb][14], mine[rb], t[rb][14]);
-        acc[rb][15] = scale_into<15>(acc[rb][15], mine[rb], t[rb][15]);
+        scale_into_all(acc[rb], mine[rb], t[rb]);
       }
       __syncthreads();
     }
@@ -1865,23 +1871,7 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream64(GemmSegs segs,
       }
 #pragma unroll
       for (int cb = 0; cb < 2; ++cb) {
-        mfma_results_settled(t[cb], mine);
-        acc[cb][0] = scale_into<0>(acc[cb][0], mine, t[cb][0]);
-        acc[cb][1] = scale_into<1>(acc[cb][1], mine, t[cb][1]);
-        acc[cb][2] = scale_into<2>(acc[cb][2], mine, t[cb][2]);
-        acc[cb][3] = scale_into<3>(acc[cb][3], mine, t[cb][3]);
-        acc[cb][4] = scale_into<4>(acc[cb][4], mine, t[cb][4]);
-        acc[cb][5] = scale_into<5>(acc[cb][5], mine, t[cb][5]);
-        acc[cb][6] = scale_into<6>(acc[cb][6], mine, t[cb][6]);
-        acc[cb][7] = scale_into<7>(acc[cb][7], mine, t[cb][7]);
-        acc[cb][8] = scale_into<8>(acc[cb][8], mine, t[cb][8]);
-        acc[cb][9] = scale_into<9>(acc[cb][9], mine, t[cb][9]);
-        acc[cb][10] = scale_into<10>(acc[cb][10], mine, t[cb][10]);
-        acc[cb][11] = scale_into<11>(acc[cb][11], mine, t[cb][11]);
-        acc[cb][12] = scale_into<12>(acc[cb][12], mine, t[cb][12]);
-        acc[cb][13] = scale_into<13>(acc[cb][13], mine, t[cb][13]);
-        acc[cb][14] = scale_into<14>(acc[cb][14], mine, t[cb][14]);
-        acc[cb][15] = scale_into<15>(acc[cb][15], mine, t[cb][15]);
+        scale_into_all(acc[cb], mine, t[cb]);
       }
       __syncthreads();
     }
@@ -2329,28 +2319,58 @@ struct StackPlan {
   int stream;  // 32-row blocks of a workgroup of the stream tile, 0: another tile
 };
 
-// The slot of arrival counts for launches on this stream of the current device; -1 when all
-// slots are taken by other streams (the splits then meet in a reduce kernel).  Launches on one
-// stream run one after the other, so they can share a slot.
+// The row of arrival counts a split launch of the stream tile uses, or -1: its splits then meet
+// in a reduce kernel, which needs no counts (and gives the same bits).  Two launches may share a
+// row only if they cannot run at the same time:
+//   - eager launches on one stream run one after the other: a row per (device, stream);
+//   - a launch recorded during stream capture runs whenever and wherever its graph is replayed,
+//     possibly beside eager work on the stream it was captured from: a row per (device,
+//     capture, stream), which no eager launch and no other graph ever gets (two replays of one
+//     graph do not overlap: the runtime orders launches of one executable graph);
+//   - the per-thread default stream is one handle for many streams: no row, -1.
+// Rows are never handed back (nothing tells the library that a graph is gone); when all 512
+// are taken, further owners get -1.
 int arrival_slot(hipStream_t st) {
+  struct Owner {
+    int dev;
+    hipStream_t st;
+    unsigned long long capture;  // 0: eager launches on st
+  };
   static std::mutex mu;
-  static std::pair<int, hipStream_t> owner[kArriveSlots];
+  static Owner owner[kArriveSlots];
   static int used = 0;
+  if (st == hipStreamPerThread) {
+    return -1;
+  }
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) {
     (void)hipGetLastError();
     return -1;
   }
+  unsigned long long capture = 0;
+  {
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    unsigned long long id = 0;
+    if (hipStreamGetCaptureInfo(st, &status, &id) != hipSuccess) {
+      (void)hipGetLastError();
+      return -1;
+    }
+    if (status == hipStreamCaptureStatusActive) {
+      capture = id + 1;  // (ids start anywhere: keep 0 for "not capturing")
+    } else if (status != hipStreamCaptureStatusNone) {
+      return -1;  // a capture that has been invalidated: the launch will fail anyway
+    }
+  }
   const std::lock_guard<std::mutex> lock(mu);
   for (int i = 0; i < used; ++i) {
-    if (owner[i].first == dev && owner[i].second == st) {
+    if (owner[i].dev == dev && owner[i].st == st && owner[i].capture == capture) {
       return i;
     }
   }
   if (used == kArriveSlots) {
     return -1;
   }
-  owner[used] = {dev, st};
+  owner[used] = {dev, st, capture};
   return used++;
 }
 

@@ -73,3 +73,16 @@ class DecodeState:
         host round trip: ``token = next``, ``position += 1``, ``finished |= eos``."""
         dv2_argmax_commit(self.arena.logits.view(-1), self.next_token, self.token, self.position,
                           self.finished, self.eos_id, commit=commit, ws=self.arena.argmax_ws)
+
+    def commit_step(self) -> None:
+        """Feed ``next_token`` back on the device (``gpu/decodev2/state.py:98-103``): the same
+        launch as ``pick_next(commit=True)``, which picks the id again from the logits it was
+        picked from and then commits it."""
+        self.pick_next(commit=True)
+
+    def rope_at_position(self) -> tuple[torch.Tensor, torch.Tensor]:
+        """Rows of the RoPE tables at the device-side position, ``[1, head_dim]`` each
+        (``gpu/decodev2/state.py:105-107``); the step's kernels index the tables themselves,
+        this is for callers that want the rows."""
+        at = self.position.reshape(1)
+        return self.cos.index_select(0, at), self.sin.index_select(0, at)

@@ -115,9 +115,12 @@ void chr_nf4_set_tuning(int32_t path, int32_t split_k, int32_t one_wave);
 /* Which prefill launches run the tile whose workgroups finish their rows themselves:
  * 0 where the planner's cost model prefers it (the default), > 0 wherever it fits, < 0 never.
  * Process-wide, like chr_nf4_set_tuning.  Launches of that tile that split K count their
- * arrivals in a table the library owns, one slot per stream (32 streams; further streams get
- * a reduce launch instead): launches that may overlap in time must be made on different
- * streams, and graphs captured from one stream must not be replayed concurrently.
+ * arrivals in a table the library owns: one row per stream for eager launches, one row per
+ * capture and stream for launches recorded into a graph (so a graph may be replayed on any
+ * stream, beside eager launches on the stream it was captured from and beside other graphs),
+ * none for the per-thread default stream; when the 512 rows are taken, and on that stream,
+ * the splits meet in a reduce launch instead (same bits).  What the caller must not do is
+ * replay one executable graph concurrently with itself, which the HIP runtime orders anyway.
  * No counterpart in the reference. */
 void chr_nf4_gemm_stream_policy(int32_t policy);
 

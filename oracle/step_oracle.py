@@ -158,9 +158,10 @@ def teacher_logits(model, token_ids: Sequence[int]) -> np.ndarray:
 
 
 def greedy_ids(model, prompt_ids: Sequence[int], n_new: int, *, ignore_eos: bool = False,
-               return_margins: bool = False):
+               return_margins: bool = False, return_tops: bool = False):
     """Greedy continuation (``oracle.py:151-166``).  With ``return_margins`` also the
-    top-1 minus top-2 logit gap of every pick, which says how thin each decision is."""
+    top-1 minus top-2 logit gap of every pick, which says how thin each decision is; with
+    ``return_tops`` (and margins) the top-1 logit of every pick as a third list."""
     if not len(prompt_ids):
         raise ValueError("prompt_ids must be non-empty")
     cache = OracleCache(model.spec)
@@ -169,16 +170,20 @@ def greedy_ids(model, prompt_ids: Sequence[int], n_new: int, *, ignore_eos: bool
         last = step_logits(model, cache, int(t))
     out: list[int] = []
     margins: list[float] = []
+    tops: list[float] = []
     eos = int(model.spec.eos_id)
     tok = int(last.argmax())
     for _ in range(int(n_new)):
         out.append(tok)
         top2 = np.partition(last, -2)[-2:]
         margins.append(float(top2[1] - top2[0]))
+        tops.append(float(top2[1]))
         if tok == eos and not ignore_eos:
             break
         if cache.pos >= model.spec.max_seq:
             break
         last = step_logits(model, cache, tok)
         tok = int(last.argmax())
+    if return_margins and return_tops:
+        return out, margins, tops
     return (out, margins) if return_margins else out

@@ -762,9 +762,9 @@ def test_gemm_stream_tile_random_shapes():
 
 
 def test_gemm_stream_splits_on_many_streams():
-    """Launches whose workgroups share K count their arrivals in a slot of a table the library
-    owns, one slot per stream; streams beyond its 32 slots get the reduce kernel on the same
-    partials.  Forty streams, each launching twice: every result equals the first bit for bit."""
+    """Launches whose workgroups share K count their arrivals in a row of a table the library
+    owns, one row per stream (owners beyond its 512 rows get the reduce kernel on the same
+    partials).  Forty streams, each launching twice: every result equals the first bit for bit."""
     m, k, n = 5120, 13824, 8
     say("gemm stream, many streams", m, k, n)
     assert nf4.nf4_plan(m, k, n)["grid_y"] == 3 and nf4.nf4_plan(m, k, n)["block"] == 1024
@@ -809,6 +809,48 @@ def test_gemm_stream_splits_in_a_replayed_graph():
             assert (bf16_bits(o) == want).all()
         m, k, n = shapes[0]
         assert (bf16_bits(nf4.nf4_gemm(mats[0][0], mats[0][1], xs[0], m, k, k)) == eager[0]).all()
+
+
+def test_gemm_stream_graph_replayed_beside_eager_launches():
+    """A split launch recorded during capture owns a row of arrival counts of its own, so the
+    graph can be replayed on a second stream while eager split launches of the same shape run
+    on the stream it was captured from: all results equal those of the same launches made one
+    at a time, bit for bit, on every one of several overlapping rounds."""
+    m, k, n = 5120, 13824, 8
+    say("gemm stream, graph beside eager", m, k, n)
+    assert nf4.nf4_plan(m, k, n)["grid_y"] == 3 and nf4.nf4_plan(m, k, n)["block"] == 1024
+    p, s, dp, ds = blobs(m, k, 78)
+    p2, s2, dp2, ds2 = blobs(m, k, 79)
+    xa, xb = bf16_tensor(rand_x(k, n, 6)), bf16_tensor(rand_x(k, n, 7))
+    # the same launches one at a time on an idle device (their sums are the reduce kernel's, in
+    # split order whoever arrives last: test_gemm_add_sq compares the two bit for bit)
+    want_a = bf16_bits(nf4.nf4_gemm(dp, ds, xa, m, k, k))
+    torch.cuda.synchronize()
+    want_b = bf16_bits(nf4.nf4_gemm(dp2, ds2, xb, m, k, k))
+    torch.cuda.synchronize()
+    cap = torch.cuda.Stream()
+    other = torch.cuda.Stream()
+    with torch.cuda.stream(cap):
+        nf4.nf4_gemm(dp, ds, xa, m, k, k)  # eager launches on the capture stream own its row
+        cap.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        graph.capture_begin()
+        held = [nf4.nf4_gemm(dp, ds, xa, m, k, k) for _ in range(6)]
+        graph.capture_end()
+    torch.cuda.synchronize()
+    for _ in range(5):
+        eager = []
+        with torch.cuda.stream(other):
+            graph.replay()
+        with torch.cuda.stream(cap):
+            for _ in range(6):
+                eager.append(nf4.nf4_gemm(dp2, ds2, xb, m, k, k))
+        torch.cuda.synchronize()
+        for o in held:
+            assert (bf16_bits(o) == want_a).all()
+            o.zero_()
+        for o in eager:
+            assert (bf16_bits(o) == want_b).all()
 
 
 @pytest.mark.parametrize("n", [5, 8, 16, 24, 32, 40, 64])
