@@ -58,11 +58,18 @@ def main() -> None:
     workers = int(sys.argv[3]) if len(sys.argv) > 3 else 6
     with ProcessPoolExecutor(workers) as pool:
         rows = list(pool.map(one, range(first, first + count), chunksize=8))
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "greedy_margin_seeds.json")
+    scanned = [[first, first + count]]
+    if os.path.exists(path):  # a further range: keep the best of both
+        with open(path) as f:
+            old = json.load(f)
+        seen = {r["seed"] for r in rows}
+        rows += [r for r in old["streams"] if r["seed"] not in seen]
+        scanned = old["seeds_scanned"] + scanned
     rows.sort(key=lambda r: -r["min_gap_bf16_steps"])
     out = {"spec": "longrun (4 layers, hidden 512, 8 query / 2 kv heads of 64, ffn 1536, vocab 2048)",
-           "prompt": PROMPT, "n_new": N_NEW, "seeds_scanned": [first, first + count],
+           "prompt": PROMPT, "n_new": N_NEW, "seeds_scanned": scanned,
            "streams": rows[:KEEP]}
-    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "greedy_margin_seeds.json")
     with open(path, "w") as f:
         json.dump(out, f, indent=1)
     print("widest smallest gaps (bf16 steps):", [round(r["min_gap_bf16_steps"], 2) for r in rows[:KEEP]])

@@ -232,7 +232,7 @@ def near_tie(logits: np.ndarray) -> bool:
 #: near-tie a stream lands on then changes with the summation order of the kernel that
 #: serves a row length, and no stream is promised to stay identical for 64 picks (every
 #: difference is still checked to sit at a near-tie of the oracle).
-IDENTICAL_FLOOR = {"plain": 1, "fold_rms": 1, "fp32_levels": 1, "one_term": 0}
+IDENTICAL_FLOOR = {"plain": 1, "fold_rms": 1, "fp32_levels": 1, "two_term": 1, "one_term": 0}
 
 
 def _streams_64(monkeypatch, form: str) -> tuple[int, list[str]]:
@@ -240,7 +240,7 @@ def _streams_64(monkeypatch, form: str) -> tuple[int, list[str]]:
     a first difference at a pick that is a near-tie for the oracle itself.  Returns how many
     were identical all the way, and a line per stream."""
     env = {"plain": {}, "fold_rms": {}, "fp32_levels": {"CHR_NF4_GEMV_STAGED": "0"},
-           "one_term": {"CHR_NF4_GEMV_TERMS": "1"}}[form]
+           "two_term": {"CHR_NF4_GEMV_TERMS": "2"}, "one_term": {"CHR_NF4_GEMV_TERMS": "1"}}[form]
     for k, v in env.items():
         monkeypatch.setenv(k, v)
     prompt = [11, 200, 37, 1999, 5, 640, 3, 77]
@@ -249,7 +249,7 @@ def _streams_64(monkeypatch, form: str) -> tuple[int, list[str]]:
         for seed in (0, 1, 2, 3):
             model, state, weights = session(LONGRUN, seed, packed_embed)
             # fp32_levels forces the plain kernel, which has no fused norm: reference sequence
-            sched = "fold_rms" if form in ("fold_rms", "one_term") else "plain"
+            sched = "fold_rms" if form in ("fold_rms", "two_term", "one_term") else "plain"
             want, margins = so.greedy_ids(model, prompt, 64, ignore_eos=True, return_margins=True)
             assert len(want) == 64
             state.reset()
@@ -272,16 +272,63 @@ def _streams_64(monkeypatch, form: str) -> tuple[int, list[str]]:
     return identical, lines
 
 
-@pytest.mark.parametrize("form", ["plain", "fold_rms", "fp32_levels", "one_term"])
+@pytest.mark.parametrize("form", ["plain", "fold_rms", "fp32_levels", "two_term", "one_term"])
 def test_greedy_64_tokens_identical_to_the_oracle(form, monkeypatch):
     """64 generated tokens on random-init weights, ignore-EOS, eager and graph, eight
-    streams per launch form: the reference's call sequence (``plain``), the folded one
-    (``fold_rms``), the plain GEMV kernel with fp32 levels, and the one-term (bf16) levels."""
+    streams per launch form: the reference's call sequence (``plain``) and the folded one
+    (``fold_rms``) with the default binary16 levels, the plain GEMV kernel with fp32 levels,
+    the two-term and the one-term bf16 levels.  These eight seeds were not chosen: most of their
+    streams pass a pick that is a near-tie for the oracle itself, which is where a stream may
+    leave the oracle's (the test below has the streams that pass none)."""
     say("64-token streams,", form)
     identical, lines = _streams_64(monkeypatch, form)
     say("\n".join(lines))
     say(f"  {form}: {identical} of 8 streams identical over 64 tokens")
     assert identical >= IDENTICAL_FLOOR[form], (form, identical)
+
+
+#: Streams picked on the CPU by the oracle alone (tests/golden/scan_greedy_margins.py): seeds of the
+#: same 4-layer model whose every one of the 64 picks has a top-1 / top-2 gap of at least
+#: WIDE_GAP_STEPS bf16 steps of the top logit.  Where the oracle itself never decides on less than
+#: that, every launch form must reproduce all 64 ids, eager and from the captured graph: a hard
+#: assertion, no floor.
+WIDE_GAP_STEPS = 2.0
+WIDE_GAP_STREAMS = 8
+
+
+def wide_gap_streams():
+    import json
+    import os
+
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "greedy_margin_seeds.json")) as f:
+        fixture = json.load(f)
+    rows = [r for r in fixture["streams"] if r["min_gap_bf16_steps"] >= WIDE_GAP_STEPS][:WIDE_GAP_STREAMS]
+    assert len(rows) == WIDE_GAP_STREAMS, "the fixture holds fewer streams of that gap than the test wants"
+    return fixture, rows
+
+
+@pytest.mark.parametrize("form", ["fold_rms", "plain", "fp32_levels", "two_term", "one_term"])
+def test_greedy_64_tokens_identical_on_wide_gap_streams(form, monkeypatch):
+    say("64-token streams with wide gaps,", form)
+    env = {"plain": {}, "fold_rms": {}, "fp32_levels": {"CHR_NF4_GEMV_STAGED": "0"},
+           "two_term": {"CHR_NF4_GEMV_TERMS": "2"}, "one_term": {"CHR_NF4_GEMV_TERMS": "1"}}[form]
+    for k, v in env.items():
+        monkeypatch.setenv(k, v)
+    sched = "plain" if form in ("plain", "fp32_levels") else "fold_rms"
+    fixture, rows = wide_gap_streams()
+    prompt, n_new = fixture["prompt"], fixture["n_new"]
+    for row in rows:
+        model, state, weights = session(LONGRUN, row["seed"])
+        state.reset()
+        step = lambda s, w: dv2.greedy_decode(s, w, schedule=sched)  # noqa: E731
+        got = dv2.generate(state, weights, prompt, n_new, step=step, ignore_eos=True)
+        assert got == row["ids"], (form, row["seed"], row["min_gap_bf16_steps"],
+                                   next(i for i, (a, b) in enumerate(zip(got, row["ids"])) if a != b))
+        state.reset()
+        graph = dv2.capture_greedy(state, weights, warmup=1, schedule=sched)
+        state.reset()
+        assert dv2.generate(state, weights, prompt, n_new, step=graph, ignore_eos=True) == got, (form, row["seed"])
+        say(f"  seed {row['seed']}: identical, eager and graph (smallest gap {row['min_gap_bf16_steps']:.2f} bf16 steps)")
 
 
 def _two_layers(spec, **over):

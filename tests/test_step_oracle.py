@@ -140,3 +140,26 @@ def test_greedy_oracle_runs_and_is_reproducible(spec, seed, prompt):
     so.step_logits(model, c2, 1)
     c2.k[:, -1], c2.v[:, -1] = 1e4, 1e4
     assert np.allclose(so.step_logits(model, c1, 3), so.step_logits(model, c2, 3))
+
+
+def test_wide_gap_stream_fixture_is_what_the_oracle_gives():
+    """``tests/golden/greedy_margin_seeds.json`` (made by ``scan_greedy_margins.py``): two of its
+    streams recomputed here, ids and smallest gap; the list is sorted by that gap."""
+    import importlib.util
+    import json
+    import os
+
+    here = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    with open(os.path.join(here, "greedy_margin_seeds.json")) as f:
+        fixture = json.load(f)
+    spec = importlib.util.spec_from_file_location("scan_greedy_margins",
+                                                  os.path.join(here, "scan_greedy_margins.py"))
+    scan = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(scan)
+    assert fixture["prompt"] == scan.PROMPT and fixture["n_new"] == scan.N_NEW
+    gaps = [r["min_gap_bf16_steps"] for r in fixture["streams"]]
+    assert gaps == sorted(gaps, reverse=True) and len(gaps) >= 8 and gaps[7] >= 2.0
+    for row in (fixture["streams"][0], fixture["streams"][7]):
+        again = scan.one(row["seed"])
+        assert again["ids"] == row["ids"] and len(row["ids"]) == 64
+        assert abs(again["min_gap_bf16_steps"] - row["min_gap_bf16_steps"]) < 1e-9
