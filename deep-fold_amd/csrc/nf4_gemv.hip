@@ -225,8 +225,8 @@ __device__ __forceinline__ void zero_unused_slots(uint4 *xs, int K_pad) {
 // x piece i (8 consecutive dims of one head) merged from the per-part softmax states:
 // x = sum_p e^{m_p - M} o_p / sum_p e^{m_p - M} l_p, rounded to bf16 as the attention
 // launch itself would have stored it.  An empty part has m = -1e30, l = 0: weight zero.
+template <int kBatch>  // parts whose states are fetched together (one memory round trip)
 __device__ __forceinline__ uint4 merged_attn_piece(const StreamArgs &a, int i) {
-  constexpr int kBatch = 8;  // parts whose states are fetched together (one memory round trip)
   const int hd = a.attn_hd;
   const int k = i << 3;
   const int head = k / hd;
@@ -327,11 +327,18 @@ __device__ __forceinline__ void x_store(const StreamArgs &a, uint4 *xs, StagedLd
   zero_unused_slots(xs, a.K_pad);
   float inv = 1.f;
   int power = 0;
+  // first vector index of this wavefront: a wavefront (or a round j of all of them) past the
+  // end of x skips the arithmetic as a whole (a scalar branch) and only joins the barriers;
+  // at K = 5120 ten of the sixteen wavefronts hold a vector, in the first round only
+  const int wave_first = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) & ~(kWave - 1));
   if (a.rms_w != nullptr) {
     float ss = 0.f;
     uint32_t xm = 0u, gm = 0u;  // largest magnitudes of x and of the norm weights, per dword half
 #pragma unroll
     for (int j = 0; j < kXKeep; ++j) {
+      if (wave_first + j * kStagedThreads >= nk) {
+        continue;
+      }
       const int i = threadIdx.x + j * kStagedThreads;
       const uint32_t u[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
       const uint32_t gw[4] = {g[j].x, g[j].y, g[j].z, g[j].w};
@@ -366,7 +373,9 @@ __device__ __forceinline__ void x_store(const StreamArgs &a, uint4 *xs, StagedLd
     uint32_t xm = 0u;
 #pragma unroll
     for (int j = 0; j < kXKeep; ++j) {
-      xm = mag_max(mag_max(mag_max(mag_max(xm, v[j].x), v[j].y), v[j].z), v[j].w);
+      if (wave_first + j * kStagedThreads < nk) {
+        xm = mag_max(mag_max(mag_max(mag_max(xm, v[j].x), v[j].y), v[j].z), v[j].w);
+      }
     }
     float none = 0.f;
     block_fold<false>(none, xm, lds.part, lds.vmax);
@@ -374,6 +383,9 @@ __device__ __forceinline__ void x_store(const StreamArgs &a, uint4 *xs, StagedLd
   }
 #pragma unroll
   for (int j = 0; j < kXKeep; ++j) {
+    if (wave_first + j * kStagedThreads >= nvec) {
+      continue;
+    }
     const int i = threadIdx.x + j * kStagedThreads;
     if (i < nvec) {
       uint4 o = i < nk ? v[j] : make_uint4(0, 0, 0, 0);
@@ -431,8 +443,34 @@ __device__ __forceinline__ void stage_x(const StreamArgs &a, uint4 *xs, StagedLd
   float *part = lds.part;
   zero_unused_slots(xs, a.K_pad);
   if (a.attn_state != nullptr) {
-    for (int i = threadIdx.x; i < (a.K_pad >> 3); i += kStagedThreads) {
-      xs[x_slot(i)] = merged_attn_piece(a, i);
+    const int nvec = a.K_pad >> 3;
+    if (nvec <= kStagedThreads) {
+      // one piece a thread at most (K <= 8192): it stays in registers from the merge to the
+      // store (binary16: through the search for the largest magnitude and the conversion)
+      const int i = threadIdx.x;
+      uint4 piece = make_uint4(0, 0, 0, 0);
+      if (i < nvec) {
+        piece = a.attn_parts <= 4 ? merged_attn_piece<4>(a, i) : merged_attn_piece<8>(a, i);
+      }
+      if constexpr (F16) {
+        uint32_t xm = mag_max(mag_max(mag_max(mag_max(0u, piece.x), piece.y), piece.z), piece.w);
+        float none = 0.f;
+        block_fold<false>(none, xm, lds.part, lds.vmax);
+        const int power = x_power_for(larger_half_bf16(xm));
+        if (threadIdx.x == 0) {
+          lds.xexp = power;
+        }
+        piece = make_uint4(bf16x2_to_f16x2(piece.x, power), bf16x2_to_f16x2(piece.y, power),
+                           bf16x2_to_f16x2(piece.z, power), bf16x2_to_f16x2(piece.w, power));
+      }
+      if (i < nvec) {
+        xs[x_slot(i)] = piece;
+      }
+      __syncthreads();
+      return;
+    }
+    for (int i = threadIdx.x; i < nvec; i += kStagedThreads) {
+      xs[x_slot(i)] = a.attn_parts <= 4 ? merged_attn_piece<4>(a, i) : merged_attn_piece<8>(a, i);
     }
     __syncthreads();
     if constexpr (F16) {
