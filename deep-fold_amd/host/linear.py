@@ -33,11 +33,11 @@ def nf4_linear(x: torch.Tensor, packed: torch.Tensor, scale: torch.Tensor, M: in
                K_pad: int, bias: torch.Tensor | None = None) -> torch.Tensor:  # noqa: N803
     """``y[..., M] = x[..., K] @ dequant(packed, scale).T (+ bias)`` in bf16."""
     if x.shape[-1] != K:
-        raise ValueError(f"x has {x.shape[-1]} features, this linear takes K={K}")
+        raise ValueError(f"the last dimension of x is {x.shape[-1]}, the matrix multiplies K={K}")
     lead = x.shape[:-1]
     n = math.prod(lead)
     if n < 1:
-        raise ValueError(f"CompressedLinear: empty leading dims x{tuple(x.shape)}")
+        raise ValueError(f"x{tuple(x.shape)} holds no token to multiply")
     rows = x.to(torch.bfloat16).reshape(n, K)
     if n == 1:
         out = nf4_gemm(packed, scale, rows.reshape(K, 1), M, K, K_pad).reshape(1, M)
@@ -63,7 +63,7 @@ class CompressedLinear(nn.Module):
         super().__init__()
         self.in_features, self.out_features = int(in_features), int(out_features)
         if min(self.in_features, self.out_features) < 1:
-            raise ValueError(f"bad shape: in={in_features} out={out_features}")
+            raise ValueError(f"in_features={in_features} and out_features={out_features} must both be positive")
         self.K, self.M = self.in_features, self.out_features
         self.K_pad = k_pad(self.K)
         self.n_groups = self.K_pad // GROUP_SIZE
@@ -77,7 +77,7 @@ class CompressedLinear(nn.Module):
         self.chr_name: str | None = None
         self.host_image: HostImage | None = None
 
-    # ---- the weight that is not there ---------------------------------------------------
+    # ---- what stands in for nn.Linear.weight --------------------------------------------
     @property
     def weight(self) -> torch.Tensor:
         """0 elements of the compute dtype on the layer's device, for code that asks a
@@ -107,17 +107,17 @@ class CompressedLinear(nn.Module):
     # ---- attaching ----------------------------------------------------------------------
     def _check_shape(self, what: str, m: int, k: int, pad: int) -> None:
         if (int(m), int(k)) != (self.M, self.K):
-            raise ValueError(f"{what} is [{m},{k}], this linear is [{self.M},{self.K}]")
+            raise ValueError(f"{what} has {m} rows of {k}, this seat holds {self.M} rows of {self.K}")
         if int(pad) != self.K_pad:
-            raise ValueError(f"{what}: K_pad {pad} != {self.K_pad}")
+            raise ValueError(f"{what} pads its rows to {pad} codes, this seat to {self.K_pad}")
 
     def attach(self, matrix: ChrMatrix) -> None:
         """Use ``matrix``'s tensors as they are (shared, not copied: tied layers can hold
         one matrix)."""
         self._check_shape(f"{matrix.name}: matrix", matrix.M, matrix.K, matrix.K_pad)
         if matrix.packed.dtype != torch.uint8 or matrix.scale.dtype != torch.float16:
-            raise TypeError(f"{matrix.name}: expected uint8 packed / float16 scale, got "
-                            f"{matrix.packed.dtype} / {matrix.scale.dtype}")
+            raise TypeError(f"{matrix.name}: codes must be uint8 and scales float16, not "
+                            f"{matrix.packed.dtype} and {matrix.scale.dtype}")
         self.packed, self.scale = matrix.packed, matrix.scale
         self.chr_name, self.host_image = matrix.name, None
 
@@ -131,9 +131,9 @@ class CompressedLinear(nn.Module):
 
     def set_bias(self, bias: torch.Tensor) -> None:
         if self.bias is None:
-            raise ValueError(f"{self.chr_name or self}: built with bias=False")
+            raise ValueError(f"{self.chr_name or self} was built with bias=False: there is no bias to set")
         if tuple(bias.shape) != (self.M,):
-            raise ValueError(f"bias {tuple(bias.shape)} != {(self.M,)}")
+            raise ValueError(f"a bias of shape {tuple(bias.shape)} does not fit {self.M} output features")
         self.bias = bias.to(self.compute_dtype)
 
     # ---- forward ------------------------------------------------------------------------
@@ -144,11 +144,11 @@ class CompressedLinear(nn.Module):
             raise RuntimeError(f"{label} is host-resident; a CopyRing has to stream it, "
                                "forward does no silent host-to-device copy")
         if where == "empty":
-            raise RuntimeError(f"{label} has no weights: attach a ChrMatrix first")
+            raise RuntimeError(f"{label} has no weights yet: attach() a ChrMatrix before calling it")
         bias = self.bias if self.bias is not None and self.bias.numel() else None
         return nf4_linear(x, self.packed, self.scale, self.M, self.K, self.K_pad, bias)
 
     def extra_repr(self) -> str:
         return (f"in_features={self.in_features}, out_features={self.out_features}, "
-                f"bias={self.bias is not None}, codec=nf4-g{GROUP_SIZE}, K_pad={self.K_pad}, "
-                f"home={self.home}, loaded={self.is_loaded}")
+                f"bias={self.bias is not None}, home={self.home}, weight=NF4 in groups of {GROUP_SIZE} "
+                f"(K_pad={self.K_pad})")

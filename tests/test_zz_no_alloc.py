@@ -33,10 +33,17 @@ def _both(lib, m, k, n, seed, ws, ws_floats):
     y_na = torch.ones((m, n), dtype=torch.bfloat16, device="cuda")
     rc_ws = lib.chr_nf4_gemm_ws(ctypes.byref(dev), x.data_ptr(), y_ws.data_ptr(), n, ws.data_ptr(),
                                 ws_floats, stream)
-    before = torch.cuda.memory_allocated()
-    rc_na = lib.chr_nf4_gemm_noalloc(ctypes.byref(dev), x.data_ptr(), y_na.data_ptr(), n, stream)
-    assert torch.cuda.memory_allocated() == before
+    # neither torch's allocator nor the driver hands out memory during the call: the allocator's
+    # own count, and the device's free bytes as the driver reports them (a hipMalloc inside the
+    # library would show there and only there)
     torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated()
+    free_before, _ = torch.cuda.mem_get_info()
+    rc_na = lib.chr_nf4_gemm_noalloc(ctypes.byref(dev), x.data_ptr(), y_na.data_ptr(), n, stream)
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert torch.cuda.memory_allocated() == before
+    assert free_after >= free_before, (free_before, free_after)
     return rc_ws, rc_na, y_ws, y_na, (packed, scale, x)
 
 
@@ -86,3 +93,40 @@ def test_noalloc_refuses_partials_beyond_its_array():
         nf4.nf4_set_tuning()
     assert rc_ws == -7 and rc_na == -7
     assert bool((y_na == 1).all())          # nothing was launched
+
+
+def test_noalloc_calls_recorded_into_a_graph():
+    """What the entry point is for: its calls recorded during stream capture (after a first
+    call on the device outside capture, which looks the array's address up) and replayed, with
+    eager work between the replays; every replay gives the workspace entry's bits."""
+    lib = nf4._load_ext()
+    ws_floats = int(lib.chr_nf4_gemm_noalloc_max_floats())
+    ws = torch.empty(ws_floats, dtype=torch.float32, device="cuda")
+    shapes = [(5120, 13824, 32, 21), (640, 2048, 5, 22)]
+    want, held = [], []
+    for m, k, n, seed in shapes:
+        rc_ws, rc_na, y_ws, y_na, (packed, scale, x) = _both(lib, m, k, n, seed, ws, ws_floats)
+        assert rc_ws == 0 and rc_na == 0
+        want.append(y_ws.clone())
+        held.append((nf4._dev(packed, scale, m, k, oc.k_pad(k)), packed, scale, x,
+                     torch.zeros((m, n), dtype=torch.bfloat16, device="cuda"), n))
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        graph = torch.cuda.CUDAGraph()
+        graph.capture_begin()
+        for dev, _, _, x, y, n in held:
+            assert lib.chr_nf4_gemm_noalloc(ctypes.byref(dev), x.data_ptr(), y.data_ptr(), n, nf4._stream()) == 0
+        graph.capture_end()
+    torch.cuda.synchronize()
+    for rep in range(3):
+        for _, _, _, _, y, _ in held:
+            y.fill_(1)
+        graph.replay()
+        torch.cuda.synchronize()
+        for (_, _, _, _, y, _), w in zip(held, want):
+            assert torch.equal(y.view(torch.int16), w.view(torch.int16)), rep
+        # eager work of the same kind between the replays
+        m, k, n, seed = shapes[1]
+        rc_ws, rc_na, y_ws, y_na, _ = _both(lib, m, k, n, seed, ws, ws_floats)
+        assert rc_ws == 0 and rc_na == 0 and torch.equal(y_ws.view(torch.int16), y_na.view(torch.int16))
