@@ -23,8 +23,9 @@
 // Numerics.  Plain: weight = fp32 LUT * fp32(scale) never rounded below fp32, x widened
 // bf16->fp32 (gpu/nf4/nf4_gemv.cu:70-101, 217-245).  Staged and ring kernels, by the form of
 // the levels (CHR_NF4_GEMV_TERMS): 3, the default: levels rounded to binary16 (2^-12 relative)
-// against x staged as binary16 times a power of two, which holds every bf16 element within
-// 2^-29 of the largest exactly; 2: levels as two bf16 terms (below 2^-17), 8-byte lookups;
+// against x staged as binary16, every 16 consecutive activations times a power of two of
+// their own, which holds every bf16 element within 2^-29 of the largest of its 16 exactly;
+// 2: levels as two bf16 terms (below 2^-17), 8-byte lookups;
 // 1: levels rounded to bf16 (2^-9), the precision class of the reference's tensor-core path
 // (gpu/nf4/nf4_gemm.cu:322).  In all three the products are exact and the fp16 scale is
 // applied in fp32 to each 16-weight partial.  Both families: fp32 accumulation, residual /
@@ -50,11 +51,8 @@ struct GemvLds {
   float ksum[kMaxWaves][4];  // K-split: per-wavefront partial dot products of a row group
 };
 
-// The kernels that stage x in LDS keep two things more in their slot of small statics.
-struct StagedLds : GemvLds {
-  float vmax[kMaxWaves];  // per-wavefront maxima (x staged as binary16)
-  int xexp;               // x staged as binary16: the power of two it was multiplied by
-};
+// The small statics of the kernels that stage x in LDS (their slot of kStagedSmallBytes).
+struct StagedLds : GemvLds {};
 
 __device__ __forceinline__ float fma8(const Levels8 &v, const float *xf, float acc) {
 #pragma unroll
@@ -104,9 +102,17 @@ __device__ __forceinline__ float block_sum(float v, float *part) {
   return s;
 }
 
-// ---- largest magnitude of a staged vector, on the bf16 bit patterns ------------------------
-// The magnitude bits of a bf16 value order like the value's magnitude, so the largest element is
-// an unsigned 16-bit maximum: one packed instruction per two elements.
+// ---- x as binary16 -------------------------------------------------------------------
+// With levels kept as binary16 (11 significant bits against bf16's 8) the products need x as
+// binary16 too.  A bf16 value has 8 significant bits, so it is a binary16 value exactly
+// whenever its exponent fits.  The 16 activations one lane multiplies in one half step (two
+// 16-byte pieces, staged by two neighbouring threads) are therefore multiplied by the power
+// of two that puts the largest of them in [2^14, 2^15): every one within 2^-29 of that
+// largest converts exactly, smaller ones land on binary16's subnormal grid (absolute error
+// below 2^-39 of the largest: far under the fp32 accumulation's own rounding).  The inverse
+// power is kept beside x as a float, one per pair of pieces, and multiplies the fp16 scale of
+// the lane's 16 weights before it meets their sum.  A pair of zeros, or one that holds
+// something not finite: power 0 (what is not finite stays so through the products).
 typedef uint16_t U16x2 __attribute__((ext_vector_type(2)));
 
 __device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
@@ -114,75 +120,26 @@ __device__ __forceinline__ uint32_t pk_max_u16(uint32_t a, uint32_t b) {
                                                                 __builtin_bit_cast(U16x2, b)));
 }
 
-// running maximum of the magnitudes of two bf16 values, per half of the dword
-__device__ __forceinline__ uint32_t mag_max(uint32_t acc, uint32_t pair) {
-  return pk_max_u16(acc, pair & 0x7FFF7FFFu);
-}
-
 template <int CTRL>
 __device__ __forceinline__ uint32_t dpp_u32(uint32_t v) {
   return static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), CTRL, 0xF, 0xF, true));
 }
 
-// maximum per 16-bit half over each row of 16 lanes, in every lane of the row
-__device__ __forceinline__ uint32_t row_pk_max(uint32_t v) {
-  v = pk_max_u16(v, dpp_u32<kDppQuadXor1>(v));
-  v = pk_max_u16(v, dpp_u32<kDppQuadXor2>(v));
-  v = pk_max_u16(v, dpp_u32<kDppRowHalfMirror>(v));
-  v = pk_max_u16(v, dpp_u32<kDppRowMirror>(v));
-  return v;
-}
-
-// Sum of `sum` and per-half maximum of `pk` over the workgroup (16 wavefronts), the same in
-// every thread, with one barrier: wavefront totals go to LDS, lane l reads the total of
-// wavefront l % 16, and a row of 16 lanes folds them.  The caller's next barrier is what
-// separates this use of the two arrays from any later one.
-template <bool WITH_SUM>
-__device__ __forceinline__ void block_fold(float &sum, uint32_t &pk, float *part, float *vmax) {
-  static_assert(kStagedThreads == 16 * kWave, "one total per lane of a 16-lane row");
-  uint32_t *vm = reinterpret_cast<uint32_t *>(vmax);
-  if constexpr (WITH_SUM) {
-    sum = wave_sum(sum);
-  }
-  pk = row_pk_max(pk);
-  const uint32_t r0 = __builtin_amdgcn_readlane(pk, 0), r1 = __builtin_amdgcn_readlane(pk, 16);
-  const uint32_t r2 = __builtin_amdgcn_readlane(pk, 32), r3 = __builtin_amdgcn_readlane(pk, 48);
-  pk = pk_max_u16(pk_max_u16(r0, r1), pk_max_u16(r2, r3));
-  const int lane = threadIdx.x & (kWave - 1);
-  if (lane == 0) {
-    if constexpr (WITH_SUM) {
-      part[threadIdx.x >> 6] = sum;
-    }
-    vm[threadIdx.x >> 6] = pk;
-  }
-  __syncthreads();
-  if constexpr (WITH_SUM) {
-    sum = group_sum<16>(part[lane & 15]);
-  }
-  pk = row_pk_max(vm[lane & 15]);
-}
-
-// the larger half of a packed pair of bf16 magnitudes, as a float
-__device__ __forceinline__ float larger_half_bf16(uint32_t pk) {
-  return bits_to_f32(max(pk & 0xFFFFu, pk >> 16) << 16);
-}
-
-// ---- x as binary16 -------------------------------------------------------------------
-// With levels kept as binary16 (11 significant bits against bf16's 8) the products need x as
-// binary16 too.  A bf16 value has 8 significant bits, so it is a binary16 value exactly
-// whenever its exponent fits; the staged vector is therefore multiplied by the power of two
-// that puts its largest magnitude in [2^14, 2^15): every element within 2^-29 of the largest
-// converts exactly, smaller ones land on binary16's subnormal grid (absolute error below
-// 2^-39 of the largest element: far under the fp32 accumulation's own rounding).  The row
-// sums are multiplied by the inverse power at the end.  Largest magnitude 0 (or not finite):
-// power 0 (what is not finite stays so through the products).
-__device__ __forceinline__ int x_power_for(float largest) {
-  const uint32_t b = f32_to_bits(largest) & 0x7FFFFFFFu;
-  if (b == 0u || b >= 0x7F800000u) {
+// The power for the pair of pieces this thread and its neighbour (lane ^ 1) hold: the
+// magnitude bits of a bf16 value order like its magnitude, so the largest of the 16 is an
+// unsigned 16-bit maximum.  Every lane of the wavefront must be active (the neighbour's
+// value is read across lanes); a thread without a piece passes zeros.
+__device__ __forceinline__ int pair_power(const uint4 &piece) {
+  const uint32_t mask = 0x7FFF7FFFu;
+  uint32_t m = pk_max_u16(pk_max_u16(piece.x & mask, piece.y & mask), pk_max_u16(piece.z & mask, piece.w & mask));
+  m = max(m & 0xFFFFu, m >> 16);
+  m = max(m, dpp_u32<kDppQuadXor1>(m));
+  if (m == 0u || m >= 0x7F80u) {
     return 0;
   }
-  // -113 (the largest bf16) .. 141 (a subnormal reads as exponent -127 and ends up below 2^15 too)
-  return 14 - (static_cast<int>(b >> 23) - 127);
+  // exponent field -127: -113 for the largest bf16, 141 for a subnormal (read as exponent
+  // -127; it ends up below 2^15 too)
+  return 14 - (static_cast<int>(m >> 7) - 127);
 }
 
 // two bf16 values (one dword) -> the same two values times 2^power as a binary16 pair
@@ -190,6 +147,11 @@ __device__ __forceinline__ uint32_t bf16x2_to_f16x2(uint32_t pair, int power) {
   const float lo = __builtin_ldexpf(bf16_lo(pair), power);
   const float hi = __builtin_ldexpf(bf16_hi(pair), power);
   return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(lo, hi));
+}
+
+__device__ __forceinline__ uint4 piece_to_f16(const uint4 &piece, int power) {
+  return make_uint4(bf16x2_to_f16x2(piece.x, power), bf16x2_to_f16x2(piece.y, power),
+                    bf16x2_to_f16x2(piece.z, power), bf16x2_to_f16x2(piece.w, power));
 }
 
 // ---- activations staged in LDS ------------------------------------------------------
@@ -315,25 +277,59 @@ __device__ __forceinline__ void x_request(const StreamArgs &a, uint4 (&v)[kXKeep
   }
 }
 
+// The inverse powers of two of the binary16 form, one float per pair of pieces (= per lane and
+// half step, laid out [t][lane] like the lanes read them), behind the x pieces in LDS.
+__device__ __forceinline__ float *x_factors(uint4 *xs, int K_pad) {
+  return reinterpret_cast<float *>(xs + x_pieces(K_pad));
+}
+
+// One piece on its way to LDS: stored as it is, or (F16) as binary16 times the pair's power,
+// whose inverse the pair's even thread leaves in the factor array.  Called by all lanes of a
+// wavefront together (pair_power reads the neighbour lane); `live` says whether this thread
+// has a piece to store.
+template <bool F16>
+__device__ __forceinline__ void store_piece(uint4 *xs, float *xf, int i, bool live, uint4 piece) {
+  if constexpr (F16) {
+    const int power = pair_power(live ? piece : make_uint4(0, 0, 0, 0));
+    if (live) {
+      xs[x_slot(i)] = piece_to_f16(piece, power);
+      if ((i & 1) == 0) {
+        xf[i >> 1] = __builtin_ldexpf(1.f, -power);
+      }
+    }
+  } else {
+    if (live) {
+      xs[x_slot(i)] = piece;
+    }
+  }
+}
+
 // Fast staging, second half: normalise if asked, store the pieces, barrier.  With rms_w
 // the value stored is bf16( (w*x) * rsqrt(mean(x^2)+eps) ), i.e. what a separate RMSNorm
 // launch would have handed over (gpu/nf4/nf4_gemv.cu:264-289).  F16: those bf16 values are
-// stored as binary16 times a power of two (x_power_for), which lds.xexp then holds.
+// stored as binary16, pair by pair times a power of two (store_piece).
 template <bool F16>
 __device__ __forceinline__ void x_store(const StreamArgs &a, uint4 *xs, StagedLds &lds,
                                         const uint4 (&v)[kXKeep], const uint4 (&g)[kXKeep]) {
   const int nk = a.K >> 3;
   const int nvec = a.K_pad >> 3;
+  float *xf = x_factors(xs, a.K_pad);
   zero_unused_slots(xs, a.K_pad);
+  if constexpr (F16) {
+    // (the pairs of the last half step that no piece maps to: their lanes are switched off where
+    // the scale is applied, but what they multiply must be finite)
+    const int pairs = x_half_steps(a.K_pad) << 6;
+    for (int h = (nvec + 1) / 2 + threadIdx.x; h < pairs; h += kStagedThreads) {
+      xf[h] = 1.f;
+    }
+  }
   float inv = 1.f;
-  int power = 0;
   // first vector index of this wavefront: a wavefront (or a round j of all of them) past the
   // end of x skips the arithmetic as a whole (a scalar branch) and only joins the barriers;
   // at K = 5120 ten of the sixteen wavefronts hold a vector, in the first round only
   const int wave_first = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) & ~(kWave - 1));
   if (a.rms_w != nullptr) {
     float ss = 0.f;
-    uint32_t xm = 0u, gm = 0u;  // largest magnitudes of x and of the norm weights, per dword half
 #pragma unroll
     for (int j = 0; j < kXKeep; ++j) {
       if (wave_first + j * kStagedThreads >= nk) {
@@ -341,45 +337,16 @@ __device__ __forceinline__ void x_store(const StreamArgs &a, uint4 *xs, StagedLd
       }
       const int i = threadIdx.x + j * kStagedThreads;
       const uint32_t u[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
-      const uint32_t gw[4] = {g[j].x, g[j].y, g[j].z, g[j].w};
       float s4 = 0.f;
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         s4 = fmaf(bf16_lo(u[q]), bf16_lo(u[q]), s4);
         s4 = fmaf(bf16_hi(u[q]), bf16_hi(u[q]), s4);
-        if constexpr (F16) {
-          // (a vector past the end repeats the last one: the same maxima)
-          xm = mag_max(xm, u[q]);
-          gm = mag_max(gm, gw[q]);
-        }
       }
       ss += i < nk ? s4 : 0.f;
     }
-    if constexpr (F16) {
-      // one word: the weights' maximum in the high half, x's in the low half
-      uint32_t pk = (max(gm & 0xFFFFu, gm >> 16) << 16) | max(xm & 0xFFFFu, xm >> 16);
-      block_fold<true>(ss, pk, lds.part, lds.vmax);
-      inv = rsqrtf(ss / static_cast<float>(a.K) + a.rms_eps);
-      // No normalised value is larger than bf16((G * X) * inv) with G, X the two maxima: the
-      // product of two bf16 values is exact in fp32, and multiplying by inv and the two
-      // roundings keep the order of magnitudes.
-      const float bound = (bits_to_f32(pk & 0xFFFF0000u) * bits_to_f32(pk << 16)) * inv;
-      power = x_power_for(bf16_to_f32(f32_to_bf16(bound)));
-    } else {
-      ss = block_sum(ss, lds.part);
-      inv = rsqrtf(ss / static_cast<float>(a.K) + a.rms_eps);
-    }
-  } else if constexpr (F16) {
-    uint32_t xm = 0u;
-#pragma unroll
-    for (int j = 0; j < kXKeep; ++j) {
-      if (wave_first + j * kStagedThreads < nk) {
-        xm = mag_max(mag_max(mag_max(mag_max(xm, v[j].x), v[j].y), v[j].z), v[j].w);
-      }
-    }
-    float none = 0.f;
-    block_fold<false>(none, xm, lds.part, lds.vmax);
-    power = x_power_for(larger_half_bf16(xm));
+    ss = block_sum(ss, lds.part);
+    inv = rsqrtf(ss / static_cast<float>(a.K) + a.rms_eps);
   }
 #pragma unroll
   for (int j = 0; j < kXKeep; ++j) {
@@ -387,52 +354,37 @@ __device__ __forceinline__ void x_store(const StreamArgs &a, uint4 *xs, StagedLd
       continue;
     }
     const int i = threadIdx.x + j * kStagedThreads;
-    if (i < nvec) {
-      uint4 o = i < nk ? v[j] : make_uint4(0, 0, 0, 0);
-      if (a.rms_w != nullptr && i < nk) {
-        const uint32_t u[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
-        const uint32_t gw[4] = {g[j].x, g[j].y, g[j].z, g[j].w};
-        uint32_t r[4];
+    uint4 o = i < nk ? v[j] : make_uint4(0, 0, 0, 0);
+    if (a.rms_w != nullptr) {
+      const uint32_t u[4] = {o.x, o.y, o.z, o.w};
+      const uint32_t gw[4] = {g[j].x, g[j].y, g[j].z, g[j].w};
+      uint32_t r[4];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          r[q] = f32x2_to_bf16x2((bf16_lo(gw[q]) * bf16_lo(u[q])) * inv, (bf16_hi(gw[q]) * bf16_hi(u[q])) * inv);
-        }
-        o = make_uint4(r[0], r[1], r[2], r[3]);
+      for (int q = 0; q < 4; ++q) {
+        r[q] = f32x2_to_bf16x2((bf16_lo(gw[q]) * bf16_lo(u[q])) * inv, (bf16_hi(gw[q]) * bf16_hi(u[q])) * inv);
       }
-      if constexpr (F16) {
-        o = make_uint4(bf16x2_to_f16x2(o.x, power), bf16x2_to_f16x2(o.y, power),
-                       bf16x2_to_f16x2(o.z, power), bf16x2_to_f16x2(o.w, power));
-      }
-      xs[x_slot(i)] = o;
+      o = make_uint4(r[0], r[1], r[2], r[3]);
     }
-  }
-  if constexpr (F16) {
-    if (threadIdx.x == 0) {
-      lds.xexp = power;
-    }
+    store_piece<F16>(xs, xf, i, i < nvec, o);
   }
   __syncthreads();
 }
 
-// F16 staging of what the loops below left as bf16: the largest magnitude, then the conversion,
-// every thread on the pieces it alone touches.
-__device__ __forceinline__ void staged_to_f16(const StreamArgs &a, uint4 *xs, StagedLds &lds) {
-  const int nvec = a.K_pad >> 3;
-  uint32_t xm = 0u;
-  for (int i = threadIdx.x; i < nvec; i += kStagedThreads) {
-    const uint4 q = xs[x_slot(i)];
-    xm = mag_max(mag_max(mag_max(mag_max(xm, q.x), q.y), q.z), q.w);
-  }
-  float none = 0.f;
-  block_fold<false>(none, xm, lds.part, lds.vmax);
-  const int power = x_power_for(larger_half_bf16(xm));
-  for (int i = threadIdx.x; i < nvec; i += kStagedThreads) {
-    const uint4 q = xs[x_slot(i)];
-    xs[x_slot(i)] = make_uint4(bf16x2_to_f16x2(q.x, power), bf16x2_to_f16x2(q.y, power),
-                               bf16x2_to_f16x2(q.z, power), bf16x2_to_f16x2(q.w, power));
-  }
-  if (threadIdx.x == 0) {
-    lds.xexp = power;
+// F16 staging of what the loops below left as bf16: every thread takes whole pairs of pieces.
+__device__ __forceinline__ void staged_to_f16(const StreamArgs &a, uint4 *xs) {
+  float *xf = x_factors(xs, a.K_pad);
+  const int pairs = x_half_steps(a.K_pad) << 6;  // every slot pair of the staged half steps
+  for (int h = threadIdx.x; h < pairs; h += kStagedThreads) {
+    const int s0 = ((h >> 6) << 7) + (h & 63);  // slots of pieces 2 h and 2 h + 1
+    const uint4 p0 = xs[s0], p1 = xs[s0 + 64];
+    const uint32_t mask = 0x7FFF7FFFu;
+    uint32_t m = pk_max_u16(pk_max_u16(pk_max_u16(p0.x & mask, p0.y & mask), pk_max_u16(p0.z & mask, p0.w & mask)),
+                            pk_max_u16(pk_max_u16(p1.x & mask, p1.y & mask), pk_max_u16(p1.z & mask, p1.w & mask)));
+    m = max(m & 0xFFFFu, m >> 16);
+    const int power = (m == 0u || m >= 0x7F80u) ? 0 : 14 - (static_cast<int>(m >> 7) - 127);
+    xs[s0] = piece_to_f16(p0, power);
+    xs[s0 + 64] = piece_to_f16(p1, power);
+    xf[h] = __builtin_ldexpf(1.f, -power);
   }
   __syncthreads();
 }
@@ -444,27 +396,15 @@ __device__ __forceinline__ void stage_x(const StreamArgs &a, uint4 *xs, StagedLd
   zero_unused_slots(xs, a.K_pad);
   if (a.attn_state != nullptr) {
     const int nvec = a.K_pad >> 3;
-    if (nvec <= kStagedThreads) {
-      // one piece a thread at most (K <= 8192): it stays in registers from the merge to the
-      // store (binary16: through the search for the largest magnitude and the conversion)
+    if (nvec <= kStagedThreads && (nvec & 127) == 0) {
+      // one piece a thread at most (K <= 8192, whole half steps): it stays in registers from
+      // the merge to the store
+      float *xf = x_factors(xs, a.K_pad);
       const int i = threadIdx.x;
-      uint4 piece = make_uint4(0, 0, 0, 0);
-      if (i < nvec) {
-        piece = a.attn_parts <= 4 ? merged_attn_piece<4>(a, i) : merged_attn_piece<8>(a, i);
-      }
-      if constexpr (F16) {
-        uint32_t xm = mag_max(mag_max(mag_max(mag_max(0u, piece.x), piece.y), piece.z), piece.w);
-        float none = 0.f;
-        block_fold<false>(none, xm, lds.part, lds.vmax);
-        const int power = x_power_for(larger_half_bf16(xm));
-        if (threadIdx.x == 0) {
-          lds.xexp = power;
-        }
-        piece = make_uint4(bf16x2_to_f16x2(piece.x, power), bf16x2_to_f16x2(piece.y, power),
-                           bf16x2_to_f16x2(piece.z, power), bf16x2_to_f16x2(piece.w, power));
-      }
-      if (i < nvec) {
-        xs[x_slot(i)] = piece;
+      const int wave_first = __builtin_amdgcn_readfirstlane(i & ~(kWave - 1));
+      if (wave_first < nvec) {
+        const uint4 piece = a.attn_parts <= 4 ? merged_attn_piece<4>(a, i) : merged_attn_piece<8>(a, i);
+        store_piece<F16>(xs, xf, i, true, piece);
       }
       __syncthreads();
       return;
@@ -474,7 +414,7 @@ __device__ __forceinline__ void stage_x(const StreamArgs &a, uint4 *xs, StagedLd
     }
     __syncthreads();
     if constexpr (F16) {
-      staged_to_f16(a, xs, lds);
+      staged_to_f16(a, xs);
     }
     return;
   }
@@ -503,7 +443,7 @@ __device__ __forceinline__ void stage_x(const StreamArgs &a, uint4 *xs, StagedLd
   }
   __syncthreads();
   if constexpr (F16) {
-    staged_to_f16(a, xs, lds);
+    staged_to_f16(a, xs);
   }
 }
 
@@ -844,16 +784,6 @@ __device__ __forceinline__ void fill_level_table(uint4 *dyn_lds, int wave, int l
   }
 }
 
-// A row sum of the binary16 form is the sum over x * 2^power: divide the power out again.
-template <int TERMS>
-__device__ __forceinline__ float unscaled(float sum, int power) {
-  if constexpr (TERMS == 3) {
-    return __builtin_ldexpf(sum, -power);
-  } else {
-    return sum;
-  }
-}
-
 // ---- staged kernel: x in LDS, pair table, weight requests one item ahead -----------
 // Request half step t of R rows: 8 packed bytes per lane.  Lanes past the end of the row
 // read the row's last half chunk instead (in bounds, one instruction form for every
@@ -875,9 +805,11 @@ __device__ __forceinline__ void load_step(const uint8_t *const (&prow)[R],
 // binary16 against x staged as binary16 (same table shape as TERMS == 1).
 template <int R, int TERMS>
 __device__ __forceinline__ void dot_step(const uint2 (&w)[R], const uint16_t (&sc)[R],
-                                         const uint4 *xs, int n_half, int t, int lane,
+                                         const uint4 *xs, const float *xf, int n_half, int t, int lane,
                                          float (&acc)[R]) {
   const bool on = (t << 6) + lane < n_half;
+  // binary16 x: the inverse of the power of two this lane's 16 activations were staged with
+  const float factor = TERMS == 3 ? xf[(t << 6) + lane] : 1.f;
   const uint4 *xp = xs + (t << 7) + lane;
   const uint4 x0 = xp[0], x1 = xp[64];
   if constexpr (TERMS != 2) {
@@ -893,7 +825,7 @@ __device__ __forceinline__ void dot_step(const uint2 (&w)[R], const uint16_t (&s
       pb = dot2_levels<TERMS>(pair_at<1>(w[r].y, lane4), x1.y, pb);
       pa = dot2_levels<TERMS>(pair_at<2>(w[r].y, lane4), x1.z, pa);
       pb = dot2_levels<TERMS>(pair_at<3>(w[r].y, lane4), x1.w, pb);
-      const float scale = on ? f16_to_f32(sc[r]) : 0.f;
+      const float scale = on ? f16_to_f32(sc[r]) * factor : 0.f;
       acc[r] = fmaf(scale, pa + pb, acc[r]);
     }
   } else {
@@ -951,6 +883,7 @@ __global__ __launch_bounds__(1024) void gemv_staged(const StreamArgs a) {
   char *base = reinterpret_cast<char *>(dyn_lds);
   StagedLds &lds = *reinterpret_cast<StagedLds *>(base + kPairTableBytes);
   uint4 *xs = reinterpret_cast<uint4 *>(base + kPairTableBytes + kStagedSmallBytes);
+  const float *xf = x_factors(xs, a.K_pad);
   constexpr int U = SWIGLU ? R / 2 : R;
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
@@ -1016,8 +949,6 @@ __global__ __launch_bounds__(1024) void gemv_staged(const StreamArgs a) {
     fill_table();
     stage_x<TERMS == 3>(a, xs, lds);
   }
-  // binary16 x: the power of two the row sums are divided by again
-  const int xexp = TERMS == 3 ? __builtin_amdgcn_readfirstlane(lds.xexp) : 0;
 
   // compute cursor: half step ci of the list = step ct of group cg
   int ci = 0, cg = first, ct = 0;
@@ -1029,8 +960,8 @@ __global__ __launch_bounds__(1024) void gemv_staged(const StreamArgs a) {
     if constexpr (SWIGLU) {
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        const float gsum = unscaled<TERMS>(wave_sum(acc[u]), xexp);
-        const float usum = unscaled<TERMS>(wave_sum(acc[U + u]), xexp);
+        const float gsum = wave_sum(acc[u]);
+        const float usum = wave_sum(acc[U + u]);
         const int r = row0 + u;
         if (lane == u && r < M) {
           a.y[0][r] = f32_to_bf16(silu(gsum) * usum);
@@ -1041,7 +972,7 @@ __global__ __launch_bounds__(1024) void gemv_staged(const StreamArgs a) {
       uint16_t *y = a.y[seg];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        float v = unscaled<TERMS>(wave_sum(acc[u]), xexp);
+        float v = wave_sum(acc[u]);
         const int r = row0 + u;
         if (add != nullptr) {
           v += uniform_bf16(add + min(r, M - 1));
@@ -1060,7 +991,7 @@ __global__ __launch_bounds__(1024) void gemv_staged(const StreamArgs a) {
 #define CHR_COMPUTE(W, SC)                                              \
   _Pragma("unroll") for (int j = 0; j < S; ++j) {                       \
     if (ci < n_steps_all) {                                             \
-      dot_step<R, TERMS>(W[j], SC[j], xs, n_half, ct, lane, acc);              \
+      dot_step<R, TERMS>(W[j], SC[j], xs, xf, n_half, ct, lane, acc);          \
       ++ci;                                                             \
       if (++ct == nsteps) {                                             \
         finish_group(cg);                                               \
@@ -1267,6 +1198,9 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
   const uint32_t v_wl = static_cast<uint32_t>(min(lane, rem - 1)) << 3;
   const uint32_t v_sl = static_cast<uint32_t>(min(lane, rem - 1) >> 2) << 1;
   const uint32_t x_lane = kXsAddr + (static_cast<uint32_t>(lane) << 4);
+  // binary16 x: the lane's inverse powers, one float per half step, behind the x pieces
+  const uint32_t f_lane = kXsAddr + (static_cast<uint32_t>(x_pieces(a.K_pad)) << 4) +
+                          (static_cast<uint32_t>(lane) << 2);
   const uint32_t lane_off = TERMS != 2 ? static_cast<uint32_t>(lane) << 2
                                        : static_cast<uint32_t>(lane & 31) << 3;
   const uint64_t last_lanes = ragged ? ((uint64_t{1} << rem) - 1) : ~uint64_t{0};
@@ -1424,8 +1358,6 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
     fill_level_table<TERMS>(dyn_lds, wave, lane);
     stage_x<TERMS == 3>(a, xs, lds);
   }
-  // binary16 x: the power of two the row sums are divided by again
-  const int xexp = TERMS == 3 ? __builtin_amdgcn_readfirstlane(lds.xexp) : 0;
 #undef CHR_RING_FENCE
 #undef CHR_RING_FILL
 #undef CHR_RING_FILL_B
@@ -1437,8 +1369,8 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
   float acc[R] = {};
   auto finish_group = [&](int grp) {
     if constexpr (SWIGLU) {
-      const float gsum = unscaled<TERMS>(wave_sum(acc[0]), xexp);
-      const float usum = unscaled<TERMS>(wave_sum(acc[1]), xexp);
+      const float gsum = wave_sum(acc[0]);
+      const float usum = wave_sum(acc[1]);
       if (lane == 0) {
         a.y[0][grp] = f32_to_bf16(silu(gsum) * usum);
       }
@@ -1452,7 +1384,7 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
         add = third ? a.add[2] : a.add[1];
         row -= third ? seg_end1 : seg_end0;
       }
-      float v = unscaled<TERMS>(wave_sum(acc[0]), xexp);
+      float v = wave_sum(acc[0]);
       if (add != nullptr) {
         v += uniform_bf16(add + row);
       }
@@ -1484,7 +1416,7 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
   // (REQUEST), and only then look the levels up and multiply: the new request travels while
   // this half step is computed.  MASK_IF says whether the lanes past the row's end are to be
   // switched off.
-#define CHR_RING_STEP(I, X0, X1, WAIT, REQUEST, MASK_IF, EMPTY_IF)                        \
+#define CHR_RING_STEP(I, X0, X1, F, WAIT, REQUEST, MASK_IF, EMPTY_IF)                     \
   if (EMPTY_IF) {                                                                         \
     WAIT                                                                                  \
     REQUEST                                                                               \
@@ -1502,6 +1434,11 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
         CHR_RING_MASKED(sg_, sg_, last_lanes);                                            \
         CHR_RING_MASKED(su_, su_, last_lanes);                                            \
       }                                                                                   \
+      if constexpr (TERMS == 3) {                                                         \
+        const float f_ = F;                                                               \
+        sg_ *= f_;                                                                        \
+        su_ *= f_;                                                                        \
+      }                                                                                   \
       acc[0] = fmaf(sg_, ring_row_dot<TERMS>(ag, xw), acc[0]);                            \
       acc[1] = fmaf(su_, ring_row_dot<TERMS>(au, xw), acc[1]);                            \
     } else {                                                                              \
@@ -1511,6 +1448,9 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
       REQUEST                                                                             \
       if (MASK_IF) {                                                                      \
         CHR_RING_MASKED(sw_, sw_, last_lanes);                                            \
+      }                                                                                   \
+      if constexpr (TERMS == 3) {                                                         \
+        sw_ *= F;                                                                         \
       }                                                                                   \
       acc[0] = fmaf(sw_, ring_row_dot<TERMS>(aw, xw), acc[0]);                            \
     }                                                                                     \
@@ -1528,28 +1468,35 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
   // XREG (a row is one piece of at most 5 half steps): the lane's x pieces of the whole row
   // stay in registers, which takes two 16-byte LDS reads out of every half step.
   uint4 x_row[XREG ? 2 * NS : 1];
+  float f_row[XREG && TERMS == 3 ? NS : 1];
   if constexpr (XREG) {
     if (c_left > 0) {
 #pragma unroll
       for (int i = 0; i < NS; ++i) {
         x_row[2 * i] = lds0_u128(x_lane + i * 2048);
         x_row[2 * i + 1] = lds0_u128(x_lane + i * 2048 + 1024);
+        if constexpr (TERMS == 3) {
+          f_row[i] = lds0_at(f_lane + i * 256);
+        }
       }
     }
   }
 #define CHR_RING_OWN_STEP(I, WAIT, REQUEST)                                               \
   if constexpr (NS > (I)) {                                                               \
     if constexpr (XREG) {                                                                 \
-      CHR_RING_STEP(I, x_row[2 * ((I) % NS)], x_row[2 * ((I) % NS) + 1], WAIT, REQUEST,   \
+      CHR_RING_STEP(I, x_row[2 * ((I) % NS)], x_row[2 * ((I) % NS) + 1],                  \
+                    f_row[TERMS == 3 ? (I) % NS : 0], WAIT, REQUEST,                      \
                     (I) == NS - 1 && ragged, false)                                       \
     } else {                                                                              \
-      CHR_RING_STEP(I, lds0_u128(xa + (I) * 2048), lds0_u128(xa + (I) * 2048 + 1024), WAIT, \
+      CHR_RING_STEP(I, lds0_u128(xa + (I) * 2048), lds0_u128(xa + (I) * 2048 + 1024),     \
+                    lds0_at(fa + (I) * 256), WAIT,                                        \
                     REQUEST, (I) == kLastReal && ragged && c_last, (I) > kLastReal && c_last) \
     }                                                                                     \
   }
 #define CHR_RING_PIECE(WAIT, REQUEST_OF, AFTER_REQUESTS)                                  \
   {                                                                                       \
     const uint32_t xa = x_lane + static_cast<uint32_t>(c_part) * (NS * 2048);             \
+    const uint32_t fa = f_lane + static_cast<uint32_t>(c_part) * (NS * 256);              \
     const bool c_last = c_part == pieces - 1;                                             \
     CHR_RING_OWN_STEP(0, WAIT, REQUEST_OF(0))                                             \
     CHR_RING_OWN_STEP(1, WAIT, REQUEST_OF(1))                                             \
@@ -1569,6 +1516,7 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
       ++c_part;                                                                           \
     }                                                                                     \
     (void)xa;                                                                             \
+    (void)fa;                                                                             \
   }
 #define CHR_RING_REQUEST_NEXT(I) CHR_RING_REQUEST(I, q_part == pieces - 1)
 #define CHR_RING_REQUEST_NONE(I)
@@ -1771,9 +1719,10 @@ int prep_lds(Kern kern, size_t dyn) {
 // more again (10.4, 11.0 us) -- deeper request queues do not pay on this memory system.
 constexpr int kItemSteps = 2;
 
-// pair table, small statics, x pieces
+// pair table, small statics, x pieces, the binary16 form's inverse powers (a float per lane and half step)
 inline size_t staged_lds_bytes(int K_pad) {
-  return kPairTableBytes + kStagedSmallBytes + static_cast<size_t>(x_pieces(K_pad)) * 16;
+  return kPairTableBytes + kStagedSmallBytes + static_cast<size_t>(x_pieces(K_pad)) * 16 +
+         static_cast<size_t>(x_half_steps(K_pad)) * kWave * sizeof(float);
 }
 
 // Whether staged launches go to the ring kernels where those take the row length: yes.

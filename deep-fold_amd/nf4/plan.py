@@ -102,9 +102,10 @@ _MAX_DYN_LDS = 150 * 1024
 
 
 def staged_lds_bytes(k_pad_: int) -> int:
-    """LDS of a staged GEMV launch: table, reduction scratch, x in half steps of 1024 codes."""
+    """LDS of a staged GEMV launch: table, reduction scratch, x in half steps of 1024 codes and
+    one float per lane and half step (the powers of two of the binary16 form)."""
     half_steps = _ceil_div(int(k_pad_) // 16, 64)
-    return _STAGED_TABLE_BYTES + _STAGED_SMALL_BYTES + half_steps * 128 * 16
+    return _STAGED_TABLE_BYTES + _STAGED_SMALL_BYTES + half_steps * 128 * 16 + half_steps * 64 * 4
 
 
 def ring_piece_steps(half_steps: int, pairs: bool = False) -> int:

@@ -129,11 +129,12 @@ void chr_nf4_gemm_stream_policy(int32_t policy);
  * rounded to bf16, is what the dots consume.
  * Arithmetic: fp32 accumulation, one bf16 rounding of y.  Launches of fewer than 16M codes
  * multiply fp32 levels (as nf4_gemv.cu:70-101); launches from 16M codes up, and every
- * launch with rms_w or K != K_pad, stage x in LDS (K_pad * 2 <= 85 KB; -6 when rms_w or a
+ * launch with rms_w or K != K_pad, stage x in LDS (K_pad * 2.25 <= 85 KB; -6 when rms_w or a
  * ragged K require it and it does not fit) and multiply the levels in the form
  * CHR_NF4_GEMV_TERMS names: 3 or unset, levels rounded to binary16 (2^-12 relative) against x
- * held as binary16 times a power of two (exact for every bf16 element within 2^-29 of the
- * largest); 2, levels as two bf16 terms (below 2^-17); 1, levels rounded to bf16 (2^-9, the
+ * held as binary16, every 16 consecutive activations times a power of two of their own (exact
+ * for every bf16 element within 2^-29 of the largest of its 16); 2, levels as two bf16 terms
+ * (below 2^-17); 1, levels rounded to bf16 (2^-9, the
  * precision of the reference's tensor-core path, nf4_gemm.cu:322).  CHR_NF4_GEMV_STAGED=0|1
  * in the environment forces either kernel family where both are possible.
  * Replaces chr_nf4_gemv (chr_gpu.h:92-93; nf4_gemv.cu:790-834). */

@@ -73,8 +73,9 @@ def env_terms() -> int:
 
 def staged_levels(terms: int | None = None) -> np.ndarray:
     """The 16 levels as the staged GEMV multiplies them, in float64: rounded to binary16
-    (form 3, the default; x is staged as binary16 times a power of two, which is exact for every
-    element within 2^-29 of the largest, so the model leaves x alone), head = bf16(level) plus
+    (form 3, the default; x is staged as binary16, every 16 consecutive elements times a power
+    of two of their own, which is exact for every element within 2^-29 of the largest of its
+    16, so the model leaves x alone), head = bf16(level) plus
     tail = bf16(level - head) (form 2), or the head alone (form 1)."""
     if terms is None:
         terms = env_terms()

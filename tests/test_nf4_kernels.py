@@ -433,11 +433,12 @@ def test_ring_gemv(m, k, terms, monkeypatch):
     check_linear(y, to_f32(y0), what=f"ring {m}x{k} vs pipelined", ulps=1)
 
 
-# Form 3 stages x as binary16 times the power of two that puts its largest magnitude in
-# [2^14, 2^15).  Every element within 2^-29 of the largest converts exactly; the cases below are
-# the ones a fixed binary16 conversion would break (overflow above 65504, underflow of a vector
-# that is tiny as a whole) and the ones the scaling itself could (all zero, one huge outlier among
-# tiny elements, elements so far below the largest that they land on the subnormal grid).
+# Form 3 stages x as binary16, every 16 consecutive elements times the power of two that puts
+# the largest of them in [2^14, 2^15).  Every element within 2^-29 of that largest converts
+# exactly; the cases below are the ones a fixed binary16 conversion would break (overflow above
+# 65504, underflow of a vector that is tiny as a whole) and the ones the scaling itself could
+# (all zero, one huge outlier among tiny elements, elements so far below their neighbours that
+# they land on the subnormal grid, neighbouring groups of 16 of very different size).
 def _x_cases(k):
     rng = np.random.default_rng(5)
     base = rng.standard_normal(k).astype(np.float32)
