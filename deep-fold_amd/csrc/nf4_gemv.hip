@@ -1151,13 +1151,17 @@ __device__ __forceinline__ float ring_row_dot(const uint32_t (&adr)[8], const ui
 // many.  Those slots are requested like the others (a fixed number of requests per piece is
 // what makes the waits exact), from the piece's first half step, which is there and cached,
 // and never computed.
-template <int NS, bool SWIGLU, int TERMS, bool XREG, int PAD = 0>
+//
+// SEQ (single rows): a group is a gate row and the up row of the same index, walked one after
+// the other through the same ring (same x, same registers as a plain row); the gate's sum
+// waits in a register for the up row's, and the pair leaves silu(gate) * up.
+template <int NS, int TERMS, bool XREG, int PAD = 0, bool SEQ = false>
 __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
-  static_assert(NS >= 2 && NS <= (SWIGLU ? 6 : 8), "slots of the ring that have registers");
+  static_assert(NS >= 2 && NS <= 8, "slots of the ring that have registers");
   static_assert(!XREG || NS <= 5, "x of a whole row in 8 * NS registers");
   static_assert(PAD >= 0 && PAD < NS && !(XREG && PAD > 0), "slots left empty in a row's last piece");
   constexpr int kLastReal = NS - 1 - PAD;  // last slot of a row's last piece that holds a half step
-  constexpr int R = SWIGLU ? 2 : 1;
+  constexpr int R = 1;                 // rows in the ring at a time
   constexpr int D = NS;                // slots of the ring
   constexpr int kStepLoads = 2 * R;    // vector memory operations of one half step
   // LDS byte address of the x pieces (the pair table starts at LDS address 0)
@@ -1188,7 +1192,7 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
   const uint64_t row_scale_bytes = static_cast<uint64_t>(a.K_pad >> 6) << 1;
   const int seg_end0 = a.groups[0];
   const int seg_end1 = a.groups[0] + a.groups[1];
-  const bool one_segment = SWIGLU || a.groups[1] + a.groups[2] == 0;
+  const bool one_segment = SEQ || a.groups[1] + a.groups[2] == 0;
 
   // per-lane loop constants: byte offsets into a half step of packed bytes / of scales (and
   // their clamped forms for a ragged last step), the x pieces' LDS address, the lane's copy
@@ -1212,13 +1216,15 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
 
   // ---- request cursor: piece q_part of group q_group at wq / sq --------------------------
   uint64_t wq[R], sq[R];
-  int q_left = my_groups * pieces, q_part = 0, q_group = first;
+  constexpr int kRowsPerGroup = SEQ ? 2 : 1;
+  int q_left = my_groups * pieces * kRowsPerGroup, q_part = 0, q_group = first;
+  int q_sub = 0;  // SEQ: 0 the gate row of the group, 1 its up row
   auto q_locate = [&]() {
-    if constexpr (SWIGLU) {
-      wq[0] = reinterpret_cast<uint64_t>(a.packed[0]) + static_cast<uint32_t>(q_group) * row_bytes;
-      sq[0] = reinterpret_cast<uint64_t>(a.scale[0]) + static_cast<uint32_t>(q_group) * row_scale_bytes;
-      wq[R - 1] = reinterpret_cast<uint64_t>(a.packed2) + static_cast<uint32_t>(q_group) * row_bytes;
-      sq[R - 1] = reinterpret_cast<uint64_t>(a.scale2) + static_cast<uint32_t>(q_group) * row_scale_bytes;
+    if constexpr (SEQ) {
+      const uint8_t *pk = q_sub == 0 ? a.packed[0] : a.packed2;
+      const uint16_t *sc = q_sub == 0 ? a.scale[0] : a.scale2;
+      wq[0] = reinterpret_cast<uint64_t>(pk) + static_cast<uint32_t>(q_group) * row_bytes;
+      sq[0] = reinterpret_cast<uint64_t>(sc) + static_cast<uint32_t>(q_group) * row_scale_bytes;
     } else {
       int row = q_group;
       const uint8_t *pk = a.packed[0];
@@ -1247,7 +1253,14 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
       return;
     }
     q_part = 0;
-    q_group += stride;
+    if constexpr (SEQ) {
+      q_sub ^= 1;
+      if (q_sub == 0) {
+        q_group += stride;
+      }
+    } else {
+      q_group += stride;
+    }
     q_locate();
   };
   if (q_left > 0) {
@@ -1268,13 +1281,8 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
       : "v"(VW), "s"(WP), "v"(VS), "s"(SP), "n"((I) * 512), "n"((I) * 32)                 \
       : CLOB);
   // slot I: half step I of the piece at wq / sq; LASTP = the piece ends its row
-#define CHR_RING_REQUEST_FORM(I, VW, VS, OFF)                                             \
-  if constexpr (SWIGLU) {                                                                 \
-    CHR_RING_LOAD(RR2_W(I, 0), RR2_S(I, 0), RR2_CLOB(I, 0), VW, VS, wq[0], sq[0], OFF)    \
-    CHR_RING_LOAD(RR2_W(I, 1), RR2_S(I, 1), RR2_CLOB(I, 1), VW, VS, wq[R - 1], sq[R - 1], OFF) \
-  } else {                                                                                \
-    CHR_RING_LOAD(RR1_W(I), RR1_S(I), RR1_CLOB(I), VW, VS, wq[0], sq[0], OFF)             \
-  }
+#define CHR_RING_REQUEST_FORM(I, VW, VS, OFF) \
+  CHR_RING_LOAD(RR1_W(I), RR1_S(I), RR1_CLOB(I), VW, VS, wq[0], sq[0], OFF)
 #define CHR_RING_REQUEST(I, LASTP)                                                        \
   if ((I) > kLastReal && (LASTP)) {                                                       \
     CHR_RING_REQUEST_FORM(I, v_w, v_s, 0)                                                 \
@@ -1367,12 +1375,15 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
 #undef CHR_RING_FILL_STEP
 
   float acc[R] = {};
+  float gate_sum = 0.f;  // SEQ: the gate row's sum while the up row is walked
+  int c_sub = 0;
   auto finish_group = [&](int grp) {
-    if constexpr (SWIGLU) {
-      const float gsum = wave_sum(acc[0]);
-      const float usum = wave_sum(acc[1]);
-      if (lane == 0) {
-        a.y[0][grp] = f32_to_bf16(silu(gsum) * usum);
+    if constexpr (SEQ) {
+      const float sum = wave_sum(acc[0]);
+      if (c_sub == 0) {
+        gate_sum = sum;
+      } else if (lane == 0) {
+        a.y[0][grp] = f32_to_bf16(silu(gate_sum) * sum);
       }
     } else {
       int row = grp;
@@ -1405,12 +1416,7 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
   // The sums go through the chain of asm statements once per half step, which keeps a half
   // step's products ahead of the next half step's wait: left to itself the compiler sinks
   // all products of a piece to its end and holds every level it has looked up until then.
-#define CHR_RING_PIN                                                                      \
-  if constexpr (SWIGLU) {                                                                 \
-    asm("" : "+v"(acc[0]), "+v"(acc[R - 1]), "+s"(tok));                                  \
-  } else {                                                                                \
-    asm("" : "+v"(acc[0]), "+s"(tok));                                                    \
-  }
+#define CHR_RING_PIN asm("" : "+v"(acc[0]), "+s"(tok));
   // The half step in slot I, its x pieces X0 / X1: wait for it (WAIT), turn its packed bytes
   // into lookup addresses, which frees the slot's registers, request the slot again at once
   // (REQUEST), and only then look the levels up and multiply: the new request travels while
@@ -1424,24 +1430,7 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
     const uint4 x0 = X0, x1 = X1;                                                         \
     const uint32_t xw[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};              \
     WAIT                                                                                  \
-    if constexpr (SWIGLU) {                                                               \
-      uint32_t ag[8], au[8];                                                              \
-      float sg_, su_;                                                                     \
-      CHR_RING_ADDRESSES(RR2_X(I, 0), RR2_Y(I, 0), RR2_S(I, 0), ag, sg_, lane_off, tok);  \
-      CHR_RING_ADDRESSES(RR2_X(I, 1), RR2_Y(I, 1), RR2_S(I, 1), au, su_, lane_off, tok);  \
-      REQUEST                                                                             \
-      if (MASK_IF) {                                                                      \
-        CHR_RING_MASKED(sg_, sg_, last_lanes);                                            \
-        CHR_RING_MASKED(su_, su_, last_lanes);                                            \
-      }                                                                                   \
-      if constexpr (TERMS == 3) {                                                         \
-        const float f_ = F;                                                               \
-        sg_ *= f_;                                                                        \
-        su_ *= f_;                                                                        \
-      }                                                                                   \
-      acc[0] = fmaf(sg_, ring_row_dot<TERMS>(ag, xw), acc[0]);                            \
-      acc[1] = fmaf(su_, ring_row_dot<TERMS>(au, xw), acc[1]);                            \
-    } else {                                                                              \
+    {                                                                                     \
       uint32_t aw[8];                                                                     \
       float sw_;                                                                          \
       CHR_RING_ADDRESSES(RR1_X(I), RR1_Y(I), RR1_S(I), aw, sw_, lane_off, tok);           \
@@ -1464,7 +1453,7 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
 #define CHR_RING_WAIT_ALL asm("s_waitcnt vmcnt(0)" : "+s"(tok));
 
   // ---- the groups, a piece per turn --------------------------------------------------------
-  int c_left = my_groups * pieces, c_part = 0, c_group = first;
+  int c_left = my_groups * pieces * kRowsPerGroup, c_part = 0, c_group = first;
   // XREG (a row is one piece of at most 5 half steps): the lane's x pieces of the whole row
   // stay in registers, which takes two 16-byte LDS reads out of every half step.
   uint4 x_row[XREG ? 2 * NS : 1];
@@ -1510,7 +1499,14 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
     --c_left;                                                                             \
     if (c_last) {                                                                         \
       finish_group(c_group);                                                              \
-      c_group += stride;                                                                  \
+      if constexpr (SEQ) {                                                                \
+        c_sub ^= 1;                                                                       \
+        if (c_sub == 0) {                                                                 \
+          c_group += stride;                                                              \
+        }                                                                                 \
+      } else {                                                                            \
+        c_group += stride;                                                                \
+      }                                                                                   \
       c_part = 0;                                                                         \
     } else {                                                                              \
       ++c_part;                                                                           \
@@ -1548,16 +1544,10 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
 // The compiler's VGPR budget stops where the ring's fixed registers begin.  (On this target
 // the attribute counts vector and accumulation registers together and is ignored when the
 // sum exceeds what the launch bounds allow, so it names half the vector registers meant.)
-template <int NS, int TERMS, bool XREG, int PAD = 0>
+template <int NS, int TERMS, bool XREG, int PAD = 0, bool SEQ = false>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_num_vgpr(52))) void gemv_ring_rows(
     const StreamArgs a) {
-  gemv_ring_body<NS, false, TERMS, XREG, PAD>(a);
-}
-
-template <int NS, int TERMS, bool XREG>
-__global__ __launch_bounds__(1024) __attribute__((amdgpu_num_vgpr(46))) void gemv_ring_pairs(
-    const StreamArgs a) {
-  gemv_ring_body<NS, true, TERMS, XREG>(a);
+  gemv_ring_body<NS, TERMS, XREG, PAD, SEQ>(a);
 }
 
 // Half steps of a piece (= slots of the ring, 512 bytes per row each) for a row of nsteps
@@ -1571,13 +1561,13 @@ struct RingPiece {
   int steps;
   int pad;
 };
-RingPiece ring_piece_steps(int nsteps, bool pairs) {
-  for (int ns = pairs ? 6 : 8; ns >= 4; --ns) {
+RingPiece ring_piece_steps(int nsteps) {
+  for (int ns = 8; ns >= 4; --ns) {
     if (nsteps % ns == 0) {
       return {ns, 0};
     }
   }
-  if (!pairs && nsteps > 8) {
+  if (nsteps > 8) {
     for (int ns = 8; ns >= 5; --ns) {
       if ((nsteps + 1) % ns == 0) {
         return {ns, 1};
@@ -1759,12 +1749,12 @@ int pick_family(const StreamArgs &a, int m_total) {
 // wavefront of 256 compute units work; the ring kernel (one row) where ring_wanted says so
 // and it takes the row length; else two rows from 32768 up (lm_head 152064x5120: 75 us
 // against 81 us).
-int staged_rows_for_m(int M, int K_pad, bool pairs) {
+int staged_rows_for_m(int M, int K_pad) {
   const int f = forced_rows();
   if (f > 0) {
     return f;
   }
-  if (ring_wanted() && ring_piece_steps(x_half_steps(K_pad), pairs).steps > 0) {
+  if (ring_wanted() && ring_piece_steps(x_half_steps(K_pad)).steps > 0) {
     return 1;  // the ring kernel walks one row (or one gate/up pair) per group
   }
   return M >= 32768 ? 2 : 1;
@@ -1783,9 +1773,9 @@ int launch_stream(StreamArgs &a, int n_seg, bool staged, hipStream_t st) {
     const int waves = kStagedThreads / kWave;
     const int grid = std::min(device_cu_count(), (total + waves - 1) / waves);
     const int terms = level_terms();
-    constexpr bool kRingShape = (SWIGLU && R == 2) || (!SWIGLU && R == 1);
+    constexpr bool kRingShape = (SWIGLU && R == 2) || (!SWIGLU && R == 1);  // one row, or one gate/up pair, a group
     const RingPiece ring = kRingShape && ring_wanted()
-                               ? ring_piece_steps(x_half_steps(a.K_pad), SWIGLU) : RingPiece{0, 0};
+                               ? ring_piece_steps(x_half_steps(a.K_pad)) : RingPiece{0, 0};
     const int ring_ns = ring.steps;
     if (ring_ns > 0) {
       const int per_pass = grid * waves;
@@ -1808,15 +1798,21 @@ int launch_stream(StreamArgs &a, int n_seg, bool staged, hipStream_t st) {
 #define CHR_GO_ROWS(NS, XREG, PAD)                                                        \
   (terms == 1 ? go(gemv_ring_rows<NS, 1, XREG, PAD>)                                      \
    : terms == 3 ? go(gemv_ring_rows<NS, 3, XREG, PAD>) : go(gemv_ring_rows<NS, 2, XREG, PAD>))
-#define CHR_GO_PAIRS(NS, XREG_OK)                                                         \
-  (terms == 2 ? go(gemv_ring_pairs<NS, 2, false>)                                         \
-   : terms == 1 ? ((XREG_OK) && one_piece ? go(gemv_ring_pairs<NS, 1, XREG_OK>) : go(gemv_ring_pairs<NS, 1, false>)) \
-                : ((XREG_OK) && one_piece ? go(gemv_ring_pairs<NS, 3, XREG_OK>) : go(gemv_ring_pairs<NS, 3, false>)))
+#define CHR_GO_SEQ(NS, XREG, PAD)                                                         \
+  (terms == 1 ? go(gemv_ring_rows<NS, 1, XREG, PAD, true>)                                \
+   : terms == 3 ? go(gemv_ring_rows<NS, 3, XREG, PAD, true>) : go(gemv_ring_rows<NS, 2, XREG, PAD, true>))
         if constexpr (SWIGLU) {
-          switch (ring_ns) {
-            case 4: rc = CHR_GO_PAIRS(4, true); break;
-            case 5: rc = CHR_GO_PAIRS(5, true); break;
-            case 6: rc = CHR_GO_PAIRS(6, false); break;
+          // gate row, then up row of the same index, through the single-row ring
+          switch (ring.pad > 0 ? -ring_ns : ring_ns) {
+            case -5: rc = CHR_GO_SEQ(5, false, 1); break;
+            case -6: rc = CHR_GO_SEQ(6, false, 1); break;
+            case -7: rc = CHR_GO_SEQ(7, false, 1); break;
+            case -8: rc = CHR_GO_SEQ(8, false, 1); break;
+            case 4: rc = one_piece ? CHR_GO_SEQ(4, true, 0) : CHR_GO_SEQ(4, false, 0); break;
+            case 5: rc = one_piece ? CHR_GO_SEQ(5, true, 0) : CHR_GO_SEQ(5, false, 0); break;
+            case 6: rc = CHR_GO_SEQ(6, false, 0); break;
+            case 7: rc = CHR_GO_SEQ(7, false, 0); break;
+            case 8: rc = CHR_GO_SEQ(8, false, 0); break;
           }
         } else {
           switch (ring.pad > 0 ? -ring_ns : ring_ns) {
@@ -1831,7 +1827,7 @@ int launch_stream(StreamArgs &a, int n_seg, bool staged, hipStream_t st) {
             case 8: rc = CHR_GO_ROWS(8, false, 0); break;
           }
         }
-#undef CHR_GO_PAIRS
+#undef CHR_GO_SEQ
 #undef CHR_GO_ROWS
         if (rc != 0) {
           return rc;
@@ -1876,7 +1872,7 @@ int launch_rows(StreamArgs &a, int n_seg, int m_for_policy, hipStream_t st) {
     return -6;
   }
   const bool staged = family == 1;
-  switch (staged ? staged_rows_for_m(m_for_policy, a.K_pad, false) : rows_for_m(m_for_policy)) {
+  switch (staged ? staged_rows_for_m(m_for_policy, a.K_pad) : rows_for_m(m_for_policy)) {
     case 4:
       return launch_stream<4, false>(a, n_seg, staged, st);
     case 2:
@@ -1894,7 +1890,7 @@ int launch_pairs(StreamArgs &a, int m_pairs, hipStream_t st) {
     return -6;
   }
   const bool staged = family == 1;
-  const int rows = staged ? 2 * staged_rows_for_m(m_pairs, a.K_pad, true) : (rows_for_m(2 * m_pairs) >= 2 ? 4 : 2);
+  const int rows = staged ? 2 * staged_rows_for_m(m_pairs, a.K_pad) : (rows_for_m(2 * m_pairs) >= 2 ? 4 : 2);
   if (rows >= 4) {
     return launch_stream<4, true>(a, 1, staged, st);
   }
@@ -1972,7 +1968,7 @@ bool gemv_plan_staged(int M, int K, int K_pad) {
 }
 
 int gemv_rows_per_wg(int M, int K, int K_pad) {
-  return gemv_plan_staged(M, K, K_pad) ? (kStagedThreads / kWave) * staged_rows_for_m(M, K_pad, false)
+  return gemv_plan_staged(M, K, K_pad) ? (kStagedThreads / kWave) * staged_rows_for_m(M, K_pad)
                                        : (kThreads / kWave) * rows_for_m(M);
 }
 

@@ -108,15 +108,15 @@ def staged_lds_bytes(k_pad_: int) -> int:
     return _STAGED_TABLE_BYTES + _STAGED_SMALL_BYTES + half_steps * 128 * 16 + half_steps * 64 * 4
 
 
-def ring_piece_steps(half_steps: int, pairs: bool = False) -> int:
+def ring_piece_steps(half_steps: int) -> int:
     """Half steps per piece of the ring GEMV kernel for a row of ``half_steps``: the largest
-    divisor in 4..8 (4..6 for gate/up pairs); for single rows longer than a piece also the
-    largest of 8..5 that divides ``half_steps + 1`` (the last piece then ends in one empty
-    slot); 0 when that kernel does not take the row."""
-    for ns in range(6 if pairs else 8, 3, -1):
+    divisor in 4..8; for rows longer than a piece also the largest of 8..5 that divides
+    ``half_steps + 1`` (the last piece then ends in one empty slot); 0 when that kernel does
+    not take the row.  Gate/up pairs go through the same ring, one row after the other."""
+    for ns in range(8, 3, -1):
         if half_steps % ns == 0:
             return ns
-    if not pairs and half_steps > 8:
+    if half_steps > 8:
         for ns in range(8, 4, -1):
             if (half_steps + 1) % ns == 0:
                 return ns

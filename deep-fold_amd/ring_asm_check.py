@@ -25,9 +25,9 @@ import re
 import subprocess
 import tempfile
 
-KERNEL = re.compile(r"^(_ZN3chr12_GLOBAL__N_1\d+gemv_ring_(rows|pairs)\w+):", re.M)
+KERNEL = re.compile(r"^(_ZN3chr12_GLOBAL__N_1\d+gemv_ring_(rows)\w+):", re.M)
 #: first fixed register of each kernel family (``csrc/nf4_gemv_ring_regs.h``)
-BUDGET = {"rows": 104, "pairs": 92}
+BUDGET = {"rows": 104}
 HAZARD_WAIT_STATES = 5
 
 

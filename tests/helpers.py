@@ -111,7 +111,7 @@ def staged_gemv_model(packed: np.ndarray, scale: np.ndarray, m: int, k: int,
 
 
 def check_linear(y: torch.Tensor, y_ref: np.ndarray, *, what: str = "", ulps: float = 1.0,
-                 model: np.ndarray | None = None) -> dict:
+                 model: np.ndarray | None = None, floor: bool = True) -> dict:
     """y (bf16 on GPU) against a float32/float64 oracle result of the same shape.
 
     Three bounds: the reference's floor-1 bound max(0.05, ULP/2); max-rel 1e-2;
@@ -126,7 +126,8 @@ def check_linear(y: torch.Tensor, y_ref: np.ndarray, *, what: str = "", ulps: fl
     err = np.abs(got - ref)
     u = ulp_bf16(ref)
     rms = float(np.sqrt((ref ** 2).mean())) if ref.size else 0.0
-    assert (err <= np.maximum(MAXABS_FLOOR, 0.5 * u) + 1e-12).all(), f"{what}: maxabs {err.max():.6f}"
+    if floor:  # (a bound for one linear at rms(x) ~ 1; not for a product of two long ones)
+        assert (err <= np.maximum(MAXABS_FLOOR, 0.5 * u) + 1e-12).all(), f"{what}: maxabs {err.max():.6f}"
     denom = np.abs(ref).max()
     if denom > 0:
         assert err.max() / denom <= MAX_REL, f"{what}: max-rel {err.max() / denom:.3e}"
