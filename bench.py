@@ -17,6 +17,7 @@ Extra objects on the same line:
   decode        resident greedy decode of the 14B-shaped model: tokens/s from
                 graph replays and its fraction of the bandwidth roofline
   prefill       MFMA GEMM chunks at the 14B linear shapes, N in {8, 16, 32}
+  layer_launches  the five launches of one 14B decode layer, each on its own
 """
 
 from __future__ import annotations
@@ -214,6 +215,94 @@ def bench_gemv_shapes(torch, nf4):
                      "hbm_frac": by / ms / 1e6 / HBM_PEAK_GBPS})
         del weights
         torch.cuda.empty_cache()
+    return rows
+
+
+def bench_layer_launches(torch, nf4, contexts=(640, 2047)):
+    """The five launches of one 14B-architecture decode layer, each on its own (graph replays,
+    rotating weights and caches): q/k/v with the folded RMSNorm and biases, the attention at the
+    given cache lengths, the o projection that merges the attention's states and adds the
+    residual, gate/up with the folded RMSNorm and SwiGLU, down with the residual."""
+    from deepfold_amd.decodev2.rope import rope_tables_torch
+
+    k5, ffn, n_q, n_kv, hd, max_seq = 5120, 13824, 40, 8, 128, 2048
+    rows = []
+    dev = "cuda"
+    x = torch.randn(k5, device=dev).to(torch.bfloat16)
+    g = (1 + 0.05 * torch.randn(k5, device=dev)).to(torch.bfloat16)
+    res = torch.randn(k5, device=dev).to(torch.bfloat16)
+
+    def add(name, launch, nbytes, n=120):
+        ms = graph_time(torch, launch, n)
+        rows.append({"launch": name, "us": ms * 1e3, "bytes": nbytes, "gbps": nbytes / ms / 1e6,
+                     "hbm_frac": nbytes / ms / 1e6 / HBM_PEAK_GBPS})
+
+    c = 24
+    q = make_weights(torch, nf4, n_q * hd, k5, c, 1)
+    kk = make_weights(torch, nf4, n_kv * hd, k5, c, 2)
+    v = make_weights(torch, nf4, n_kv * hd, k5, c, 3)
+    yq = torch.empty(n_q * hd, dtype=torch.bfloat16, device=dev)
+    yk = torch.empty(n_kv * hd, dtype=torch.bfloat16, device=dev)
+    yv = torch.empty(n_kv * hd, dtype=torch.bfloat16, device=dev)
+    bq, bk, bv = (torch.randn(t.numel(), device=dev).to(torch.bfloat16) for t in (yq, yk, yv))
+
+    def qkv(i):
+        j = i % c
+        nf4.nf4_qkv(q[j][0], q[j][1], kk[j][0], kk[j][1], v[j][0], v[j][1], x, n_q * hd, n_kv * hd, n_kv * hd,
+                    k5, k5, yq, yk, yv, bq, bk, bv, rms_w=g)
+
+    add("q/k/v 7168x5120 + RMSNorm + biases", qkv, algorithmic_bytes((n_q + 2 * n_kv) * hd, k5))
+    del q, kk, v
+    torch.cuda.empty_cache()
+
+    layers = 48
+    kc = torch.randn(layers, max_seq, n_kv, hd, device=dev).to(torch.bfloat16)
+    vc = torch.randn(layers, max_seq, n_kv, hd, device=dev).to(torch.bfloat16)
+    qa = torch.randn(n_q, hd, device=dev).to(torch.bfloat16)
+    ka = torch.randn(n_kv, hd, device=dev).to(torch.bfloat16)
+    va = torch.randn(n_kv, hd, device=dev).to(torch.bfloat16)
+    cos, sin = rope_tables_torch(max_seq, hd, 1e6, device=dev, dtype=torch.bfloat16)
+    state = torch.zeros(nf4.dv2_attn_state_floats(n_q, hd), dtype=torch.float32, device=dev)
+    for ctx in contexts:
+        vl = torch.full((), ctx, dtype=torch.int32, device=dev)
+        pos = torch.full((), ctx, dtype=torch.int64, device=dev)
+
+        def attn(i, vl=vl, pos=pos):
+            layer = i % layers
+            nf4.dv2_attn_parts(qa, kc[layer], vc[layer], vl, hd ** -0.5, state, k_act=ka, v_act=va, cos=cos,
+                               sin=sin, position=pos)
+
+        add(f"attention, {ctx} cache rows (RoPE, cache write, states for the o projection)", attn,
+            2 * ctx * n_kv * hd * 2, n=96)
+    del kc, vc
+    torch.cuda.empty_cache()
+
+    o = make_weights(torch, nf4, k5, k5, 40, 5)
+    yo = torch.empty(k5, dtype=torch.bfloat16, device=dev)
+    st = torch.randn(nf4.dv2_attn_state_floats(n_q, hd), device=dev).abs()
+    add("o 5120x5120 + attention merge + residual",
+        lambda i: nf4.dv2_gemv_attn(o[i % 40][0], o[i % 40][1], st, n_q, hd, k5, k5, k5, yo, res),
+        algorithmic_bytes(k5, k5) + st.numel() * 4)
+    del o
+    torch.cuda.empty_cache()
+
+    ga = make_weights(torch, nf4, ffn, k5, 10, 6)
+    up = make_weights(torch, nf4, ffn, k5, 10, 7)
+    ys = torch.empty(ffn, dtype=torch.bfloat16, device=dev)
+    add("gate/up 2 x 13824x5120 + RMSNorm + SwiGLU",
+        lambda i: nf4.nf4_swiglu(ga[i % 10][0], ga[i % 10][1], up[i % 10][0], up[i % 10][1], x, ffn, k5, k5, ys,
+                                 rms_w=g),
+        2 * algorithmic_bytes(ffn, k5) - 2 * k5 - 2 * ffn)
+    del ga, up
+    torch.cuda.empty_cache()
+
+    d = make_weights(torch, nf4, k5, ffn, 18, 8)
+    xd = torch.randn(ffn, device=dev).to(torch.bfloat16)
+    add("down 5120x13824 + residual",
+        lambda i: nf4.nf4_gemv(d[i % 18][0], d[i % 18][1], xd, k5, ffn, ffn, yo, res),
+        algorithmic_bytes(k5, ffn) + 2 * k5)
+    del d
+    torch.cuda.empty_cache()
     return rows
 
 
@@ -487,6 +576,8 @@ def main() -> int:
     ap.add_argument("--prefill-widths", default="8,16,32,64", help="chunk widths of the prefill sweep")
     ap.add_argument("--decode-models", default="3b,14b,20b,32b", help="comma list of 3b,14b,20b,32b")
     ap.add_argument("--no-shapes", action="store_true", help="skip the GEMV sweep over other shapes")
+    ap.add_argument("--no-layer", action="store_true",
+                    help="skip the five launches of a 14B decode layer measured one by one")
     ap.add_argument("--schedule", default=None, help="decode launch schedule: plain or fold_rms")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="MiB",
                     help="first run four plain device copies of this size (a kernel of known "
@@ -589,6 +680,10 @@ def main() -> int:
         out["gemv_shapes"] = bench_gemv_shapes(torch, nf4)
         for row in out["gemv_shapes"]:
             out["roofline"]["other"][f"gemv_{row['M']}x{row['K']}_frac"] = row["hbm_frac"]
+    if not args.no_layer:
+        out["layer_launches"] = bench_layer_launches(torch, nf4)
+        out["roofline"]["other"]["layer_14b_sum_us"] = sum(
+            r["us"] for r in out["layer_launches"] if "2047" not in r["launch"])
     if not args.no_decode:
         rows = []
         for name in (n.strip() for n in args.decode_models.split(",")):
