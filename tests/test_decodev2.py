@@ -293,7 +293,7 @@ def test_greedy_64_tokens_identical_to_the_oracle(form, monkeypatch):
 #: that, every launch form must reproduce all 64 ids, eager and from the captured graph: a hard
 #: assertion, no floor.
 WIDE_GAP_STEPS = 2.0
-WIDE_GAP_STREAMS = 8
+WIDE_GAP_STREAMS = 16
 
 
 def wide_gap_streams():
