@@ -13,6 +13,8 @@
 // current key stay fp32; older keys and all values come from the bf16 cache;
 // running max starts at -1e30; exp is the fast hardware exponential.
 
+#include <cstdlib>
+
 #include "nf4_common.h"
 
 namespace chr {
@@ -85,7 +87,33 @@ struct AttnArgs {
   // q + t*q_tok_stride, sees *valid_len + t cache rows, and writes dim d of a head to
   // out[t*out_tok_stride + (head*hd + d)*out_dim_stride]
   int q_tok_stride, out_tok_stride, out_dim_stride;
+  // one-workgroup forms: workgroups are dealt to the eight dies of the chip in turn (workgroup
+  // b runs on die b % 8, each with its own L2).  With xcd_map the (head, part) of a workgroup
+  // follows from b so that the query heads of one KV head that walk the same cache rows (the
+  // same part) share a die: a cache row is then fetched from memory by one L2 instead of by
+  // each die that holds one of those heads.  Placement only: what a (head, part) computes and
+  // where it writes does not change.
+  int xcd_map;
 };
+
+constexpr int kDies = 8;
+
+// (head, part) of workgroup b of a one-workgroup-form launch (n_q * n_parts workgroups a
+// token).  xcd_map: die X = b % 8 holds the (KV head, part) pairs c = X, X + 8, .. (c = KV
+// head * n_parts + part), each with its n_rep query heads next to each other.
+__device__ __forceinline__ void locate_head(const AttnArgs &a, int b, int n_rep, int &head, int &part) {
+  if (a.xcd_map) {
+    const int die = b % kDies, idx = b / kDies;
+    const int j = idx / n_rep, r = idx - j * n_rep;
+    const int c = die + kDies * j;
+    const int g = c / a.n_parts;
+    part = c - g * a.n_parts;
+    head = g * n_rep + r;
+  } else {
+    part = b % a.n_parts;
+    head = b / a.n_parts;
+  }
+}
 
 constexpr int kMaxWgSplits = 16;  // wavefronts of a one-workgroup-per-head launch
 
@@ -163,16 +191,17 @@ __global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flas
   constexpr int TPW = kWave / LPT;  // time steps per wavefront iteration
   const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
   const int wg_waves = static_cast<int>(blockDim.x >> 6);
-  const int part = INWG ? static_cast<int>(blockIdx.x) % a.n_parts : 0;
-  const int head = INWG ? static_cast<int>(blockIdx.x) / a.n_parts
-                        : static_cast<int>(blockIdx.x) / a.n_split;
+  const int n_rep = a.n_q / a.n_kv;
+  int part = 0, head = static_cast<int>(blockIdx.x) / a.n_split;
+  if constexpr (INWG) {
+    locate_head(a, static_cast<int>(blockIdx.x), n_rep, head, part);
+  }
   const int split = INWG ? part * wg_waves + wave : static_cast<int>(blockIdx.x) % a.n_split;
   const int lane = threadIdx.x & (kWave - 1);
   const int li = lane % LPT;  // which 8 dims of the head
   const int grp = lane / LPT; // which time step of the iteration
   const int hd = a.hd;
   const int d0 = li * 8;
-  const int n_rep = a.n_q / a.n_kv;
   const int kv_head = head / n_rep;
   const int tok = INWG ? static_cast<int>(blockIdx.y) : 0;
   const int vl = min(*a.valid_len + tok, a.max_seq);
@@ -520,14 +549,15 @@ __global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flas
     const AttnArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
   const int wg_waves = static_cast<int>(blockDim.x >> 6);
-  const int part = INWG ? static_cast<int>(blockIdx.x) % a.n_parts : 0;
-  const int head = INWG ? static_cast<int>(blockIdx.x) / a.n_parts
-                        : static_cast<int>(blockIdx.x) / a.n_split;
+  const int n_rep = a.n_q / a.n_kv;
+  int part = 0, head = static_cast<int>(blockIdx.x) / a.n_split;
+  if constexpr (INWG) {
+    locate_head(a, static_cast<int>(blockIdx.x), n_rep, head, part);
+  }
   const int split = INWG ? part * wg_waves + wave : static_cast<int>(blockIdx.x) % a.n_split;
   const int lane = threadIdx.x & (kWave - 1);
   const int hd = a.hd;
   const int half = hd / 2;
-  const int n_rep = a.n_q / a.n_kv;
   const int kv_head = head / n_rep;
   const int tok = INWG ? static_cast<int>(blockIdx.y) : 0;
   const int vl = min(*a.valid_len + tok, a.max_seq);
@@ -815,6 +845,13 @@ int attn_common(const void *q, const void *k, const void *v, void *out, const vo
   a.q_tok_stride = n_q * hd;
   a.out_tok_stride = out_tok_stride;
   a.out_dim_stride = out_dim_stride;
+  // heads that share cache rows on one die, where the (KV head, part) pairs deal out evenly
+  // over the dies (CHR_ATTN_XCD_MAP=0: workgroups in head order, for comparison)
+  static const bool xcd_map_on = [] {
+    const char *e = std::getenv("CHR_ATTN_XCD_MAP");
+    return e == nullptr || e[0] != '0';
+  }();
+  a.xcd_map = (xcd_map_on && mode != 0 && (n_kv * a.n_parts) % kDies == 0) ? 1 : 0;
   hipStream_t st = static_cast<hipStream_t>(stream);
   // The vector path needs 16-byte aligned rows and 16-byte aligned fp32 partials.
   const bool vec_ok = aligned16(q) && aligned16(k) && aligned16(v) &&
