@@ -248,6 +248,19 @@ __device__ __forceinline__ uint4 merged_attn_piece(const StreamArgs &a, int i) {
 
 constexpr int kXKeep = 4;  // 16-byte vectors of x a thread keeps between request and use
 
+// Threads the 16-byte vectors of x are dealt over in the fast staging (vector i to thread
+// i % deal, its round i / deal): the first eight wavefronts where x fits their kXKeep rounds,
+// all sixteen beyond.  The wavefronts that hold no x write their share of the level table and
+// wait at the barrier; with eight rather than sixteen (or the ten that 640 vectors would take
+// at one each) asking for x, its requests queue behind fewer of the first weight requests:
+// 5120x13824 10.35 -> 10.0 us, 13824x5120 9.35 -> 9.25 us, 14B decode +1% (256 and 384
+// threads: no better).
+constexpr int kXDeal = 512;
+static_assert(kXDeal <= kStagedThreads && kXDeal % 128 == 0, "whole pairs of wavefront lanes");
+__device__ __forceinline__ int x_deal(int nk) {
+  return nk <= kXKeep * kXDeal ? kXDeal : kStagedThreads;
+}
+
 // The common case of staging: K a multiple of 8, aligned pointers, x short enough to sit in
 // registers between its request and its use, no attention merge.
 __device__ __forceinline__ bool stage_fast_ok(const StreamArgs &a) {
@@ -263,12 +276,14 @@ __device__ __forceinline__ bool stage_fast_ok(const StreamArgs &a) {
 __device__ __forceinline__ void x_request(const StreamArgs &a, uint4 (&v)[kXKeep],
                                           uint4 (&g)[kXKeep]) {
   const int nk = a.K >> 3;
+  const int deal = x_deal(a.K_pad >> 3);
+  const int wave_first = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) & ~(kWave - 1));
 #pragma unroll
   for (int j = 0; j < kXKeep; ++j) {
     v[j] = make_uint4(0, 0, 0, 0);
     g[j] = make_uint4(0, 0, 0, 0);
-    if (j * kStagedThreads < nk) {
-      const int i = min(static_cast<int>(threadIdx.x) + j * kStagedThreads, nk - 1);
+    if (j * deal < nk && wave_first < deal) {
+      const int i = min(static_cast<int>(threadIdx.x) + j * deal, nk - 1);
       v[j] = reinterpret_cast<const uint4 *>(a.x)[i];
       if (a.rms_w != nullptr) {
         g[j] = reinterpret_cast<const uint4 *>(a.rms_w)[i];
@@ -326,16 +341,17 @@ __device__ __forceinline__ void x_store(const StreamArgs &a, uint4 *xs, StagedLd
   float inv = 1.f;
   // first vector index of this wavefront: a wavefront (or a round j of all of them) past the
   // end of x skips the arithmetic as a whole (a scalar branch) and only joins the barriers;
-  // at K = 5120 ten of the sixteen wavefronts hold a vector, in the first round only
+  // at K = 5120 eight wavefronts hold a vector, two of them a second one
   const int wave_first = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) & ~(kWave - 1));
+  const int deal = x_deal(nvec);
   if (a.rms_w != nullptr) {
     float ss = 0.f;
 #pragma unroll
     for (int j = 0; j < kXKeep; ++j) {
-      if (wave_first + j * kStagedThreads >= nk) {
+      if (wave_first + j * deal >= nk || wave_first >= deal) {
         continue;
       }
-      const int i = threadIdx.x + j * kStagedThreads;
+      const int i = threadIdx.x + j * deal;
       const uint32_t u[4] = {v[j].x, v[j].y, v[j].z, v[j].w};
       float s4 = 0.f;
 #pragma unroll
@@ -350,10 +366,10 @@ __device__ __forceinline__ void x_store(const StreamArgs &a, uint4 *xs, StagedLd
   }
 #pragma unroll
   for (int j = 0; j < kXKeep; ++j) {
-    if (wave_first + j * kStagedThreads >= nvec) {
+    if (wave_first + j * deal >= nvec || wave_first >= deal) {
       continue;
     }
-    const int i = threadIdx.x + j * kStagedThreads;
+    const int i = threadIdx.x + j * deal;
     uint4 o = i < nk ? v[j] : make_uint4(0, 0, 0, 0);
     if (a.rms_w != nullptr) {
       const uint32_t u[4] = {o.x, o.y, o.z, o.w};
@@ -1040,7 +1056,7 @@ __global__ __launch_bounds__(1024) void gemv_staged(const StreamArgs a) {
 // ones are in flight, and its slot is requested again as soon as its bytes have been turned
 // into lookup addresses.  Work is dealt as in the staged kernel's comment.
 struct XRegs {
-  U32x4 v[kXKeep];  // x, 16-byte vectors i = thread + j * 1024
+  U32x4 v[kXKeep];  // x, 16-byte vectors i = thread + j * x_deal()
   U32x4 g[kXKeep];  // the RMSNorm weights at the same places (fused norm only)
 };
 
@@ -1052,12 +1068,14 @@ __device__ __forceinline__ void request16(U32x4 &d, const void *p, uint32_t &tok
 
 __device__ __forceinline__ void ring_x_request(const StreamArgs &a, XRegs &x, uint32_t &tok) {
   const int nk = a.K >> 3;
+  const int deal = x_deal(a.K_pad >> 3);
+  const int wave_first = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) & ~(kWave - 1));
 #pragma unroll
   for (int j = 0; j < kXKeep; ++j) {
     x.v[j] = U32x4{0u, 0u, 0u, 0u};
     x.g[j] = U32x4{0u, 0u, 0u, 0u};
-    if (j * kStagedThreads < nk) {
-      const int i = min(static_cast<int>(threadIdx.x) + j * kStagedThreads, nk - 1);
+    if (j * deal < nk && wave_first < deal) {
+      const int i = min(static_cast<int>(threadIdx.x) + j * deal, nk - 1);
       request16(x.v[j], reinterpret_cast<const uint4 *>(a.x) + i, tok);
       if (a.rms_w != nullptr) {
         request16(x.g[j], reinterpret_cast<const uint4 *>(a.rms_w) + i, tok);
