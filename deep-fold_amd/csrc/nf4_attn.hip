@@ -94,6 +94,9 @@ struct AttnArgs {
   // each die that holds one of those heads.  Placement only: what a (head, part) computes and
   // where it writes does not change.
   int xcd_map;
+  // n_q / n_kv, and reciprocals for the index arithmetic ahead of the first cache request
+  int n_rep;
+  float inv_rep, inv_parts;
 };
 
 constexpr int kDies = 8;
@@ -101,17 +104,27 @@ constexpr int kDies = 8;
 // (head, part) of workgroup b of a one-workgroup-form launch (n_q * n_parts workgroups a
 // token).  xcd_map: die X = b % 8 holds the (KV head, part) pairs c = X, X + 8, .. (c = KV
 // head * n_parts + part), each with its n_rep query heads next to each other.
-__device__ __forceinline__ void locate_head(const AttnArgs &a, int b, int n_rep, int &head, int &part) {
+// x / d for the small non-negative indices of a launch, d also given as 1.f / d: three vector
+// instructions where the integer division is some thirty, on the way to a kernel's first
+// memory request.  Exact for x < 2^22 and d <= 256 (every such pair checked on the CPU: (x + 0.5)
+// / d is at least 0.5 / d from the next integer, the float error far below that); the host
+// passes inv_d = 0 outside that range and the integer division runs.
+__device__ __forceinline__ int small_div(int x, int d, float inv_d) {
+  return inv_d != 0.f ? static_cast<int>((static_cast<float>(x) + 0.5f) * inv_d) : x / d;
+}
+
+__device__ __forceinline__ void locate_head(const AttnArgs &a, int b, int &head, int &part, int &kv_head) {
   if (a.xcd_map) {
     const int die = b % kDies, idx = b / kDies;
-    const int j = idx / n_rep, r = idx - j * n_rep;
+    const int j = small_div(idx, a.n_rep, a.inv_rep), r = idx - j * a.n_rep;
     const int c = die + kDies * j;
-    const int g = c / a.n_parts;
-    part = c - g * a.n_parts;
-    head = g * n_rep + r;
+    kv_head = small_div(c, a.n_parts, a.inv_parts);
+    part = c - kv_head * a.n_parts;
+    head = kv_head * a.n_rep + r;
   } else {
-    part = b % a.n_parts;
-    head = b / a.n_parts;
+    head = small_div(b, a.n_parts, a.inv_parts);
+    part = b - head * a.n_parts;
+    kv_head = small_div(head, a.n_rep, a.inv_rep);
   }
 }
 
@@ -180,21 +193,100 @@ __device__ __forceinline__ void merge_head(const float *m_s, const float *l_s, c
   }
 }
 
+// Fold the kWave / LPT lane groups of a wavefront: lanes with equal lane % LPT hold online-softmax
+// states (m, l, acc[8]) of different time-step subsets; afterwards every lane holds the state of
+// their union.  (The row-swap instructions in place of the shuffles for offsets 16 and 32 were
+// measured: no faster.)
+template <int LPT>
+__device__ __forceinline__ void fold_lane_groups(float &m, float &l, float (&acc)[8]) {
+  if constexpr (LPT < kWave) {
+    float mg = m;
+#pragma unroll
+    for (int off = LPT; off < kWave; off <<= 1) {
+      mg = fmaxf(mg, __shfl_xor(mg, off, kWave));
+    }
+    const float w = __expf(m - mg);
+    l *= w;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      acc[i] *= w;
+    }
+#pragma unroll
+    for (int off = LPT; off < kWave; off <<= 1) {
+      l += __shfl_xor(l, off, kWave);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        acc[i] += __shfl_xor(acc[i], off, kWave);
+      }
+    }
+    m = mg;
+  }
+}
+
+// The same merge for states that sit in LDS, by the workgroup that left them there (after its
+// barrier): thread d takes dim d and walks the n <= 16 states itself, in state order -- no
+// cross-lane traffic, every read independent -- instead of one wavefront doing the whole head
+// with a shuffle per state and dim (1.3 us of a 5.3 us launch at 8 states of 128 dims; this
+// form 0.3).  m and l of the states are broadcast reads; every thread computes the same
+// weights.
+__device__ __forceinline__ void merge_wg(const float *sm, const float *sl, const float *so,
+                                         uint16_t *dst, int hd, int n, int d, float *state,
+                                         int dstride) {
+  float m = kNegBig;
+#pragma unroll
+  for (int s = 0; s < kMaxWgSplits; ++s) {
+    m = fmaxf(m, sm[min(s, n - 1)]);
+  }
+  float l = 0.f, acc = 0.f;
+  for (int s0 = 0; s0 < n; s0 += 8) {
+    float w[8], v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int sc = min(s0 + j, n - 1);
+      w[j] = s0 + j < n ? __expf(sm[sc] - m) : 0.f;
+      v[j] = so[sc * hd + d];
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int sc = min(s0 + j, n - 1);
+      l = fmaf(w[j], sl[sc], l);
+      acc = fmaf(w[j], v[j], acc);
+    }
+  }
+  if (state != nullptr) {
+    if (d == 0) {
+      state[0] = m;
+      state[1] = l;
+    }
+    state[4 + d] = acc;  // unnormalised: the later merge divides
+  } else {
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    dst[static_cast<size_t>(d) * dstride] = f32_to_bf16(l > 0.f ? acc * inv : 0.f);
+  }
+}
+
 // LPT lanes per time step, 8 dims per lane: hd == 8*LPT.
 // INWG == false: one wavefront per (head, split), partials to global memory, merged by a
 //                second launch (attn_merge).
 // INWG == true : one workgroup per head, wavefront w takes split w of n_split =
-//                blockDim.x/64 <= 16, partials meet in LDS and wavefront 0 merges them:
-//                no workspace and no second launch.
-template <int LPT, bool INWG>
-__global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flash(const AttnArgs a) {
+//                blockDim.x/64 <= 16, partials meet in LDS and the workgroup merges them:
+//                no workspace and no second launch.  WMAX = the most wavefronts a workgroup of
+//                the instantiation is launched with: up to 8 leave every lane 256 registers,
+//                enough to hold the next block of cache rows while the current one is
+//                computed (at 2047 rows an iteration took 1.5 us, 0.7 of arithmetic after
+//                0.8 of waiting for its rows: 11.2 -> 10.2 us).
+template <int LPT, bool INWG, int WMAX = kMaxWgSplits>
+__global__ __launch_bounds__(INWG ? kWave * WMAX : kWave) void attn_flash(const AttnArgs a) {
   constexpr int TPW = kWave / LPT;  // time steps per wavefront iteration
+  constexpr bool AHEAD = INWG && WMAX <= 8;
   const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
   const int wg_waves = static_cast<int>(blockDim.x >> 6);
-  const int n_rep = a.n_q / a.n_kv;
-  int part = 0, head = static_cast<int>(blockIdx.x) / a.n_split;
+  const int n_rep = a.n_rep;
+  int part = 0, head = static_cast<int>(blockIdx.x) / a.n_split, kv_head;
   if constexpr (INWG) {
-    locate_head(a, static_cast<int>(blockIdx.x), n_rep, head, part);
+    locate_head(a, static_cast<int>(blockIdx.x), head, part, kv_head);
+  } else {
+    kv_head = head / n_rep;
   }
   const int split = INWG ? part * wg_waves + wave : static_cast<int>(blockIdx.x) % a.n_split;
   const int lane = threadIdx.x & (kWave - 1);
@@ -202,7 +294,6 @@ __global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flas
   const int grp = lane / LPT; // which time step of the iteration
   const int hd = a.hd;
   const int d0 = li * 8;
-  const int kv_head = head / n_rep;
   const int tok = INWG ? static_cast<int>(blockIdx.y) : 0;
   const int vl = min(*a.valid_len + tok, a.max_seq);
 
@@ -216,17 +307,20 @@ __global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flas
   const size_t row_stride = static_cast<size_t>(a.n_kv) * hd;
   // plain dwords: arrays of vector structs would not stay in registers
   uint32_t kraw[UNR][4], vraw[UNR][4];
-  auto load_block = [&](int t0, int limit) {
+  // AHEAD: a second register set, so that the next block is in flight while one is computed
+  uint32_t knext[AHEAD ? UNR : 1][4], vnext[AHEAD ? UNR : 1][4];
+  // Every request is unconditional (a row index past `limit` reads row limit - 1 again, and the
+  // values are dropped below, live[]): under a branch the number of requests in flight would
+  // be unknown and every wait for an older block a wait for all of them.
+  auto load_block = [&](auto &kraw, auto &vraw, int t0, int limit) {
 #pragma unroll
     for (int u = 0; u < UNR; ++u) {
-      const int t = t0 + grp * a.n_split + u * stride;
-      uint4 kv = make_uint4(0, 0, 0, 0), vv = make_uint4(0, 0, 0, 0);
-      if (t < limit) {  // the row at *position may be mid-write: it is replaced below
-        const size_t off =
-            static_cast<size_t>(t) * row_stride + static_cast<size_t>(kv_head) * hd + d0;
-        kv = *reinterpret_cast<const uint4 *>(a.k_cache + off);
-        vv = *reinterpret_cast<const uint4 *>(a.v_cache + off);
-      }
+      // (the row at *position may be mid-write: it is replaced below)
+      const int t = max(min(t0 + grp * a.n_split + u * stride, limit - 1), 0);
+      const size_t off =
+          static_cast<size_t>(t) * row_stride + static_cast<size_t>(kv_head) * hd + d0;
+      const uint4 kv = *reinterpret_cast<const uint4 *>(a.k_cache + off);
+      const uint4 vv = *reinterpret_cast<const uint4 *>(a.v_cache + off);
       kraw[u][0] = kv.x;
       kraw[u][1] = kv.y;
       kraw[u][2] = kv.z;
@@ -241,7 +335,7 @@ __global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flas
   // length, a device scalar: its requests leave with the first instructions of the kernel
   // instead of after a round trip for that scalar.  Rows past the valid length are
   // allocated memory with arbitrary contents; they are dropped below (live[]) unused.
-  load_block(split, a.max_seq);
+  load_block(kraw, vraw, split, a.max_seq);
 
   float qf[8];
   float kcur[8];
@@ -281,10 +375,8 @@ __global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flas
   float m = kNegBig;
   float l = 0.f;
   float acc[8] = {};
-  for (int t0 = split; t0 < vl; t0 += UNR * stride) {
-    if (t0 != split) {
-      load_block(t0, vl);
-    }
+  // one block of rows (UNR slots of TPW time steps) into the running state
+  auto take_block = [&](auto &kraw, auto &vraw, int t0) {
     bool live[UNR], cur[UNR];
 #pragma unroll
     for (int u = 0; u < UNR; ++u) {
@@ -294,6 +386,12 @@ __global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flas
     }
 #pragma unroll
     for (int u = 0; u < UNR; ++u) {
+      // the rows of slot u start at t0 + u * stride for the wavefront's first lane group: past
+      // the valid length no lane has a live row in this slot or a later one (a scalar branch;
+      // at 640 rows the second round of 512 keeps one slot of four)
+      if (t0 + u * stride >= vl) {
+        break;
+      }
       float kf[8], vf[8];
       widen8(make_uint4(kraw[u][0], kraw[u][1], kraw[u][2], kraw[u][3]), kf);
       widen8(make_uint4(vraw[u][0], vraw[u][1], vraw[u][2], vraw[u][3]), vf);
@@ -314,40 +412,43 @@ __global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flas
         const float m2 = fmaxf(m, dot);
         const float alpha = __expf(m - m2);
         const float e = __expf(dot - m2);
-        l = l * alpha + e;
+        // (explicit fused multiply-adds: written a * b + c * d the compiler chooses per kernel
+        // which product to fuse, and the chunk kernel must round exactly like this one)
+        l = fmaf(l, alpha, e);
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-          acc[i] = acc[i] * alpha + e * vf[i];
+          acc[i] = fmaf(e, vf[i], acc[i] * alpha);
         }
         m = m2;
       }
     }
-  }
-
-  // Fold the TPW lane groups: lanes with equal li hold states of different
-  // time-step subsets.
-  if constexpr (TPW > 1) {
-    float mg = m;
+  };
+  const int step = UNR * stride;
+  if constexpr (AHEAD) {
+    // (two blocks ahead, the loop written out over three named buffers, was slower: 6.8 / 11.0 us
+    // at 640 / 2047 rows against 6.4 / 10.2 on the same box)
+    for (int t0 = split; t0 < vl; t0 += step) {
+      load_block(knext, vnext, t0 + step, vl);
+      take_block(kraw, vraw, t0);
 #pragma unroll
-    for (int off = LPT; off < kWave; off <<= 1) {
-      mg = fmaxf(mg, __shfl_xor(mg, off, kWave));
-    }
-    const float w = __expf(m - mg);
-    l *= w;
+      for (int u = 0; u < UNR; ++u) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      acc[i] *= w;
-    }
-#pragma unroll
-    for (int off = LPT; off < kWave; off <<= 1) {
-      l += __shfl_xor(l, off, kWave);
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        acc[i] += __shfl_xor(acc[i], off, kWave);
+        for (int i = 0; i < 4; ++i) {
+          kraw[u][i] = knext[u][i];
+          vraw[u][i] = vnext[u][i];
+        }
       }
     }
-    m = mg;
+  } else {
+    for (int t0 = split; t0 < vl; t0 += step) {
+      if (t0 != split) {
+        load_block(kraw, vraw, t0, vl);
+      }
+      take_block(kraw, vraw, t0);
+    }
   }
+
+  fold_lane_groups<LPT>(m, l, acc);
 
   if constexpr (INWG) {
     __shared__ float sm[kMaxWgSplits], sl[kMaxWgSplits];
@@ -362,13 +463,13 @@ __global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flas
       *reinterpret_cast<float4 *>(oh + 4) = make_float4(acc[4], acc[5], acc[6], acc[7]);
     }
     __syncthreads();
-    if (wave == 0) {
-      float *st = a.state == nullptr
-                      ? nullptr
-                      : a.state + (static_cast<size_t>(head) * a.n_parts + part) * (hd + 4);
-      uint16_t *dst = a.out + static_cast<size_t>(tok) * a.out_tok_stride +
-                      static_cast<size_t>(head) * hd * a.out_dim_stride;
-      merge_head(sm, sl, so, dst, 0, hd, wg_waves, lane, st, a.out_dim_stride);
+    float *st = a.state == nullptr
+                    ? nullptr
+                    : a.state + (static_cast<size_t>(head) * a.n_parts + part) * (hd + 4);
+    uint16_t *dst = a.out + static_cast<size_t>(tok) * a.out_tok_stride +
+                    static_cast<size_t>(head) * hd * a.out_dim_stride;
+    for (int d = threadIdx.x; d < hd; d += blockDim.x) {
+      merge_wg(sm, sl, so, dst, hd, wg_waves, d, st, a.out_dim_stride);
     }
   } else {
     const size_t slot = static_cast<size_t>(head) * a.n_split + split;
@@ -456,6 +557,9 @@ __global__ __launch_bounds__(kWave * kMaxGqaWaves) void attn_chunk_gqa(const Att
     load_block(nxt, t0 + UNR * stride);
 #pragma unroll
     for (int u = 0; u < UNR; ++u) {
+      if (t0 + u * stride >= vl) {  // no live row in this slot or a later one, for any lane
+        break;
+      }
       const bool live = t0 + grp * wg_waves + u * stride < vl;
       float kf[8], vf[8];
       widen8(make_uint4(cur.k[u][0], cur.k[u][1], cur.k[u][2], cur.k[u][3]), kf);
@@ -472,10 +576,10 @@ __global__ __launch_bounds__(kWave * kMaxGqaWaves) void attn_chunk_gqa(const Att
           const float m2 = fmaxf(m[r], dot);
           const float alpha = __expf(m[r] - m2);
           const float e = __expf(dot - m2);
-          l[r] = l[r] * alpha + e;
+          l[r] = fmaf(l[r], alpha, e);
 #pragma unroll
           for (int i = 0; i < 8; ++i) {
-            acc[r][i] = acc[r][i] * alpha + e * vf[i];
+            acc[r][i] = fmaf(e, vf[i], acc[r][i] * alpha);
           }
           m[r] = m2;
         }
@@ -488,28 +592,7 @@ __global__ __launch_bounds__(kWave * kMaxGqaWaves) void attn_chunk_gqa(const Att
   __shared__ __align__(16) float so[REP][kMaxGqaWaves * HD];
 #pragma unroll
   for (int r = 0; r < REP; ++r) {
-    if constexpr (TPW > 1) {  // fold the lane groups (different time steps, same dims)
-      float mg = m[r];
-#pragma unroll
-      for (int off = LPT; off < kWave; off <<= 1) {
-        mg = fmaxf(mg, __shfl_xor(mg, off, kWave));
-      }
-      const float w = __expf(m[r] - mg);
-      l[r] *= w;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        acc[r][i] *= w;
-      }
-#pragma unroll
-      for (int off = LPT; off < kWave; off <<= 1) {
-        l[r] += __shfl_xor(l[r], off, kWave);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          acc[r][i] += __shfl_xor(acc[r][i], off, kWave);
-        }
-      }
-      m[r] = mg;
-    }
+    fold_lane_groups<LPT>(m[r], l[r], acc[r]);  // (different time steps, same dims)
     if (lane == 0) {
       sm[r][wave] = m[r];
       sl[r][wave] = l[r];
@@ -521,10 +604,11 @@ __global__ __launch_bounds__(kWave * kMaxGqaWaves) void attn_chunk_gqa(const Att
     }
   }
   __syncthreads();
-  for (int r = wave; r < REP; r += wg_waves) {
+  for (int item = threadIdx.x; item < REP * HD; item += blockDim.x) {
+    const int r = item / HD, d = item - r * HD;
     uint16_t *dst = a.out + static_cast<size_t>(tok) * a.out_tok_stride +
                     static_cast<size_t>(kv_head * REP + r) * HD * a.out_dim_stride;
-    merge_head(sm[r], sl[r], so[r], dst, 0, HD, wg_waves, lane, nullptr, a.out_dim_stride);
+    merge_wg(sm[r], sl[r], so[r], dst, HD, wg_waves, d, nullptr, a.out_dim_stride);
   }
 }
 
@@ -549,16 +633,17 @@ __global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flas
     const AttnArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
   const int wg_waves = static_cast<int>(blockDim.x >> 6);
-  const int n_rep = a.n_q / a.n_kv;
-  int part = 0, head = static_cast<int>(blockIdx.x) / a.n_split;
+  const int n_rep = a.n_rep;
+  int part = 0, head = static_cast<int>(blockIdx.x) / a.n_split, kv_head;
   if constexpr (INWG) {
-    locate_head(a, static_cast<int>(blockIdx.x), n_rep, head, part);
+    locate_head(a, static_cast<int>(blockIdx.x), head, part, kv_head);
+  } else {
+    kv_head = head / n_rep;
   }
   const int split = INWG ? part * wg_waves + wave : static_cast<int>(blockIdx.x) % a.n_split;
   const int lane = threadIdx.x & (kWave - 1);
   const int hd = a.hd;
   const int half = hd / 2;
-  const int kv_head = head / n_rep;
   const int tok = INWG ? static_cast<int>(blockIdx.y) : 0;
   const int vl = min(*a.valid_len + tok, a.max_seq);
   const uint16_t *qh = a.q + static_cast<size_t>(tok) * a.q_tok_stride + static_cast<size_t>(head) * hd;
@@ -635,10 +720,10 @@ __global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flas
     const float m2 = fmaxf(m, dot);
     const float alpha = __expf(m - m2);
     const float e = __expf(dot - m2);
-    l = l * alpha + e;
+    l = fmaf(l, alpha, e);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      acc[i] = acc[i] * alpha + e * vf[i];
+      acc[i] = fmaf(e, vf[i], acc[i] * alpha);
     }
     m = m2;
   }
@@ -657,13 +742,13 @@ __global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flas
       }
     }
     __syncthreads();
-    if (wave == 0) {
-      float *st = a.state == nullptr
-                      ? nullptr
-                      : a.state + (static_cast<size_t>(head) * a.n_parts + part) * (hd + 4);
-      uint16_t *dst = a.out + static_cast<size_t>(tok) * a.out_tok_stride +
-                      static_cast<size_t>(head) * hd * a.out_dim_stride;
-      merge_head(sm, sl, so, dst, 0, hd, wg_waves, lane, st, a.out_dim_stride);
+    float *st = a.state == nullptr
+                    ? nullptr
+                    : a.state + (static_cast<size_t>(head) * a.n_parts + part) * (hd + 4);
+    uint16_t *dst = a.out + static_cast<size_t>(tok) * a.out_tok_stride +
+                    static_cast<size_t>(head) * hd * a.out_dim_stride;
+    for (int d = threadIdx.x; d < hd; d += blockDim.x) {
+      merge_wg(sm, sl, so, dst, hd, wg_waves, d, st, a.out_dim_stride);
     }
   } else {
     const size_t slot = static_cast<size_t>(head) * a.n_split + split;
@@ -774,10 +859,19 @@ void launch_flash(const AttnArgs &a, bool vec_ok, hipStream_t st, int n_tok = 1)
   const dim3 grid(static_cast<unsigned>(INWG ? a.n_q * a.n_parts : a.n_q * a.n_split),
                   static_cast<unsigned>(INWG ? n_tok : 1));
   const dim3 block(static_cast<unsigned>(INWG ? kWave * (a.n_split / a.n_parts) : kWave));
+  const bool few = INWG && block.x <= 8 * kWave;  // the form that reads a block ahead
   if (vec_ok && a.hd == 128) {
-    attn_flash<16, INWG><<<grid, block, 0, st>>>(a);
+    if (few) {
+      attn_flash<16, INWG, 8><<<grid, block, 0, st>>>(a);
+    } else {
+      attn_flash<16, INWG><<<grid, block, 0, st>>>(a);
+    }
   } else if (vec_ok && a.hd == 64) {
-    attn_flash<8, INWG><<<grid, block, 0, st>>>(a);
+    if (few) {
+      attn_flash<8, INWG, 8><<<grid, block, 0, st>>>(a);
+    } else {
+      attn_flash<8, INWG><<<grid, block, 0, st>>>(a);
+    }
   } else if (vec_ok && a.hd == 256) {
     attn_flash<32, INWG><<<grid, block, 0, st>>>(a);
   } else if (vec_ok && a.hd == 32) {
@@ -852,6 +946,10 @@ int attn_common(const void *q, const void *k, const void *v, void *out, const vo
     return e == nullptr || e[0] != '0';
   }();
   a.xcd_map = (xcd_map_on && mode != 0 && (n_kv * a.n_parts) % kDies == 0) ? 1 : 0;
+  a.n_rep = n_q / n_kv;
+  const bool small = static_cast<long long>(n_q) * a.n_parts < (1 << 22) && a.n_rep <= 256 && a.n_parts <= 256;
+  a.inv_rep = small ? 1.f / static_cast<float>(a.n_rep) : 0.f;
+  a.inv_parts = small ? 1.f / static_cast<float>(a.n_parts) : 0.f;
   hipStream_t st = static_cast<hipStream_t>(stream);
   // The vector path needs 16-byte aligned rows and 16-byte aligned fp32 partials.
   const bool vec_ok = aligned16(q) && aligned16(k) && aligned16(v) &&

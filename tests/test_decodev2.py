@@ -223,16 +223,14 @@ def near_tie(logits: np.ndarray) -> bool:
     return float(top[1] - top[0]) <= 4 * 2.0 ** (np.floor(np.log2(max(abs(top[1]), 1e-30))) - 7)
 
 
-#: streams of 64 tokens that must come out identical to the oracle's, per launch form, out
-#: of the 8 (4 seeds x dense / packed embedding table).  Random-init logits have a median
-#: top-1/top-2 gap of ~0.1 and a minimum over 64 picks that is usually below one bf16 step
-#: of the logit, so some streams meet a coin-toss pick; these are the counts measured with
-#: the levels kept as two bf16 terms (fp32-class weights), asserted as floors.
-#: One-term (bf16) levels carry 2^-9 of weight rounding into every logit: which side of a
-#: near-tie a stream lands on then changes with the summation order of the kernel that
-#: serves a row length, and no stream is promised to stay identical for 64 picks (every
-#: difference is still checked to sit at a near-tie of the oracle).
-IDENTICAL_FLOOR = {"plain": 1, "fold_rms": 1, "fp32_levels": 1, "two_term": 1, "one_term": 0}
+#: How many of the 8 streams below (4 seeds x dense / packed embedding table) stay identical to the
+#: oracle's for all 64 picks is printed, not asserted.  Random-init logits have a median top-1 /
+#: top-2 gap of ~0.1 and a minimum over 64 picks that is usually below one bf16 step of the logit,
+#: so most of these streams meet a coin-toss pick, and which side of it a stream lands on changes
+#: with any change of summation order in any kernel (the counts have been 0 .. 2 of 8 for every
+#: form, fp32 levels included).  What is asserted for them: a stream leaves the oracle's only at a
+#: pick that is a near-tie for the oracle itself.  The streams that must be identical, all 64
+#: picks, every form, are the wide-gap ones further down.
 
 
 def _streams_64(monkeypatch, form: str) -> tuple[int, list[str]]:
@@ -273,7 +271,7 @@ def _streams_64(monkeypatch, form: str) -> tuple[int, list[str]]:
 
 
 @pytest.mark.parametrize("form", ["plain", "fold_rms", "fp32_levels", "two_term", "one_term"])
-def test_greedy_64_tokens_identical_to_the_oracle(form, monkeypatch):
+def test_greedy_64_tokens_leave_the_oracle_only_at_near_ties(form, monkeypatch):
     """64 generated tokens on random-init weights, ignore-EOS, eager and graph, eight
     streams per launch form: the reference's call sequence (``plain``) and the folded one
     (``fold_rms``) with the default binary16 levels, the plain GEMV kernel with fp32 levels,
@@ -284,7 +282,6 @@ def test_greedy_64_tokens_identical_to_the_oracle(form, monkeypatch):
     identical, lines = _streams_64(monkeypatch, form)
     say("\n".join(lines))
     say(f"  {form}: {identical} of 8 streams identical over 64 tokens")
-    assert identical >= IDENTICAL_FLOOR[form], (form, identical)
 
 
 #: Streams picked on the CPU by the oracle alone (tests/golden/scan_greedy_margins.py): seeds of the
