@@ -1069,7 +1069,11 @@ def test_rope_kv(n_q, n_kv, hd, pos):
 
 @pytest.mark.parametrize("n_q,n_kv,hd,max_seq,pos", [(4, 2, 16, 16, 0), (16, 2, 128, 128, 100),
                                                      (40, 8, 128, 2048, 1500), (4, 2, 48, 32, 9),
-                                                     (40, 8, 128, 2048, 2047)])
+                                                     (40, 8, 128, 2048, 2047),
+                                                     # 264 query heads on one KV head: past the
+                                                     # range of the kernel's reciprocal index
+                                                     # arithmetic, the integer division runs
+                                                     (264, 1, 16, 64, 20)])
 def test_dv2_attn_equals_the_two_launch_form(n_q, n_kv, hd, max_seq, pos):
     """One workgroup per head against split kernel + merge: the same online softmax over
     another partition of the rows, so the outputs agree to bf16 rounding; the cache row
@@ -1147,7 +1151,10 @@ def test_begin_step(vocab, k):
 
 @pytest.mark.parametrize("n_q,n_kv,hd,max_seq,pos,parts,waves", [
     (4, 2, 16, 16, 0, 8, 4), (16, 2, 128, 128, 100, 8, 4), (40, 8, 128, 2048, 1500, 8, 4),
-    (4, 2, 48, 32, 9, 3, 2), (40, 8, 128, 2048, 2047, 5, 16), (8, 8, 64, 64, 33, 1, 1)])
+    (4, 2, 48, 32, 9, 3, 2), (40, 8, 128, 2048, 2047, 5, 16), (8, 8, 64, 64, 33, 1, 1),
+    # what the decode step launches (4 parts of 8 wavefronts: heads placed by die, a block of rows
+    # read ahead), at a context of one block, of two, and of the whole cache
+    (40, 8, 128, 2048, 300, 4, 8), (40, 8, 128, 2048, 700, 4, 8), (40, 8, 128, 2048, 2047, 4, 8)])
 def test_attention_merged_by_the_o_projection(n_q, n_kv, hd, max_seq, pos, parts, waves):
     """dv2_attn_parts + dv2_gemv_attn against nf4_attn + nf4_gemv(add) (each checked against
     float64 above): the same softmax over another partition of the rows, merged inside the
