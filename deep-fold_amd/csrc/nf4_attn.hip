@@ -97,6 +97,9 @@ struct AttnArgs {
   // n_q / n_kv, and reciprocals for the index arithmetic ahead of the first cache request
   int n_rep;
   float inv_rep, inv_parts;
+  // wavefronts of a workgroup (the block size is a hidden kernel argument: read from there it
+  // is a second trip to the scalar cache ahead of the first cache request)
+  int wg_waves;
 };
 
 constexpr int kDies = 8;
@@ -229,12 +232,13 @@ __device__ __forceinline__ void fold_lane_groups(float &m, float &l, float (&acc
 // with a shuffle per state and dim (1.3 us of a 5.3 us launch at 8 states of 128 dims; this
 // form 0.3).  m and l of the states are broadcast reads; every thread computes the same
 // weights.
+template <int NMAX = kMaxWgSplits>  // the most states there can be
 __device__ __forceinline__ void merge_wg(const float *sm, const float *sl, const float *so,
                                          uint16_t *dst, int hd, int n, int d, float *state,
                                          int dstride) {
   float m = kNegBig;
 #pragma unroll
-  for (int s = 0; s < kMaxWgSplits; ++s) {
+  for (int s = 0; s < NMAX; ++s) {
     m = fmaxf(m, sm[min(s, n - 1)]);
   }
   float l = 0.f, acc = 0.f;
@@ -280,7 +284,7 @@ __global__ __launch_bounds__(INWG ? kWave * WMAX : kWave) void attn_flash(const 
   constexpr int TPW = kWave / LPT;  // time steps per wavefront iteration
   constexpr bool AHEAD = INWG && WMAX <= 8;
   const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
-  const int wg_waves = static_cast<int>(blockDim.x >> 6);
+  const int wg_waves = a.wg_waves;
   const int n_rep = a.n_rep;
   int part = 0, head = static_cast<int>(blockIdx.x) / a.n_split, kv_head;
   if constexpr (INWG) {
@@ -468,8 +472,8 @@ __global__ __launch_bounds__(INWG ? kWave * WMAX : kWave) void attn_flash(const 
                     : a.state + (static_cast<size_t>(head) * a.n_parts + part) * (hd + 4);
     uint16_t *dst = a.out + static_cast<size_t>(tok) * a.out_tok_stride +
                     static_cast<size_t>(head) * hd * a.out_dim_stride;
-    for (int d = threadIdx.x; d < hd; d += blockDim.x) {
-      merge_wg(sm, sl, so, dst, hd, wg_waves, d, st, a.out_dim_stride);
+    for (int d = threadIdx.x; d < hd; d += wg_waves * kWave) {
+      merge_wg<WMAX>(sm, sl, so, dst, hd, wg_waves, d, st, a.out_dim_stride);
     }
   } else {
     const size_t slot = static_cast<size_t>(head) * a.n_split + split;
@@ -498,7 +502,7 @@ __global__ __launch_bounds__(kWave * kMaxGqaWaves) void attn_chunk_gqa(const Att
   constexpr int UNR = 4;
   constexpr int HD = 8 * LPT;
   const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
-  const int wg_waves = static_cast<int>(blockDim.x >> 6);
+  const int wg_waves = a.wg_waves;
   const int kv_head = static_cast<int>(blockIdx.x);
   const int tok = static_cast<int>(blockIdx.y);
   const int lane = threadIdx.x & (kWave - 1);
@@ -604,11 +608,11 @@ __global__ __launch_bounds__(kWave * kMaxGqaWaves) void attn_chunk_gqa(const Att
     }
   }
   __syncthreads();
-  for (int item = threadIdx.x; item < REP * HD; item += blockDim.x) {
+  for (int item = threadIdx.x; item < REP * HD; item += wg_waves * kWave) {
     const int r = item / HD, d = item - r * HD;
     uint16_t *dst = a.out + static_cast<size_t>(tok) * a.out_tok_stride +
                     static_cast<size_t>(kv_head * REP + r) * HD * a.out_dim_stride;
-    merge_wg(sm[r], sl[r], so[r], dst, HD, wg_waves, d, nullptr, a.out_dim_stride);
+    merge_wg<kMaxGqaWaves>(sm[r], sl[r], so[r], dst, HD, wg_waves, d, nullptr, a.out_dim_stride);
   }
 }
 
@@ -632,7 +636,7 @@ template <bool INWG>
 __global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flash_generic(
     const AttnArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
-  const int wg_waves = static_cast<int>(blockDim.x >> 6);
+  const int wg_waves = a.wg_waves;
   const int n_rep = a.n_rep;
   int part = 0, head = static_cast<int>(blockIdx.x) / a.n_split, kv_head;
   if constexpr (INWG) {
@@ -747,7 +751,7 @@ __global__ __launch_bounds__(INWG ? kWave * kMaxWgSplits : kWave) void attn_flas
                     : a.state + (static_cast<size_t>(head) * a.n_parts + part) * (hd + 4);
     uint16_t *dst = a.out + static_cast<size_t>(tok) * a.out_tok_stride +
                     static_cast<size_t>(head) * hd * a.out_dim_stride;
-    for (int d = threadIdx.x; d < hd; d += blockDim.x) {
+    for (int d = threadIdx.x; d < hd; d += wg_waves * kWave) {
       merge_wg(sm, sl, so, dst, hd, wg_waves, d, st, a.out_dim_stride);
     }
   } else {
@@ -916,6 +920,7 @@ int attn_common(const void *q, const void *k, const void *v, void *out, const vo
   a.v_cache = static_cast<const uint16_t *>(v);
   a.n_parts = mode == 2 ? n_parts : 1;
   a.n_split = mode == 2 ? n_split * n_parts : n_split;  // wavefronts that share a head
+  a.wg_waves = mode == 0 ? 1 : n_split;
   if (mode == 0) {
     const int nml = n_q * n_split;
     a.m_s = ws;
