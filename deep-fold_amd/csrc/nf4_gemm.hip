@@ -438,6 +438,10 @@ struct GemmSegs {
   int M[3];       // rows of each matrix
   int blocks[3];  // row blocks (of kBM rows) of each
   int row0[3];    // first output row of each
+  // the stream tiles: workgroups that share K (grid.y) and the chunks each of them takes, from
+  // the host (read from the grid size, a hidden kernel argument, and divided in the kernel they
+  // were a trip to the scalar cache and an integer division ahead of the first requests)
+  int splits, per_split;
 };
 
 template <int NB>
@@ -1184,7 +1188,8 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
   // grid.y splits K by whole chunks: this workgroup takes n_ch of them from chunk c0 on, and
   // from here on x, K, row_bytes and groups describe what is left of K from that chunk on
   const int n_ch_all = (K_pad + CK - 1) / CK;
-  const int per_split = (n_ch_all + static_cast<int>(gridDim.y) - 1) / static_cast<int>(gridDim.y);
+  const int per_split = segs.per_split;
+  const unsigned int n_splits = static_cast<unsigned int>(segs.splits);
   const int c0 = static_cast<int>(blockIdx.y) * per_split;
   const int n_ch = min(per_split, n_ch_all - c0);
   const int row_stride = K_pad >> 1;  // bytes of a packed row
@@ -1545,7 +1550,7 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
       unsigned int *count = &stream_arrivals[arrive_slot][blockIdx.x];
       const unsigned int before =
           __hip_atomic_fetch_add(count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      const bool all_in = before + 1 == gridDim.y;
+      const bool all_in = before + 1 == n_splits;
       if (all_in) {
         __hip_atomic_store(count, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
@@ -1559,16 +1564,16 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
     for (int rb = 0; rb < RB; ++rb) {
       // (four requests at a time: a loop of single ones waits a round trip for each)
       float sum = 0.f;
-      for (unsigned int j0 = 0; j0 < gridDim.y; j0 += 4) {
+      for (unsigned int j0 = 0; j0 < n_splits; j0 += 4) {
         float v[4];
 #pragma unroll
         for (unsigned int u = 0; u < 4; ++u) {
-          v[u] = __hip_atomic_load(partial + min(j0 + u, gridDim.y - 1) * slab + at[rb], __ATOMIC_RELAXED,
+          v[u] = __hip_atomic_load(partial + min(j0 + u, n_splits - 1) * slab + at[rb], __ATOMIC_RELAXED,
                                    __HIP_MEMORY_SCOPE_AGENT);
         }
 #pragma unroll
         for (unsigned int u = 0; u < 4; ++u) {
-          sum = j0 + u == 0 ? v[0] : (j0 + u < gridDim.y ? sum + v[u] : sum);
+          sum = j0 + u == 0 ? v[0] : (j0 + u < n_splits ? sum + v[u] : sum);
         }
       }
       o32[rb] = sum;
@@ -1683,7 +1688,8 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream64(GemmSegs segs,
   // grid.y splits K by whole chunks (see gemm_stream): from here on x, K, row_bytes and groups
   // describe what is left of K from this workgroup's first chunk on
   const int n_ch_all = (K_pad + CK - 1) / CK;
-  const int per_split = (n_ch_all + static_cast<int>(gridDim.y) - 1) / static_cast<int>(gridDim.y);
+  const int per_split = segs.per_split;
+  const unsigned int n_splits = static_cast<unsigned int>(segs.splits);
   const int c0 = static_cast<int>(blockIdx.y) * per_split;
   const int n_ch = min(per_split, n_ch_all - c0);
   const int row_stride = K_pad >> 1;
@@ -1943,7 +1949,7 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream64(GemmSegs segs,
       unsigned int *count = &stream_arrivals[arrive_slot][blockIdx.x];
       const unsigned int before =
           __hip_atomic_fetch_add(count, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      const bool all_in = before + 1 == gridDim.y;
+      const bool all_in = before + 1 == n_splits;
       if (all_in) {
         __hip_atomic_store(count, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
@@ -1956,16 +1962,16 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream64(GemmSegs segs,
 #pragma unroll
     for (int o = 0; o < 4; ++o) {
       float sum = 0.f;
-      for (unsigned int j0 = 0; j0 < gridDim.y; j0 += 4) {
+      for (unsigned int j0 = 0; j0 < n_splits; j0 += 4) {
         float v[4];
 #pragma unroll
         for (unsigned int u = 0; u < 4; ++u) {
-          v[u] = __hip_atomic_load(partial + min(j0 + u, gridDim.y - 1) * slab + at[o], __ATOMIC_RELAXED,
+          v[u] = __hip_atomic_load(partial + min(j0 + u, n_splits - 1) * slab + at[o], __ATOMIC_RELAXED,
                                    __HIP_MEMORY_SCOPE_AGENT);
         }
 #pragma unroll
         for (unsigned int u = 0; u < 4; ++u) {
-          sum = j0 + u == 0 ? v[0] : (j0 + u < gridDim.y ? sum + v[u] : sum);
+          sum = j0 + u == 0 ? v[0] : (j0 + u < n_splits ? sum + v[u] : sum);
         }
       }
       o32[o] = sum;
@@ -2487,6 +2493,12 @@ int gemm_launch(const chr_nf4_dev_t *const *w, int nseg, const void *x, void *y,
   float *partial = (sp.grid_y > 1 || (swiglu && !pair)) ? ws : nullptr;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const dim3 grid(static_cast<unsigned>(sp.grid_x), static_cast<unsigned>(sp.grid_y));
+  if (sp.stream != 0) {
+    // whole chunks of K per workgroup of a row block: chunks of 256 at 64 columns, of 512 below
+    const int chunk_k = (sp.stream == 2 && N == 64) ? kWideChunkK : kStreamChunkK;
+    sp.segs.splits = sp.grid_y;
+    sp.segs.per_split = ceil_div(ceil_div(h[0].K_pad, chunk_k), sp.grid_y);
+  }
   // 16-byte activation vectors need N in {8, 16, 32, 64}; x is 16-byte aligned (checked above)
   const bool vec = N == 8 || N == 16 || N == 32 || N == 64;
   if (gemm_lds_ready() != 0) {
