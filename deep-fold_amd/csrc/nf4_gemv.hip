@@ -41,6 +41,7 @@ namespace chr {
 namespace {
 
 constexpr int kMaxWaves = 16;  // wavefronts per workgroup, upper bound
+constexpr int kThreads = 256;          // workgroup of the plain kernel, fixed
 constexpr int kStagedThreads = 1024;  // workgroup of the kernel that stages x in LDS, fixed
 
 // Static LDS of the GEMV kernels.  The codebook comes first so that its LDS
@@ -709,7 +710,7 @@ __global__ __launch_bounds__(256) void gemv_stream(const StreamArgs a) {
   // The wavefront index is the same in every lane: saying so keeps the row-group and
   // segment arithmetic, and the kernel-argument reads indexed by it, on the scalar unit.
   const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
-  const int waves = blockDim.x >> 6;
+  constexpr int waves = kThreads >> 6;  // (every launch of this kernel has kThreads threads)
 
   if (threadIdx.x < 16) {
     lds.lut[threadIdx.x] = bits_to_f32(kLutBits[threadIdx.x]);
@@ -905,11 +906,14 @@ __global__ __launch_bounds__(1024) void gemv_staged(const StreamArgs a) {
   const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
   constexpr int waves = kStagedThreads >> 6;
   const int total = a.groups[0] + a.groups[1] + a.groups[2];
-  const int first = wave * static_cast<int>(gridDim.x) + static_cast<int>(blockIdx.x);
-  const int stride = static_cast<int>(gridDim.x) * waves;
+  // (the grid size and how the groups split into passes come from the host: read from the
+  // hidden kernel arguments and divided here they were a trip to the scalar cache and an integer
+  // division ahead of the first requests)
+  const int first = wave * a.ring_grid + static_cast<int>(blockIdx.x);
+  const int stride = a.ring_grid * waves;
   const int n_half = a.K_pad >> 4;
   const int nsteps = x_half_steps(a.K_pad);
-  const int my_groups = first < total ? (total - first + stride - 1) / stride : 0;
+  const int my_groups = a.ring_passes + (first < a.ring_left ? 1 : 0);
   const int n_steps_all = my_groups * nsteps;      // half steps of this wavefront, in order
   const int n_items = (n_steps_all + S - 1) / S;   // S of them per item, across group borders
 
@@ -1703,7 +1707,6 @@ int level_terms() {
   return CHR_NF4_DEFAULT_TERMS;
 }
 
-constexpr int kThreads = 256;
 constexpr size_t kMaxDynLds = 150 * 1024;
 
 template <typename Kern>
@@ -1795,11 +1798,13 @@ int launch_stream(StreamArgs &a, int n_seg, bool staged, hipStream_t st) {
     const RingPiece ring = kRingShape && ring_wanted()
                                ? ring_piece_steps(x_half_steps(a.K_pad)) : RingPiece{0, 0};
     const int ring_ns = ring.steps;
+    // wavefront w of workgroup b walks groups w * grid + b, + 16 * grid, ..: full passes, and one
+    // more for the first ring_left wavefronts
+    const int per_pass = grid * waves;
+    a.ring_grid = grid;
+    a.ring_passes = total / per_pass;
+    a.ring_left = total % per_pass;
     if (ring_ns > 0) {
-      const int per_pass = grid * waves;
-      a.ring_grid = grid;
-      a.ring_passes = total / per_pass;
-      a.ring_left = total % per_pass;
       if constexpr (kRingShape) {
         auto go = [&](auto kern) {
           if (prep_lds(kern, dyn) != 0) {
