@@ -1572,25 +1572,26 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_num_vgpr(52))) void gem
   gemv_ring_body<NS, TERMS, XREG, PAD, SEQ>(a);
 }
 
-// Half steps of a piece (= slots of the ring, 512 bytes per row each) for a row of nsteps
-// half steps: the largest divisor the registers hold, at least 4 so that 1.5 KB per row stay
-// in flight (a pure streaming read of a 35 MB matrix by this grid is fastest with 2 KB per
-// wavefront on the way and loses 15% at 4 KB).  A row kernel also takes a length one half
-// step short of a multiple of 5..8 (11 = 2 * 6 - 1, 27 = 4 * 7 - 1), its last piece ending in
-// one empty slot.  steps == 0: the ring kernel does not take this row length (the
-// compiler-pipelined kernel does).
+// Half steps of a piece (= slots of the ring, 544 bytes per row each) for a row of nsteps
+// half steps: the largest divisor in 7..4, so that 2 to 4 KB per wavefront are in flight (a
+// pure streaming read of a 35 MB matrix by this grid is fastest with 2 KB per wavefront on the
+// way and loses 15% at 4 KB; eight slots, 4.3 KB, measured 9.36 against 8.92 us with four at
+// 8192x8192 and 11.73 against 11.56 at 6144x16384, while six beat four at 5120x12288, 8.5
+// against 8.7).  A row kernel also takes a length one half step short of a multiple of 5..8
+// (11 = 2 * 6 - 1, 27 = 4 * 7 - 1), its last piece ending in one empty slot.  steps == 0: the
+// ring kernel does not take this row length (the compiler-pipelined kernel does).
 struct RingPiece {
   int steps;
   int pad;
 };
 RingPiece ring_piece_steps(int nsteps) {
-  for (int ns = 8; ns >= 4; --ns) {
+  for (int ns = 7; ns >= 4; --ns) {
     if (nsteps % ns == 0) {
       return {ns, 0};
     }
   }
   if (nsteps > 8) {
-    for (int ns = 8; ns >= 5; --ns) {
+    for (const int ns : {7, 6, 5, 8}) {
       if ((nsteps + 1) % ns == 0) {
         return {ns, 1};
       }
@@ -1835,7 +1836,6 @@ int launch_stream(StreamArgs &a, int n_seg, bool staged, hipStream_t st) {
             case 5: rc = one_piece ? CHR_GO_SEQ(5, true, 0) : CHR_GO_SEQ(5, false, 0); break;
             case 6: rc = CHR_GO_SEQ(6, false, 0); break;
             case 7: rc = CHR_GO_SEQ(7, false, 0); break;
-            case 8: rc = CHR_GO_SEQ(8, false, 0); break;
           }
         } else {
           switch (ring.pad > 0 ? -ring_ns : ring_ns) {
@@ -1847,7 +1847,6 @@ int launch_stream(StreamArgs &a, int n_seg, bool staged, hipStream_t st) {
             case 5: rc = one_piece ? CHR_GO_ROWS(5, true, 0) : CHR_GO_ROWS(5, false, 0); break;
             case 6: rc = CHR_GO_ROWS(6, false, 0); break;
             case 7: rc = CHR_GO_ROWS(7, false, 0); break;
-            case 8: rc = CHR_GO_ROWS(8, false, 0); break;
           }
         }
 #undef CHR_GO_SEQ

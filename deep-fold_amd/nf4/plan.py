@@ -110,14 +110,15 @@ def staged_lds_bytes(k_pad_: int) -> int:
 
 def ring_piece_steps(half_steps: int) -> int:
     """Half steps per piece of the ring GEMV kernel for a row of ``half_steps``: the largest
-    divisor in 4..8; for rows longer than a piece also the largest of 8..5 that divides
-    ``half_steps + 1`` (the last piece then ends in one empty slot); 0 when that kernel does
-    not take the row.  Gate/up pairs go through the same ring, one row after the other."""
-    for ns in range(8, 3, -1):
+    divisor in 4..7 (eight slots keep more bytes in flight than pays); for rows longer than a
+    piece also the first of 7, 6, 5, 8 that divides ``half_steps + 1`` (the last piece then ends
+    in one empty slot); 0 when that kernel does not take the row.  Gate/up pairs go through the
+    same ring, one row after the other."""
+    for ns in range(7, 3, -1):
         if half_steps % ns == 0:
             return ns
     if half_steps > 8:
-        for ns in range(8, 4, -1):
+        for ns in (7, 6, 5, 8):
             if (half_steps + 1) % ns == 0:
                 return ns
     return 0

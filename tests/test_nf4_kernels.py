@@ -385,8 +385,8 @@ def test_swiglu_equals_pair(m, k):
 
 
 # ----------------------------------------------------------------- ring GEMV kernels
-# The ring kernels take every staged launch whose row length is a multiple of 4..8 half steps
-# of 1024 weights (4..6 for gate/up pairs) or, for single rows, one half step short of a
+# The ring kernels take every staged launch whose row length is a multiple of 4..7 half steps
+# of 1024 weights or one half step short of a
 # multiple of 5..8; CHR_NF4_GEMV_RING=0 keeps such launches on the compiler-pipelined kernel.
 RING_ROWS = [
     (4100, 4096),   # 4 half steps, x of the row in registers; a pass and four rows more
@@ -551,7 +551,7 @@ def test_ring_gemv_fused_rms(m, k, terms, monkeypatch):
 @pytest.mark.parametrize("terms", [1, 2, 3])
 @pytest.mark.parametrize("m,k", [
     (4100, 4096), (4400, 5120), (20, 5120), (2300, 6144), (1100, 12288), (2100, 5056),
-    (2200, 7168), (2100, 8192),    # rows of 7 and of 8 half steps
+    (2200, 7168), (2100, 8192),    # rows of 7 half steps, and of 8 (two pieces of 4)
     (700, 13824),                  # two pieces of 7
     (2200, 11008),                 # 11 half steps: two pieces of 6, the last with an empty slot
     (2100, 4000),                  # K below K_pad
