@@ -1056,9 +1056,10 @@ __global__ __launch_bounds__(1024) void gemv_staged(const StreamArgs a) {
 // operations complete in order, so "at most N outstanding" means everything but the N
 // youngest has arrived: every wait below is exact by construction.
 //
-// NS slots of one half step each form a ring: while the oldest is computed, NS-1 younger
-// ones are in flight, and its slot is requested again as soon as its bytes have been turned
-// into lookup addresses.  Work is dealt as in the staged kernel's comment.
+// NS slots of one half step each form a ring: while the oldest is computed, NS-1-LAG younger
+// ones are in flight; a slot is free once its bytes have been turned into lookup addresses
+// and is requested again LAG steps later (LAG is chosen per ring length in the body).  Work is
+// dealt as in the staged kernel's comment.
 struct XRegs {
   U32x4 v[kXKeep];  // x, 16-byte vectors i = thread + j * x_deal()
   U32x4 g[kXKeep];  // the RMSNorm weights at the same places (fused norm only)
@@ -1186,6 +1187,17 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
   constexpr int R = 1;                 // rows in the ring at a time
   constexpr int D = NS;                // slots of the ring
   constexpr int kStepLoads = 2 * R;    // vector memory operations of one half step
+  // A slot is requested again LAG steps after the step that consumed it, so NS - LAG half steps
+  // of a wavefront are in flight or being computed, not NS: this memory system serves a launch
+  // fastest with about 2 KB per wavefront on the way (ring_piece_steps), a half step is 544
+  // bytes.  Measured, us per launch at lag 0 / 1 / 2 / 3 (a dash: not measured): five slots
+  // 13824x5120 9.11 / 8.76 / 9.05 / -, 152064x5120 69.3 / 68.4 / 67.0 / -; six slots 8192x6144
+  // - / 7.98 / 7.21 / 7.28, 16384x6144 - / 12.8 / 11.6 .. 12.3 / 11.7, 20B decode 324 / - / 333 /
+  // 336 tok/s; seven slots 5120x13824 - / 10.06 / 9.52 / 9.59, 8192x7168 - / 9.65 / 8.63 / 8.01,
+  // 5120x27648 - / 16.1 / 16.2 / 16.9; four slots 8192x4096 6.00 / 5.90, 6144x16384 11.9 / 12.3.
+  // 14B decode 392 -> 399 tok/s, 20B 324 -> 336.
+  constexpr int LAG = NS == 4 ? 0 : NS == 5 ? 1 : NS == 6 ? 3 : NS == 7 ? 2 : 3;
+  static_assert(LAG >= 0 && LAG < NS - 2, "at least two half steps in flight");
   // LDS byte address of the x pieces (the pair table starts at LDS address 0)
   constexpr uint32_t kXsAddr = kPairTableBytes + kStagedSmallBytes;
   extern __shared__ uint4 dyn_lds[];  // [pair table][GemvLds][x pieces]
@@ -1319,7 +1331,7 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
   // nothing.
   const bool any_work = q_left > 0;
 #define CHR_RING_FILL_STEP(I) \
-  if constexpr (NS > (I)) { CHR_RING_REQUEST(I, pieces == 1) }
+  if constexpr (NS - LAG > (I)) { CHR_RING_REQUEST(I, pieces == 1) }
   // The first kRingEarlySlots slots are requested right after x, the others after the level
   // table has been written: x then queues behind two half steps per wavefront instead of the
   // whole ring (all slots at once: 7168x5120 7.2-7.4 us and 5120x5120 6.1 us against 7.0 and
@@ -1350,7 +1362,9 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
     CHR_RING_FILL_B_STEP(5)                                                               \
     CHR_RING_FILL_B_STEP(6)                                                               \
     CHR_RING_FILL_B_STEP(7)                                                               \
-    q_advance();                                                                          \
+    if constexpr (LAG == 0) {                                                             \
+      q_advance();                                                                        \
+    }                                                                                     \
   }
 #define CHR_RING_FILL CHR_RING_FILL_A CHR_RING_FILL_B
   // nothing of the compiler's own memory traffic crosses this, nor any statement of the chain
@@ -1373,7 +1387,7 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
     if (!any_work) {
       asm("s_waitcnt vmcnt(0)" : "+s"(tok));
     }
-    ring_x_wait<NS * kStepLoads>(xr, tok);
+    ring_x_wait<(NS - LAG) * kStepLoads>(xr, tok);
     uint4 xv[kXKeep], xg[kXKeep];
 #pragma unroll
     for (int j = 0; j < kXKeep; ++j) {
@@ -1440,9 +1454,9 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
   // all products of a piece to its end and holds every level it has looked up until then.
 #define CHR_RING_PIN asm("" : "+v"(acc[0]), "+s"(tok));
   // The half step in slot I, its x pieces X0 / X1: wait for it (WAIT), turn its packed bytes
-  // into lookup addresses, which frees the slot's registers, request the slot again at once
-  // (REQUEST), and only then look the levels up and multiply: the new request travels while
-  // this half step is computed.  MASK_IF says whether the lanes past the row's end are to be
+  // into lookup addresses, which frees the slot's registers, issue this step's request
+  // (REQUEST: the slot freed LAG steps ago), and only then look the levels up and multiply: the
+  // new request travels while this half step is computed.  MASK_IF says whether the lanes past the row's end are to be
   // switched off.
 #define CHR_RING_STEP(I, X0, X1, F, WAIT, REQUEST, MASK_IF, EMPTY_IF)                     \
   if (EMPTY_IF) {                                                                         \
@@ -1468,11 +1482,14 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
     CHR_RING_PIN                                                                          \
   }
 
-  // every step so far has requested its slot again: D-1 younger half steps are in flight
-#define CHR_RING_WAIT_FULL \
-  asm("s_waitcnt vmcnt(%1)" : "+s"(tok) : "n"((D - 1) * kStepLoads));
-  // the last piece requests nothing: its steps wait for whatever is still on its way
-#define CHR_RING_WAIT_ALL asm("s_waitcnt vmcnt(0)" : "+s"(tok));
+  // steady state: D-1-LAG younger half steps are in flight when a step waits for its own
+#define CHR_RING_WAIT_FULL(I) \
+  asm("s_waitcnt vmcnt(%1)" : "+s"(tok) : "n"((D - 1 - LAG) * kStepLoads));
+  // the last piece requests only its own last LAG slots (in its first LAG steps): step I has
+  // D-1-I younger half steps behind it at most
+#define CHR_RING_WAIT_LAST(I)              \
+  asm("s_waitcnt vmcnt(%1)" : "+s"(tok) \
+      : "n"(((D - 1 - (I)) < (D - 1 - LAG) ? (D - 1 - (I)) : (D - 1 - LAG)) * kStepLoads));
 
   // ---- the groups, a piece per turn --------------------------------------------------------
   int c_left = my_groups * pieces * kRowsPerGroup, c_part = 0, c_group = first;
@@ -1504,20 +1521,19 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
                     REQUEST, (I) == kLastReal && ragged && c_last, (I) > kLastReal && c_last) \
     }                                                                                     \
   }
-#define CHR_RING_PIECE(WAIT, REQUEST_OF, AFTER_REQUESTS)                                  \
+#define CHR_RING_PIECE(WAIT_OF, REQUEST_OF)                                               \
   {                                                                                       \
     const uint32_t xa = x_lane + static_cast<uint32_t>(c_part) * (NS * 2048);             \
     const uint32_t fa = f_lane + static_cast<uint32_t>(c_part) * (NS * 256);              \
     const bool c_last = c_part == pieces - 1;                                             \
-    CHR_RING_OWN_STEP(0, WAIT, REQUEST_OF(0))                                             \
-    CHR_RING_OWN_STEP(1, WAIT, REQUEST_OF(1))                                             \
-    CHR_RING_OWN_STEP(2, WAIT, REQUEST_OF(2))                                             \
-    CHR_RING_OWN_STEP(3, WAIT, REQUEST_OF(3))                                             \
-    CHR_RING_OWN_STEP(4, WAIT, REQUEST_OF(4))                                             \
-    CHR_RING_OWN_STEP(5, WAIT, REQUEST_OF(5))                                             \
-    CHR_RING_OWN_STEP(6, WAIT, REQUEST_OF(6))                                             \
-    CHR_RING_OWN_STEP(7, WAIT, REQUEST_OF(7))                                             \
-    AFTER_REQUESTS                                                                        \
+    CHR_RING_OWN_STEP(0, WAIT_OF(0), REQUEST_OF(0))                                       \
+    CHR_RING_OWN_STEP(1, WAIT_OF(1), REQUEST_OF(1))                                       \
+    CHR_RING_OWN_STEP(2, WAIT_OF(2), REQUEST_OF(2))                                       \
+    CHR_RING_OWN_STEP(3, WAIT_OF(3), REQUEST_OF(3))                                       \
+    CHR_RING_OWN_STEP(4, WAIT_OF(4), REQUEST_OF(4))                                       \
+    CHR_RING_OWN_STEP(5, WAIT_OF(5), REQUEST_OF(5))                                       \
+    CHR_RING_OWN_STEP(6, WAIT_OF(6), REQUEST_OF(6))                                       \
+    CHR_RING_OWN_STEP(7, WAIT_OF(7), REQUEST_OF(7))                                       \
     --c_left;                                                                             \
     if (c_last) {                                                                         \
       finish_group(c_group);                                                              \
@@ -1536,24 +1552,43 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
     (void)xa;                                                                             \
     (void)fa;                                                                             \
   }
-#define CHR_RING_REQUEST_NEXT(I) CHR_RING_REQUEST(I, q_part == pieces - 1)
-#define CHR_RING_REQUEST_NONE(I)
-  // while a piece is left to request, every step requests its slot again
-  while (q_left > 0) {
-    CHR_RING_PIECE(CHR_RING_WAIT_FULL, CHR_RING_REQUEST_NEXT, q_advance();)
+  // slot S (a constant expression) of the piece at the request cursor; the cursor moves on
+  // with the piece's last slot
+#define CHR_RING_REQUEST_SLOT(S)                                                          \
+  {                                                                                       \
+    const bool lastp = q_part == pieces - 1;                                              \
+    if constexpr ((S) == 0) { CHR_RING_REQUEST(0, lastp) }                                \
+    if constexpr ((S) == 1) { CHR_RING_REQUEST(1, lastp) }                                \
+    if constexpr ((S) == 2) { CHR_RING_REQUEST(2, lastp) }                                \
+    if constexpr ((S) == 3) { CHR_RING_REQUEST(3, lastp) }                                \
+    if constexpr ((S) == 4) { CHR_RING_REQUEST(4, lastp) }                                \
+    if constexpr ((S) == 5) { CHR_RING_REQUEST(5, lastp) }                                \
+    if constexpr ((S) == 6) { CHR_RING_REQUEST(6, lastp) }                                \
+    if constexpr ((S) == 7) { CHR_RING_REQUEST(7, lastp) }                                \
+    if constexpr ((S) == NS - 1) { q_advance(); }                                         \
+  }
+  // step I asks again for the slot that step I - LAG consumed
+#define CHR_RING_REQUEST_NEXT(I) CHR_RING_REQUEST_SLOT(((I) + NS - LAG) % NS)
+  // the last piece: its own last LAG slots, then nothing
+#define CHR_RING_REQUEST_LAST(I) \
+  if constexpr ((I) < LAG) { CHR_RING_REQUEST_SLOT(NS - LAG + (I)) }
+  // while a piece after the one being computed is left to request
+  while (q_left > (LAG > 0 ? 1 : 0)) {
+    CHR_RING_PIECE(CHR_RING_WAIT_FULL, CHR_RING_REQUEST_NEXT)
   }
   // the last piece
   if (c_left > 0) {
-    CHR_RING_PIECE(CHR_RING_WAIT_ALL, CHR_RING_REQUEST_NONE, )
+    CHR_RING_PIECE(CHR_RING_WAIT_LAST, CHR_RING_REQUEST_LAST)
   }
   // nothing may still be on its way into the fixed registers when the wavefront ends (this
   // statement is volatile: it is what keeps the token chain, and with it every request, alive)
   asm volatile("s_waitcnt vmcnt(0)" : "+s"(tok));
-#undef CHR_RING_REQUEST_NONE
+#undef CHR_RING_REQUEST_LAST
 #undef CHR_RING_REQUEST_NEXT
+#undef CHR_RING_REQUEST_SLOT
 #undef CHR_RING_PIECE
 #undef CHR_RING_OWN_STEP
-#undef CHR_RING_WAIT_ALL
+#undef CHR_RING_WAIT_LAST
 #undef CHR_RING_WAIT_FULL
 #undef CHR_RING_STEP
 #undef CHR_RING_PIN
@@ -1815,8 +1850,7 @@ int launch_stream(StreamArgs &a, int n_seg, bool staged, hipStream_t st) {
           return 0;
         };
         int rc = -6;
-        // a row that is one piece of at most 5 half steps keeps its x in registers (the pair
-        // kernel only with single-lookup levels: two rows of two-term lookups leave no room)
+        // a row that is one piece of at most 5 half steps keeps its x in registers
         const bool one_piece = x_half_steps(a.K_pad) == ring_ns && ring_ns <= 5;
         // the kernel for NS slots by the form of the levels
 #define CHR_GO_ROWS(NS, XREG, PAD)                                                        \
