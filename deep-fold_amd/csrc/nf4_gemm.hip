@@ -113,7 +113,14 @@ constexpr int kStreamBlock = 1024;
 constexpr int kStreamStagers = 512;  // threads of the wavefronts that stage (the other eight multiply)
 constexpr int kStreamRows = 32;
 constexpr int kStreamChunkK = 512;
-constexpr int kStreamRing = 4;
+// Chunks of loads a staging thread keeps in flight in registers.  Two: with four (three at 32
+// and 64 columns) a compute unit had 64 to 100 KB on the way, and this memory system serves a
+// launch fastest with about 32 KB per compute unit in flight (the GEMV's ring: 2 KB a
+// wavefront).  Measured at 4 (3) / 2 / 1, us per launch: 7168x5120 N = 8 10.1 / 9.6 / 12.5, N = 16
+// 10.7 / 10.0 / 11.9, N = 32 12.7 / 11.9 / 13.5, N = 64 20.5 / 19.8 / 20.2; 13824x5120 15.8 / 14.6 /
+// 15.5, 16.5 / 15.3 / 15.4, 17.4 / 16.4 / 16.8, 22.7 / 22.5 / 25.0; 5120x13824 17.2 / 16.2 / 16.6,
+// 18.1 / 17.0 / 17.2, 19.4 / 18.4 / 18.7, 27.4 / 27.3 / 29.0.
+constexpr int kStreamRing = 2;
 constexpr int kStreamBodies = 12;   // chunks of the longest K the tile takes, written out one by one
 constexpr int kStreamMaxGroups = kStreamBodies * kStreamChunkK / 64;  // groups of the longest K
 constexpr int kStreamXS = kStreamChunkK + kXPad;       // bf16 elements of a token row of one chunk
@@ -1005,7 +1012,7 @@ __global__ __launch_bounds__(kRowsBlock) void gemm_rows(const GemmSegs segs,
 // staging thread (two k x eight columns each), or at 32 columns four whole-line pieces,
 // interleaved into the transposed chunk buffer.
 //
-// Pipeline: a staging thread keeps its loads of four chunks (three above 16 columns) in
+// Pipeline: a staging thread keeps its loads of kStreamRing chunks in
 // flight in registers and stores a chunk to LDS (two buffers) one chunk ahead of its use.
 // Every request is unconditional -- past the end of K it repeats the last chunk, unused --
 // and the chunks of a workgroup (at most kStreamBodies) are written out nested, chunk c + 1
@@ -1345,10 +1352,9 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream(const GemmSegs segs,
         sc + static_cast<size_t>(min(row_base + (PAIR ? srow & 31 : srow), M - 1)) * groups_all + 8 * c0 +
         4 * (i - srow * quads));
   }
-  // chunks a staging thread keeps in flight: with 64 bytes of x a chunk, three are what 128
-  // registers hold
-  // (deeper rings measured slower in every form: 6 / 4 chunks with 32 rows, 5 / 4 with 64)
-  constexpr int R = XI >= 2 ? 3 : kStreamRing;
+  // chunks a staging thread keeps in flight (kStreamRing: deeper rings measured slower in every
+  // form)
+  constexpr int R = kStreamRing;
   Item ring[R];
   // (native vectors: the struct type's assignment would pin them in memory; the second block's
   // are idle with one block)
@@ -1781,7 +1787,7 @@ __global__ __launch_bounds__(kStreamBlock) void gemm_stream64(GemmSegs segs,
         sc + static_cast<size_t>(min(row_base + (PAIR ? srow & 31 : srow), M - 1)) * groups_all + 4 * c0 +
         4 * (i - srow * quads));
   }
-  constexpr int R = 3;
+  constexpr int R = kStreamRing;
   Item ring[R];
   U32x4 ring_w[R];
   if (stager) {
