@@ -306,7 +306,9 @@ __global__ __launch_bounds__(INWG ? kWave * WMAX : kWave) void attn_flash(const 
   // and iteration: their loads are independent and all in flight together, so the trip count
   // (and with it the exposed memory latency) shrinks; the one-workgroup form has fewer
   // wavefronts per head and unrolls further.
-  constexpr int UNR = INWG ? 4 : 2;
+  // (with a block read ahead, two: 5.8 / 9.8 us at 640 / 2047 rows with four, 5.4 / 9.5 with two,
+  // 5.55 / 12.3 with one)
+  constexpr int UNR = INWG && !AHEAD ? 4 : 2;
   const int stride = a.n_split * TPW;
   const size_t row_stride = static_cast<size_t>(a.n_kv) * hd;
   // plain dwords: arrays of vector structs would not stay in registers
@@ -499,7 +501,7 @@ constexpr int kMaxGqaWaves = 8;
 template <int LPT, int REP>
 __global__ __launch_bounds__(kWave * kMaxGqaWaves) void attn_chunk_gqa(const AttnArgs a) {
   constexpr int TPW = kWave / LPT;
-  constexpr int UNR = 4;
+  constexpr int UNR = 2;  // (4: the same within 0.5% on a prefill, 8: 1 to 5% slower)
   constexpr int HD = 8 * LPT;
   const int wave = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x >> 6));
   const int wg_waves = a.wg_waves;
