@@ -36,7 +36,7 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes one GEMV launch of the primary workload moves, from FETCH_SIZE + WRITE_SIZE
 # hardware counters scaled by a plain device copy (profiles/gemv_ring_rows_13824x5120_pmc.txt
 # has the runs and the arithmetic).  Hardware counters cannot be read inside this process.
-GEMV_TRAFFIC_BYTES = 39_409_786
+GEMV_TRAFFIC_BYTES = 39_428_626
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
 M, K = 13824, 5120  # headline layer: 14B gate/up projection
