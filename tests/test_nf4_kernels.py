@@ -392,9 +392,9 @@ RING_ROWS = [
     (4100, 4096),   # 4 half steps, x of the row in registers; a pass and four rows more
     (9000, 5120),   # 5 half steps, two passes and a part of a third
     (3, 5120),      # fewer rows than wavefronts
-    (4500, 6144), (4200, 7168), (4100, 8192),
+    (4500, 6144), (4200, 7168), (4100, 8192),   # one piece of 6, of 7; two pieces of 4
     (700, 13824),   # two pieces of 7 half steps
-    (300, 16384),   # two pieces of 8
+    (300, 16384),   # four pieces of 4
     (4300, 6208),   # last half step partly filled (4 of 64 lanes)
     (4200, 5056),   # the same with x in registers
     (4100, 4000),   # K below K_pad
@@ -402,7 +402,8 @@ RING_ROWS = [
     (600, 27648),   # 27: four pieces of 7, the last with an empty slot
     (4200, 10950),  # 11 half steps, the last partly filled, then the empty slot
     (500, 19456),   # 19: four pieces of 5 with an empty slot (x stays in LDS)
-    (400, 23552),   # 23: three pieces of 8 with an empty slot
+    (400, 23552),   # 23: four pieces of 6 with an empty slot
+    (300, 31744),   # 31: four pieces of 8 with an empty slot (the only lengths that take 8)
 ]
 
 
@@ -431,6 +432,36 @@ def test_ring_gemv(m, k, terms, monkeypatch):
     monkeypatch.setenv("CHR_NF4_GEMV_RING", "0")
     y0 = nf4.nf4_gemv(dp, ds, bf16_tensor(x), m, k, oc.k_pad(k))
     check_linear(y, to_f32(y0), what=f"ring {m}x{k} vs pipelined", ulps=1)
+
+
+@pytest.mark.parametrize("m,k", [(70000, 5120), (45000, 6144), (33000, 7168), (20000, 13824), (12000, 16384)])
+def test_ring_gemv_many_rows_per_wavefront(m, k, monkeypatch):
+    """The ring in its steady state (4 to 17 rows per wavefront, every slot requested again a
+    few steps after it was consumed, waits by count): against the compiler-pipelined kernel,
+    whose waits are the compiler's own, to one bf16 step, sampled rows against the fp64 oracle,
+    and the same bits on every one of five launches."""
+    say("ring gemv, many rows", m, k)
+    monkeypatch.setenv("CHR_NF4_GEMV_STAGED", "1")
+    monkeypatch.setenv("CHR_NF4_GEMV_TERMS", "3")
+    g = torch.Generator(device=DEV).manual_seed(m + k)
+    w = torch.randn((m, k), generator=g, device=DEV, dtype=torch.float32) * 0.02
+    dp, ds = nf4.nf4_quantize(w)
+    del w
+    x = rand_x(k, None, 31)
+    dx = bf16_tensor(x)
+    monkeypatch.setenv("CHR_NF4_GEMV_RING", "1")
+    runs = [nf4.nf4_gemv(dp, ds, dx, m, k, oc.k_pad(k)) for _ in range(5)]
+    torch.cuda.synchronize()
+    for r in runs[1:]:
+        assert torch.equal(runs[0].view(torch.int16), r.view(torch.int16))
+    monkeypatch.setenv("CHR_NF4_GEMV_RING", "0")
+    y0 = nf4.nf4_gemv(dp, ds, dx, m, k, oc.k_pad(k))
+    check_linear(runs[0], to_f32(y0), what=f"ring {m}x{k} vs pipelined", ulps=1)
+    rows = torch.arange(0, m, 997, device=DEV)
+    wd = nf4.nf4_dequant(dp, ds, m, k, oc.k_pad(k))[rows].double()
+    want = (wd @ torch.from_numpy(x.astype(np.float64)).to(DEV)).cpu().numpy()
+    got = to_f32(runs[0][rows]).reshape(-1)
+    assert np.abs(got - want).max() <= 1e-2 * np.abs(want).max() + 0.05
 
 
 # Form 3 stages x as binary16, every 16 consecutive elements times the power of two that puts
