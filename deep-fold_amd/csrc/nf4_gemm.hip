@@ -240,8 +240,10 @@ constexpr int kArriveBlocks = 1024;  // row blocks of a launch whose splits meet
 // the caller brought a workspace; at most four rounds of workgroups, and more than one only
 // with 3072 of K or more to spread a round's fixed time over and the rounds four fifths full,
 // and splits over several rounds only from 24 columns on), the one a cost model fitted to measurements calls cheapest, in hundredths of a
-// microsecond: a round of 32-row workgroups 5.2 us + 0.55 / 0.67 / 0.86 / 1.06 us a chunk at
-// 8 / 16 / 24 / 32 columns, of 64-row workgroups 6.5 us + 1.00 / 1.06 / 1.22 / 1.38 us a chunk,
+// microsecond: a round of 32-row workgroups 4.5 us + 0.50 / 0.52 / 0.62 / 0.73 us a chunk at
+// 8 / 16 / 24 / 32 columns, of 64-row workgroups 6.0 us + 0.86 / 0.93 / 1.00 / 1.06 us a chunk
+// (refitted with two chunks of loads in flight per staging thread; before, 5.2 + 0.55 .. 1.06
+// and 6.5 + 1.00 .. 1.38),
 // 2.3 us for the meeting of a split's partials (at most 8 splits; a split has to win by 3%).
 // codes: weights of the launch; with 2^24 or fewer the split tiles keep it (measured at
 // 8 / 32 columns, this tile against those: 256x5120 8.2 / 8.8 us against 7.5 / 8.5, 2048x2048
@@ -250,8 +252,8 @@ constexpr int kArriveBlocks = 1024;  // row blocks of a launch whose splits meet
 // shapes below).  At 64 columns, where the split tiles are slower, above 2^20 weights
 // (512x2048 14.9 us against 17.7, 2560x2048 13.6 against 19.1, 4096x4096 16.3 against 20.5;
 // 256x1024 10.9 against 10.4).  At the 14B shapes:
-// q/k/v 32 rows x all of K up to 24 columns and 64 rows x 2 splits at 32; o 32 rows x all of K
-// up to 16 columns, 64 rows x 3 splits above; gate or up 64 rows; gate+up stacked 64 rows in two
+// q/k/v and o 32 rows x all of K up to 32 columns (o at 32 columns: 11.7 us against 12.4 with
+// 64 rows x 3 splits), 64 rows x 2 or 3 splits at 64; gate or up 64 rows; gate+up stacked 64 rows in two
 // rounds; down (K = 13824) 64 rows x 3 splits.  CHR_NF4_GEMM_STREAM_ROWS=32 or 64 allows only
 // that form, CHR_NF4_GEMM_STREAM_SPLIT=0 no splits.
 StreamPlan stream_plan(int N, int K_pad, int blocks32, int blocks64, int have_ws, int64_t codes) {
@@ -261,8 +263,8 @@ StreamPlan stream_plan(int N, int K_pad, int blocks32, int blocks64, int have_ws
   if (!stream_columns(N) || tuning().split_k != 0 || K_pad % kBK != 0) {
     return best;
   }
-  static constexpr int kFixed[2] = {520, 650};
-  static constexpr int kChunk[2][4] = {{55, 67, 86, 106}, {100, 106, 122, 138}};
+  static constexpr int kFixed[2] = {450, 600};
+  static constexpr int kChunk[2][4] = {{50, 52, 62, 73}, {86, 93, 100, 106}};
   constexpr int kWideChunk = 110;  // a 256-wide chunk of the 64-column form
   constexpr int kMeet = 230, kMaxSplit = 8;
   const int cus = resolved_one_wave();

@@ -246,8 +246,8 @@ def _stream_columns(N: int, policy: int) -> bool:  # noqa: N803
 _STREAM_SPLITS: bool | None = None
 #: the stream tile's cost model, hundredths of a microsecond: a round of workgroups of 32 / 64
 #: rows, a 512-wide chunk at 8 / 16 / 24 / 32 columns, the meeting of a split's partials
-_STREAM_FIXED = (520, 650)
-_STREAM_CHUNK = ((55, 67, 86, 106), (100, 106, 122, 138))
+_STREAM_FIXED = (450, 600)
+_STREAM_CHUNK = ((50, 52, 62, 73), (86, 93, 100, 106))
 _STREAM_CHUNK_64 = 110      # a 256-wide chunk of the 64-column form (64 rows a workgroup)
 _STREAM_MEET = 230
 _STREAM_MAX_SPLIT = 8

@@ -829,7 +829,7 @@ def test_gemm_stream_splits_in_a_replayed_graph():
     """Three launches with K shared by workgroups, captured in one graph: every replay, with
     eager launches of the same tile between the replays, gives the eager results bit for bit
     (the arrival counts must be back at zero after every launch)."""
-    shapes = [(5120, 13824, 8), (5120, 5120, 32), (3072, 8192, 16)]
+    shapes = [(5120, 13824, 8), (5120, 13824, 32), (3072, 8192, 16)]
     mats, xs, eager = [], [], []
     for i, (m, k, n) in enumerate(shapes):
         say("gemm stream, graph", m, k, n)
@@ -944,9 +944,8 @@ def test_gemm_full_14b_shapes(name, m, k):
         y = nf4.nf4_gemm(dp, ds, bf16_tensor(x), m, k, k)
         plan = nf4.nf4_plan(m, k, n)
         # every one of them on the tile whose workgroups finish their rows themselves: 32 rows
-        # and all of K (q/k/v, o to 24 columns), 64 rows (gate, up), 64 rows and K over three
-        # workgroups (o at 32 columns, down)
-        form = {"qkv": (32, 1), "o": (64, 3) if n == 32 else (32, 1), "gate_up": (64, 1), "down": (64, 3)}
+        # and all of K (q/k/v, o), 64 rows (gate, up), 64 rows and K over three workgroups (down)
+        form = {"qkv": (32, 1), "o": (32, 1), "gate_up": (64, 1), "down": (64, 3)}
         assert (plan["bm"], plan["grid_y"]) == form[name], name
         assert plan["block"] == 1024
         ref = oc.c_matmul_f64(exact_w, x)
