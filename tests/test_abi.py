@@ -8,6 +8,7 @@ import ctypes
 import os
 import re
 
+import numpy as np
 import pytest
 
 from deepfold_amd import nf4
@@ -145,3 +146,15 @@ def test_no_cpu_fallback():
         nf4.nf4_gemv(packed, scale, x, 128, 256, 256)
     with pytest.raises(RuntimeError, match="CUDA"):
         nf4.nf4_gemm(packed, scale, x.reshape(256, 1).repeat(1, 2), 128, 256, 256)
+
+
+def test_attention_index_division_by_reciprocal_is_exact_where_the_kernel_uses_it():
+    """The decode attention finds (head, part) of a workgroup with ``int((x + 0.5f) * (1.f / d))``
+    instead of an integer division (``small_div`` in ``csrc/nf4_attn.hip``); the host passes the
+    reciprocal only for x < 2^22 and d <= 256.  The same float32 arithmetic here, every such
+    pair."""
+    x = np.arange(0, 1 << 22, dtype=np.int64)
+    xf = x.astype(np.float32) + np.float32(0.5)
+    for d in range(1, 257):
+        q = (xf * (np.float32(1.0) / np.float32(d))).astype(np.int64)
+        assert np.array_equal(q, x // d), d
