@@ -12,7 +12,7 @@
 namespace chr {
 
 int gemv_attn_entry(const chr_nf4_dev_t *w, const float *state, int n_q, int hd, int n_parts,
-                    void *y, const void *add, void *stream);
+                    void *y, const void *add, void *stream, float *sq_out);
 
 namespace {
 
@@ -27,7 +27,7 @@ __global__ __launch_bounds__(kBeginBlock) void begin_step(
     const uint8_t *__restrict__ packed, const uint16_t *__restrict__ scale, int M, int K, int K_pad,
     const int64_t *__restrict__ token, const int64_t *__restrict__ position,
     int32_t *__restrict__ valid_len, uint16_t *__restrict__ x, const uint16_t *__restrict__ norm_w,
-    float eps, uint16_t *__restrict__ h) {
+    float eps, uint16_t *__restrict__ h, float *__restrict__ sq_out, int sq_parts) {
   __shared__ float lut[16];
   __shared__ float part[kBeginBlock / kWave];
   if (threadIdx.x < 16) {
@@ -61,10 +61,20 @@ __global__ __launch_bounds__(kBeginBlock) void begin_step(
   if ((threadIdx.x & (kWave - 1)) == 0) {
     part[threadIdx.x >> 6] = sq;
   }
-  if (norm_w == nullptr) {
+  if (norm_w == nullptr && sq_out == nullptr) {
     return;
   }
   __syncthreads();  // also orders this workgroup's x stores before the reads below
+  if (sq_out != nullptr) {
+    // the sum of squares of x in the form the GEMVs hand it on: the wavefronts' sums as the
+    // first parts, zeros behind them
+    for (int i = threadIdx.x; i < sq_parts; i += kBeginBlock) {
+      sq_out[i] = i < kBeginBlock / kWave ? part[i] : 0.f;
+    }
+  }
+  if (norm_w == nullptr) {
+    return;
+  }
   float sum = 0.f;
 #pragma unroll
   for (int i = 0; i < kBeginBlock / kWave; ++i) {
@@ -298,9 +308,11 @@ __global__ __launch_bounds__(kArgmaxParts) void argmax_final(
 
 using namespace chr;
 
-extern "C" int chr_dv2_begin_step(const chr_nf4_dev_t *table, const void *token,
-                                  const void *position, void *valid_len, void *x,
-                                  const void *norm_w, float eps, void *h, void *stream) {
+namespace chr {
+namespace {
+int begin_step_entry(const chr_nf4_dev_t *table, const void *token, const void *position,
+                     void *valid_len, void *x, const void *norm_w, float eps, void *h, void *stream,
+                     float *sq_out) {
   if (table == nullptr || token == nullptr || position == nullptr || valid_len == nullptr ||
       x == nullptr || (norm_w != nullptr && h == nullptr)) {
     return -1;
@@ -318,14 +330,38 @@ extern "C" int chr_dv2_begin_step(const chr_nf4_dev_t *table, const void *token,
       table->packed, table->scale, table->M, table->K, table->K_pad,
       static_cast<const int64_t *>(token), static_cast<const int64_t *>(position),
       static_cast<int32_t *>(valid_len), static_cast<uint16_t *>(x),
-      static_cast<const uint16_t *>(norm_w), eps, static_cast<uint16_t *>(h));
+      static_cast<const uint16_t *>(norm_w), eps, static_cast<uint16_t *>(h), sq_out, kSumsqParts);
   return launch_rc();
+}
+}  // namespace
+}  // namespace chr
+
+extern "C" int chr_dv2_begin_step(const chr_nf4_dev_t *table, const void *token,
+                                  const void *position, void *valid_len, void *x,
+                                  const void *norm_w, float eps, void *h, void *stream) {
+  return begin_step_entry(table, token, position, valid_len, x, norm_w, eps, h, stream, nullptr);
+}
+
+extern "C" int chr_dv2_begin_step_sumsq(const chr_nf4_dev_t *table, const void *token,
+                                        const void *position, void *valid_len, void *x,
+                                        void *stream, float *sumsq_out) {
+  if (sumsq_out == nullptr || (reinterpret_cast<uintptr_t>(sumsq_out) & 3u) != 0) {
+    return sumsq_out == nullptr ? -1 : -5;
+  }
+  return begin_step_entry(table, token, position, valid_len, x, nullptr, 0.f, nullptr, stream,
+                          sumsq_out);
 }
 
 extern "C" int chr_dv2_gemv_attn(const chr_nf4_dev_t *w, const float *state, int32_t n_q,
                                  int32_t hd, int32_t n_parts, void *y, const void *add,
                                  void *stream) {
-  return gemv_attn_entry(w, state, n_q, hd, n_parts, y, add, stream);
+  return gemv_attn_entry(w, state, n_q, hd, n_parts, y, add, stream, nullptr);
+}
+
+extern "C" int chr_dv2_gemv_attn_sumsq(const chr_nf4_dev_t *w, const float *state, int32_t n_q,
+                                       int32_t hd, int32_t n_parts, void *y, const void *add,
+                                       void *stream, float *sumsq_out) {
+  return gemv_attn_entry(w, state, n_q, hd, n_parts, y, add, stream, sumsq_out);
 }
 
 extern "C" int chr_dv2_mark_written(const void *position, void *valid_len, void *stream) {

@@ -12,6 +12,10 @@ namespace chr {
 
 constexpr int kGroup = 64;  // weights per scale
 constexpr int kWave = 64;   // lanes per wavefront on gfx950
+// Floats of a sum of squares handed from the launch that writes a vector to the launch that
+// normalises it (one part per workgroup of the writer, zeros behind them; a lane of the reader
+// takes four).
+constexpr int kSumsqParts = 256;
 
 // binary32 bit patterns of the QLoRA NF4 levels (internal/nf4/nf4.go:18-35,
 // bits as listed in internal/nf4/nf4_test.go:12-29).

@@ -52,7 +52,7 @@
 namespace chr {
 
 int gemv_entry(const chr_nf4_dev_t *w, const void *x, void *y, void *stream, const void *add,
-               const void *rms_w, float rms_eps);
+               const void *rms_w, float rms_eps, const float *sq_in, float *sq_out);
 int gemv_rows_per_wg(int M, int K, int K_pad);
 int gemv_threads_per_wg(int M, int K, int K_pad);
 int gemv_grid_x(int M, int K, int K_pad);
@@ -2469,7 +2469,7 @@ int gemm_launch(const chr_nf4_dev_t *const *w, int nseg, const void *x, void *y,
     if (bias != nullptr || res != nullptr || nseg != 1) {
       return -2;  // the fused epilogue and the stacking belong to the tiles (N >= 2)
     }
-    return gemv_entry(&h[0], x, y, stream, nullptr, nullptr, 0.f);
+    return gemv_entry(&h[0], x, y, stream, nullptr, nullptr, 0.f, nullptr, nullptr);
   }
   const int have_ws = (ws != nullptr && ws_floats > 0) ? 1 : 0;
   bool scales_aligned8 = true;

@@ -85,6 +85,12 @@ struct StreamArgs {
   float rms_eps;
   // ring kernels: grid size, full passes of 16 * grid groups, and the groups left after them
   int ring_grid, ring_passes, ring_left;
+  // Sum of squares handed from the launch that writes a vector to the launch that normalises
+  // it: kSumsqParts floats, workgroup b of the writer leaving the sum over its rows' stored
+  // bf16 values at [b] (zeros where no workgroup writes).  sq_out: this launch writes them for
+  // its y; sq_in (with rms_w): this launch takes mean(x^2) from them instead of summing x.
+  float *sq_out;
+  const float *sq_in;
 };
 
 // Sum of a value over a workgroup of kStagedThreads threads, the same in every thread.
@@ -275,10 +281,17 @@ __device__ __forceinline__ bool stage_fast_ok(const StreamArgs &a) {
 // the last vector and is dropped at the use), so later code can wait for these loads by
 // count while younger loads are still in flight.
 __device__ __forceinline__ void x_request(const StreamArgs &a, uint4 (&v)[kXKeep],
-                                          uint4 (&g)[kXKeep]) {
+                                          uint4 (&g)[kXKeep], uint4 &sq) {
   const int nk = a.K >> 3;
   const int deal = x_deal(a.K_pad >> 3);
   const int wave_first = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) & ~(kWave - 1));
+  // (the parts of the sum of squares, or, without them, a vector of x that is dropped: a load
+  // under a condition of its own would make the wait for x a wait for everything)
+  sq = make_uint4(0, 0, 0, 0);
+  if (wave_first < deal) {
+    sq = a.sq_in != nullptr ? reinterpret_cast<const uint4 *>(a.sq_in)[threadIdx.x & (kWave - 1)]
+                            : reinterpret_cast<const uint4 *>(a.x)[0];
+  }
 #pragma unroll
   for (int j = 0; j < kXKeep; ++j) {
     v[j] = make_uint4(0, 0, 0, 0);
@@ -326,7 +339,8 @@ __device__ __forceinline__ void store_piece(uint4 *xs, float *xf, int i, bool li
 // stored as binary16, pair by pair times a power of two (store_piece).
 template <bool F16>
 __device__ __forceinline__ void x_store(const StreamArgs &a, uint4 *xs, StagedLds &lds,
-                                        const uint4 (&v)[kXKeep], const uint4 (&g)[kXKeep]) {
+                                        const uint4 (&v)[kXKeep], const uint4 (&g)[kXKeep],
+                                        const uint4 sq) {
   const int nk = a.K >> 3;
   const int nvec = a.K_pad >> 3;
   float *xf = x_factors(xs, a.K_pad);
@@ -345,7 +359,15 @@ __device__ __forceinline__ void x_store(const StreamArgs &a, uint4 *xs, StagedLd
   // at K = 5120 eight wavefronts hold a vector, two of them a second one
   const int wave_first = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) & ~(kWave - 1));
   const int deal = x_deal(nvec);
-  if (a.rms_w != nullptr) {
+  if (a.rms_w != nullptr && a.sq_in != nullptr) {
+    // the writer of x left the sum in kSumsqParts parts: lane l holds parts 4l .. 4l+3 (only
+    // the wavefronts that hold x need the factor; no barrier)
+    if (wave_first < deal) {
+      const float ss = wave_sum(((__uint_as_float(sq.x) + __uint_as_float(sq.y)) + __uint_as_float(sq.z)) +
+                                __uint_as_float(sq.w));
+      inv = rsqrtf(ss / static_cast<float>(a.K) + a.rms_eps);
+    }
+  } else if (a.rms_w != nullptr) {
     float ss = 0.f;
 #pragma unroll
     for (int j = 0; j < kXKeep; ++j) {
@@ -947,16 +969,16 @@ __global__ __launch_bounds__(1024) void gemv_staged(const StreamArgs a) {
   // (the two copies of the stores and barriers are the price): a path that merged
   // "weights requested" with "nothing requested" would make the wait a wait for all.
   if (stage_fast_ok(a)) {
-    uint4 xv[kXKeep], xg[kXKeep];
-    x_request(a, xv, xg);
+    uint4 xv[kXKeep], xg[kXKeep], xq;
+    x_request(a, xv, xg, xq);
     if (n_items > 0) {
       group_pointers<R, SWIGLU>(a, first, prow, srow);
       CHR_REQUEST(wa, sa)
       fill_table();
-      x_store<TERMS == 3>(a, xs, lds, xv, xg);
+      x_store<TERMS == 3>(a, xs, lds, xv, xg, xq);
     } else {
       fill_table();
-      x_store<TERMS == 3>(a, xs, lds, xv, xg);
+      x_store<TERMS == 3>(a, xs, lds, xv, xg, xq);
     }
   } else {
     // The other staging forms read what they need in loops of their own; the first item
@@ -1063,6 +1085,7 @@ __global__ __launch_bounds__(1024) void gemv_staged(const StreamArgs a) {
 struct XRegs {
   U32x4 v[kXKeep];  // x, 16-byte vectors i = thread + j * x_deal()
   U32x4 g[kXKeep];  // the RMSNorm weights at the same places (fused norm only)
+  U32x4 q;          // four of the sum-of-squares parts a writer left (sq_in only)
 };
 
 // A request whose destination keeps its value where the request is skipped: in/out operand,
@@ -1075,6 +1098,10 @@ __device__ __forceinline__ void ring_x_request(const StreamArgs &a, XRegs &x, ui
   const int nk = a.K >> 3;
   const int deal = x_deal(a.K_pad >> 3);
   const int wave_first = __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) & ~(kWave - 1));
+  x.q = U32x4{0u, 0u, 0u, 0u};
+  if (a.sq_in != nullptr && wave_first < deal) {
+    request16(x.q, reinterpret_cast<const uint4 *>(a.sq_in) + (threadIdx.x & (kWave - 1)), tok);
+  }
 #pragma unroll
   for (int j = 0; j < kXKeep; ++j) {
     x.v[j] = U32x4{0u, 0u, 0u, 0u};
@@ -1093,9 +1120,9 @@ __device__ __forceinline__ void ring_x_request(const StreamArgs &a, XRegs &x, ui
 template <int YOUNGER>
 __device__ __forceinline__ void ring_x_wait(XRegs &x, uint32_t &tok) {
   static_assert(kXKeep == 4, "operand list below");
-  asm("s_waitcnt vmcnt(%9) ; covers %0 %1 %2 %3 %4 %5 %6 %7"
+  asm("s_waitcnt vmcnt(%10) ; covers %0 %1 %2 %3 %4 %5 %6 %7 %8"
       : "+v"(x.v[0]), "+v"(x.v[1]), "+v"(x.v[2]), "+v"(x.v[3]), "+v"(x.g[0]), "+v"(x.g[1]),
-        "+v"(x.g[2]), "+v"(x.g[3]), "+s"(tok)
+        "+v"(x.g[2]), "+v"(x.g[3]), "+v"(x.q), "+s"(tok)
       : "n"(YOUNGER));
 }
 
@@ -1394,7 +1421,7 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
       xv[j] = make_uint4(xr.v[j].x, xr.v[j].y, xr.v[j].z, xr.v[j].w);
       xg[j] = make_uint4(xr.g[j].x, xr.g[j].y, xr.g[j].z, xr.g[j].w);
     }
-    x_store<TERMS == 3>(a, xs, lds, xv, xg);
+    x_store<TERMS == 3>(a, xs, lds, xv, xg, make_uint4(xr.q.x, xr.q.y, xr.q.z, xr.q.w));
   } else {
     // The other staging forms read what they need in loops of their own (loads the compiler
     // counts: its waits then also cover the half steps requested here, which are older).
@@ -1411,6 +1438,7 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
 #undef CHR_RING_FILL_STEP
 
   float acc[R] = {};
+  float sq_acc = 0.f;    // sq_out: sum of squares of what this wavefront has stored
   float gate_sum = 0.f;  // SEQ: the gate row's sum while the up row is walked
   int c_sub = 0;
   auto finish_group = [&](int grp) {
@@ -1435,8 +1463,13 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
       if (add != nullptr) {
         v += uniform_bf16(add + row);
       }
+      const uint16_t stored = f32_to_bf16(v);
       if (lane == 0) {
-        y[row] = f32_to_bf16(v);
+        y[row] = stored;
+      }
+      if (a.sq_out != nullptr) {
+        const float r = bf16_to_f32(stored);
+        sq_acc = fmaf(r, r, sq_acc);
       }
     }
 #pragma unroll
@@ -1583,6 +1616,26 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
   // nothing may still be on its way into the fixed registers when the wavefront ends (this
   // statement is volatile: it is what keeps the token chain, and with it every request, alive)
   asm volatile("s_waitcnt vmcnt(0)" : "+s"(tok));
+  if constexpr (!SEQ) {
+    if (a.sq_out != nullptr) {
+      // the wavefronts' sums meet in their own order; the workgroup's part, and zeros at the
+      // places no workgroup writes
+      if (lane == 0) {
+        lds.part[wave] = sq_acc;
+      }
+      __syncthreads();
+      if (wave == 0 && lane == 0) {
+        float s = 0.f;
+        for (int w = 0; w < waves; ++w) {
+          s += lds.part[w];
+        }
+        a.sq_out[block] = s;
+        for (int b = block + grid; b < kSumsqParts; b += grid) {
+          a.sq_out[b] = 0.f;
+        }
+      }
+    }
+  }
 #undef CHR_RING_REQUEST_LAST
 #undef CHR_RING_REQUEST_NEXT
 #undef CHR_RING_REQUEST_SLOT
@@ -1817,9 +1870,23 @@ int staged_rows_for_m(int M, int K_pad) {
   return M >= 32768 ? 2 : 1;
 }
 
+// Whether a launch can take its mean(x^2) from parts a writer left: the staging that keeps x in
+// registers between its request and its use (the device's stage_fast_ok), on a staged kernel.
+bool sumsq_in_ok(const StreamArgs &a, bool staged) {
+  return staged && a.rms_w != nullptr && a.attn_state == nullptr && (a.K & 7) == 0 &&
+         aligned16(a.x) && aligned16(a.rms_w) && aligned16(a.sq_in) &&
+         (a.K_pad >> 3) <= kXKeep * kStagedThreads;
+}
+
 template <int R, bool SWIGLU>
 int launch_stream(StreamArgs &a, int n_seg, bool staged, hipStream_t st) {
   constexpr int U = SWIGLU ? R / 2 : R;
+  if (a.sq_in != nullptr && !sumsq_in_ok(a, staged)) {
+    return -8;
+  }
+  if (a.sq_out != nullptr && !staged) {
+    return -8;  // only the ring kernel of single rows writes the parts (checked again below)
+  }
   int total = 0;
   for (int i = 0; i < 3; ++i) {
     a.groups[i] = i < n_seg ? (a.M[i] + U - 1) / U : 0;
@@ -1840,6 +1907,11 @@ int launch_stream(StreamArgs &a, int n_seg, bool staged, hipStream_t st) {
     a.ring_grid = grid;
     a.ring_passes = total / per_pass;
     a.ring_left = total % per_pass;
+    if (a.sq_out != nullptr &&
+        !(ring_ns > 0 && !SWIGLU && n_seg == 1 && grid <= kSumsqParts &&
+          (reinterpret_cast<uintptr_t>(a.sq_out) & 3u) == 0)) {
+      return -8;
+    }
     if (ring_ns > 0) {
       if constexpr (kRingShape) {
         auto go = [&](auto kern) {
@@ -1957,9 +2029,12 @@ int launch_pairs(StreamArgs &a, int m_pairs, hipStream_t st) {
 
 // Shared with the GEMM entry points, which route N == 1 here.
 int gemv_entry(const chr_nf4_dev_t *w, const void *x, void *y, void *stream, const void *add,
-               const void *rms_w, float rms_eps) {
+               const void *rms_w, float rms_eps, const float *sq_in, float *sq_out) {
   if (w == nullptr || x == nullptr || y == nullptr) {
     return -1;
+  }
+  if (sq_in != nullptr && rms_w == nullptr) {
+    return -8;
   }
   if (w->M < 1 || w->K < 1 || w->packed == nullptr || w->scale == nullptr) {
     return -3;
@@ -1981,12 +2056,14 @@ int gemv_entry(const chr_nf4_dev_t *w, const void *x, void *y, void *stream, con
   a.K = w->K;
   a.K_pad = w->K_pad;
   a.rms_eps = rms_eps;
+  a.sq_in = sq_in;
+  a.sq_out = sq_out;
   return launch_rows(a, 1, w->M, static_cast<hipStream_t>(stream));
 }
 
 // y = W @ merge(states) (+ add): the o projection consuming what chr_dv2_attn_parts left.
 int gemv_attn_entry(const chr_nf4_dev_t *w, const float *state, int n_q, int hd, int n_parts,
-                    void *y, const void *add, void *stream) {
+                    void *y, const void *add, void *stream, float *sq_out) {
   if (w == nullptr || state == nullptr || y == nullptr) {
     return -1;
   }
@@ -2011,7 +2088,28 @@ int gemv_attn_entry(const chr_nf4_dev_t *w, const float *state, int n_q, int hd,
   a.attn_state = state;
   a.attn_parts = n_parts;
   a.attn_hd = hd;
+  a.sq_out = sq_out;
   return launch_rows(a, 1, w->M, static_cast<hipStream_t>(stream));
+}
+
+// Whether a single-matrix GEMV of this shape (merging attention states or not) runs on the
+// kernel that can leave the sum of squares of its output (chr_dv2_sumsq_ok).
+bool gemv_sumsq_out_ok(int M, int K, int K_pad, bool merges_attention) {
+  if (M < 1 || K < 1 || !k_pad_ok(K, K_pad)) {
+    return false;
+  }
+  StreamArgs a{};
+  a.K = K;
+  a.K_pad = K_pad;
+  if (merges_attention) {
+    a.attn_state = reinterpret_cast<const float *>(&a);  // only tested against nullptr
+  }
+  if (pick_family(a, M) != 1 || staged_rows_for_m(M, K_pad) != 1 || !ring_wanted() ||
+      ring_piece_steps(x_half_steps(K_pad)).steps == 0) {
+    return false;
+  }
+  const int waves = kStagedThreads / kWave;
+  return std::min(device_cu_count(), (M + waves - 1) / waves) <= kSumsqParts;
 }
 
 // Launch geometry of the N=1 path, reported by the planner: what chr_nf4_gemv launches for
@@ -2052,13 +2150,29 @@ using namespace chr;
 
 extern "C" int chr_nf4_gemv(const chr_nf4_dev_t *w, const void *x, void *y, void *stream,
                             const void *add, const void *rms_w, float rms_eps) {
-  return gemv_entry(w, x, y, stream, add, rms_w, rms_eps);
+  return gemv_entry(w, x, y, stream, add, rms_w, rms_eps, nullptr, nullptr);
 }
 
-extern "C" int chr_nf4_gemv_qkv(const chr_nf4_dev_t *q, const chr_nf4_dev_t *k,
-                                const chr_nf4_dev_t *v, const void *x, void *yq, void *yk,
-                                void *yv, const void *bq, const void *bk, const void *bv,
-                                void *stream, const void *rms_w, float rms_eps) {
+extern "C" int chr_dv2_gemv_sumsq(const chr_nf4_dev_t *w, const void *x, void *y, void *stream,
+                                  const void *add, const void *rms_w, float rms_eps,
+                                  const float *sumsq_in, float *sumsq_out) {
+  return gemv_entry(w, x, y, stream, add, rms_w, rms_eps, sumsq_in, sumsq_out);
+}
+
+extern "C" int32_t chr_dv2_sumsq_parts(void) { return kSumsqParts; }
+
+extern "C" int32_t chr_dv2_sumsq_ok(int32_t M, int32_t K, int32_t K_pad, int32_t merges_attention) {
+  return gemv_sumsq_out_ok(M, K, K_pad, merges_attention != 0) ? 1 : 0;
+}
+
+namespace chr {
+namespace {
+int qkv_entry(const chr_nf4_dev_t *q, const chr_nf4_dev_t *k, const chr_nf4_dev_t *v, const void *x,
+              void *yq, void *yk, void *yv, const void *bq, const void *bk, const void *bv,
+              void *stream, const void *rms_w, float rms_eps, const float *sq_in) {
+  if (sq_in != nullptr && rms_w == nullptr) {
+    return -8;
+  }
   if (q == nullptr || k == nullptr || v == nullptr || x == nullptr || yq == nullptr ||
       yk == nullptr || yv == nullptr) {
     return -1;
@@ -2093,12 +2207,15 @@ extern "C" int chr_nf4_gemv_qkv(const chr_nf4_dev_t *q, const chr_nf4_dev_t *k,
   a.K = q->K;
   a.K_pad = q->K_pad;
   a.rms_eps = rms_eps;
+  a.sq_in = sq_in;
   return launch_rows(a, 3, q->M + k->M + v->M, static_cast<hipStream_t>(stream));
 }
 
-extern "C" int chr_nf4_gemv_swiglu(const chr_nf4_dev_t *gate, const chr_nf4_dev_t *up,
-                                   const void *x, void *y, void *stream, const void *rms_w,
-                                   float rms_eps) {
+int swiglu_entry(const chr_nf4_dev_t *gate, const chr_nf4_dev_t *up, const void *x, void *y,
+                 void *stream, const void *rms_w, float rms_eps, const float *sq_in) {
+  if (sq_in != nullptr && rms_w == nullptr) {
+    return -8;
+  }
   if (gate == nullptr || up == nullptr || x == nullptr || y == nullptr) {
     return -1;
   }
@@ -2125,7 +2242,37 @@ extern "C" int chr_nf4_gemv_swiglu(const chr_nf4_dev_t *gate, const chr_nf4_dev_
   a.K = gate->K;
   a.K_pad = gate->K_pad;
   a.rms_eps = rms_eps;
+  a.sq_in = sq_in;
   return launch_pairs(a, gate->M, static_cast<hipStream_t>(stream));
+}
+}  // namespace
+}  // namespace chr
+
+extern "C" int chr_nf4_gemv_qkv(const chr_nf4_dev_t *q, const chr_nf4_dev_t *k,
+                                const chr_nf4_dev_t *v, const void *x, void *yq, void *yk,
+                                void *yv, const void *bq, const void *bk, const void *bv,
+                                void *stream, const void *rms_w, float rms_eps) {
+  return qkv_entry(q, k, v, x, yq, yk, yv, bq, bk, bv, stream, rms_w, rms_eps, nullptr);
+}
+
+extern "C" int chr_dv2_gemv_qkv_sumsq(const chr_nf4_dev_t *q, const chr_nf4_dev_t *k,
+                                      const chr_nf4_dev_t *v, const void *x, void *yq, void *yk,
+                                      void *yv, const void *bq, const void *bk, const void *bv,
+                                      void *stream, const void *rms_w, float rms_eps,
+                                      const float *sumsq_in) {
+  return qkv_entry(q, k, v, x, yq, yk, yv, bq, bk, bv, stream, rms_w, rms_eps, sumsq_in);
+}
+
+extern "C" int chr_nf4_gemv_swiglu(const chr_nf4_dev_t *gate, const chr_nf4_dev_t *up,
+                                   const void *x, void *y, void *stream, const void *rms_w,
+                                   float rms_eps) {
+  return swiglu_entry(gate, up, x, y, stream, rms_w, rms_eps, nullptr);
+}
+
+extern "C" int chr_dv2_gemv_swiglu_sumsq(const chr_nf4_dev_t *gate, const chr_nf4_dev_t *up,
+                                         const void *x, void *y, void *stream, const void *rms_w,
+                                         float rms_eps, const float *sumsq_in) {
+  return swiglu_entry(gate, up, x, y, stream, rms_w, rms_eps, sumsq_in);
 }
 
 extern "C" int chr_nf4_rms(const void *x, const void *w, void *y, int32_t n, float eps,

@@ -7,7 +7,7 @@ from dataclasses import dataclass
 
 import torch
 
-from ..nf4 import ATTN_SPLIT, dv2_argmax_ws_bytes, dv2_attn_state_floats
+from ..nf4 import ATTN_SPLIT, dv2_argmax_ws_bytes, dv2_attn_state_floats, dv2_sumsq_parts
 from .plan import ArchSpec
 
 __all__ = ["Arena"]
@@ -28,6 +28,7 @@ class Arena:
     attn_ws: torch.Tensor
     attn_state: torch.Tensor     # softmax states of the attention whose merge the o projection does
     argmax_ws: torch.Tensor      # per-slice candidates of the two-launch argmax
+    sumsq: torch.Tensor          # sum of squares of x, in parts, from the launch that wrote x to the one that normalises it
 
     @classmethod
     def allocate(cls, spec: ArchSpec, *, device, dtype: torch.dtype = torch.bfloat16) -> "Arena":
@@ -50,4 +51,5 @@ class Arena:
             attn_state=torch.zeros(dv2_attn_state_floats(spec.n_q, spec.head_dim), dtype=torch.float32,
                                    device=device),
             argmax_ws=torch.zeros(dv2_argmax_ws_bytes() // 8, dtype=torch.int64, device=device),
+            sumsq=torch.zeros(dv2_sumsq_parts(), dtype=torch.float32, device=device),
         )

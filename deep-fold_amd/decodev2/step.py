@@ -16,15 +16,19 @@ Two launch schedules compute that sequence:
               attention splits runs inside the o projection, and the embedding
               gather also sets the KV length: five launches per layer.  A
               dependent launch costs about 5 us on an MI355X whatever it does, so
-              the launch count is what this buys.
+              the launch count is what this buys.  Where every launch that writes the
+              residual stream can do so, it also leaves the sum of squares of what it
+              wrote for the launch that normalises it (``_sumsq_handover``).
 """
 
 from __future__ import annotations
 
+import os
+
 import torch
 
-from ..nf4 import (ATTN_SPLIT, dv2_attn_parts, dv2_begin_step, dv2_gemv_attn, nf4_attn, nf4_gemv,
-                   nf4_qkv, nf4_rms, nf4_swiglu)
+from ..nf4 import (ATTN_SPLIT, dv2_attn_parts, dv2_begin_step, dv2_gemv_attn, dv2_sumsq_ok, nf4_attn,
+                   nf4_gemv, nf4_qkv, nf4_rms, nf4_swiglu)
 from .embed import PackedEmbed, gather_embed
 from .linear import DeviceLayer, DeviceLinear, DeviceWeights
 from .state import DecodeState
@@ -32,30 +36,53 @@ from .state import DecodeState
 __all__ = ["forward_decode", "greedy_decode", "teacher_force_token", "SCHEDULES"]
 
 
-def _gemv_accum(mat: DeviceLinear, src: torch.Tensor, dest: torch.Tensor) -> None:
-    """``dest += W @ src`` in one launch (residual added in fp32 before rounding)."""
+def _gemv_accum(mat: DeviceLinear, src: torch.Tensor, dest: torch.Tensor,
+                sumsq_out: torch.Tensor | None = None) -> None:
+    """``dest += W @ src`` in one launch (residual added in fp32 before rounding); with
+    ``sumsq_out`` the launch leaves the sum of squares of the new ``dest`` (no bias then)."""
     d = dest.view(-1)
-    nf4_gemv(mat.packed, mat.scale, src.view(-1), mat.M, mat.K, mat.K_pad, d, d)
+    nf4_gemv(mat.packed, mat.scale, src.view(-1), mat.M, mat.K, mat.K_pad, d, d, sumsq_out=sumsq_out)
     if mat.bias is not None:
         d.add_(mat.bias)
 
 
-def _qkv(state: DecodeState, layer: DeviceLayer, h: torch.Tensor, rms_w: torch.Tensor | None = None):
+def _sumsq_handover(weights: DeviceWeights) -> bool:
+    """Whether the folded step hands the sum of squares of the residual stream from the launch
+    that writes it (prologue, o projection, down projection) to the launch that normalises it
+    (q/k/v, gate/up, lm_head), which then skips its own sum over the workgroup (two barriers
+    ahead of its first product: 0.7 us of a 7 us launch).  Every writer must be the last to
+    touch the stream (no separate bias add) and run on the kernel that leaves the sum.
+    ``CHR_DV2_SUMSQ=0`` keeps every launch summing for itself."""
+    if os.environ.get("CHR_DV2_SUMSQ", "1") == "0":
+        return False
+    shapes = getattr(weights, "_sumsq_writers", None)
+    if shapes is None:
+        shapes = set()
+        for layer in weights.layers:
+            for mat, merges in ((layer.o, True), (layer.down, False)):
+                shapes.add((mat.M, mat.K, mat.K_pad, merges, mat.bias is None))
+        weights._sumsq_writers = shapes
+    return all(no_bias and dv2_sumsq_ok(m, k, k_pad, merges) for m, k, k_pad, merges, no_bias in shapes)
+
+
+def _qkv(state: DecodeState, layer: DeviceLayer, h: torch.Tensor, rms_w: torch.Tensor | None = None,
+         sumsq_in: torch.Tensor | None = None):
     """q, k, v of the current token as contiguous ``[heads*hd]`` views; with ``rms_w``
-    the GEMV normalises ``h`` itself."""
+    the GEMV normalises ``h`` itself (from the sum of squares in ``sumsq_in`` when given)."""
     ar = state.arena
     spec = state.spec
     eps = spec.rms_eps
     if layer.wqkv is not None:
         m = layer.wqkv
         nf4_gemv(m.packed, m.scale, h.view(-1), m.M, m.K, m.K_pad, ar.qkv.view(-1),
-                 None if m.bias is None else m.bias, rms_w, eps)
+                 None if m.bias is None else m.bias, rms_w, eps, sumsq_in=sumsq_in)
         flat = ar.qkv.view(-1)
         return (flat[: spec.q_dim], flat[spec.q_dim: spec.q_dim + spec.kv_dim],
                 flat[spec.q_dim + spec.kv_dim:])
     q, k, v = layer.q, layer.k, layer.v
     nf4_qkv(q.packed, q.scale, k.packed, k.scale, v.packed, v.scale, h.view(-1), q.M, k.M, v.M, q.K,
-            q.K_pad, ar.q.view(-1), ar.k.view(-1), ar.v.view(-1), q.bias, k.bias, v.bias, rms_w, eps)
+            q.K_pad, ar.q.view(-1), ar.k.view(-1), ar.v.view(-1), q.bias, k.bias, v.bias, rms_w, eps,
+            sumsq_in=sumsq_in)
     return ar.q.view(-1), ar.k.view(-1), ar.v.view(-1)
 
 
@@ -64,7 +91,8 @@ SCHEDULES = ("plain", "fold_rms")
 DEFAULT_SCHEDULE = "fold_rms"
 
 
-def _attend_into_o(state: DecodeState, li: int, layer: DeviceLayer, q, k, v) -> None:
+def _attend_into_o(state: DecodeState, li: int, layer: DeviceLayer, q, k, v,
+                   sumsq_out: torch.Tensor | None = None) -> None:
     """Attention + o projection + residual as two launches: the attention workgroups (several
     per head, so a head's cache rows stream through several compute units) leave their
     softmax states, and the o GEMV merges them while it stages its activations."""
@@ -77,7 +105,7 @@ def _attend_into_o(state: DecodeState, li: int, layer: DeviceLayer, q, k, v) -> 
                    position=state.position)
     o = layer.o
     d = ar.x.view(-1)
-    dv2_gemv_attn(o.packed, o.scale, ar.attn_state, n_q, hd, o.M, o.K, o.K_pad, d, d)
+    dv2_gemv_attn(o.packed, o.scale, ar.attn_state, n_q, hd, o.M, o.K, o.K_pad, d, d, sumsq_out=sumsq_out)
     if o.bias is not None:
         d.add_(o.bias)
 
@@ -99,38 +127,40 @@ def _forward_calls(state: DecodeState, weights: DeviceWeights, commit: bool, fol
     ar = state.arena
     eps = spec.rms_eps
     emb = weights.embed
+    merge_in_o = fold and spec.head_dim % 8 == 0
+    # sq: the parts buffer when every writer of ar.x leaves its sum of squares for the next reader
+    sq = ar.sumsq if (merge_in_o and isinstance(emb, PackedEmbed) and _sumsq_handover(weights)) else None
     if fold and isinstance(emb, PackedEmbed):
         dv2_begin_step(emb.packed, emb.scale, emb.hidden, state.token, state.position,
-                       state.valid_len, ar.x.view(-1))
+                       state.valid_len, ar.x.view(-1), sumsq_out=sq)
     else:
         gather_embed(emb, state.token.reshape(1), out=ar.x)
         state.kv.mark_written(state.position)
-    merge_in_o = fold and spec.head_dim % 8 == 0
     for li, layer in enumerate(weights.layers):
         if fold:
-            q, k, v = _qkv(state, layer, ar.x, layer.norm1)
+            q, k, v = _qkv(state, layer, ar.x, layer.norm1, sq)
         else:
             nf4_rms(ar.x, layer.norm1, ar.h, eps)
             q, k, v = _qkv(state, layer, ar.h)
         if merge_in_o:
-            _attend_into_o(state, li, layer, q, k, v)
+            _attend_into_o(state, li, layer, q, k, v, sq)
         else:
             _attend(state, li, q, k, v)
             _gemv_accum(layer.o, ar.attn, ar.x)
         g, u = layer.gate, layer.up
         if fold:
             nf4_swiglu(g.packed, g.scale, u.packed, u.scale, ar.x.view(-1), g.M, g.K, g.K_pad,
-                       ar.down_in.view(-1), layer.norm2, eps)
+                       ar.down_in.view(-1), layer.norm2, eps, sumsq_in=sq)
         else:
             nf4_rms(ar.x, layer.norm2, ar.h, eps)
             nf4_swiglu(g.packed, g.scale, u.packed, u.scale, ar.h.view(-1), g.M, g.K, g.K_pad,
                        ar.down_in.view(-1))
-        _gemv_accum(layer.down, ar.down_in, ar.x)
+        _gemv_accum(layer.down, ar.down_in, ar.x, sq)
     head = weights.lm_head
     bias = None if head.bias is None else head.bias
     if fold:
         nf4_gemv(head.packed, head.scale, ar.x.view(-1), head.M, head.K, head.K_pad,
-                 ar.logits.view(-1), bias, weights.final_norm, eps)
+                 ar.logits.view(-1), bias, weights.final_norm, eps, sumsq_in=sq)
     else:
         nf4_rms(ar.x, weights.final_norm, ar.h, eps)
         nf4_gemv(head.packed, head.scale, ar.h.view(-1), head.M, head.K, head.K_pad,

@@ -48,6 +48,8 @@ __all__ = [
     "dv2_attn_state_floats",
     "dv2_attn_parts",
     "dv2_gemv_attn",
+    "dv2_sumsq_ok",
+    "dv2_sumsq_parts",
     "dv2_attn",
     "dv2_rms_cols",
     "dv2_sq_blocks",
@@ -125,6 +127,14 @@ EXPORTS = (
     ("chr_nf4_embed_rows", ctypes.c_int, [_DP, _P, _I, _P, _P]),
     ("chr_nf4_quantize", ctypes.c_int, [_P, _DP, _P, _P]),
     ("chr_dv2_begin_step", ctypes.c_int, [_DP, _P, _P, _P, _P, _P, _F, _P, _P]),
+    ("chr_dv2_begin_step_sumsq", ctypes.c_int, [_DP, _P, _P, _P, _P, _P, _P]),
+    ("chr_dv2_sumsq_parts", ctypes.c_int32, []),
+    ("chr_dv2_sumsq_ok", ctypes.c_int32, [_I, _I, _I, _I]),
+    ("chr_dv2_gemv_sumsq", ctypes.c_int, [_DP, _P, _P, _P, _P, _P, _F, _P, _P]),
+    ("chr_dv2_gemv_qkv_sumsq", ctypes.c_int,
+     [_DP, _DP, _DP, _P, _P, _P, _P, _P, _P, _P, _P, _P, _F, _P]),
+    ("chr_dv2_gemv_swiglu_sumsq", ctypes.c_int, [_DP, _DP, _P, _P, _P, _P, _F, _P]),
+    ("chr_dv2_gemv_attn_sumsq", ctypes.c_int, [_DP, _P, _I, _I, _I, _P, _P, _P, _P]),
     ("chr_dv2_attn", ctypes.c_int,
      [_P, _P, _P, _P, _P, _I, _I, _I, _I, _F, _P, _P, _P, _P, _P, _P, _I]),
     ("chr_dv2_attn_state_floats", ctypes.c_int64, [_I, _I, _I]),
@@ -187,6 +197,7 @@ _ERR = {
     -5: "packed or x not 16-byte aligned",
     -6: "HIP launch / func attribute failed",
     -7: "split-K workspace smaller than the plan asked for",
+    -8: "this launch cannot serve the sum-of-squares hand-over asked for",
 }
 
 
@@ -364,15 +375,42 @@ def dv2_sq_blocks(rows: int, n: int) -> int:
     return -(-int(rows) // per) if per > 0 else 0
 
 
+def dv2_sumsq_parts() -> int:
+    """Floats of a sum-of-squares hand-over buffer (``sumsq_in`` / ``sumsq_out`` below)."""
+    return int(_load_ext().chr_dv2_sumsq_parts())
+
+
+def dv2_sumsq_ok(M: int, K: int, K_pad: int, merges_attention: bool = False) -> bool:  # noqa: N803
+    """Whether a single-matrix GEMV of this shape runs on the kernel that can write
+    ``sumsq_out`` (it reads the environment switches a launch reads)."""
+    return bool(_load_ext().chr_dv2_sumsq_ok(int(M), int(K), int(K_pad), int(bool(merges_attention))))
+
+
+def _opt_sumsq(t: torch.Tensor | None, what: str):
+    """Device pointer of a sum-of-squares hand-over buffer, or None."""
+    if t is None:
+        return None
+    _need(t.is_cuda and t.dtype == torch.float32 and t.is_contiguous()
+          and t.numel() >= dv2_sumsq_parts() and t.data_ptr() % 16 == 0,
+          f"{what} must be a contiguous, 16-byte aligned CUDA float32 tensor of dv2_sumsq_parts() elements")
+    return t.data_ptr()
+
+
 def nf4_gemv(packed: torch.Tensor, scale: torch.Tensor, x: torch.Tensor, M: int, K: int,  # noqa: N803
              K_pad: int, out: torch.Tensor | None = None, add: torch.Tensor | None = None,  # noqa: N803
-             rms_w: torch.Tensor | None = None, rms_eps: float = 1e-6) -> torch.Tensor:
+             rms_w: torch.Tensor | None = None, rms_eps: float = 1e-6,
+             sumsq_in: torch.Tensor | None = None, sumsq_out: torch.Tensor | None = None) -> torch.Tensor:
     """N=1 GEMV.  ``x`` is bf16 ``[K, 1]`` or ``[K]``; ``y`` is ``[M, 1]``.
 
     Optional ``out`` is the destination (numel >= M).  Optional ``add`` is a
     residual of numel >= M; ``out`` and ``add`` may alias.  Optional ``rms_w``
     applies RMSNorm(x, rms_w, rms_eps) in the same launch
-    (``gpu/nf4/__init__.py:179-206``, ``bindings.cpp:127-204``)."""
+    (``gpu/nf4/__init__.py:179-206``, ``bindings.cpp:127-204``).
+
+    ``sumsq_out``: the launch also leaves the sum of squares of what it stored, in parts, for
+    the launch that normalises ``y``; ``sumsq_in`` (with ``rms_w``): mean(x^2) comes from the
+    parts the writer of ``x`` left instead of a sum over ``x`` (``chr_dv2_gemv_sumsq``; no
+    reference counterpart)."""
     n = 1 if x.dim() == 1 else int(x.size(-1))
     if n != 1:
         raise RuntimeError(f"chr_nf4_gemv is N=1 only, got N={n}")
@@ -398,18 +436,25 @@ def nf4_gemv(packed: torch.Tensor, scale: torch.Tensor, x: torch.Tensor, M: int,
     add_keep, add_ptr = _opt_bf16(add, M, "add", exact=False)
     rms_keep, rms_ptr = _opt_bf16(rms_w, K, "rms_w", exact=True)
     w = _dev(packed, scale, M, K, K_pad)
-    rc = _load_ext().chr_nf4_gemv(ctypes.byref(w), x.data_ptr(), y.data_ptr(), _stream(), add_ptr,
-                                  rms_ptr, float(rms_eps))
-    _check_rc("chr_nf4_gemv", rc)
+    if sumsq_in is None and sumsq_out is None:
+        rc = _load_ext().chr_nf4_gemv(ctypes.byref(w), x.data_ptr(), y.data_ptr(), _stream(), add_ptr,
+                                      rms_ptr, float(rms_eps))
+        _check_rc("chr_nf4_gemv", rc)
+    else:
+        rc = _load_ext().chr_dv2_gemv_sumsq(ctypes.byref(w), x.data_ptr(), y.data_ptr(), _stream(),
+                                            add_ptr, rms_ptr, float(rms_eps),
+                                            _opt_sumsq(sumsq_in, "sumsq_in"),
+                                            _opt_sumsq(sumsq_out, "sumsq_out"))
+        _check_rc("chr_dv2_gemv_sumsq", rc)
     del add_keep, rms_keep
     return y
 
 
 def nf4_qkv(q_packed, q_scale, k_packed, k_scale, v_packed, v_scale, x, Mq: int, Mk: int,  # noqa: N803
             Mv: int, K: int, K_pad: int, out_q, out_k, out_v, q_bias=None, k_bias=None,  # noqa: N803
-            v_bias=None, rms_w=None, rms_eps: float = 1e-6):
+            v_bias=None, rms_w=None, rms_eps: float = 1e-6, sumsq_in=None):
     """One launch: q/k/v GEMVs sharing x.  Writes ``out_*`` (numel >= M)
-    (``gpu/nf4/__init__.py:209-257``, ``bindings.cpp:281-324``)."""
+    (``gpu/nf4/__init__.py:209-257``, ``bindings.cpp:281-324``).  ``sumsq_in``: see ``nf4_gemv``."""
     Mq, Mk, Mv, K, K_pad = int(Mq), int(Mk), int(Mv), int(K), int(K_pad)
     _check_packed(q_packed, q_scale, Mq, K, K_pad, "q")
     _check_packed(k_packed, k_scale, Mk, K, K_pad, "k")
@@ -427,18 +472,25 @@ def nf4_qkv(q_packed, q_scale, k_packed, k_scale, v_packed, v_scale, x, Mq: int,
     q = _dev(q_packed, q_scale, Mq, K, K_pad)
     k = _dev(k_packed, k_scale, Mk, K, K_pad)
     v = _dev(v_packed, v_scale, Mv, K, K_pad)
-    rc = _load_ext().chr_nf4_gemv_qkv(ctypes.byref(q), ctypes.byref(k), ctypes.byref(v),
-                                      x.data_ptr(), yq.data_ptr(), yk.data_ptr(), yv.data_ptr(),
-                                      bq, bk, bv, _stream(), rms_ptr, float(rms_eps))
-    _check_rc("chr_nf4_gemv_qkv", rc)
+    if sumsq_in is None:
+        rc = _load_ext().chr_nf4_gemv_qkv(ctypes.byref(q), ctypes.byref(k), ctypes.byref(v),
+                                          x.data_ptr(), yq.data_ptr(), yk.data_ptr(), yv.data_ptr(),
+                                          bq, bk, bv, _stream(), rms_ptr, float(rms_eps))
+        _check_rc("chr_nf4_gemv_qkv", rc)
+    else:
+        rc = _load_ext().chr_dv2_gemv_qkv_sumsq(ctypes.byref(q), ctypes.byref(k), ctypes.byref(v),
+                                                x.data_ptr(), yq.data_ptr(), yk.data_ptr(),
+                                                yv.data_ptr(), bq, bk, bv, _stream(), rms_ptr,
+                                                float(rms_eps), _opt_sumsq(sumsq_in, "sumsq_in"))
+        _check_rc("chr_dv2_gemv_qkv_sumsq", rc)
     del qb_keep, kb_keep, vb_keep, rms_keep
     return (yq, yk, yv)
 
 
 def nf4_swiglu(g_packed, g_scale, u_packed, u_scale, x, M: int, K: int, K_pad: int, out,  # noqa: N803
-               rms_w=None, rms_eps: float = 1e-6) -> torch.Tensor:
+               rms_w=None, rms_eps: float = 1e-6, sumsq_in=None) -> torch.Tensor:
     """One launch: ``silu(gate @ x) * (up @ x)`` into ``out``
-    (``gpu/nf4/__init__.py:260-287``, ``bindings.cpp:326-354``)."""
+    (``gpu/nf4/__init__.py:260-287``, ``bindings.cpp:326-354``).  ``sumsq_in``: see ``nf4_gemv``."""
     M, K, K_pad = int(M), int(K), int(K_pad)
     _check_packed(g_packed, g_scale, M, K, K_pad, "gate")
     _check_packed(u_packed, u_scale, M, K, K_pad, "up")
@@ -450,9 +502,15 @@ def nf4_swiglu(g_packed, g_scale, u_packed, u_scale, x, M: int, K: int, K_pad: i
     rms_keep, rms_ptr = _opt_bf16(rms_w, K, "rms_w", exact=True)
     g = _dev(g_packed, g_scale, M, K, K_pad)
     u = _dev(u_packed, u_scale, M, K, K_pad)
-    rc = _load_ext().chr_nf4_gemv_swiglu(ctypes.byref(g), ctypes.byref(u), x.data_ptr(),
-                                         y.data_ptr(), _stream(), rms_ptr, float(rms_eps))
-    _check_rc("chr_nf4_gemv_swiglu", rc)
+    if sumsq_in is None:
+        rc = _load_ext().chr_nf4_gemv_swiglu(ctypes.byref(g), ctypes.byref(u), x.data_ptr(),
+                                             y.data_ptr(), _stream(), rms_ptr, float(rms_eps))
+        _check_rc("chr_nf4_gemv_swiglu", rc)
+    else:
+        rc = _load_ext().chr_dv2_gemv_swiglu_sumsq(ctypes.byref(g), ctypes.byref(u), x.data_ptr(),
+                                                   y.data_ptr(), _stream(), rms_ptr, float(rms_eps),
+                                                   _opt_sumsq(sumsq_in, "sumsq_in"))
+        _check_rc("chr_dv2_gemv_swiglu_sumsq", rc)
     del rms_keep
     return y
 
@@ -687,9 +745,10 @@ def dv2_argmax_ws_bytes() -> int:
 def dv2_begin_step(packed: torch.Tensor, scale: torch.Tensor, K: int, token: torch.Tensor,  # noqa: N803
                    position: torch.Tensor, valid_len: torch.Tensor, x: torch.Tensor,
                    norm_w: torch.Tensor | None = None, eps: float = 1e-6,
-                   h: torch.Tensor | None = None) -> None:
+                   h: torch.Tensor | None = None, sumsq_out: torch.Tensor | None = None) -> None:
     """First launch of a decode step: ``valid_len = position + 1``, ``x`` = the packed
-    embedding row ``token`` and, with ``norm_w``, ``h = RMSNorm(x, norm_w, eps)``."""
+    embedding row ``token`` and, with ``norm_w``, ``h = RMSNorm(x, norm_w, eps)``; with
+    ``sumsq_out`` (and no ``norm_w``) the sum of squares of ``x`` in parts, see ``nf4_gemv``."""
     M, K, K_pad = int(packed.size(0)), int(K), int(packed.size(1)) * 2
     _check_packed(packed, scale, M, K, K_pad, "embed")
     _need(packed.is_contiguous() and scale.is_contiguous(), "embed blobs must be contiguous")
@@ -701,6 +760,13 @@ def dv2_begin_step(packed: torch.Tensor, scale: torch.Tensor, K: int, token: tor
         _need(t is None or (t.is_cuda and t.dtype == torch.bfloat16 and t.is_contiguous()
                             and t.numel() == K), f"{name} must be contiguous CUDA bf16 with K elements")
     w = _dev(packed, scale, M, K, K_pad)
+    if sumsq_out is not None:
+        _need(norm_w is None, "sumsq_out goes without norm_w")
+        rc = _load_ext().chr_dv2_begin_step_sumsq(ctypes.byref(w), token.data_ptr(), position.data_ptr(),
+                                                  valid_len.data_ptr(), x.data_ptr(), _stream(),
+                                                  _opt_sumsq(sumsq_out, "sumsq_out"))
+        _check_rc("chr_dv2_begin_step_sumsq", rc)
+        return
     rc = _load_ext().chr_dv2_begin_step(ctypes.byref(w), token.data_ptr(), position.data_ptr(),
                                         valid_len.data_ptr(), x.data_ptr(),
                                         None if norm_w is None else norm_w.data_ptr(), float(eps),
@@ -777,9 +843,10 @@ def dv2_attn_parts(q, k, v, valid_len, scale: float, state, n_parts: int = ATTN_
 
 def dv2_gemv_attn(packed: torch.Tensor, scale: torch.Tensor, state: torch.Tensor, n_q: int, hd: int,
                   M: int, K: int, K_pad: int, out: torch.Tensor, add: torch.Tensor | None = None,  # noqa: N803
-                  n_parts: int = ATTN_PARTS) -> torch.Tensor:
+                  n_parts: int = ATTN_PARTS, sumsq_out: torch.Tensor | None = None) -> torch.Tensor:
     """``out = W @ merge(state) (+ add)``: the o projection that also merges the softmax
-    states of ``dv2_attn_parts``.  ``K == n_q * hd`` and a multiple of 64; ``hd % 8 == 0``."""
+    states of ``dv2_attn_parts``.  ``K == n_q * hd`` and a multiple of 64; ``hd % 8 == 0``.
+    ``sumsq_out``: see ``nf4_gemv``."""
     M, K, K_pad = int(M), int(K), int(K_pad)
     _check_packed(packed, scale, M, K, K_pad)
     _need(packed.is_contiguous() and scale.is_contiguous(), "blobs must be contiguous")
@@ -791,10 +858,17 @@ def dv2_gemv_attn(packed: torch.Tensor, scale: torch.Tensor, state: torch.Tensor
         _need(t is None or (t.is_cuda and t.dtype == torch.bfloat16 and t.is_contiguous()
                             and t.numel() >= M), f"{name} must be contiguous CUDA bf16 with M elements")
     w = _dev(packed, scale, M, K, K_pad)
-    rc = _load_ext().chr_dv2_gemv_attn(ctypes.byref(w), state.data_ptr(), int(n_q), int(hd),
-                                       int(n_parts), out.data_ptr(),
-                                       None if add is None else add.data_ptr(), _stream())
-    _check_rc("chr_dv2_gemv_attn", rc)
+    if sumsq_out is None:
+        rc = _load_ext().chr_dv2_gemv_attn(ctypes.byref(w), state.data_ptr(), int(n_q), int(hd),
+                                           int(n_parts), out.data_ptr(),
+                                           None if add is None else add.data_ptr(), _stream())
+        _check_rc("chr_dv2_gemv_attn", rc)
+    else:
+        rc = _load_ext().chr_dv2_gemv_attn_sumsq(ctypes.byref(w), state.data_ptr(), int(n_q), int(hd),
+                                                 int(n_parts), out.data_ptr(),
+                                                 None if add is None else add.data_ptr(), _stream(),
+                                                 _opt_sumsq(sumsq_out, "sumsq_out"))
+        _check_rc("chr_dv2_gemv_attn_sumsq", rc)
     return out
 
 

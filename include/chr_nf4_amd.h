@@ -15,6 +15,7 @@
  *       -2 N out of range             (scale not 2-byte aligned)
  *       -3 bad dims / null blobs   -6 launch failure
  *       -4 K_pad != 64*ceil(K/64)  -7 split-K workspace too small
+ *       -8 a sum-of-squares hand-over (chr_dv2_*_sumsq) this launch cannot serve
  *     (chr_gpu.h:30-33; gpu/nf4/nf4_gemm.cu:1621-1644, 1683-1698)
  *
  * Naming follows the reference: M = out features, K = in features,
@@ -254,6 +255,44 @@ int chr_dv2_attn_parts(const void *q, const void *k, const void *v, const void *
                        const void *position, int32_t max_seq);
 int chr_dv2_gemv_attn(const chr_nf4_dev_t *w, const float *state, int32_t n_q, int32_t hd,
                       int32_t n_parts, void *y, const void *add, void *stream);
+
+/* The sum of squares of a vector handed from the launch that writes it to the launch that
+ * normalises it, for a decode step that folds every RMSNorm into the GEMV that consumes it
+ * (the rms_w argument of chr_nf4_gemv, gpu/nf4/nf4_gemv.cu:264-289): with rms_w alone the
+ * consuming launch sums x^2 over its workgroup, two barriers between x arriving and the first
+ * product (0.7 us of a 7 us launch); here the writer, which has every element in hand as it
+ * stores it, leaves the sum in chr_dv2_sumsq_parts() floats (its workgroups' sums over the bf16
+ * values they stored, in a fixed order, zeros behind them: a 16-byte aligned buffer of that
+ * many floats, the caller's), and the reader's wavefronts add the parts up themselves.  No
+ * reference counterpart.
+ *   sumsq_out (chr_dv2_gemv_sumsq, chr_dv2_gemv_attn_sumsq, chr_dv2_begin_step_sumsq): this
+ *     launch writes the parts for its y (after `add`).  Only the GEMV kernel of single rows
+ *     does: chr_dv2_sumsq_ok(M, K, K_pad, merges_attention) says whether a matrix of that shape
+ *     runs on it (it reads the same environment switches a launch reads); else -8.
+ *   sumsq_in (chr_dv2_gemv_sumsq, chr_dv2_gemv_qkv_sumsq, chr_dv2_gemv_swiglu_sumsq): with
+ *     rms_w, mean(x^2) comes from the parts that the writer of x left.  Needs K % 8 == 0 and
+ *     x, rms_w and the parts 16-byte aligned; else -8.  The parts must be those of this x:
+ *     nothing checks it.
+ * Either pointer NULL: the entry behaves as the one it extends.  The values differ from the
+ * reader's own sum by the order of the additions only. */
+int32_t chr_dv2_sumsq_parts(void);
+int32_t chr_dv2_sumsq_ok(int32_t M, int32_t K, int32_t K_pad, int32_t merges_attention);
+int chr_dv2_gemv_sumsq(const chr_nf4_dev_t *w, const void *x, void *y, void *stream,
+                       const void *add, const void *rms_w, float rms_eps, const float *sumsq_in,
+                       float *sumsq_out);
+int chr_dv2_gemv_qkv_sumsq(const chr_nf4_dev_t *q, const chr_nf4_dev_t *k, const chr_nf4_dev_t *v,
+                           const void *x, void *yq, void *yk, void *yv, const void *bq,
+                           const void *bk, const void *bv, void *stream, const void *rms_w,
+                           float rms_eps, const float *sumsq_in);
+int chr_dv2_gemv_swiglu_sumsq(const chr_nf4_dev_t *gate, const chr_nf4_dev_t *up, const void *x,
+                              void *y, void *stream, const void *rms_w, float rms_eps,
+                              const float *sumsq_in);
+int chr_dv2_gemv_attn_sumsq(const chr_nf4_dev_t *w, const float *state, int32_t n_q, int32_t hd,
+                            int32_t n_parts, void *y, const void *add, void *stream,
+                            float *sumsq_out);
+/* chr_dv2_begin_step without its RMSNorm, leaving the parts for the first layer's q/k/v. */
+int chr_dv2_begin_step_sumsq(const chr_nf4_dev_t *table, const void *token, const void *position,
+                             void *valid_len, void *x, void *stream, float *sumsq_out);
 
 /* ---- Chunked prefill glue on the GEMM's own layout -----------------------------------------
  * The reference's prefill (gpu/decodev2/prefill.py:58-133) runs everything but its linears as

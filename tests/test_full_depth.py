@@ -16,6 +16,7 @@ import pytest
 import torch
 
 from deepfold_amd import decodev2 as dv2
+from deepfold_amd.decodev2 import step as step_mod
 
 pytestmark = pytest.mark.gpu
 
@@ -35,7 +36,7 @@ def say(*a):
 
 
 @pytest.mark.parametrize("name,spec,prompt_len,width", CONFIGS, ids=[c[0] for c in CONFIGS])
-def test_full_depth_decode(name, spec, prompt_len, width):
+def test_full_depth_decode(name, spec, prompt_len, width, monkeypatch):
     say("full depth", name, spec.n_layers, "layers, prompt", prompt_len, "chunks of", width or 64)
     weights = dv2.DeviceWeights.random(spec, seed=2027)
     state = dv2.DecodeState.allocate(spec, device="cuda")
@@ -98,5 +99,24 @@ def test_full_depth_decode(name, spec, prompt_len, width):
         state.token.fill_(eager[i])   # stay on the folded schedule's stream
     say(f"  {name}: graph == eager over {N_NEW} steps; plain against folded schedule: worst logit "
         f"difference {worst:.3f}, bound {bound:.3f} (logit scale {scale:.2f})")
+
+    # the folded schedule with every launch summing x^2 for itself instead of taking the sum from
+    # the launch that wrote x (the hand-over is taken where the model's shapes allow it: not at
+    # the 3B model's rows of 2048): the same statistic added in another order, so a few of the
+    # normalised activations round the other way and the logits drift as they do between the
+    # two schedules above
+    assert step_mod._sumsq_handover(weights) == (name != "3b")
+    monkeypatch.setenv("CHR_DV2_SUMSQ", "0")
+    assert not step_mod._sumsq_handover(weights)
+    assert prefill() == first
+    worst = 0.0
+    for i in range(N_NEW):
+        dv2.greedy_decode(state, weights)
+        diff = float((state.arena.logits.float() - eager_logits[i].float()).abs().max())
+        worst = max(worst, diff)
+        assert diff <= (0.0 if name == "3b" else bound + 1e-3), (name, i, diff, bound, scale)
+        state.token.fill_(eager[i])
+    say(f"  {name}: without the sum-of-squares hand-over: worst logit difference {worst:.3f}")
+    monkeypatch.delenv("CHR_DV2_SUMSQ")
     del graph, pre, state, weights
     torch.cuda.empty_cache()

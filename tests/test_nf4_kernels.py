@@ -613,6 +613,169 @@ def test_ring_swiglu(m, k, terms, monkeypatch):
     assert (bf16_bits(out) == bf16_bits(out2)).all()
 
 
+# ------------------------------------ sum of squares handed from a vector's writer to its reader
+def gpu_blobs(m, k, seed):
+    """Quantised N(0, 0.02) weights made on the GPU (shapes too large for the toy blobs)."""
+    g = torch.Generator(device=DEV)
+    g.manual_seed(seed)
+    w = torch.randn((m, k), generator=g, device=DEV, dtype=torch.float32) * 0.02
+    return nf4.nf4_quantize(w)
+
+
+def parts_of(y, grid):
+    """What the writer leaves: workgroup b sums the squares of rows b, b + grid, ..."""
+    sq = to_f32(y).reshape(-1).astype(np.float64) ** 2
+    parts = np.zeros(nf4.dv2_sumsq_parts())
+    for b in range(min(grid, sq.size)):
+        parts[b] = sq[b::grid].sum()
+    return parts
+
+
+@pytest.mark.parametrize("terms", [1, 3])
+@pytest.mark.parametrize("m,k,merges", [(5120, 13824, False), (5120, 5120, True), (2100, 8192, False),
+                                        (6144, 16384, False), (1040, 27648, False)])
+def test_gemv_leaves_the_sum_of_squares_of_what_it_stored(m, k, merges, terms, monkeypatch):
+    """``sumsq_out``: the same y, bit for bit, and in the parts buffer the squares of the stored
+    bf16 values, workgroup by workgroup, zeros behind them (whatever the buffer held before)."""
+    say("sumsq writer", m, k, merges, terms)
+    monkeypatch.setenv("CHR_NF4_GEMV_TERMS", str(terms))
+    assert nf4.dv2_sumsq_ok(m, k, k, merges)
+    dp, ds = gpu_blobs(m, k, 71)
+    res = bf16_tensor(np.random.default_rng(3).standard_normal(m).astype(np.float32))
+    n_parts = nf4.dv2_sumsq_parts()
+    grid = min(torch.cuda.get_device_properties(0).multi_processor_count, -(-m // 16))
+    for rep in range(2):
+        parts = torch.full((n_parts,), float("nan"), dtype=torch.float32, device=DEV)
+        y0 = torch.empty(m, dtype=torch.bfloat16, device=DEV)
+        y1 = torch.empty(m, dtype=torch.bfloat16, device=DEV)
+        if merges:
+            n_q, hd = k // 128, 128
+            st = torch.randn(nf4.dv2_attn_state_floats(n_q, hd), device=DEV).abs()
+            nf4.dv2_gemv_attn(dp, ds, st, n_q, hd, m, k, k, y0, res)
+            nf4.dv2_gemv_attn(dp, ds, st, n_q, hd, m, k, k, y1, res, sumsq_out=parts)
+        else:
+            x = bf16_tensor(rand_x(k, None, 5 + rep))
+            nf4.nf4_gemv(dp, ds, x, m, k, k, y0, res)
+            nf4.nf4_gemv(dp, ds, x, m, k, k, y1, res, sumsq_out=parts)
+        assert (bf16_bits(y0) == bf16_bits(y1)).all()
+        got = parts.cpu().numpy().astype(np.float64)
+        want = parts_of(y1, grid)
+        assert np.isfinite(got).all() and (got[grid:] == 0).all()
+        assert np.abs(got - want).max() <= 1e-5 * want.max(), (rep, np.abs(got - want).max(), want.max())
+
+
+def test_sumsq_hand_over_is_refused_where_no_kernel_serves_it(monkeypatch):
+    """A shape the single-row ring kernel does not take (too few codes: the plain kernel; rows of
+    2 half steps), a reader without a norm, the ring switched off: error -8, nothing launched."""
+    parts = torch.zeros(nf4.dv2_sumsq_parts(), dtype=torch.float32, device=DEV)
+    for m, k in [(300, 7168), (4096, 2048)]:
+        assert not nf4.dv2_sumsq_ok(m, k, k)
+        dp, ds = gpu_blobs(m, k, 72)
+        x = bf16_tensor(rand_x(k, None, 6))
+        with pytest.raises(RuntimeError, match="-8"):
+            nf4.nf4_gemv(dp, ds, x, m, k, k, sumsq_out=parts)
+        with pytest.raises(RuntimeError, match="-8"):
+            nf4.nf4_gemv(dp, ds, x, m, k, k, sumsq_in=parts)          # no rms_w
+    m, k = 5120, 5120
+    dp, ds = gpu_blobs(m, k, 73)
+    x = bf16_tensor(rand_x(k, None, 7))
+    assert nf4.dv2_sumsq_ok(m, k, k)
+    monkeypatch.setenv("CHR_NF4_GEMV_RING", "0")
+    assert not nf4.dv2_sumsq_ok(m, k, k)
+    with pytest.raises(RuntimeError, match="-8"):
+        nf4.nf4_gemv(dp, ds, x, m, k, k, sumsq_out=parts)
+    with pytest.raises(RuntimeError):
+        nf4.nf4_gemv(dp, ds, x, m, k, k, sumsq_in=parts[1:])            # not 16-byte aligned, too short
+
+
+@pytest.mark.parametrize("ring", ["1", "0"])
+@pytest.mark.parametrize("terms", [1, 3])
+@pytest.mark.parametrize("k", [5120, 6144, 2048])
+def test_norm_folded_into_a_gemv_takes_the_sum_of_squares_it_is_handed(k, terms, ring, monkeypatch):
+    """``sumsq_in``: q/k/v, gate/up and a single matrix normalise x with the sum the parts hold
+    instead of summing x: with the parts of x itself the result is the launch's own to the last
+    bf16 step of a few elements (another order of the same additions); with four times those
+    parts it is the result for x / 2: the parts are what is used."""
+    say("sumsq reader", k, terms, ring)
+    monkeypatch.setenv("CHR_NF4_GEMV_TERMS", str(terms))
+    monkeypatch.setenv("CHR_NF4_GEMV_RING", ring)
+    monkeypatch.setenv("CHR_NF4_GEMV_STAGED", "1")
+    rng = np.random.default_rng(k)
+    xh = oc.bf16_round(rng.standard_normal(k).astype(np.float32) * 3)
+    x = bf16_tensor(xh)
+    g = bf16_tensor(oc.bf16_round(1 + 0.1 * rng.standard_normal(k).astype(np.float32)))
+    n_parts = nf4.dv2_sumsq_parts()
+    sq = xh.astype(np.float64) ** 2
+    own = np.zeros(n_parts)
+    for b in range(n_parts):
+        own[b] = sq[b::n_parts].sum()
+    parts = torch.tensor(own, dtype=torch.float32, device=DEV)
+    m = 4100
+    dp, ds = gpu_blobs(m, k, 74)
+    mq, mk = 2048, 512
+    dq, sq_ = gpu_blobs(mq, k, 75)
+    dk, sk = gpu_blobs(mk, k, 76)
+    dv, sv = gpu_blobs(mk, k, 77)
+    bias = [bf16_tensor(rng.standard_normal(n).astype(np.float32)) for n in (mq, mk, mk)]
+
+    def run(p):
+        kw = {} if p is None else {"sumsq_in": p}
+        y = nf4.nf4_gemv(dp, ds, x, m, k, k, rms_w=g, **kw).reshape(-1).clone()
+        o = [torch.empty(n, dtype=torch.bfloat16, device=DEV) for n in (mq, mk, mk)]
+        nf4.nf4_qkv(dq, sq_, dk, sk, dv, sv, x, mq, mk, mk, k, k, *o, *bias, rms_w=g, **kw)
+        s = torch.empty(mq, dtype=torch.bfloat16, device=DEV)
+        nf4.nf4_swiglu(dq, sq_, dp[:mq], ds[:mq], x, mq, k, k, s, rms_w=g, **kw)
+        return [y, *o, s]
+
+    base, handed, scaled = run(None), run(parts), run(parts * 4)
+    for a, b, c in zip(base, handed, scaled):
+        fa, fb, fc = to_f32(a).reshape(-1), to_f32(b).reshape(-1), to_f32(c).reshape(-1)
+        lim = 2.0 ** -7 * np.maximum(np.abs(fa), 2.0 ** -6 * np.abs(fa).max())
+        assert (np.abs(fa - fb) <= lim).all(), np.abs(fa - fb).max()
+        assert (bf16_bits(a) != bf16_bits(b)).mean() <= 0.02
+        # x / 2 (no bias rows only: the single matrix and the SwiGLU's gate * up ~ 1/4 .. 1/2)
+    y, y4 = to_f32(base[0]).reshape(-1), to_f32(scaled[0]).reshape(-1)
+    assert np.abs(y4 - 0.5 * y).max() <= 2.0 ** -6 * np.abs(y).max()
+
+
+def test_sum_of_squares_from_the_writer_to_the_reader(monkeypatch):
+    """The hand-over as the decode step uses it, at the 14B shapes: the down projection (residual
+    added) leaves the parts, gate/up of the next layer normalises with them; the prologue leaves
+    them for the first q/k/v.  Against the reader summing for itself."""
+    k5, ffn = 5120, 13824
+    dd, sd = gpu_blobs(k5, ffn, 81)
+    dg, sg = gpu_blobs(4096, k5, 82)
+    du, su = gpu_blobs(4096, k5, 83)
+    rng = np.random.default_rng(9)
+    xin = bf16_tensor(rand_x(ffn, None, 10))
+    res = bf16_tensor(rng.standard_normal(k5).astype(np.float32))
+    g = bf16_tensor(oc.bf16_round(1 + 0.1 * rng.standard_normal(k5).astype(np.float32)))
+    parts = torch.zeros(nf4.dv2_sumsq_parts(), dtype=torch.float32, device=DEV)
+    h = torch.empty(k5, dtype=torch.bfloat16, device=DEV)
+    nf4.nf4_gemv(dd, sd, xin, k5, ffn, ffn, h, res, sumsq_out=parts)
+    assert abs(float(parts.double().sum()) - float((h.double() ** 2).sum())) <= 1e-5 * float((h.double() ** 2).sum())
+    a = torch.empty(4096, dtype=torch.bfloat16, device=DEV)
+    b = torch.empty(4096, dtype=torch.bfloat16, device=DEV)
+    nf4.nf4_swiglu(dg, sg, du, su, h, 4096, k5, k5, a, rms_w=g)
+    nf4.nf4_swiglu(dg, sg, du, su, h, 4096, k5, k5, b, rms_w=g, sumsq_in=parts)
+    fa, fb = to_f32(a).reshape(-1), to_f32(b).reshape(-1)
+    assert (np.abs(fa - fb) <= 2.0 ** -7 * np.maximum(np.abs(fa), 2.0 ** -6 * np.abs(fa).max())).all()
+    # the prologue: the embedding row and its sum of squares
+    emb_p, emb_s = gpu_blobs(1000, k5, 84)
+    tok = torch.tensor(123, dtype=torch.int64, device=DEV)
+    pos = torch.tensor(17, dtype=torch.int64, device=DEV)
+    vl0 = torch.zeros((), dtype=torch.int32, device=DEV)
+    vl1 = torch.zeros((), dtype=torch.int32, device=DEV)
+    x0 = torch.empty(k5, dtype=torch.bfloat16, device=DEV)
+    x1 = torch.empty(k5, dtype=torch.bfloat16, device=DEV)
+    parts.fill_(float("nan"))
+    nf4.dv2_begin_step(emb_p, emb_s, k5, tok, pos, vl0, x0)
+    nf4.dv2_begin_step(emb_p, emb_s, k5, tok, pos, vl1, x1, sumsq_out=parts)
+    assert torch.equal(x0, x1) and int(vl0) == int(vl1) == 18
+    want = float((x1.double() ** 2).sum())
+    assert abs(float(parts.double().sum()) - want) <= 1e-5 * want and float(parts[16:].abs().max()) == 0.0
+
+
 # ------------------------------------------------------------------------ RMS
 @pytest.mark.parametrize("n", [64, 2048, 5120, 6144, 100])
 def test_rms(n):
