@@ -224,7 +224,9 @@ def bench_layer_launches(torch, nf4, contexts=(640, 2047)):
     """The five launches of one 14B-architecture decode layer, each on its own (graph replays,
     rotating weights and caches): q/k/v with the folded RMSNorm and biases, the attention at the
     given cache lengths, the o projection that merges the attention's states and adds the
-    residual, gate/up with the folded RMSNorm and SwiGLU, down with the residual."""
+    residual, gate/up with the folded RMSNorm and SwiGLU, down with the residual.  As in the
+    step, the two launches that write the residual stream leave its sum of squares and the two
+    that normalise it take it from there."""
     from deepfold_amd.decodev2.rope import rope_tables_torch
 
     k5, ffn, n_q, n_kv, hd, max_seq = 5120, 13824, 40, 8, 128, 2048
@@ -233,6 +235,8 @@ def bench_layer_launches(torch, nf4, contexts=(640, 2047)):
     x = torch.randn(k5, device=dev).to(torch.bfloat16)
     g = (1 + 0.05 * torch.randn(k5, device=dev)).to(torch.bfloat16)
     res = torch.randn(k5, device=dev).to(torch.bfloat16)
+    parts = torch.zeros(nf4.dv2_sumsq_parts(), dtype=torch.float32, device=dev)
+    parts[0] = float((x.float() ** 2).sum())
 
     def add(name, launch, nbytes, n=120):
         ms = graph_time(torch, launch, n)
@@ -251,7 +255,7 @@ def bench_layer_launches(torch, nf4, contexts=(640, 2047)):
     def qkv(i):
         j = i % c
         nf4.nf4_qkv(q[j][0], q[j][1], kk[j][0], kk[j][1], v[j][0], v[j][1], x, n_q * hd, n_kv * hd, n_kv * hd,
-                    k5, k5, yq, yk, yv, bq, bk, bv, rms_w=g)
+                    k5, k5, yq, yk, yv, bq, bk, bv, rms_w=g, sumsq_in=parts)
 
     add("q/k/v 7168x5120 + RMSNorm + biases", qkv, algorithmic_bytes((n_q + 2 * n_kv) * hd, k5))
     del q, kk, v
@@ -282,8 +286,10 @@ def bench_layer_launches(torch, nf4, contexts=(640, 2047)):
     o = make_weights(torch, nf4, k5, k5, 40, 5)
     yo = torch.empty(k5, dtype=torch.bfloat16, device=dev)
     st = torch.randn(nf4.dv2_attn_state_floats(n_q, hd), device=dev).abs()
+    parts_out = torch.zeros_like(parts)
     add("o 5120x5120 + attention merge + residual",
-        lambda i: nf4.dv2_gemv_attn(o[i % 40][0], o[i % 40][1], st, n_q, hd, k5, k5, k5, yo, res),
+        lambda i: nf4.dv2_gemv_attn(o[i % 40][0], o[i % 40][1], st, n_q, hd, k5, k5, k5, yo, res,
+                                    sumsq_out=parts_out),
         algorithmic_bytes(k5, k5) + st.numel() * 4)
     del o
     torch.cuda.empty_cache()
@@ -293,7 +299,7 @@ def bench_layer_launches(torch, nf4, contexts=(640, 2047)):
     ys = torch.empty(ffn, dtype=torch.bfloat16, device=dev)
     add("gate/up 2 x 13824x5120 + RMSNorm + SwiGLU",
         lambda i: nf4.nf4_swiglu(ga[i % 10][0], ga[i % 10][1], up[i % 10][0], up[i % 10][1], x, ffn, k5, k5, ys,
-                                 rms_w=g),
+                                 rms_w=g, sumsq_in=parts),
         2 * algorithmic_bytes(ffn, k5) - 2 * k5 - 2 * ffn)
     del ga, up
     torch.cuda.empty_cache()
@@ -301,7 +307,7 @@ def bench_layer_launches(torch, nf4, contexts=(640, 2047)):
     d = make_weights(torch, nf4, k5, ffn, 18, 8)
     xd = torch.randn(ffn, device=dev).to(torch.bfloat16)
     add("down 5120x13824 + residual",
-        lambda i: nf4.nf4_gemv(d[i % 18][0], d[i % 18][1], xd, k5, ffn, ffn, yo, res),
+        lambda i: nf4.nf4_gemv(d[i % 18][0], d[i % 18][1], xd, k5, ffn, ffn, yo, res, sumsq_out=parts_out),
         algorithmic_bytes(k5, ffn) + 2 * k5)
     del d
     torch.cuda.empty_cache()
