@@ -109,6 +109,28 @@ __device__ __forceinline__ float block_sum(float v, float *part) {
   return s;
 }
 
+// sq_out at the end of a launch (every wavefront of the workgroup calls it): the wavefronts' sums
+// of squares meet in their own order, the workgroup stores its part, and zeros at the places
+// that no workgroup of this grid writes.
+__device__ __forceinline__ void store_sumsq_part(const StreamArgs &a, StagedLds &lds, float sq_acc,
+                                                 int wave, int lane) {
+  if (lane == 0) {
+    lds.part[wave] = sq_acc;
+  }
+  __syncthreads();
+  if (wave == 0 && lane == 0) {
+    float s = 0.f;
+    for (int w = 0; w < (kStagedThreads >> 6); ++w) {
+      s += lds.part[w];
+    }
+    const int block = static_cast<int>(blockIdx.x);
+    a.sq_out[block] = s;
+    for (int b = block + a.ring_grid; b < kSumsqParts; b += a.ring_grid) {
+      a.sq_out[b] = 0.f;
+    }
+  }
+}
+
 // ---- x as binary16 -------------------------------------------------------------------
 // With levels kept as binary16 (11 significant bits against bf16's 8) the products need x as
 // binary16 too.  A bf16 value has 8 significant bits, so it is a binary16 value exactly
@@ -995,6 +1017,7 @@ __global__ __launch_bounds__(1024) void gemv_staged(const StreamArgs a) {
   // compute cursor: half step ci of the list = step ct of group cg
   int ci = 0, cg = first, ct = 0;
   float acc[R] = {};
+  float sq_acc = 0.f;  // sq_out: sum of squares of what this wavefront has stored
 
   auto finish_group = [&](int grp) {
     int seg, row0, M;
@@ -1019,8 +1042,13 @@ __global__ __launch_bounds__(1024) void gemv_staged(const StreamArgs a) {
         if (add != nullptr) {
           v += uniform_bf16(add + min(r, M - 1));
         }
+        const uint16_t stored = f32_to_bf16(v);
         if (lane == u && r < M) {
-          y[r] = f32_to_bf16(v);
+          y[r] = stored;
+        }
+        if (a.sq_out != nullptr && r < M) {
+          const float rf = bf16_to_f32(stored);
+          sq_acc = fmaf(rf, rf, sq_acc);
         }
       }
     }
@@ -1066,6 +1094,11 @@ __global__ __launch_bounds__(1024) void gemv_staged(const StreamArgs a) {
   }
 #undef CHR_COMPUTE
 #undef CHR_REQUEST
+  if constexpr (!SWIGLU) {
+    if (a.sq_out != nullptr) {
+      store_sumsq_part(a, lds, sq_acc, wave, lane);
+    }
+  }
 }
 
 // ---- ring kernel: weight requests and their waits written by hand ----------------------
@@ -1618,22 +1651,7 @@ __device__ __forceinline__ void gemv_ring_body(const StreamArgs &a) {
   asm volatile("s_waitcnt vmcnt(0)" : "+s"(tok));
   if constexpr (!SEQ) {
     if (a.sq_out != nullptr) {
-      // the wavefronts' sums meet in their own order; the workgroup's part, and zeros at the
-      // places no workgroup writes
-      if (lane == 0) {
-        lds.part[wave] = sq_acc;
-      }
-      __syncthreads();
-      if (wave == 0 && lane == 0) {
-        float s = 0.f;
-        for (int w = 0; w < waves; ++w) {
-          s += lds.part[w];
-        }
-        a.sq_out[block] = s;
-        for (int b = block + grid; b < kSumsqParts; b += grid) {
-          a.sq_out[b] = 0.f;
-        }
-      }
+      store_sumsq_part(a, lds, sq_acc, wave, lane);
     }
   }
 #undef CHR_RING_REQUEST_LAST
@@ -1884,8 +1902,9 @@ int launch_stream(StreamArgs &a, int n_seg, bool staged, hipStream_t st) {
   if (a.sq_in != nullptr && !sumsq_in_ok(a, staged)) {
     return -8;
   }
-  if (a.sq_out != nullptr && !staged) {
-    return -8;  // only the ring kernel of single rows writes the parts (checked again below)
+  if (a.sq_out != nullptr && (!staged || SWIGLU || n_seg != 1 ||
+                              (reinterpret_cast<uintptr_t>(a.sq_out) & 3u) != 0)) {
+    return -8;  // the staged kernels of a single matrix write the parts
   }
   int total = 0;
   for (int i = 0; i < 3; ++i) {
@@ -1907,9 +1926,7 @@ int launch_stream(StreamArgs &a, int n_seg, bool staged, hipStream_t st) {
     a.ring_grid = grid;
     a.ring_passes = total / per_pass;
     a.ring_left = total % per_pass;
-    if (a.sq_out != nullptr &&
-        !(ring_ns > 0 && !SWIGLU && n_seg == 1 && grid <= kSumsqParts &&
-          (reinterpret_cast<uintptr_t>(a.sq_out) & 3u) == 0)) {
+    if (a.sq_out != nullptr && grid > kSumsqParts) {
       return -8;
     }
     if (ring_ns > 0) {
@@ -2104,12 +2121,12 @@ bool gemv_sumsq_out_ok(int M, int K, int K_pad, bool merges_attention) {
   if (merges_attention) {
     a.attn_state = reinterpret_cast<const float *>(&a);  // only tested against nullptr
   }
-  if (pick_family(a, M) != 1 || staged_rows_for_m(M, K_pad) != 1 || !ring_wanted() ||
-      ring_piece_steps(x_half_steps(K_pad)).steps == 0) {
+  if (pick_family(a, M) != 1) {
     return false;
   }
   const int waves = kStagedThreads / kWave;
-  return std::min(device_cu_count(), (M + waves - 1) / waves) <= kSumsqParts;
+  const int groups = (M + staged_rows_for_m(M, K_pad) - 1) / staged_rows_for_m(M, K_pad);
+  return std::min(device_cu_count(), (groups + waves - 1) / waves) <= kSumsqParts;
 }
 
 // Launch geometry of the N=1 path, reported by the planner: what chr_nf4_gemv launches for

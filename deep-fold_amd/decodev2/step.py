@@ -51,7 +51,7 @@ def _sumsq_handover(weights: DeviceWeights) -> bool:
     that writes it (prologue, o projection, down projection) to the launch that normalises it
     (q/k/v, gate/up, lm_head), which then skips its own sum over the workgroup (two barriers
     ahead of its first product: 0.7 us of a 7 us launch).  Every writer must be the last to
-    touch the stream (no separate bias add) and run on the kernel that leaves the sum.
+    touch the stream (no separate bias add) and run on a kernel that leaves the sum.
     ``CHR_DV2_SUMSQ=0`` keeps every launch summing for itself."""
     if os.environ.get("CHR_DV2_SUMSQ", "1") == "0":
         return False

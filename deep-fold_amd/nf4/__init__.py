@@ -381,8 +381,8 @@ def dv2_sumsq_parts() -> int:
 
 
 def dv2_sumsq_ok(M: int, K: int, K_pad: int, merges_attention: bool = False) -> bool:  # noqa: N803
-    """Whether a single-matrix GEMV of this shape runs on the kernel that can write
-    ``sumsq_out`` (it reads the environment switches a launch reads)."""
+    """Whether a single-matrix GEMV of this shape runs on a kernel that can write
+    ``sumsq_out`` (those that stage x in LDS; it reads the environment switches a launch reads)."""
     return bool(_load_ext().chr_dv2_sumsq_ok(int(M), int(K), int(K_pad), int(bool(merges_attention))))
 
 

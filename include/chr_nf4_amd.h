@@ -266,9 +266,10 @@ int chr_dv2_gemv_attn(const chr_nf4_dev_t *w, const float *state, int32_t n_q, i
  * many floats, the caller's), and the reader's wavefronts add the parts up themselves.  No
  * reference counterpart.
  *   sumsq_out (chr_dv2_gemv_sumsq, chr_dv2_gemv_attn_sumsq, chr_dv2_begin_step_sumsq): this
- *     launch writes the parts for its y (after `add`).  Only the GEMV kernel of single rows
- *     does: chr_dv2_sumsq_ok(M, K, K_pad, merges_attention) says whether a matrix of that shape
- *     runs on it (it reads the same environment switches a launch reads); else -8.
+ *     launch writes the parts for its y (after `add`).  Only the GEMV kernels that stage x in LDS
+ *     do (launches of 16 M codes and more, and every launch that merges attention states):
+ *     chr_dv2_sumsq_ok(M, K, K_pad, merges_attention) says whether a matrix of that shape runs
+ *     on one (it reads the same environment switches a launch reads); else -8.
  *   sumsq_in (chr_dv2_gemv_sumsq, chr_dv2_gemv_qkv_sumsq, chr_dv2_gemv_swiglu_sumsq): with
  *     rms_w, mean(x^2) comes from the parts that the writer of x left.  Needs K % 8 == 0 and
  *     x, rms_w and the parts 16-byte aligned; else -8.  The parts must be those of this x:

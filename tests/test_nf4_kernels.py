@@ -632,13 +632,18 @@ def parts_of(y, grid):
 
 
 @pytest.mark.parametrize("terms", [1, 3])
-@pytest.mark.parametrize("m,k,merges", [(5120, 13824, False), (5120, 5120, True), (2100, 8192, False),
-                                        (6144, 16384, False), (1040, 27648, False)])
-def test_gemv_leaves_the_sum_of_squares_of_what_it_stored(m, k, merges, terms, monkeypatch):
+@pytest.mark.parametrize("m,k,merges,ring", [
+    (5120, 13824, False, "1"), (5120, 5120, True, "1"), (2100, 8192, False, "1"), (6144, 16384, False, "1"),
+    (1040, 27648, False, "1"),
+    (5120, 5120, True, "0"), (2100, 8192, False, "0"),   # the compiler-pipelined kernel
+    (2048, 2048, True, "1"), (8200, 2048, False, "1"),   # rows of 2 half steps: no ring kernel takes them
+])
+def test_gemv_leaves_the_sum_of_squares_of_what_it_stored(m, k, merges, ring, terms, monkeypatch):
     """``sumsq_out``: the same y, bit for bit, and in the parts buffer the squares of the stored
     bf16 values, workgroup by workgroup, zeros behind them (whatever the buffer held before)."""
-    say("sumsq writer", m, k, merges, terms)
+    say("sumsq writer", m, k, merges, ring, terms)
     monkeypatch.setenv("CHR_NF4_GEMV_TERMS", str(terms))
+    monkeypatch.setenv("CHR_NF4_GEMV_RING", ring)
     assert nf4.dv2_sumsq_ok(m, k, k, merges)
     dp, ds = gpu_blobs(m, k, 71)
     res = bf16_tensor(np.random.default_rng(3).standard_normal(m).astype(np.float32))
@@ -665,8 +670,8 @@ def test_gemv_leaves_the_sum_of_squares_of_what_it_stored(m, k, merges, terms, m
 
 
 def test_sumsq_hand_over_is_refused_where_no_kernel_serves_it(monkeypatch):
-    """A shape the single-row ring kernel does not take (too few codes: the plain kernel; rows of
-    2 half steps), a reader without a norm, the ring switched off: error -8, nothing launched."""
+    """A launch of the plain kernel (too few codes for the kernels that stage x), a reader
+    without a norm, a launch forced onto the plain kernel: error -8, nothing launched."""
     parts = torch.zeros(nf4.dv2_sumsq_parts(), dtype=torch.float32, device=DEV)
     for m, k in [(300, 7168), (4096, 2048)]:
         assert not nf4.dv2_sumsq_ok(m, k, k)
@@ -680,7 +685,7 @@ def test_sumsq_hand_over_is_refused_where_no_kernel_serves_it(monkeypatch):
     dp, ds = gpu_blobs(m, k, 73)
     x = bf16_tensor(rand_x(k, None, 7))
     assert nf4.dv2_sumsq_ok(m, k, k)
-    monkeypatch.setenv("CHR_NF4_GEMV_RING", "0")
+    monkeypatch.setenv("CHR_NF4_GEMV_STAGED", "0")
     assert not nf4.dv2_sumsq_ok(m, k, k)
     with pytest.raises(RuntimeError, match="-8"):
         nf4.nf4_gemv(dp, ds, x, m, k, k, sumsq_out=parts)
