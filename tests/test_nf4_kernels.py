@@ -637,6 +637,8 @@ def parts_of(y, grid):
     (1040, 27648, False, "1"),
     (5120, 5120, True, "0"), (2100, 8192, False, "0"),   # the compiler-pipelined kernel
     (2048, 2048, True, "1"), (8200, 2048, False, "1"),   # rows of 2 half steps: no ring kernel takes them
+    (4099, 5120, False, "1"), (4099, 5120, False, "0"),  # a last workgroup pass that is not full
+    (300, 5120, True, "1"),                              # fewer workgroups than parts: zeros behind them
 ])
 def test_gemv_leaves_the_sum_of_squares_of_what_it_stored(m, k, merges, ring, terms, monkeypatch):
     """``sumsq_out``: the same y, bit for bit, and in the parts buffer the squares of the stored
@@ -695,7 +697,7 @@ def test_sumsq_hand_over_is_refused_where_no_kernel_serves_it(monkeypatch):
 
 @pytest.mark.parametrize("ring", ["1", "0"])
 @pytest.mark.parametrize("terms", [1, 3])
-@pytest.mark.parametrize("k", [5120, 6144, 2048])
+@pytest.mark.parametrize("k", [5120, 6144, 2048, 4000, 13824])
 def test_norm_folded_into_a_gemv_takes_the_sum_of_squares_it_is_handed(k, terms, ring, monkeypatch):
     """``sumsq_in``: q/k/v, gate/up and a single matrix normalise x with the sum the parts hold
     instead of summing x: with the parts of x itself the result is the launch's own to the last
@@ -723,13 +725,15 @@ def test_norm_folded_into_a_gemv_takes_the_sum_of_squares_it_is_handed(k, terms,
     dv, sv = gpu_blobs(mk, k, 77)
     bias = [bf16_tensor(rng.standard_normal(n).astype(np.float32)) for n in (mq, mk, mk)]
 
+    kp = oc.k_pad(k)
+
     def run(p):
         kw = {} if p is None else {"sumsq_in": p}
-        y = nf4.nf4_gemv(dp, ds, x, m, k, k, rms_w=g, **kw).reshape(-1).clone()
+        y = nf4.nf4_gemv(dp, ds, x, m, k, kp, rms_w=g, **kw).reshape(-1).clone()
         o = [torch.empty(n, dtype=torch.bfloat16, device=DEV) for n in (mq, mk, mk)]
-        nf4.nf4_qkv(dq, sq_, dk, sk, dv, sv, x, mq, mk, mk, k, k, *o, *bias, rms_w=g, **kw)
+        nf4.nf4_qkv(dq, sq_, dk, sk, dv, sv, x, mq, mk, mk, k, kp, *o, *bias, rms_w=g, **kw)
         s = torch.empty(mq, dtype=torch.bfloat16, device=DEV)
-        nf4.nf4_swiglu(dq, sq_, dp[:mq], ds[:mq], x, mq, k, k, s, rms_w=g, **kw)
+        nf4.nf4_swiglu(dq, sq_, dp[:mq], ds[:mq], x, mq, k, kp, s, rms_w=g, **kw)
         return [y, *o, s]
 
     base, handed, scaled = run(None), run(parts), run(parts * 4)
