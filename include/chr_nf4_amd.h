@@ -357,12 +357,18 @@ int chr_dv2_gemm_add(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N, 
 /* chr_dv2_gemm_add that also leaves, for the RMSNorm that reads y next, the column sums of
  * squares of the values it stored: with R = chr_dv2_sq_rows(N) = 1024 / N rows per block,
  * colsq[b * N + n] = sum over rows R b .. R b + R - 1 of y[row][n]^2 (fp32,
- * ceil(M / R) * N elements, no NULL).  The sums are taken in the split-K reduction, so they
- * exist only when the launch has one and N divides 256: returns 0 when colsq was written, 1
- * when the product was computed but colsq was not (the caller then normalises with
- * chr_dv2_rms_cols), a negative code as chr_dv2_gemm_add.  chr_dv2_sq_rows gives 0 for an N
- * that does not divide 1024.  No reference counterpart (the reference's prefill normalises
- * with a torch op, gpu/decodev2/prefill.py:58-133). */
+ * ceil(M / R) * N elements, no NULL).  The sums are taken where the stored values are made: in
+ * the tile that finishes its rows itself (32 and 64 columns) or in the split-K reduction, so
+ * they exist only when the launch runs one of the two and N divides 256: returns 0 when colsq
+ * was written, 1 when the product was computed but colsq was not (the caller then normalises
+ * with chr_dv2_rms_cols), a negative code as chr_dv2_gemm_add.  The two places add a block's
+ * squares in different orders (the tile by wavefront and lane, the reduction by row), each
+ * fixed: a launch repeats its bits, but which place a launch takes follows its plan (shape,
+ * chr_nf4_gemm_stream_policy, whether a row of arrival counts was left for its stream), so
+ * colsq, and through it single elements of the next RMSNorm's bf16 output, are reproducible
+ * for one plan and not across plans.  chr_dv2_sq_rows gives 0 for an N that does not divide
+ * 1024.  No reference counterpart (the reference's prefill normalises with a torch op,
+ * gpu/decodev2/prefill.py:58-133). */
 int chr_dv2_gemm_add_sq(const chr_nf4_dev_t *w, const void *x, void *y, int32_t N, float *ws,
                         int64_t ws_floats, const void *bias, const void *residual, float *colsq,
                         void *stream);
