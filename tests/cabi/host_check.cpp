@@ -10,6 +10,7 @@
 // Exit status 0 and a last line "host_check: OK" mean every check passed.
 #include <hip/hip_runtime_api.h>
 
+#include <algorithm>
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
@@ -215,6 +216,57 @@ void on_device() {
   EXPECT(e1 <= 1e-2, "gemv max-rel %.3e", e1);
   EXPECT(en <= 1e-2, "gemm max-rel %.3e", en);
   EXPECT(ew <= 1e-2, "gemm_ws max-rel %.3e", ew);
+
+  // The sum of squares handed from the launch that writes a vector to the launch that
+  // normalises it: the GEMV leaves the parts for its y (same y, bit for bit), a GEMV with a
+  // norm takes mean(x^2) from parts, and a launch that can serve neither says -8.
+  {
+    const int n_parts = chr_dv2_sumsq_parts();
+    EXPECT(n_parts >= 64 && n_parts % 4 == 0, "parts %d", n_parts);
+    float *dParts;
+    uint16_t *dG, *dY2;
+    HIP_OK(hipMalloc(&dParts, n_parts * 4));
+    HIP_OK(hipMalloc(&dG, K * 2));
+    HIP_OK(hipMalloc(&dY2, M * 2));
+    EXPECT(chr_dv2_sumsq_ok(M, K, K_pad, 0) == 1, "a ragged K runs on a kernel that stages x");
+    EXPECT(chr_dv2_gemv_sumsq(&w, dX1, dY2, stream, nullptr, nullptr, 0.f, nullptr, dParts) == 0,
+           "gemv with sumsq_out");
+    HIP_OK(hipStreamSynchronize(stream));
+    std::vector<float> parts(n_parts);
+    std::vector<uint16_t> y2(M);
+    HIP_OK(hipMemcpy(parts.data(), dParts, n_parts * 4, hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(y2.data(), dY2, M * 2, hipMemcpyDeviceToHost));
+    EXPECT(y2 == y1, "sumsq_out changed y");
+    double left = 0.0, want = 0.0;
+    for (float v : parts) left += v;
+    for (uint16_t v : y2) want += (double)bf16_to_float(v) * bf16_to_float(v);
+    EXPECT(std::fabs(left - want) <= 1e-5 * want, "parts add up to %.6g, y^2 to %.6g", left, want);
+
+    std::vector<uint16_t> g(K, float_to_bf16(1.0f));
+    double xx = 0.0;
+    for (uint16_t v : x1) xx += (double)bf16_to_float(v) * bf16_to_float(v);
+    std::fill(parts.begin(), parts.end(), 0.f);
+    parts[0] = (float)xx;
+    HIP_OK(hipMemcpy(dG, g.data(), K * 2, hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(dParts, parts.data(), n_parts * 4, hipMemcpyHostToDevice));
+    EXPECT(chr_nf4_gemv(&w, dX1, dY1, stream, nullptr, dG, 1e-6f) == 0, "gemv with a norm");
+    EXPECT(chr_dv2_gemv_sumsq(&w, dX1, dY2, stream, nullptr, dG, 1e-6f, dParts, nullptr) == 0,
+           "gemv with a norm and sumsq_in");
+    HIP_OK(hipStreamSynchronize(stream));
+    std::vector<uint16_t> ya(M), yb(M);
+    HIP_OK(hipMemcpy(ya.data(), dY1, M * 2, hipMemcpyDeviceToHost));
+    HIP_OK(hipMemcpy(yb.data(), dY2, M * 2, hipMemcpyDeviceToHost));
+    double peak = 0.0, apart = 0.0;
+    for (int r = 0; r < M; ++r) {
+      peak = std::fmax(peak, std::fabs(bf16_to_float(ya[r])));
+      apart = std::fmax(apart, std::fabs(bf16_to_float(ya[r]) - bf16_to_float(yb[r])));
+    }
+    EXPECT(peak > 0.0 && apart <= peak / 128, "handed sum: %.3g apart at a peak of %.3g", apart, peak);
+    EXPECT(chr_dv2_gemv_sumsq(&w, dX1, dY2, stream, nullptr, nullptr, 0.f, dParts, nullptr) == -8,
+           "sumsq_in without a norm");
+    HIP_OK(hipStreamSynchronize(stream));
+    for (void *p : {(void *)dParts, (void *)dG, (void *)dY2}) HIP_OK(hipFree(p));
+  }
 
   // Refusals that must come back as codes, not as faults.
   EXPECT(chr_nf4_gemm(&w, dXn, dYn, 33, stream) == -2, "N=33 has no tile");
